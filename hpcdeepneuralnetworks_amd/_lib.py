@@ -1,0 +1,110 @@
+"""ctypes binding of ``libhpcdnn.so`` (the C ABI declared in ``include/hpcdnn.h``).
+
+There is no CPU fallback: if the library has not been built, or a call returns
+a non-zero status, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libhpcdnn.so")
+CSRC = os.path.join(_PKG, "csrc")
+
+OP_SGEMM = 0
+OP_SDOT = 1
+FT_TILE_M = 256
+FT_TILE_N = 128
+
+# every symbol include/hpcdnn.h declares
+EXPORTS = (
+    "hpcdnn_version",
+    "hpcdnn_error_string",
+    "hpcdnn_sgemm",
+    "hpcdnn_sgemm_ex",
+    "hpcdnn_sgemm_num_tiles",
+    "hpcdnn_sgemm_tile_info",
+    "hpcdnn_ft_sgemm",
+    "hpcdnn_ft_num_tiles",
+    "hpcdnn_ft_default_tau",
+    "hpcdnn_saxpy",
+    "hpcdnn_sdot",
+    "hpcdnn_workspace_bytes",
+    "hpcdnn_workspace_init",
+    "hpcdnn_fill_uniform",
+    "hpcdnn_fill_uniform_matrix",
+    "hpcdnn_cpu_gemm",
+)
+
+
+class Fault(C.Structure):
+    _fields_ = [("tile", C.c_int32), ("row", C.c_int32), ("col", C.c_int32), ("delta", C.c_float)]
+
+
+class HpcdnnError(RuntimeError):
+    pass
+
+
+def build(jobs: int = 8) -> str:
+    """Compile the HIP sources for gfx950 (cross-compiles without a GPU) into ``lib/libhpcdnn.so``."""
+    subprocess.run(["make", "-C", CSRC, f"-j{jobs}"], check=True)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HpcdnnError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            f"or `make -C {CSRC}`; there is no CPU fallback"
+        )
+    L = C.CDLL(LIB_PATH)
+    vp, fp, i, f, sz, i64, u64 = C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_int64, C.c_uint64
+    L.hpcdnn_version.restype = C.c_char_p
+    L.hpcdnn_version.argtypes = []
+    L.hpcdnn_error_string.restype = C.c_char_p
+    L.hpcdnn_error_string.argtypes = [i]
+    L.hpcdnn_sgemm.restype = i
+    L.hpcdnn_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, vp, sz, vp]
+    L.hpcdnn_sgemm_ex.restype = i
+    L.hpcdnn_sgemm_ex.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, vp, sz, i, i, vp]
+    L.hpcdnn_sgemm_num_tiles.restype = i
+    L.hpcdnn_sgemm_num_tiles.argtypes = []
+    L.hpcdnn_sgemm_tile_info.restype = i
+    L.hpcdnn_sgemm_tile_info.argtypes = [i, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
+    L.hpcdnn_ft_sgemm.restype = i
+    L.hpcdnn_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp]
+    L.hpcdnn_ft_num_tiles.restype = i
+    L.hpcdnn_ft_num_tiles.argtypes = [i, i]
+    L.hpcdnn_ft_default_tau.restype = f
+    L.hpcdnn_ft_default_tau.argtypes = [i]
+    L.hpcdnn_saxpy.restype = i
+    L.hpcdnn_saxpy.argtypes = [i64, f, fp, fp, vp]
+    L.hpcdnn_sdot.restype = i
+    L.hpcdnn_sdot.argtypes = [i64, fp, fp, fp, vp, sz, vp]
+    L.hpcdnn_workspace_bytes.restype = sz
+    L.hpcdnn_workspace_bytes.argtypes = [i, i, i, i]
+    L.hpcdnn_workspace_init.restype = i
+    L.hpcdnn_workspace_init.argtypes = [vp, sz, vp]
+    L.hpcdnn_fill_uniform.restype = i
+    L.hpcdnn_fill_uniform.argtypes = [fp, i64, u64, vp]
+    L.hpcdnn_fill_uniform_matrix.restype = i
+    L.hpcdnn_fill_uniform_matrix.argtypes = [fp, i, i, i, u64, vp]
+    L.hpcdnn_cpu_gemm.restype = None
+    L.hpcdnn_cpu_gemm.argtypes = [f, f, vp, vp, i, vp]
+    _lib = L
+    return L
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = lib().hpcdnn_error_string(code).decode()
+        raise HpcdnnError(f"{what} failed: {msg} (code {code})")

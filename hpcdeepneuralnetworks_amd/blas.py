@@ -1,0 +1,176 @@
+"""Host-side mirror of the reference's entry points, on torch device tensors.
+
+The reference's "API" is a set of ``__global__`` kernels launched from its
+drivers with arguments ``(dims, A, B, C, alpha, beta)`` / ``(n, alpha, x, y)`` /
+``(n, x, y, out)``.  The functions here keep those names and that argument
+order, take FP32 CUDA(HIP) tensors in place of raw device pointers, and call
+the C ABI of ``libhpcdnn.so`` on torch's current stream.  torch only provides
+device memory and streams; all arithmetic is in the HIP library.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import FT_TILE_M, FT_TILE_N, Fault, HpcdnnError, check
+
+FT_STATUS_DTYPE = np.dtype(
+    [
+        ("flag", "<i4"),
+        ("row", "<i4"),
+        ("col", "<i4"),
+        ("n_bad_rows", "<i4"),
+        ("n_bad_cols", "<i4"),
+        ("row_residual", "<f4"),
+        ("col_residual", "<f4"),
+        ("max_clean_residual", "<f4"),
+    ]
+)
+
+_sdot_ws: dict = {}
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, name: str) -> int:
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32):
+        raise HpcdnnError(f"{name} must be a float32 tensor on the GPU")
+    return t.data_ptr()
+
+
+def _matrix(t: torch.Tensor, rows: int, cols: int, name: str):
+    """Pointer and leading dimension of a row-major (possibly row-strided) 2-D view."""
+    ptr = _dev(t, name)
+    if t.dim() != 2 or t.shape[0] < rows or t.shape[1] < cols:
+        raise HpcdnnError(f"{name} must be 2-D with at least {rows}x{cols} elements, got {tuple(t.shape)}")
+    if t.shape[1] > 1 and t.stride(1) != 1:
+        raise HpcdnnError(f"{name} must be row-major (unit stride along columns)")
+    ld = t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+    return ptr, max(int(ld), 1)
+
+
+def workspace(nbytes: int, device=None) -> torch.Tensor:
+    """A zero-initialised scratch buffer (zeroed by the library's own fill kernel)."""
+    ws = torch.empty(max((nbytes + 3) // 4, 1), dtype=torch.int32, device=device or "cuda")
+    check(_lib.lib().hpcdnn_workspace_init(ws.data_ptr(), ws.numel() * 4, _stream()), "hpcdnn_workspace_init")
+    return ws
+
+
+def sgemm_workspace_bytes(M: int, N: int, K: int) -> int:
+    return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_SGEMM, M, N, K))
+
+
+def tile_table():
+    L = _lib.lib()
+    out = []
+    for t in range(L.hpcdnn_sgemm_num_tiles()):
+        bm, bn, bk = C.c_int(), C.c_int(), C.c_int()
+        check(L.hpcdnn_sgemm_tile_info(t, C.byref(bm), C.byref(bn), C.byref(bk)), "hpcdnn_sgemm_tile_info")
+        out.append((bm.value, bn.value, bk.value))
+    return out
+
+
+def sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
+          ws: torch.Tensor | None = None, tile: int = -1, split_k: int = 0) -> None:
+    """In place ``C = alpha*A@B + beta*C`` (row-major; leading dimensions are the tensors' row strides).
+
+    Counterpart of ``sgemm_k<<<...>>>(N, A, B, C, alpha, beta)`` (kernel/sgemm/sgemm.cu:120-141) and
+    ``sgemm_<shape><<<...>>>(M, N, K, A, B, C, alpha, beta)`` (kernel/ft_sgemm/sgemm.cu:114-157).
+    """
+    pa, lda = _matrix(A, M, K, "A")
+    pb, ldb = _matrix(B, K, N, "B")
+    pc, ldc = _matrix(Cm, M, N, "C")
+    wsp, wsb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
+    L = _lib.lib()
+    if tile < 0 and split_k == 0:
+        rc = L.hpcdnn_sgemm(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, wsp, wsb, _stream())
+    else:
+        rc = L.hpcdnn_sgemm_ex(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, wsp, wsb, tile, split_k, _stream())
+    check(rc, "hpcdnn_sgemm")
+
+
+def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
+             tau: float = 0.0, fault=None, status: torch.Tensor | None = None) -> None:
+    """ABFT GEMM; ``fault`` = (tile, row, col, delta) or None; ``status`` = int32 tensor of 8*ft_num_tiles words.
+
+    Counterpart of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)`` (kernel/ft_sgemm/sgemm.cu:159-165).
+    """
+    pa, lda = _matrix(A, M, K, "A")
+    pb, ldb = _matrix(B, K, N, "B")
+    pc, ldc = _matrix(Cm, M, N, "C")
+    L = _lib.lib()
+    sp = None
+    if status is not None:
+        need = 8 * L.hpcdnn_ft_num_tiles(M, N)
+        if not (status.is_cuda and status.dtype == torch.int32 and status.numel() >= need and status.is_contiguous()):
+            raise HpcdnnError(f"status must be a contiguous int32 GPU tensor with >= {need} elements")
+        sp = status.data_ptr()
+    f = None
+    if fault is not None:
+        f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
+    check(L.hpcdnn_ft_sgemm(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, f, sp, _stream()), "hpcdnn_ft_sgemm")
+
+
+def ft_num_tiles(M: int, N: int) -> int:
+    return int(_lib.lib().hpcdnn_ft_num_tiles(M, N))
+
+
+def ft_default_tau(K: int) -> float:
+    return float(_lib.lib().hpcdnn_ft_default_tau(K))
+
+
+def ft_status_alloc(M: int, N: int, device=None) -> torch.Tensor:
+    return torch.zeros(8 * ft_num_tiles(M, N), dtype=torch.int32, device=device or "cuda")
+
+
+def ft_status_numpy(status: torch.Tensor) -> np.ndarray:
+    return status.cpu().numpy().view(FT_STATUS_DTYPE)
+
+
+def saxpy(n: int, alpha: float, x: torch.Tensor, y: torch.Tensor) -> None:
+    """In place ``y = alpha*x + y`` (one FMA per element).  Counterpart of kernel/saxpy/saxpy.cu:38-48."""
+    px, py = _dev(x, "x"), _dev(y, "y")
+    if x.numel() < n or y.numel() < n or not (x.is_contiguous() and y.is_contiguous()):
+        raise HpcdnnError("x and y must be contiguous with at least n elements")
+    check(_lib.lib().hpcdnn_saxpy(n, alpha, px, py, _stream()), "hpcdnn_saxpy")
+
+
+def sdot(n: int, x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, ws: torch.Tensor | None = None) -> None:
+    """``out[0] = sum(x*y)`` on the device, deterministic.  Counterpart of kernel/sdot/sdot.cu:9-36."""
+    px, py, po = _dev(x, "x"), _dev(y, "y"), _dev(out, "out")
+    if x.numel() < n or y.numel() < n or not (x.is_contiguous() and y.is_contiguous()):
+        raise HpcdnnError("x and y must be contiguous with at least n elements")
+    if ws is None:
+        key = (out.device.index, _stream())
+        ws = _sdot_ws.get(key)
+        if ws is None:
+            ws = workspace(int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_SDOT, 0, 0, 0)), out.device)
+            _sdot_ws[key] = ws
+    check(_lib.lib().hpcdnn_sdot(n, px, py, po, ws.data_ptr(), ws.numel() * 4, _stream()), "hpcdnn_sdot")
+
+
+def fill_uniform(dst: torch.Tensor, seed: int) -> None:
+    """Seeded uniform[-1,1) fill of a contiguous vector (device-side generate_random_vector, utils/utils.cu:28-35)."""
+    p = _dev(dst, "dst")
+    if not dst.is_contiguous():
+        raise HpcdnnError("dst must be contiguous")
+    check(_lib.lib().hpcdnn_fill_uniform(p, dst.numel(), seed, _stream()), "hpcdnn_fill_uniform")
+
+
+def fill_uniform_matrix(dst: torch.Tensor, rows: int, cols: int, seed: int) -> None:
+    """Seeded fill of the leading rows x cols block of a row-major 2-D tensor (utils/utils.cu:37-44)."""
+    p, ld = _matrix(dst, rows, cols, "dst")
+    check(_lib.lib().hpcdnn_fill_uniform_matrix(p, rows, cols, ld, seed, _stream()), "hpcdnn_fill_uniform_matrix")
+
+
+def cpu_gemm(alpha: float, beta: float, mat1: np.ndarray, mat2: np.ndarray, n: int, mat3: np.ndarray) -> None:
+    """The reference's host validator (utils/utils.cu:93-103) on numpy float32 arrays, in place on ``mat3``."""
+    for a in (mat1, mat2, mat3):
+        if not (isinstance(a, np.ndarray) and a.dtype == np.float32 and a.flags.c_contiguous and a.size >= n * n):
+            raise HpcdnnError("cpu_gemm takes C-contiguous float32 numpy arrays of n*n elements")
+    _lib.lib().hpcdnn_cpu_gemm(alpha, beta, mat1.ctypes.data, mat2.ctypes.data, n, mat3.ctypes.data)

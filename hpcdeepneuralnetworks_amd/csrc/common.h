@@ -1,0 +1,75 @@
+// Shared device/host helpers for the gfx950 kernels (wave64 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hpcdnn.h"
+
+namespace hpcdnn {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return (e == hipSuccess) ? HPCDNN_OK : static_cast<int>(e);
+}
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- counter-based RNG: splitmix64 finaliser of seed*golden + index ------
+__host__ __device__ inline uint64_t mix64(uint64_t z) {
+    z ^= z >> 30; z *= 0xBF58476D1CE4E5B9ull;
+    z ^= z >> 27; z *= 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return z;
+}
+
+__host__ __device__ inline float uniform_pm1(uint64_t seed, uint64_t idx) {
+    uint64_t z = mix64(seed * 0x9E3779B97F4A7C15ull + idx + 0x632BE59BD9B4E019ull);
+    int32_t v = static_cast<int32_t>(z >> 40) - (1 << 23);
+    return static_cast<float>(v) * (1.0f / 8388608.0f);
+}
+
+// ---- cross-lane primitives (DPP / swizzle; no LDS traffic) ----------------
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i inside each 8
+constexpr int kDppMirror = 0x140;     // lane i <-> 15-i inside each 16
+constexpr int kDppBcast15 = 0x142;    // lane 15 of each row -> next row
+constexpr int kDppBcast31 = 0x143;    // lane 31 -> rows 2,3
+
+// Sum over the 16 lanes of each DPP row; every lane of the row gets the sum.
+__device__ __forceinline__ float row16_allsum(float v) {
+    v += dpp_mov<kDppXor1>(v);
+    v += dpp_mov<kDppXor2>(v);
+    v += dpp_mov<kDppHalfMirror>(v);
+    v += dpp_mov<kDppMirror>(v);
+    return v;
+}
+
+// Sum over each 32-lane half of the wave; every lane of the half gets the sum.
+__device__ __forceinline__ float half32_allsum(float v) {
+    v = row16_allsum(v);
+    // swap with lane ^ 16: bit-mask swizzle, and=0x1f or=0 xor=0x10
+    v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+    return v;
+}
+
+// Sum over the whole wave; the total is valid in lane 63 only.
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+    v = row16_allsum(v);
+    v += dpp_mov<kDppBcast15, 0xa>(v);
+    v += dpp_mov<kDppBcast31, 0xc>(v);
+    return v;
+}
+
+}  // namespace hpcdnn

@@ -1,0 +1,253 @@
+// SGEMM / ABFT-SGEMM entry points: argument checks, tile + split-K choice, launch.
+#include "sgemm_kernel.h"
+
+#include <mutex>
+
+namespace hpcdnn {
+
+struct TileConfig {
+    int bm, bn, bk;
+    int blocks_per_cu;  // resident workgroups per CU the kernel is built for
+    size_t lds_bytes;
+    void (*plain)(const GemmArgs);
+    void (*edge)(const GemmArgs);
+    float rel_speed;  // measured steady-state throughput relative to the best configuration
+};
+
+#define HPCDNN_TILE(BM, BN, BK, WGM, WGN, STAGES, OCC, SPEED)                                   \
+    {                                                                                            \
+        BM, BN, BK, OCC, gemm_lds_bytes<BM, BN, BK, STAGES>(),                                   \
+            sgemm_kernel<BM, BN, BK, WGM, WGN, STAGES, false, false, OCC>,                       \
+            sgemm_kernel<BM, BN, BK, WGM, WGN, STAGES, true, false, OCC>, SPEED                  \
+    }
+
+// The counterpart of the reference's small/medium/large/tall/wide/huge shape
+// table (kernel/ft_sgemm/code_gen/main.py:8-16), re-derived for 32x32 MFMA
+// blocks and four 64-lane waves per workgroup.
+static const TileConfig kTiles[] = {
+    HPCDNN_TILE(256, 128, 16, 2, 2, 2, 2, 1.00f),  // 0 huge
+    HPCDNN_TILE(128, 128, 16, 2, 2, 2, 2, 0.90f),  // 1 large
+    HPCDNN_TILE(128, 64, 16, 2, 2, 2, 2, 0.75f),   // 2 tall
+    HPCDNN_TILE(64, 128, 16, 2, 2, 2, 2, 0.75f),   // 3 wide
+    HPCDNN_TILE(64, 64, 16, 2, 2, 2, 4, 0.55f),    // 4 medium
+    HPCDNN_TILE(256, 128, 32, 2, 2, 2, 1, 1.00f),  // 5 huge, deep K step
+    HPCDNN_TILE(256, 256, 16, 2, 2, 2, 1, 1.00f),  // 6 giant
+    HPCDNN_TILE(192, 256, 16, 2, 2, 2, 1, 1.00f),  // 7 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
+};
+constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
+
+constexpr int kFtTile = 0;  // 256 x 128, matches HPCDNN_FT_TILE_M/N
+static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, 16, 2, 2, 2, false, true, 2>;
+static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, 16, 2, 2, 2, true, true, 2>;
+
+static int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            cus = v;
+        else
+            return 256;
+    }
+    return cus;
+}
+
+// Kernels that use more than the default 64 KiB of LDS must opt in once.
+static int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {
+    if (bytes <= 64 * 1024) return HPCDNN_OK;
+    static std::mutex mu;
+    static const void* done[4 * kNumTiles] = {};
+    std::lock_guard<std::mutex> lock(mu);
+    const void* key = reinterpret_cast<const void*>(fn);
+    for (const void* d : done)
+        if (d == key) return HPCDNN_OK;
+    hipError_t e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+    if (e != hipSuccess) return static_cast<int>(e);
+    for (const void*& d : done)
+        if (!d) { d = key; break; }
+    return HPCDNN_OK;
+}
+
+struct Plan {
+    int tile;
+    int split;
+};
+
+static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int cus) {
+    const double tiles = static_cast<double>(ceil_div(M, t.bm)) * ceil_div(N, t.bn) * split;
+    const double slots = static_cast<double>(cus) * t.blocks_per_cu;
+    const double rounds = ceil(tiles / slots);
+    // time of one round: a resident set of blocks_per_cu workgroups shares the CU's matrix cores
+    const double k_slice = ceil(static_cast<double>(ceil_div(K, split)) / t.bk) * t.bk;
+    const double per_tile = static_cast<double>(t.bm) * t.bn * (k_slice + 64.0);  // + prologue/epilogue in k-equivalents
+    double cost = rounds * per_tile * t.blocks_per_cu / t.rel_speed;
+    if (split > 1) cost += 3.0 * M * static_cast<double>(N) * split / cus * 8.0;  // partial write + ordered re-read
+    return cost;
+}
+
+static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes) {
+    const int cus = device_cus();
+    Plan best{0, 1};
+    double best_cost = 1e300;
+    for (int t = 0; t < kNumTiles; ++t) {
+        const TileConfig& cfg = kTiles[t];
+        for (int split = 1; split <= 64; split *= 2) {
+            if (split > 1) {
+                if (!allow_split) break;
+                if (ceil_div(K, split) < 4 * cfg.bk) break;
+                if (static_cast<size_t>(M) * N * split * sizeof(float) > ws_bytes) break;
+            }
+            const double c = plan_cost(cfg, M, N, K, split, cus);
+            if (c < best_cost) { best_cost = c; best = Plan{t, split}; }
+        }
+    }
+    return best;
+}
+
+static int check_gemm_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+    if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
+    if (lda < (K > 1 ? K : 1) || ldb < (N > 1 ? N : 1) || ldc < (N > 1 ? N : 1)) return HPCDNN_ERR_INVALID_VALUE;
+    if (M > 0 && N > 0 && !C) return HPCDNN_ERR_INVALID_VALUE;
+    if (M > 0 && N > 0 && K > 0 && (!A || !B)) return HPCDNN_ERR_INVALID_VALUE;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) & 3u)
+        return HPCDNN_ERR_INVALID_VALUE;
+    return HPCDNN_OK;
+}
+
+static GemmArgs make_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                          float alpha, float beta, const TileConfig& cfg) {
+    GemmArgs a{};
+    a.M = M; a.N = N; a.K = K;
+    a.A = A; a.lda = lda; a.B = B; a.ldb = ldb; a.C = C; a.ldc = ldc;
+    a.alpha = alpha; a.beta = beta;
+    a.tiles_m = static_cast<int>(ceil_div(M, cfg.bm));
+    a.tiles_n = static_cast<int>(ceil_div(N, cfg.bn));
+    a.k_chunk = static_cast<int>(ceil_div(K > 0 ? K : 1, cfg.bk)) * cfg.bk;
+    a.partial = nullptr;
+    a.vec_a = ((reinterpret_cast<uintptr_t>(A) & 15u) == 0 && lda % 4 == 0) ? 1 : 0;
+    a.vec_b = ((reinterpret_cast<uintptr_t>(B) & 15u) == 0 && ldb % 4 == 0) ? 1 : 0;
+    a.fault_tile = -1;
+    return a;
+}
+
+static bool needs_edge(const GemmArgs& a, const TileConfig& cfg, int k_slice_len_multiple_of_bk) {
+    return !(a.M % cfg.bm == 0 && a.N % cfg.bn == 0 && a.K % cfg.bk == 0 && k_slice_len_multiple_of_bk && a.vec_a && a.vec_b);
+}
+
+static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                     float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split, hipStream_t stream) {
+    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
+    if (rc != HPCDNN_OK) return rc;
+    if (tile >= kNumTiles || split < 0) return HPCDNN_ERR_INVALID_VALUE;
+    if (M == 0 || N == 0) return HPCDNN_OK;
+
+    if (tile < 0 || split == 0) {
+        Plan plan = choose_plan(M, N, K, ws != nullptr, ws ? ws_bytes : 0);
+        if (tile < 0) {
+            tile = plan.tile;
+            if (split == 0) split = plan.split;
+        } else if (split == 0) {
+            split = 1;
+        }
+    }
+    const TileConfig& cfg = kTiles[tile];
+    if (split > 1) {
+        if (!ws || static_cast<size_t>(M) * N * split * sizeof(float) > ws_bytes) return HPCDNN_ERR_WORKSPACE;
+        if (reinterpret_cast<uintptr_t>(ws) & 3u) return HPCDNN_ERR_INVALID_VALUE;
+    }
+
+    GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
+    if (split > 1) {
+        a.k_chunk = static_cast<int>(ceil_div(ceil_div(K, split), cfg.bk)) * cfg.bk;
+        split = static_cast<int>(ceil_div(K, a.k_chunk));  // drop empty slices
+        if (split > 1) a.partial = static_cast<float*>(ws);
+    }
+    const bool edge = needs_edge(a, cfg, 1);
+    void (*fn)(const GemmArgs) = edge ? cfg.edge : cfg.plain;
+    rc = enable_lds(fn, cfg.lds_bytes);
+    if (rc != HPCDNN_OK) return rc;
+
+    dim3 grid(a.tiles_m * a.tiles_n, 1, split);
+    hipLaunchKernelGGL(fn, grid, dim3(kGemmThreads), cfg.lds_bytes, stream, a);
+    rc = launch_status();
+    if (rc != HPCDNN_OK || split == 1) return rc;
+
+    const int64_t total = static_cast<int64_t>(M) * N;
+    int rgrid = static_cast<int>(ceil_div(total, 256));
+    const int cap = device_cus() * 8;
+    if (rgrid > cap) rgrid = cap;
+    splitk_reduce_kernel<<<rgrid, 256, 0, stream>>>(M, N, split, static_cast<const float*>(ws), C, ldc, alpha, beta);
+    return launch_status();
+}
+
+}  // namespace hpcdnn
+
+using namespace hpcdnn;
+
+extern "C" int hpcdnn_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                            float alpha, float beta, void* ws, size_t ws_bytes, void* stream) {
+    return run_sgemm(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, ws, ws_bytes, -1, 0, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                               float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split_k, void* stream) {
+    return run_sgemm(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, ws, ws_bytes, tile, split_k,
+                     static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hpcdnn_sgemm_num_tiles(void) { return kNumTiles; }
+
+extern "C" int hpcdnn_sgemm_tile_info(int tile, int* bm, int* bn, int* bk) {
+    if (tile < 0 || tile >= kNumTiles) return HPCDNN_ERR_INVALID_VALUE;
+    if (bm) *bm = kTiles[tile].bm;
+    if (bn) *bn = kTiles[tile].bn;
+    if (bk) *bk = kTiles[tile].bk;
+    return HPCDNN_OK;
+}
+
+extern "C" int hpcdnn_ft_num_tiles(int M, int N) {
+    if (M < 0 || N < 0) return 0;
+    return static_cast<int>(ceil_div(M, HPCDNN_FT_TILE_M) * ceil_div(N, HPCDNN_FT_TILE_N));
+}
+
+extern "C" float hpcdnn_ft_default_tau(int K) {
+    (void)K;
+    return 4e-3f;
+}
+
+extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                               float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
+                               void* stream) {
+    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
+    if (rc != HPCDNN_OK) return rc;
+    if (M == 0 || N == 0) return HPCDNN_OK;
+    const TileConfig& cfg = kTiles[kFtTile];
+    GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
+    a.tau = (tau > 0.f) ? tau : hpcdnn_ft_default_tau(K);
+    a.status = status;
+    if (inject) {
+        if (inject->tile < 0 || inject->tile >= a.tiles_m * a.tiles_n || inject->row < 0 ||
+            inject->row >= HPCDNN_FT_TILE_M || inject->col < 0 || inject->col >= HPCDNN_FT_TILE_N)
+            return HPCDNN_ERR_INVALID_VALUE;
+        a.fault_tile = inject->tile;
+        a.fault_row = inject->row;
+        a.fault_col = inject->col;
+        a.fault_delta = inject->delta;
+    }
+    const bool edge = needs_edge(a, cfg, 1);
+    void (*fn)(const GemmArgs) = edge ? kFtEdge : kFtPlain;
+    rc = enable_lds(fn, cfg.lds_bytes);
+    if (rc != HPCDNN_OK) return rc;
+    dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
+    hipLaunchKernelGGL(fn, grid, dim3(kGemmThreads), cfg.lds_bytes, stream ? static_cast<hipStream_t>(stream) : nullptr, a);
+    return launch_status();
+}
+
+namespace hpcdnn {
+size_t sgemm_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    Plan plan = choose_plan(M, N, K, true, static_cast<size_t>(-1));
+    return plan.split > 1 ? static_cast<size_t>(M) * N * plan.split * sizeof(float) : 0;
+}
+}  // namespace hpcdnn

@@ -1,0 +1,275 @@
+// SAXPY, SDOT and the seeded fill kernels: HBM-bandwidth-bound streams.
+//
+// Layout: contiguous FP32 vectors.  Algorithmic traffic: SAXPY 12 B/element
+// (two loads, one store), SDOT 8 B/element (two loads).  Both kernels are
+// grid-stride over 16-byte lanes with several independent loads in flight per
+// lane; the grid is sized to the device (CUs x resident blocks), not to n.
+#include "common.h"
+
+namespace hpcdnn {
+
+constexpr int kVecThreads = 256;
+
+// ------------------------------------------------------------------ SAXPY --
+// Stands in for saxpy / saxpy3 / _saxpy (kernel/saxpy/saxpy.cu:15-48).  The
+// reference's f128 kernels need n % 4 == 0; here the n % 4 tail is done by the
+// first lanes of block 0 and misaligned vectors take the dword kernel.
+template <int UNROLL>
+__global__ __launch_bounds__(kVecThreads) void saxpy_vec4_kernel(int64_t n, float alpha, const float* __restrict__ x,
+                                                                 float* __restrict__ y) {
+    const int64_t n4 = n >> 2;
+    const v4f* __restrict__ x4 = reinterpret_cast<const v4f*>(x);
+    v4f* __restrict__ y4 = reinterpret_cast<v4f*>(y);
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
+    int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x;
+
+    for (; i + (UNROLL - 1) * stride < n4; i += UNROLL * stride) {
+        v4f xv[UNROLL], yv[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) xv[u] = __builtin_nontemporal_load(&x4[i + u * stride]);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) yv[u] = __builtin_nontemporal_load(&y4[i + u * stride]);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            v4f r;
+            r.x = __builtin_fmaf(alpha, xv[u].x, yv[u].x);
+            r.y = __builtin_fmaf(alpha, xv[u].y, yv[u].y);
+            r.z = __builtin_fmaf(alpha, xv[u].z, yv[u].z);
+            r.w = __builtin_fmaf(alpha, xv[u].w, yv[u].w);
+            __builtin_nontemporal_store(r, &y4[i + u * stride]);
+        }
+    }
+    for (; i < n4; i += stride) {
+        v4f xv = x4[i], yv = y4[i], r;
+        r.x = __builtin_fmaf(alpha, xv.x, yv.x);
+        r.y = __builtin_fmaf(alpha, xv.y, yv.y);
+        r.z = __builtin_fmaf(alpha, xv.z, yv.z);
+        r.w = __builtin_fmaf(alpha, xv.w, yv.w);
+        y4[i] = r;
+    }
+    if (blockIdx.x == 0) {
+        const int64_t t = (n4 << 2) + threadIdx.x;
+        if (t < n) y[t] = __builtin_fmaf(alpha, x[t], y[t]);
+    }
+}
+
+__global__ __launch_bounds__(kVecThreads) void saxpy_dword_kernel(int64_t n, float alpha, const float* __restrict__ x,
+                                                                  float* __restrict__ y) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x; i < n; i += stride)
+        y[i] = __builtin_fmaf(alpha, x[i], y[i]);
+}
+
+// ------------------------------------------------------------------- SDOT --
+// Stands in for _sdot (grid-stride + shared-memory tree + float atomicAdd,
+// kernel/sdot/sdot.cu:9-36) and for the sdot + reduction multi-launch chain
+// (:38-67).  One launch, no float atomics: every block writes one partial,
+// takes a ticket, and the block that draws the last ticket adds the partials
+// in index order, so the result is reproducible bit for bit.
+//
+// Workspace layout: [0] ticket (uint32, zero between calls), [64..] one double
+// per block.
+constexpr int kSdotMaxBlocks = 4096;
+constexpr size_t kSdotPartialOffset = 64;
+
+__device__ __forceinline__ double block_sum_to_thread0(double v, double* lds) {
+    // lanes -> wave via bpermute shuffles (tail of the kernel, not hot)
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, kWave);
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
+    __syncthreads();
+    double s = 0.0;
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 0; w < kVecThreads / kWave; ++w) s += lds[w];
+    }
+    return s;
+}
+
+template <int UNROLL, bool VEC>
+__global__ __launch_bounds__(kVecThreads) void sdot_kernel(int64_t n, const float* __restrict__ x,
+                                                           const float* __restrict__ y, float* __restrict__ out,
+                                                           unsigned int* ticket, double* partials) {
+    __shared__ double lds[kVecThreads / kWave];
+    __shared__ bool is_last;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
+    int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x;
+    float acc[UNROLL][4];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) acc[u][0] = acc[u][1] = acc[u][2] = acc[u][3] = 0.0f;
+
+    if (VEC) {
+        const int64_t n4 = n >> 2;
+        const v4f* __restrict__ x4 = reinterpret_cast<const v4f*>(x);
+        const v4f* __restrict__ y4 = reinterpret_cast<const v4f*>(y);
+        for (; i + (UNROLL - 1) * stride < n4; i += UNROLL * stride) {
+            v4f xv[UNROLL], yv[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) xv[u] = __builtin_nontemporal_load(&x4[i + u * stride]);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) yv[u] = __builtin_nontemporal_load(&y4[i + u * stride]);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                acc[u][0] = __builtin_fmaf(xv[u].x, yv[u].x, acc[u][0]);
+                acc[u][1] = __builtin_fmaf(xv[u].y, yv[u].y, acc[u][1]);
+                acc[u][2] = __builtin_fmaf(xv[u].z, yv[u].z, acc[u][2]);
+                acc[u][3] = __builtin_fmaf(xv[u].w, yv[u].w, acc[u][3]);
+            }
+        }
+        for (; i < n4; i += stride) {
+            v4f xv = x4[i], yv = y4[i];
+            acc[0][0] = __builtin_fmaf(xv.x, yv.x, acc[0][0]);
+            acc[0][1] = __builtin_fmaf(xv.y, yv.y, acc[0][1]);
+            acc[0][2] = __builtin_fmaf(xv.z, yv.z, acc[0][2]);
+            acc[0][3] = __builtin_fmaf(xv.w, yv.w, acc[0][3]);
+        }
+        if (blockIdx.x == 0) {
+            const int64_t t = (n4 << 2) + threadIdx.x;
+            if (t < n) acc[0][0] = __builtin_fmaf(x[t], y[t], acc[0][0]);
+        }
+    } else {
+        for (; i < n; i += stride) acc[0][0] = __builtin_fmaf(x[i], y[i], acc[0][0]);
+    }
+
+    // Fixed-order combine of this lane's accumulators, in double from here on.
+    double v = 0.0;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+        v += (static_cast<double>(acc[u][0]) + static_cast<double>(acc[u][1])) +
+             (static_cast<double>(acc[u][2]) + static_cast<double>(acc[u][3]));
+    const double block_total = block_sum_to_thread0(v, lds);
+
+    if (threadIdx.x == 0) {
+        partials[blockIdx.x] = block_total;
+        __threadfence();  // partial visible device-wide before the ticket is drawn
+        const unsigned int t = atomicAdd(ticket, 1u);
+        is_last = (t == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (!is_last) return;
+
+    __threadfence();
+    double s = 0.0;
+    for (unsigned int b = threadIdx.x; b < gridDim.x; b += kVecThreads)
+        s += partials[b];
+    __syncthreads();  // lds reuse
+    const double total = block_sum_to_thread0(s, lds);
+    if (threadIdx.x == 0) {
+        *out = static_cast<float>(total);
+        *ticket = 0u;  // ready for the next stream-ordered call
+    }
+}
+
+// ------------------------------------------------------------------ fills --
+__global__ __launch_bounds__(kVecThreads) void fill_uniform_kernel(float* __restrict__ dst, int64_t n, uint64_t seed) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x; i < n; i += stride)
+        dst[i] = uniform_pm1(seed, static_cast<uint64_t>(i));
+}
+
+__global__ __launch_bounds__(kVecThreads) void fill_uniform_matrix_kernel(float* __restrict__ dst, int rows, int cols,
+                                                                          int ld, uint64_t seed) {
+    const int64_t total = static_cast<int64_t>(rows) * cols;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / cols, c = i - r * cols;
+        dst[r * ld + c] = uniform_pm1(seed, static_cast<uint64_t>(i));
+    }
+}
+
+__global__ __launch_bounds__(kVecThreads) void zero_words_kernel(uint32_t* __restrict__ dst, int64_t nwords) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x; i < nwords; i += stride) dst[i] = 0u;
+}
+
+// ------------------------------------------------------------- launch glue --
+static int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            cus = v;
+        else
+            return 256;
+    }
+    return cus;
+}
+
+static int stream_grid(int64_t work_items, int blocks_per_cu) {
+    int64_t want = ceil_div(work_items, kVecThreads);
+    int64_t cap = static_cast<int64_t>(device_cus()) * blocks_per_cu;
+    if (want < 1) want = 1;
+    return static_cast<int>(want < cap ? want : cap);
+}
+
+}  // namespace hpcdnn
+
+using namespace hpcdnn;
+
+extern "C" int hpcdnn_saxpy(int64_t n, float alpha, const float* x, float* y, void* stream) {
+    if (n < 0 || (n > 0 && (!x || !y))) return HPCDNN_ERR_INVALID_VALUE;
+    if (n == 0) return HPCDNN_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3u) return HPCDNN_ERR_INVALID_VALUE;
+    if (aligned) {
+        const int grid = stream_grid((n >> 2) / 4 + 1, 8);
+        saxpy_vec4_kernel<4><<<grid, kVecThreads, 0, s>>>(n, alpha, x, y);
+    } else {
+        const int grid = stream_grid(n, 16);
+        saxpy_dword_kernel<<<grid, kVecThreads, 0, s>>>(n, alpha, x, y);
+    }
+    return launch_status();
+}
+
+extern "C" int hpcdnn_sdot(int64_t n, const float* x, const float* y, float* out, void* ws, size_t ws_bytes,
+                           void* stream) {
+    if (n < 0 || !out || (n > 0 && (!x || !y))) return HPCDNN_ERR_INVALID_VALUE;
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3u) return HPCDNN_ERR_INVALID_VALUE;
+    if (!ws || ws_bytes < hpcdnn_workspace_bytes(HPCDNN_OP_SDOT, 0, 0, 0)) return HPCDNN_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned int* ticket = static_cast<unsigned int*>(ws);
+    double* partials = reinterpret_cast<double*>(static_cast<char*>(ws) + kSdotPartialOffset);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
+    if (aligned) {
+        int grid = stream_grid((n >> 2) / 4 + 1, 8);
+        if (grid > kSdotMaxBlocks) grid = kSdotMaxBlocks;
+        sdot_kernel<4, true><<<grid, kVecThreads, 0, s>>>(n, x, y, out, ticket, partials);
+    } else {
+        int grid = stream_grid(n, 16);
+        if (grid > kSdotMaxBlocks) grid = kSdotMaxBlocks;
+        sdot_kernel<1, false><<<grid, kVecThreads, 0, s>>>(n, x, y, out, ticket, partials);
+    }
+    return launch_status();
+}
+
+extern "C" int hpcdnn_workspace_init(void* ws, size_t ws_bytes, void* stream) {
+    if (ws_bytes == 0) return HPCDNN_OK;
+    if (!ws || (reinterpret_cast<uintptr_t>(ws) & 3u) || (ws_bytes & 3u)) return HPCDNN_ERR_INVALID_VALUE;
+    const int64_t words = static_cast<int64_t>(ws_bytes / 4);
+    zero_words_kernel<<<stream_grid(words, 8), kVecThreads, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<uint32_t*>(ws), words);
+    return launch_status();
+}
+
+extern "C" int hpcdnn_fill_uniform(float* dst, int64_t n, uint64_t seed, void* stream) {
+    if (n < 0 || (n > 0 && !dst)) return HPCDNN_ERR_INVALID_VALUE;
+    if (n == 0) return HPCDNN_OK;
+    fill_uniform_kernel<<<stream_grid(n, 8), kVecThreads, 0, static_cast<hipStream_t>(stream)>>>(dst, n, seed);
+    return launch_status();
+}
+
+extern "C" int hpcdnn_fill_uniform_matrix(float* dst, int rows, int cols, int ld, uint64_t seed, void* stream) {
+    if (rows < 0 || cols < 0 || ld < cols || (rows > 0 && cols > 0 && !dst)) return HPCDNN_ERR_INVALID_VALUE;
+    if (rows == 0 || cols == 0) return HPCDNN_OK;
+    const int64_t total = static_cast<int64_t>(rows) * cols;
+    fill_uniform_matrix_kernel<<<stream_grid(total, 8), kVecThreads, 0, static_cast<hipStream_t>(stream)>>>(
+        dst, rows, cols, ld, seed);
+    return launch_status();
+}
+
+namespace hpcdnn {
+size_t sdot_workspace_bytes() { return kSdotPartialOffset + sizeof(double) * kSdotMaxBlocks; }
+}  // namespace hpcdnn

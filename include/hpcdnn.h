@@ -1,0 +1,151 @@
+/*
+ * hpcdnn -- FP32 BLAS level-1/3 + ABFT-SGEMM for AMD MI355X (gfx950).
+ *
+ * C ABI of libhpcdnn.so.  Plain pointers and sizes only; every device pointer
+ * is memory the caller allocated on the current HIP device, every `stream` is
+ * a hipStream_t passed as void* (NULL = the null stream).  Calls enqueue work
+ * on `stream` and return without synchronising.  Nothing here allocates device
+ * memory: kernels that need scratch take a caller-provided workspace.
+ *
+ * The reference (shixun404/HPCDeepNeuralNetworks) exposes no library API: its
+ * boundary is "a __global__ function plus the launch geometry its driver
+ * hard-codes".  Each entry point below names the reference kernel(s) and the
+ * launch site it stands in for; argument order follows the reference
+ * (dims, A, B, C, alpha, beta) / (n, alpha, x, y) / (n, x, y, out), with
+ * leading dimensions, workspace and stream added.  All matrices are row-major:
+ * element (i,j) of A is A[i*lda + j].
+ *
+ * Return value: 0 on success, otherwise a hipError_t-compatible code
+ * (HPCDNN_ERR_INVALID_VALUE = hipErrorInvalidValue for bad arguments, or the
+ * launch error reported by the HIP runtime).  The library never exits or
+ * prints (the reference's CUDA_CALLER prints and exit(1)s, utils/utils.cuh:7-15).
+ */
+#ifndef HPCDNN_H
+#define HPCDNN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HPCDNN_OK 0
+#define HPCDNN_ERR_INVALID_VALUE 1      /* == hipErrorInvalidValue */
+#define HPCDNN_ERR_WORKSPACE 2          /* workspace missing or too small (== hipErrorOutOfMemory) */
+
+/* Output tile of the ABFT kernel: one checksum pair (256 row sums, 128 column
+ * sums) and one status record per tile, tiles numbered row-major:
+ * tile = (i / 256) * ceil(N / 128) + (j / 128). */
+#define HPCDNN_FT_TILE_M 256
+#define HPCDNN_FT_TILE_N 128
+
+/* Operation selectors for hpcdnn_workspace_bytes(). */
+#define HPCDNN_OP_SGEMM 0
+#define HPCDNN_OP_SDOT 1
+
+/* One soft error to inject: `delta` is added to the accumulator of element
+ * (row, col) of output tile `tile` after the K loop and before verification.
+ * Run-time replacement for the reference's compile-time injection
+ * (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:40,145: +1.0 into one
+ * accumulator of thread 0 of every block). */
+typedef struct hpcdnn_fault {
+    int32_t tile;
+    int32_t row;   /* tile-local, 0 .. HPCDNN_FT_TILE_M-1 */
+    int32_t col;   /* tile-local, 0 .. HPCDNN_FT_TILE_N-1 */
+    float delta;
+} hpcdnn_fault;
+
+/* Verification record of one output tile (32 bytes, device memory). */
+typedef struct hpcdnn_ft_status {
+    int32_t flag;             /* 0 clean; 1 single fault located and corrected; 2 detected, not correctable */
+    int32_t row, col;         /* tile-local location of the corrected element, -1 if none */
+    int32_t n_bad_rows;       /* lines whose |reference - observed| checksum residual exceeded the threshold */
+    int32_t n_bad_cols;
+    float row_residual;       /* signed residual of the located row (the correction that was added), else 0 */
+    float col_residual;       /* signed residual of the located column, else 0 */
+    float max_clean_residual; /* largest |residual| among the lines judged clean */
+} hpcdnn_ft_status;
+
+const char* hpcdnn_version(void);
+const char* hpcdnn_error_string(int code);
+
+/* C = alpha*A*B + beta*C, A is MxK, B is KxN, C is MxN, any M,N,K >= 0 and any
+ * lda >= K, ldb >= N, ldc >= N.  C is not read when beta == 0.
+ * Replaces sgemm_1..sgemm_14 <<<dim3(ceil(N/bt),ceil(N/bt)),256>>>(N,A,B,C,alpha,beta)
+ * (kernel/sgemm/sgemm.cu:70-141, kernel/sgemm/include/kernel_13.cuh:14) and
+ * sgemm_{small,medium,large,tall,wide,huge} <<<dim3(ceil(M/ms),ceil(N/ns)),T>>>
+ * (M,N,K,A,B,C,alpha,beta) (kernel/ft_sgemm/sgemm.cu:114-157).
+ * `ws`/`ws_bytes`: optional split-K scratch (hpcdnn_workspace_bytes); when
+ * absent or too small the K dimension is not split (slower for deep-K
+ * shapes, same result contract). */
+int hpcdnn_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                 float alpha, float beta, void* ws, size_t ws_bytes, void* stream);
+
+/* Same contract with the kernel choice pinned, for tests and sweeps:
+ * `tile` indexes the built-in tile table (hpcdnn_sgemm_tile_info), -1 = pick
+ * as hpcdnn_sgemm does; `split_k` >= 1 forces that many K slices (needs a
+ * workspace of M*N*split_k floats when > 1), 0 = pick. */
+int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                    float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split_k, void* stream);
+
+/* Number of tile configurations, and the shape of entry `tile` (returns 0, or
+ * HPCDNN_ERR_INVALID_VALUE when out of range).  Counterpart of the reference's
+ * shape table (kernel/ft_sgemm/code_gen/main.py:8-16). */
+int hpcdnn_sgemm_num_tiles(void);
+int hpcdnn_sgemm_tile_info(int tile, int* bm, int* bn, int* bk);
+
+/* SGEMM with fused online ABFT: row/column checksums of each 256x128 output
+ * tile are accumulated from A and B inside the main loop, compared with the
+ * line sums of the accumulators in the epilogue, and a single faulty element
+ * per tile is located (faulty row x faulty column) and corrected before
+ * alpha/beta are applied.  `tau` is the absolute residual threshold
+ * (<= 0 selects the default for inputs of magnitude <= 1); `inject` is a HOST
+ * pointer to one fault or NULL; `status` is DEVICE memory for
+ * hpcdnn_ft_num_tiles(M,N) records or NULL.
+ * Replaces ft_sgemm_huge <<<dim3(M/128,N/128),256>>>(M,N,K,A,B,C,alpha,beta)
+ * (kernel/ft_sgemm/sgemm.cu:159-165, kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21). */
+int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                    float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
+                    void* stream);
+int hpcdnn_ft_num_tiles(int M, int N);
+/* Threshold hpcdnn_ft_sgemm uses when tau <= 0. */
+float hpcdnn_ft_default_tau(int K);
+
+/* y = alpha*x + y, one fused multiply-add per element, any n >= 0, any 4-byte
+ * aligned x and y.  Replaces saxpy/saxpy3/_saxpy <<<ceil(n/4/tpb),tpb>>>
+ * (N,alpha,x,y) (kernel/saxpy/saxpy.cu:15-48, launch :110-114). */
+int hpcdnn_saxpy(int64_t n, float alpha, const float* x, float* y, void* stream);
+
+/* *out = sum_i x[i]*y[i] (device scalar, overwritten; deterministic: the same
+ * inputs give the same bits on every run).  `ws` must hold
+ * hpcdnn_workspace_bytes(HPCDNN_OP_SDOT,...) bytes and have been passed through
+ * hpcdnn_workspace_init once; calls sharing a workspace must be stream-ordered.
+ * Replaces _sdot <<<min(1024,ceil(n/tpb)),tpb>>>(N,x,y,out) with its
+ * pre-zeroed atomicAdd target, and the sdot + reduction multi-launch chain
+ * (kernel/sdot/sdot.cu:9-67, launches :156,:177-187). */
+int hpcdnn_sdot(int64_t n, const float* x, const float* y, float* out, void* ws, size_t ws_bytes, void* stream);
+
+/* Scratch size for an operation (SGEMM: split-K partials for the split
+ * hpcdnn_sgemm would choose, 0 if none; SDOT: block partials + ticket; M,N,K
+ * ignored for SDOT). */
+size_t hpcdnn_workspace_bytes(int op, int M, int N, int K);
+/* Zero a freshly allocated workspace (fill kernel, safe to capture). */
+int hpcdnn_workspace_init(void* ws, size_t ws_bytes, void* stream);
+
+/* Seeded i.i.d. uniform values on the grid {-1 + j*2^-23}: element i of a
+ * vector takes counter i; element (r,c) of a rows x cols matrix takes counter
+ * r*cols + c whatever `ld` is (padding is left untouched).  Device-side
+ * replacement for generate_random_vector/matrix (utils/utils.cu:28-44). */
+int hpcdnn_fill_uniform(float* dst, int64_t n, uint64_t seed, void* stream);
+int hpcdnn_fill_uniform_matrix(float* dst, int rows, int cols, int ld, uint64_t seed, void* stream);
+
+/* Host validator kept from the reference: naive row-major square
+ * C = alpha*A*B + beta*C on HOST pointers, float accumulator, one thread
+ * (utils/utils.cu:93-103; same argument order). */
+void hpcdnn_cpu_gemm(float alpha, float beta, const float* mat1, const float* mat2, int n, float* mat3);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HPCDNN_H */

@@ -1,0 +1,197 @@
+"""ctypes loader for the CPU oracle (``oracle/oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()``
+and the ``cpu_baseline`` leg of ``bench.py``; the shipped package never
+imports it.  All arrays are C-contiguous numpy arrays (float32 unless noted).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile ``oracle.c`` with the Makefile beside it."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-C", _HERE, "liboracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+class FtStatus(C.Structure):
+    _fields_ = [
+        ("flag", C.c_int32),
+        ("row", C.c_int32),
+        ("col", C.c_int32),
+        ("n_bad_rows", C.c_int32),
+        ("n_bad_cols", C.c_int32),
+        ("row_residual", C.c_float),
+        ("col_residual", C.c_float),
+        ("max_clean_residual", C.c_float),
+    ]
+
+
+FT_STATUS_DTYPE = np.dtype(
+    [
+        ("flag", "<i4"),
+        ("row", "<i4"),
+        ("col", "<i4"),
+        ("n_bad_rows", "<i4"),
+        ("n_bad_cols", "<i4"),
+        ("row_residual", "<f4"),
+        ("col_residual", "<f4"),
+        ("max_clean_residual", "<f4"),
+    ]
+)
+
+_lib = None
+
+
+def _load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = C.CDLL(_LIB_PATH)
+    fp = C.POINTER(C.c_float)
+    dp = C.POINTER(C.c_double)
+    ip = C.POINTER(C.c_int)
+    lib.oracle_uniform.restype = C.c_float
+    lib.oracle_uniform.argtypes = [C.c_uint64, C.c_uint64]
+    lib.oracle_fill_uniform.restype = None
+    lib.oracle_fill_uniform.argtypes = [fp, C.c_int64, C.c_uint64]
+    lib.oracle_fill_uniform_matrix.restype = None
+    lib.oracle_fill_uniform_matrix.argtypes = [fp, C.c_int, C.c_int, C.c_int, C.c_uint64]
+    lib.oracle_num_threads.restype = C.c_int
+    lib.oracle_cpu_gemm.restype = None
+    lib.oracle_cpu_gemm.argtypes = [C.c_float, C.c_float, fp, fp, C.c_int, fp]
+    lib.oracle_gemm_f64_rows.restype = None
+    lib.oracle_gemm_f64_rows.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int,
+                                         C.c_float, C.c_float, ip, C.c_int, dp, dp]
+    lib.oracle_gemm_max_err.restype = C.c_double
+    lib.oracle_gemm_max_err.argtypes = [C.c_int, fp, C.c_int, ip, C.c_int, dp, dp]
+    lib.oracle_saxpy.restype = None
+    lib.oracle_saxpy.argtypes = [C.c_int64, C.c_float, fp, fp]
+    lib.oracle_sdot_f64.restype = C.c_double
+    lib.oracle_sdot_f64.argtypes = [C.c_int64, fp, fp]
+    lib.oracle_sdot_f32.restype = C.c_float
+    lib.oracle_sdot_f32.argtypes = [C.c_int64, fp, fp]
+    lib.oracle_abft_residuals.restype = None
+    lib.oracle_abft_residuals.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, dp, dp]
+    lib.oracle_abft_decide.restype = C.c_float
+    lib.oracle_abft_decide.argtypes = [C.c_int, C.c_int, dp, dp, C.c_float, C.POINTER(FtStatus)]
+    lib.oracle_ft_sgemm.restype = None
+    lib.oracle_ft_sgemm.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
+                                    C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int, C.c_int, C.c_float,
+                                    C.c_void_p]
+    _lib = lib
+    return lib
+
+
+def _f(a):
+    assert a.dtype == np.float32
+    return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _d(a):
+    assert a.dtype == np.float64 and a.flags.c_contiguous
+    return a.ctypes.data_as(C.POINTER(C.c_double))
+
+
+def num_threads() -> int:
+    return int(_load().oracle_num_threads())
+
+
+def uniform(seed: int, idx: int) -> float:
+    return float(_load().oracle_uniform(seed, idx))
+
+
+def fill_uniform(n: int, seed: int) -> np.ndarray:
+    out = np.empty(n, dtype=np.float32)
+    _load().oracle_fill_uniform(_f(out), n, seed)
+    return out
+
+
+def fill_uniform_matrix(rows: int, cols: int, seed: int, ld: int | None = None, pad=np.nan) -> np.ndarray:
+    """rows x ld array whose first ``cols`` columns hold the seeded values; padding holds ``pad``."""
+    ld = cols if ld is None else ld
+    out = np.full((rows, ld), pad, dtype=np.float32)
+    _load().oracle_fill_uniform_matrix(_f(out), rows, cols, ld, seed)
+    return out
+
+
+def cpu_gemm(alpha: float, beta: float, a: np.ndarray, b: np.ndarray, n: int, c: np.ndarray) -> None:
+    """In-place C = alpha*A*B + beta*C, argument order of utils/utils.cu:93."""
+    assert a.flags.c_contiguous and b.flags.c_contiguous and c.flags.c_contiguous
+    _load().oracle_cpu_gemm(alpha, beta, _f(a), _f(b), n, _f(c))
+
+
+def gemm_f64_rows(M, N, K, a, lda, b, ldb, c0, ldc, alpha, beta, rows=None):
+    """FP64 reference and |alpha|(|A||B|)+|beta||C0| denominators for the given rows (all if None)."""
+    if rows is None:
+        rows_arr, nrows, rp = None, M, None
+    else:
+        rows_arr = np.ascontiguousarray(rows, dtype=np.int32)
+        nrows = len(rows_arr)
+        rp = rows_arr.ctypes.data_as(C.POINTER(C.c_int))
+    ref = np.empty((nrows, N), dtype=np.float64)
+    den = np.empty((nrows, N), dtype=np.float64)
+    c0p = _f(c0) if c0 is not None else None
+    _load().oracle_gemm_f64_rows(M, N, K, _f(a), lda, _f(b), ldb, c0p, ldc, alpha, beta, rp, nrows, _d(ref), _d(den))
+    return ref, den
+
+
+def gemm_max_err(N, c, ldc, ref, den, rows=None) -> float:
+    if rows is None:
+        rp, nrows = None, ref.shape[0]
+    else:
+        rows_arr = np.ascontiguousarray(rows, dtype=np.int32)
+        rp, nrows = rows_arr.ctypes.data_as(C.POINTER(C.c_int)), len(rows_arr)
+    return float(_load().oracle_gemm_max_err(N, _f(c), ldc, rp, nrows, _d(ref), _d(den)))
+
+
+def saxpy(alpha: float, x: np.ndarray, y: np.ndarray) -> None:
+    """In-place y = fmaf(alpha, x, y)."""
+    assert x.size == y.size
+    _load().oracle_saxpy(x.size, alpha, _f(x), _f(y))
+
+
+def sdot_f64(x: np.ndarray, y: np.ndarray) -> float:
+    return float(_load().oracle_sdot_f64(x.size, _f(x), _f(y)))
+
+
+def sdot_f32(x: np.ndarray, y: np.ndarray) -> float:
+    return float(_load().oracle_sdot_f32(x.size, _f(x), _f(y)))
+
+
+def abft_residuals(a_tile, lda, b_tile, ldb, acc, ldacc, tm, tn, K):
+    dr = np.empty(tm, dtype=np.float64)
+    dc = np.empty(tn, dtype=np.float64)
+    _load().oracle_abft_residuals(tm, tn, K, _f(a_tile), lda, _f(b_tile), ldb, _f(acc), ldacc, _d(dr), _d(dc))
+    return dr, dc
+
+
+def abft_decide(dr: np.ndarray, dc: np.ndarray, tau: float):
+    """Returns (status dict, correction to add to acc[row, col])."""
+    st = FtStatus()
+    dr = np.ascontiguousarray(dr, dtype=np.float64)
+    dc = np.ascontiguousarray(dc, dtype=np.float64)
+    fix = _load().oracle_abft_decide(len(dr), len(dc), _d(dr), _d(dc), tau, C.byref(st))
+    return {k: getattr(st, k) for k, _ in FtStatus._fields_}, float(fix)
+
+
+def ft_sgemm(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, tile_m, tile_n, tau, fault=None):
+    """In-place ABFT GEMM model; ``fault`` = (tile, i, j, delta) or None.  Returns the per-tile status array."""
+    ntiles = ((M + tile_m - 1) // tile_m) * ((N + tile_n - 1) // tile_n)
+    status = np.zeros(ntiles, dtype=FT_STATUS_DTYPE)
+    ft, fi, fj, fd = (-1, 0, 0, 0.0) if fault is None else fault
+    _load().oracle_ft_sgemm(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, tile_m, tile_n, tau,
+                            int(ft), int(fi), int(fj), float(fd), status.ctypes.data_as(C.c_void_p))
+    return status

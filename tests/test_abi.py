@@ -1,0 +1,107 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares,
+rejects bad arguments before touching the GPU, and its host validator agrees with the oracle."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def L():
+    from hpcdeepneuralnetworks_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build()
+    return _lib.lib()
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hpcdnn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hpcdnn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(L):
+    from hpcdeepneuralnetworks_amd import _lib
+
+    declared = _declared_symbols()
+    assert len(declared) >= 16
+    assert sorted(_lib.EXPORTS) == declared
+    for name in declared:
+        assert getattr(L, name) is not None
+
+
+def test_version_and_error_strings(L):
+    assert b"gfx950" in L.hpcdnn_version()
+    assert L.hpcdnn_error_string(0) == b"success"
+    assert b"invalid" in L.hpcdnn_error_string(1)
+    assert b"workspace" in L.hpcdnn_error_string(2)
+
+
+def test_status_and_fault_struct_sizes():
+    from hpcdeepneuralnetworks_amd import _lib
+    from hpcdeepneuralnetworks_amd.blas import FT_STATUS_DTYPE
+
+    assert C.sizeof(_lib.Fault) == 16 and FT_STATUS_DTYPE.itemsize == 32
+
+
+def test_bad_arguments_are_rejected_without_a_gpu(L):
+    INVALID, WORKSPACE = 1, 2
+    dummy = C.c_void_p(0x1000)
+    assert L.hpcdnn_saxpy(-1, 1.0, dummy, dummy, None) == INVALID
+    assert L.hpcdnn_saxpy(4, 1.0, None, dummy, None) == INVALID
+    assert L.hpcdnn_saxpy(4, 1.0, C.c_void_p(0x1002), dummy, None) == INVALID  # not 4-byte aligned
+    assert L.hpcdnn_saxpy(0, 1.0, None, None, None) == 0
+    assert L.hpcdnn_sdot(4, dummy, dummy, None, dummy, 1 << 20, None) == INVALID
+    assert L.hpcdnn_sdot(4, dummy, dummy, dummy, None, 0, None) == WORKSPACE
+    assert L.hpcdnn_sdot(4, dummy, dummy, dummy, dummy, 8, None) == WORKSPACE
+    # GEMM: negative dims, leading dimensions smaller than the row length, null operands
+    assert L.hpcdnn_sgemm(-1, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
+    assert L.hpcdnn_sgemm(4, 4, 4, dummy, 3, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
+    assert L.hpcdnn_sgemm(4, 4, 4, dummy, 4, dummy, 3, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
+    assert L.hpcdnn_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, 3, 1.0, 0.0, None, 0, None) == INVALID
+    assert L.hpcdnn_sgemm(4, 4, 4, None, 4, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
+    assert L.hpcdnn_sgemm(0, 4, 4, None, 4, None, 4, None, 4, 1.0, 0.0, None, 0, None) == 0  # empty: nothing to do
+    assert L.hpcdnn_sgemm_ex(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, 99, 1, None) == INVALID
+    assert L.hpcdnn_sgemm_ex(4, 4, 64, dummy, 64, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, 0, 2, None) == WORKSPACE
+    from hpcdeepneuralnetworks_amd._lib import Fault
+
+    bad = Fault(5, 0, 0, 1.0)  # only one tile exists
+    assert L.hpcdnn_ft_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, 0.0, C.byref(bad), None, None) == INVALID
+    bad = Fault(0, 256, 0, 1.0)
+    assert L.hpcdnn_ft_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, 0.0, C.byref(bad), None, None) == INVALID
+
+
+def test_tile_table_and_workspace_sizes(L):
+    n = L.hpcdnn_sgemm_num_tiles()
+    assert n >= 4
+    bm, bn, bk = C.c_int(), C.c_int(), C.c_int()
+    assert L.hpcdnn_sgemm_tile_info(0, C.byref(bm), C.byref(bn), C.byref(bk)) == 0
+    assert (bm.value, bn.value) == (256, 128) and bk.value % 8 == 0
+    assert L.hpcdnn_sgemm_tile_info(n, None, None, None) == 1
+    assert L.hpcdnn_ft_num_tiles(4096, 4096) == 16 * 32
+    assert L.hpcdnn_ft_num_tiles(257, 129) == 4
+    assert L.hpcdnn_workspace_bytes(1, 0, 0, 0) >= 64 + 8
+    # a square compute-bound problem needs no split-K scratch; the deep-K one does
+    assert L.hpcdnn_workspace_bytes(0, 4096, 4096, 4096) == 0
+    ws = L.hpcdnn_workspace_bytes(0, 128, 128, 65536)
+    assert ws > 0 and ws % (128 * 128 * 4) == 0
+    assert L.hpcdnn_ft_default_tau(4096) > 0
+
+
+def test_host_cpu_gemm_matches_oracle_and_numpy(L, oracle_mod):
+    n = 64
+    a = oracle_mod.fill_uniform_matrix(n, n, seed=11)
+    b = oracle_mod.fill_uniform_matrix(n, n, seed=12)
+    c0 = oracle_mod.fill_uniform_matrix(n, n, seed=13)
+    for alpha, beta in [(1.0, 0.0), (1.5, -1.0)]:
+        c_lib, c_orc = c0.copy(), c0.copy()
+        L.hpcdnn_cpu_gemm(alpha, beta, a.ctypes.data, b.ctypes.data, n, c_lib.ctypes.data)
+        oracle_mod.cpu_gemm(alpha, beta, a, b, n, c_orc)
+        assert np.array_equal(c_lib, c_orc)  # same order, same float accumulator -> same bits
+        ref = alpha * (a.astype(np.float64) @ b.astype(np.float64)) + beta * c0
+        assert np.max(np.abs(c_lib - ref)) < 5e-5

@@ -1,0 +1,253 @@
+"""Pins the CPU oracle against independent routines (numpy float64, exact rationals, closed forms).
+
+The reference holds no golden vectors for this path, so every check here is
+chosen so that a plausible slip in oracle.c (dropped term, transposed operand,
+wrong sign or index) fails it.
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+
+def _round_f32(fr: Fraction) -> np.float32:
+    """Correctly rounded (nearest-even) float32 of an exact rational."""
+    if fr == 0:
+        return np.float32(0.0)
+    guess = np.float32(float(fr))
+    cands = {guess, np.nextafter(guess, np.float32(np.inf)), np.nextafter(guess, np.float32(-np.inf))}
+    best = None
+    for c in cands:
+        d = abs(Fraction(float(c)) - fr)
+        key = (d, int(np.float32(c).view(np.uint32)) & 1)  # ties -> even mantissa
+        if best is None or key < best[0]:
+            best = (key, c)
+    return np.float32(best[1])
+
+
+def test_rng_range_grid_and_independence(oracle_mod):
+    v = oracle_mod.fill_uniform(1 << 16, seed=7)
+    assert v.dtype == np.float32 and v.min() >= -1.0 and v.max() < 1.0
+    # values sit on the 2^-23 grid
+    assert np.all(v * 8388608.0 == np.round(v * 8388608.0))
+    # first two moments of uniform[-1,1): mean 0, var 1/3
+    assert abs(float(v.mean())) < 0.01 and abs(float(v.var()) - 1.0 / 3.0) < 0.01
+    w = oracle_mod.fill_uniform(1 << 16, seed=8)
+    assert abs(float(np.corrcoef(v, w)[0, 1])) < 0.02
+    assert abs(float(np.corrcoef(v[:-1], v[1:])[0, 1])) < 0.02
+    # scalar accessor and vector fill agree, counter = index
+    assert oracle_mod.uniform(7, 12345) == float(v[12345])
+
+
+def test_rng_matrix_ignores_leading_dimension(oracle_mod):
+    a = oracle_mod.fill_uniform_matrix(5, 7, seed=3)
+    b = oracle_mod.fill_uniform_matrix(5, 7, seed=3, ld=11)
+    assert np.array_equal(a, b[:, :7]) and np.all(np.isnan(b[:, 7:]))
+    assert np.array_equal(a.ravel(), oracle_mod.fill_uniform(35, seed=3))
+
+
+def test_cpu_gemm_matches_numpy_float64(oracle_mod):
+    n = 96
+    rng = np.random.default_rng(0)
+    a = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    b = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    c0 = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    for alpha, beta in [(1.0, 0.0), (1.5, -1.0), (1.0, -1.5), (0.0, 2.0)]:
+        c = c0.copy()
+        oracle_mod.cpu_gemm(alpha, beta, a, b, n, c)
+        ref = alpha * (a.astype(np.float64) @ b.astype(np.float64)) + beta * c0.astype(np.float64)
+        assert np.max(np.abs(c - ref)) < 5e-5, (alpha, beta)
+
+
+def test_cpu_gemm_is_not_transposed(oracle_mod):
+    # A = permutation-like matrix picks rows of B: C = A@B exactly; A^T@B or B@A would differ
+    n = 8
+    a = np.zeros((n, n), dtype=np.float32)
+    for i in range(n):
+        a[i, (3 * i + 1) % n] = 1.0
+    b = np.arange(n * n, dtype=np.float32).reshape(n, n)
+    c = np.zeros((n, n), dtype=np.float32)
+    oracle_mod.cpu_gemm(1.0, 0.0, a, b, n, c)
+    assert np.array_equal(c, b[[(3 * i + 1) % n for i in range(n)], :])
+
+
+def test_cpu_gemm_float_accumulator_order(oracle_mod):
+    # float accumulate, k ascending: 2^24 + 1 + 1 stays 2^24 in float, in double it would be 2^24+2
+    n = 4
+    a = np.zeros((n, n), dtype=np.float32)
+    b = np.zeros((n, n), dtype=np.float32)
+    a[0, :3] = [16777216.0, 1.0, 1.0]
+    b[:3, 0] = 1.0
+    c = np.zeros((n, n), dtype=np.float32)
+    oracle_mod.cpu_gemm(1.0, 0.0, a, b, n, c)
+    assert c[0, 0] == np.float32(16777216.0)
+
+
+@pytest.mark.parametrize("M,N,K,lda,ldb,ldc", [(17, 9, 33, 40, 12, 10), (32, 32, 32, 32, 32, 32), (1, 1, 1, 1, 1, 1)])
+def test_gemm_f64_rows_matches_numpy(oracle_mod, M, N, K, lda, ldb, ldc):
+    rng = np.random.default_rng(1)
+    a = np.full((M, lda), np.nan, np.float32)
+    b = np.full((K, ldb), np.nan, np.float32)
+    c0 = np.full((M, ldc), np.nan, np.float32)
+    a[:, :K] = rng.uniform(-1, 1, (M, K))
+    b[:, :N] = rng.uniform(-1, 1, (K, N))
+    c0[:, :N] = rng.uniform(-1, 1, (M, N))
+    alpha, beta = 1.5, -0.5
+    ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, lda, b, ldb, c0, ldc, alpha, beta)
+    a64, b64, c64 = a[:, :K].astype(np.float64), b[:, :N].astype(np.float64), c0[:, :N].astype(np.float64)
+    assert np.allclose(ref, alpha * (a64 @ b64) + beta * c64, rtol=0, atol=1e-12)
+    assert np.allclose(den, abs(alpha) * (np.abs(a64) @ np.abs(b64)) + abs(beta) * np.abs(c64), rtol=0, atol=1e-12)
+    rows = [M - 1, 0]
+    ref2, den2 = oracle_mod.gemm_f64_rows(M, N, K, a, lda, b, ldb, c0, ldc, alpha, beta, rows=rows)
+    assert np.array_equal(ref2, ref[rows]) and np.array_equal(den2, den[rows])
+
+
+def test_gemm_max_err_is_the_componentwise_criterion(oracle_mod):
+    M = N = 4
+    ref = np.ones((M, N))
+    den = np.full((M, N), 2.0)
+    c = np.ones((M, 6), dtype=np.float32)
+    assert oracle_mod.gemm_max_err(N, c, 6, ref, den) == 0.0
+    c[2, 3] = 1.5
+    assert oracle_mod.gemm_max_err(N, c, 6, ref, den) == pytest.approx(0.25)
+    c[1, 1] = np.nan
+    assert not (oracle_mod.gemm_max_err(N, c, 6, ref, den) <= 1.0)  # NaN is never accepted
+
+
+def test_saxpy_is_one_fused_multiply_add(oracle_mod):
+    rng = np.random.default_rng(2)
+    n = 2000
+    x = rng.uniform(-1, 1, n).astype(np.float32)
+    y0 = rng.uniform(-1, 1, n).astype(np.float32)
+    alpha = np.float32(2.5)
+    y = y0.copy()
+    oracle_mod.saxpy(float(alpha), x, y)
+    exact = [_round_f32(Fraction(float(alpha)) * Fraction(float(xi)) + Fraction(float(yi))) for xi, yi in zip(x, y0)]
+    assert np.array_equal(y, np.array(exact, dtype=np.float32))
+
+
+def test_saxpy_differs_from_unfused_where_it_must(oracle_mod):
+    # a*x rounds in float when unfused; the fused result keeps the low bits: (1+2^-12)^2 - 1
+    a = np.float32(1.0 + 2.0**-12)
+    x = np.array([a], dtype=np.float32)
+    y = np.array([-1.0], dtype=np.float32)
+    oracle_mod.saxpy(float(a), x, y)
+    assert float(y[0]) == 2.0**-11 + 2.0**-24
+    assert np.float32(np.float32(a * a) + np.float32(-1.0)) != y[0]
+
+
+def test_sdot_f64_and_f32(oracle_mod):
+    rng = np.random.default_rng(3)
+    n = 100003
+    x = rng.uniform(-1, 1, n).astype(np.float32)
+    y = rng.uniform(-1, 1, n).astype(np.float32)
+    exact = float(np.dot(x.astype(np.float64), y.astype(np.float64)))
+    assert oracle_mod.sdot_f64(x, y) == pytest.approx(exact, rel=0, abs=1e-9)
+    assert oracle_mod.sdot_f32(x, y) == pytest.approx(exact, rel=0, abs=0.05)
+    # closed forms
+    ones = np.ones(1 << 12, dtype=np.float32)
+    assert oracle_mod.sdot_f64(ones, ones) == 4096.0 and oracle_mod.sdot_f32(ones, ones) == 4096.0
+    k = np.arange(1, 101, dtype=np.float32)
+    assert oracle_mod.sdot_f64(k, k) == 338350.0  # sum k^2
+    assert oracle_mod.sdot_f64(x[:0], y[:0]) == 0.0
+
+
+def _tile_problem(tm, tn, K, seed):
+    rng = np.random.default_rng(seed)
+    a = rng.uniform(-1, 1, (tm, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (K, tn)).astype(np.float32)
+    acc = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    return a, b, acc
+
+
+def test_abft_residuals_follow_the_checksum_algebra(oracle_mod):
+    tm, tn, K = 24, 16, 40
+    a, b, acc = _tile_problem(tm, tn, K, 4)
+    dr, dc = oracle_mod.abft_residuals(a, K, b, tn, acc, tn, tm, tn, K)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    # e^T(AB) = (e^T A)B and (AB)e = A(Be), each computed the "other" way round
+    cr_ref = (a64 @ b64).sum(axis=1)
+    cc_ref = (a64 @ b64).sum(axis=0)
+    assert np.allclose(dr, cr_ref - acc.astype(np.float64).sum(axis=1), atol=1e-10)
+    assert np.allclose(dc, cc_ref - acc.astype(np.float64).sum(axis=0), atol=1e-10)
+    assert np.max(np.abs(dr)) < 1e-4 and np.max(np.abs(dc)) < 1e-4  # fault-free: rounding only
+    # a fault of +delta at (i,j) shows up as -delta in row i and column j only (sign: reference - observed)
+    acc2 = acc.copy()
+    acc2[5, 9] += np.float32(0.75)
+    dr2, dc2 = oracle_mod.abft_residuals(a, K, b, tn, acc2, tn, tm, tn, K)
+    assert abs(dr2[5] + 0.75) < 1e-4 and abs(dc2[9] + 0.75) < 1e-4
+    mask_r = np.ones(tm, bool); mask_r[5] = False
+    mask_c = np.ones(tn, bool); mask_c[9] = False
+    assert np.array_equal(dr2[mask_r], dr[mask_r]) and np.array_equal(dc2[mask_c], dc[mask_c])
+
+
+def test_abft_residuals_not_transposed_for_rectangular_tiles(oracle_mod):
+    # rows and columns carry different checksums: make A's rows distinguishable from B's columns
+    tm, tn, K = 3, 5, 2
+    a = np.array([[1, 0], [0, 1], [2, 2]], dtype=np.float32)
+    b = np.array([[1, 2, 3, 4, 5], [10, 20, 30, 40, 50]], dtype=np.float32)
+    acc = np.zeros((tm, tn), dtype=np.float32)  # observed = 0 -> residual = reference checksum
+    dr, dc = oracle_mod.abft_residuals(a, K, b, tn, acc, tn, tm, tn, K)
+    assert dr.tolist() == [15.0, 150.0, 330.0]
+    assert dc.tolist() == [33.0, 66.0, 99.0, 132.0, 165.0]  # column sums of A@B
+
+
+def test_abft_reference_known_answer(oracle_mod):
+    """The one case the reference holds: +1.0 at tile-local (m=0, n=1) of a 128x128 tile, threshold 0.1
+    -> row 0 and column 1 flagged, magnitude 1 removed (ft_sgemm_huge.cuh:40,145,263,358)."""
+    tm = tn = 128
+    K = 256
+    a, b, acc = _tile_problem(tm, tn, K, 5)
+    acc[0, 1] += np.float32(1.0)
+    dr, dc = oracle_mod.abft_residuals(a, K, b, tn, acc, tn, tm, tn, K)
+    st, fix = oracle_mod.abft_decide(dr, dc, 0.1)
+    assert (st["flag"], st["row"], st["col"], st["n_bad_rows"], st["n_bad_cols"]) == (1, 0, 1, 1, 1)
+    assert round(-fix) == 1 and abs(fix + 1.0) < 1e-3  # the reference subtracts round(|residual|) = 1
+    assert st["max_clean_residual"] < 0.1
+
+
+def test_abft_decide_cases(oracle_mod):
+    tm, tn = 6, 4
+    z_r, z_c = np.zeros(tm), np.zeros(tn)
+    st, fix = oracle_mod.abft_decide(z_r, z_c, 0.01)
+    assert st["flag"] == 0 and fix == 0.0 and st["row"] == -1 and st["col"] == -1
+    # below threshold -> clean, recorded as the largest clean residual
+    r = z_r.copy(); r[2] = -0.009
+    st, fix = oracle_mod.abft_decide(r, z_c, 0.01)
+    assert st["flag"] == 0 and st["max_clean_residual"] == pytest.approx(0.009)
+    # exactly at the threshold is clean (strict >), as in the reference (fabsf(x) > err_bound)
+    r[2] = float(np.float32(0.01))
+    assert oracle_mod.abft_decide(r, z_c, np.float32(0.01))[0]["flag"] == 0
+    # single fault: correction is the signed row residual
+    r = z_r.copy(); c = z_c.copy(); r[4] = -0.5; c[1] = -0.5001
+    st, fix = oracle_mod.abft_decide(r, c, 0.01)
+    assert (st["flag"], st["row"], st["col"]) == (1, 4, 1) and fix == pytest.approx(-0.5)
+    assert st["row_residual"] == pytest.approx(-0.5) and st["col_residual"] == pytest.approx(-0.5001)
+    # row without column, or two rows: detected but not correctable
+    st, fix = oracle_mod.abft_decide(r, z_c, 0.01)
+    assert st["flag"] == 2 and fix == 0.0 and (st["n_bad_rows"], st["n_bad_cols"]) == (1, 0)
+    r[0] = 0.3
+    st, _ = oracle_mod.abft_decide(r, c, 0.01)
+    assert st["flag"] == 2 and st["n_bad_rows"] == 2
+
+
+@pytest.mark.parametrize("fault", [None, (1, 3, 2, 0.5), (2, 7, 0, -20.0)])
+def test_ft_sgemm_model_detects_and_corrects(oracle_mod, fault):
+    M, N, K, tm, tn = 20, 12, 64, 8, 8   # 3 x 2 tiles, ragged in both directions
+    rng = np.random.default_rng(6)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    c0 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    c = c0.copy()
+    st = oracle_mod.ft_sgemm(M, N, K, a, K, b, N, c, N, 1.0, 1.0, tm, tn, 1e-3, fault)
+    ref = a.astype(np.float64) @ b.astype(np.float64) + c0
+    assert np.max(np.abs(c - ref)) < 1e-4  # corrected output equals the fault-free product
+    flags = st["flag"].tolist()
+    if fault is None:
+        assert flags == [0] * 6
+    else:
+        exp = [0] * 6
+        exp[fault[0]] = 1
+        assert flags == exp
+        assert (st["row"][fault[0]], st["col"][fault[0]]) == (fault[1], fault[2])
+        assert st["row_residual"][fault[0]] == pytest.approx(-fault[3], abs=1e-4)

@@ -1,0 +1,190 @@
+"""GPU parity of SGEMM against the CPU oracle, through the C ABI.
+
+Acceptance criterion (stated tolerance): max |C - Cref| / (|alpha| (|A||B|)_ij + |beta| |C0_ij|) <= 1e-5 with Cref
+accumulated in FP64.  Small shapes are checked on every element, large ones on sampled rows plus a Freivalds
+check (C v against A (B v) in FP64) that covers every element.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+
+
+def _problem(oracle_mod, M, N, K, lda=None, ldb=None, ldc=None, seed=100):
+    lda, ldb, ldc = lda or max(K, 1), ldb or max(N, 1), ldc or max(N, 1)
+    a = oracle_mod.fill_uniform_matrix(M, K, seed, ld=lda)
+    b = oracle_mod.fill_uniform_matrix(K, N, seed + 1, ld=ldb)
+    c = oracle_mod.fill_uniform_matrix(M, N, seed + 2, ld=ldc)
+    return a, b, c
+
+
+def _check(oracle_mod, blas, M, N, K, alpha, beta, lda=None, ldb=None, ldc=None, tile=-1, split_k=0, ws=None, seed=100):
+    a, b, c0 = _problem(oracle_mod, M, N, K, lda, ldb, ldc, seed)
+    da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+    blas.sgemm(M, N, K, da, db, dc, alpha, beta, ws=ws, tile=tile, split_k=split_k)
+    c = dc.cpu().numpy()
+    if M and N:
+        ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, a.shape[1], b, b.shape[1], c0, c0.shape[1], alpha, beta)
+        err = oracle_mod.gemm_max_err(N, c, c.shape[1], ref, den)
+        assert err <= TOL, (M, N, K, alpha, beta, tile, split_k, err)
+    # padding columns of C (NaN) are never written; padding of A and B (NaN) is never used
+    assert np.all(np.isnan(c[:, N:]))
+    return c
+
+
+def test_config1_1024_cube_against_reference_cpu_gemm(blas, oracle_mod):
+    """BASELINE config 1: M=N=K=1024, alpha=1, beta=0, C zero-initialised, validated against the reference's
+    CPU triple loop (utils/utils.cu:93-103) and against the FP64 criterion."""
+    n = 1024
+    a = oracle_mod.fill_uniform_matrix(n, n, 1)
+    b = oracle_mod.fill_uniform_matrix(n, n, 2)
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    dc = torch.zeros(n, n, dtype=torch.float32, device="cuda")
+    blas.sgemm(n, n, n, da, db, dc, 1.0, 0.0)
+    c = dc.cpu().numpy()
+    c_ref = np.zeros((n, n), dtype=np.float32)
+    oracle_mod.cpu_gemm(1.0, 0.0, a, b, n, c_ref)
+    assert np.max(np.abs(c - c_ref)) < 1e-2            # the reference's own acceptance test (utils.cu:84)
+    ref, den = oracle_mod.gemm_f64_rows(n, n, n, a, n, b, n, None, n, 1.0, 0.0)
+    assert oracle_mod.gemm_max_err(n, c, n, ref, den) <= TOL
+    # the reference's calling convention: sgemm(N, A, B, C, alpha, beta) with square packed operands
+    dc2 = torch.zeros(n, n, dtype=torch.float32, device="cuda")
+    blas.sgemm(n, n, n, da, db, dc2, 1.0, 0.0, tile=1)
+    assert oracle_mod.gemm_max_err(n, dc2.cpu().numpy(), n, ref, den) <= TOL
+
+
+def _num_tiles(blas):
+    return len(blas.tile_table())
+
+
+def test_every_tile_config_small_and_ragged_shapes(blas, oracle_mod):
+    shapes = [(1, 1, 1), (5, 7, 3), (33, 31, 17), (64, 64, 64), (130, 70, 40), (257, 129, 33), (40, 300, 8), (300, 40, 100)]
+    for tile in range(_num_tiles(blas)):
+        for (M, N, K) in shapes:
+            _check(oracle_mod, blas, M, N, K, 1.0, 0.0, tile=tile, seed=200 + tile)
+
+
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (1.5, -1.0), (1.0, -1.5), (0.0, 2.0), (-0.5, 0.0)])
+def test_alpha_beta_pairs_with_padded_leading_dimensions(blas, oracle_mod, alpha, beta):
+    # 1.5/-1.0 and 1.0/-1.5 are the reference drivers' values (kernel/sgemm/sgemm.cu:33-34, ft_sgemm/sgemm.cu:32-34)
+    _check(oracle_mod, blas, 200, 150, 90, alpha, beta, lda=96, ldb=152, ldc=160)
+    _check(oracle_mod, blas, 200, 150, 90, alpha, beta, lda=91, ldb=151, ldc=153)  # odd ld: unaligned rows
+
+
+def test_beta_zero_ignores_nan_in_c(blas, oracle_mod):
+    M, N, K = 100, 60, 50
+    a, b, _ = _problem(oracle_mod, M, N, K)
+    dc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    blas.sgemm(M, N, K, torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), dc, 1.0, 0.0)
+    assert torch.isfinite(dc).all()
+
+
+def test_every_edge_residue_brute_force(blas, oracle_mod):
+    # every (M, N, K) residue class of the vector width and a few around the MFMA block size
+    vals = [1, 2, 3, 4, 5, 7, 8, 9, 31, 32, 33, 40]
+    rng = np.random.default_rng(0)
+    for _ in range(40):
+        M, N, K = (int(rng.choice(vals)) for _ in range(3))
+        _check(oracle_mod, blas, M, N, K, 1.0, 1.0, seed=int(rng.integers(1, 1000)))
+        _check(oracle_mod, blas, M, N, K, 1.0, 0.0, tile=4, seed=int(rng.integers(1, 1000)))
+
+
+def test_exact_special_cases(blas):
+    n = 192
+    dev = "cuda"
+    # identity: A @ I == A bit for bit, I @ B == B
+    a = torch.rand(n, n, device=dev) * 2 - 1
+    eye = torch.eye(n, device=dev)
+    c = torch.empty(n, n, device=dev)
+    blas.sgemm(n, n, n, a, eye, c, 1.0, 0.0)
+    assert torch.equal(c, a)
+    blas.sgemm(n, n, n, eye, a, c, 1.0, 0.0)
+    assert torch.equal(c, a)
+    # a permutation picks rows: transposed operands or a swapped k index would be caught
+    perm = torch.randperm(n, device=dev)
+    p = torch.zeros(n, n, device=dev)
+    p[torch.arange(n, device=dev), perm] = 1.0
+    blas.sgemm(n, n, n, p, a, c, 1.0, 0.0)
+    assert torch.equal(c, a[perm])
+    # all ones: C == K exactly (K <= 2^24), any accumulation order
+    M, N, K = 96, 160, 4096
+    c = torch.empty(M, N, device=dev)
+    blas.sgemm(M, N, K, torch.ones(M, K, device=dev), torch.ones(K, N, device=dev), c, 1.0, 0.0)
+    assert torch.all(c == float(K))
+    # index-valued operands: C[i][j] = i * j * K, exact in FP32 for these sizes
+    M, N, K = 70, 50, 16
+    ai = torch.arange(M, device=dev, dtype=torch.float32)[:, None].expand(M, K).contiguous()
+    bj = torch.arange(N, device=dev, dtype=torch.float32)[None, :].expand(K, N).contiguous()
+    c = torch.empty(M, N, device=dev)
+    blas.sgemm(M, N, K, ai, bj, c, 1.0, 0.0)
+    assert torch.equal(c, (torch.arange(M, device=dev)[:, None] * torch.arange(N, device=dev)[None, :] * K).float())
+    # alpha = 0, beta = 1 leaves C unchanged; K = 0 scales C by beta
+    c0 = torch.rand(M, N, device=dev)
+    c = c0.clone()
+    blas.sgemm(M, N, K, ai, bj, c, 0.0, 1.0)
+    assert torch.equal(c, c0)
+    blas.sgemm(M, N, 0, ai[:, :0], bj[:0, :], c, 1.0, 0.5)
+    assert torch.equal(c, c0 * 0.5)
+
+
+def _sampled_check(oracle_mod, blas, M, N, K, alpha, beta, nrows=48, seed=300, tile=-1, split_k=0, ws=None):
+    """Device-generated operands (same counters as the oracle), sampled-row FP64 check + Freivalds over all of C."""
+    dev = "cuda"
+    da = torch.empty(M, K, device=dev)
+    db = torch.empty(K, N, device=dev)
+    dc = torch.empty(M, N, device=dev)
+    blas.fill_uniform_matrix(da, M, K, seed)
+    blas.fill_uniform_matrix(db, K, N, seed + 1)
+    blas.fill_uniform_matrix(dc, M, N, seed + 2)
+    dc0 = dc.clone() if beta != 0.0 else None
+    blas.sgemm(M, N, K, da, db, dc, alpha, beta, ws=ws, tile=tile, split_k=split_k)
+    rng = np.random.default_rng(seed)
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, nrows)])).astype(np.int32)
+    a = oracle_mod.fill_uniform_matrix(M, K, seed)
+    b = oracle_mod.fill_uniform_matrix(K, N, seed + 1)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, seed + 2) if beta != 0.0 else None
+    ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, K, b, N, c0, N, alpha, beta, rows=rows)
+    c_rows = np.ascontiguousarray(dc[torch.from_numpy(rows).long().cuda()].cpu().numpy())
+    err = oracle_mod.gemm_max_err(N, c_rows, N, ref, den)
+    assert err <= TOL, (M, N, K, alpha, beta, err)
+    # Freivalds in FP64 over the whole matrix: C v == alpha A (B v) + beta C0 v
+    v = (torch.randint(0, 2, (N,), device=dev, dtype=torch.float64) * 2 - 1)
+    lhs = dc.double() @ v
+    rhs = alpha * (da.double() @ (db.double() @ v))
+    bound = abs(alpha) * (da.double().abs() @ (db.double().abs() @ torch.ones(N, device=dev, dtype=torch.float64)))
+    if beta != 0.0:
+        rhs = rhs + beta * (dc0.double() @ v)
+        bound = bound + abs(beta) * dc0.double().abs().sum(dim=1)
+    assert torch.all((lhs - rhs).abs() <= TOL * bound), (M, N, K)
+    return dc
+
+
+@pytest.mark.parametrize("n,beta", [(1000, 0.0), (3001, 1.0), (2048, 1.0), (4096, 0.0)])
+def test_square_sizes_from_the_sweep(blas, oracle_mod, n, beta):
+    _sampled_check(oracle_mod, blas, n, n, n, 1.0, beta)
+
+
+@pytest.mark.parametrize("n,beta", [(6000, 0.0), (6144, 0.0), (6144, 1.0)])
+def test_largest_square_sizes(blas, oracle_mod, n, beta):
+    _sampled_check(oracle_mod, blas, n, n, n, 1.0, beta, nrows=24)
+
+
+@pytest.mark.parametrize("M,N,K", [(8192, 8192, 256), (16384, 64, 4096), (128, 128, 65536)])
+def test_skinny_and_deep_shapes(blas, oracle_mod, M, N, K):
+    ws = blas.workspace(max(blas.sgemm_workspace_bytes(M, N, K), 4))
+    c1 = _sampled_check(oracle_mod, blas, M, N, K, 1.0, 0.0, nrows=16, ws=ws)
+    c2 = _sampled_check(oracle_mod, blas, M, N, K, 1.0, 0.0, nrows=16, ws=ws)
+    assert torch.equal(c1, c2)  # fixed-order split-K reduction: same bits on every run
+
+
+def test_split_k_forced_matches_and_is_deterministic(blas, oracle_mod):
+    M, N, K = 200, 136, 2000
+    ws = blas.workspace(M * N * 8 * 4)
+    outs = []
+    for split in (1, 2, 5, 8):
+        outs.append(_check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=1, split_k=split, ws=ws, ldc=144))
+    again = _check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=1, split_k=8, ws=ws, ldc=144)
+    assert np.array_equal(outs[-1][:, :N], again[:, :N])
