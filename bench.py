@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Benchmark of the SGEMM / ABFT-SGEMM / SAXPY / SDOT path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one SGEMM launch at M=N=K=6144 (alpha=1, beta=0), the size the headline metric is quoted on; operands
+are seeded synthetic data generated on the device, resident in HBM before the timed region.  One JSON line is
+printed: `value` is the SGEMM rate in GFLOP/s, `roofline` prices the SGEMM kernel against the FP32 MFMA peak,
+`cpu_baseline` times the CPU oracle's restatement of the reference's cpu_gemm on the host, and `extras` carries
+the other parts of the metric (ABFT overhead and fault campaign at 4096^3, SAXPY/SDOT GB/s at 2^28, the rest of the
+size sweep, rocBLAS/hipBLASLt through torch.matmul as a timed comparison only).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 4 SIMD x 64 flop/clk x 2.4 GHz
+PEAK_HBM_GBS = 8000.0
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extras", action="store_true", help="headline SGEMM line only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--ft-launches", type=int, default=1000, help="launches of the ABFT fault campaign")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is a single-GPU library (no collectives); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from hpcdeepneuralnetworks_amd import blas
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    dev = "cuda"
+
+    def timed(fn, steps, warmup):
+        """Average ms per call over `steps` back-to-back launches on the current stream (HIP events on that stream)."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    def median_timed(fn, steps, warmup, batches=5):
+        return statistics.median(timed(fn, steps, warmup if b == 0 else 1) for b in range(batches))
+
+    def operands(M, N, K, seed):
+        a = torch.empty(M, K, device=dev)
+        b = torch.empty(K, N, device=dev)
+        c = torch.empty(M, N, device=dev)
+        blas.fill_uniform_matrix(a, M, K, seed)
+        blas.fill_uniform_matrix(b, K, N, seed + 1)
+        blas.fill_uniform_matrix(c, M, N, seed + 2)
+        return a, b, c
+
+    # ---------------- headline: SGEMM 6144^3, exactly K timed steps between two synchronisations
+    n = 6144
+    a, b, c = operands(n, n, n, 1)
+    flop = 2.0 * n * n * n
+    for _ in range(args.warmup):
+        blas.sgemm(n, n, n, a, b, c, 1.0, 0.0)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        blas.sgemm(n, n, n, a, b, c, 1.0, 0.0)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps
+    gflops = flop / (wall_ms * 1e-3) / 1e9
+    achieved_tflops = flop / (kern_ms * 1e-3) / 1e12
+
+    result = {
+        "metric": "sgemm_fp32_gflops_6144",
+        "value": round(gflops, 1),
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded counter-based uniform[-1,1), generated on the device)",
+        "config": {
+            "workload": "SGEMM row-major FP32 M=N=K=6144, lda=ldb=ldc=6144, alpha=1, beta=0 "
+                        "(largest size of the square sweep, the size the metric is quoted on)",
+            "timing": "back-to-back launches, no per-launch sync (the reference syncs around every launch)",
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(achieved_tflops, 2),
+            "peak": PEAK_FP32_MFMA_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
+            "traffic": None,
+            "kernel": "sgemm_kernel (one launch = 2*6144^3 flop)",
+            "kernel_ms": round(kern_ms, 4),
+        },
+    }
+
+    extras = {}
+    if not args.no_extras:
+        st, wu = max(args.steps // 2, 10), 3
+        # reference-style timing: device sync before and after every launch (kernel/sgemm/sgemm.cu:161-359)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            torch.cuda.synchronize()
+            blas.sgemm(n, n, n, a, b, c, 1.0, 0.0)
+            torch.cuda.synchronize()
+        extras["sgemm_6144_sync_bracketed_gflops"] = round(flop * 10 / (time.perf_counter() - t0) / 1e9, 1)
+        ms = median_timed(lambda: blas.sgemm(n, n, n, a, b, c, 1.0, 1.0), st, wu)
+        extras["sgemm_6144_beta1_gflops"] = round(flop / ms / 1e6, 1)
+        ms = median_timed(lambda: torch.matmul(a, b, out=c), st, wu)
+        extras["rocblas_via_torch_6144_gflops"] = round(flop / ms / 1e6, 1)
+        del a, b, c
+
+        sweep = {}
+        for m in (1024, 2048, 3072, 4096, 5120):
+            a, b, c = operands(m, m, m, 10)
+            ms = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0), st, wu)
+            sweep[str(m)] = round(2.0 * m ** 3 / ms / 1e6, 1)
+        extras["sgemm_square_gflops"] = sweep
+
+        # ---- ABFT at 4096^3: overhead vs plain SGEMM and the seeded single-fault campaign
+        m = 4096
+        a, b, c = operands(m, m, m, 20)
+        status = blas.ft_status_alloc(m, m)
+        tau = blas.ft_default_tau(m)
+        ms_plain = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0), st, wu)
+        ms_plain_same_tile = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0, tile=0, split_k=1), st, wu)
+        ms_ft = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status), st, wu)
+        extras["abft_4096"] = {
+            "sgemm_gflops": round(2.0 * m ** 3 / ms_plain / 1e6, 1),
+            "sgemm_same_tile_gflops": round(2.0 * m ** 3 / ms_plain_same_tile / 1e6, 1),
+            "ft_sgemm_gflops": round(2.0 * m ** 3 / ms_ft / 1e6, 1),
+            "overhead_pct_vs_sgemm": round((ms_ft - ms_plain) / ms_plain * 100.0, 2),
+            "overhead_pct_vs_same_tile_sgemm": round((ms_ft - ms_plain_same_tile) / ms_plain_same_tile * 100.0, 2),
+            "tau": tau,
+        }
+        ntiles = blas.ft_num_tiles(m, m)
+        blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status)
+        clean = blas.ft_status_numpy(status)
+        c_clean = c.clone()
+        rng = np.random.default_rng(2024)
+        detected = located = corrected = false_pos = 0
+        worst_fix = 0.0
+        t0 = time.perf_counter()
+        for _ in range(args.ft_launches):
+            tile, i, j = int(rng.integers(ntiles)), int(rng.integers(blas.FT_TILE_M)), int(rng.integers(blas.FT_TILE_N))
+            delta = float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-2, 2)))
+            blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, fault=(tile, i, j, delta), status=status)
+            s = blas.ft_status_numpy(status)
+            hit = s["flag"][tile] != 0
+            detected += int(hit)
+            located += int(s["flag"][tile] == 1 and s["row"][tile] == i and s["col"][tile] == j)
+            others = np.delete(s["flag"], tile)
+            false_pos += int(np.count_nonzero(others))
+            fix_err = float((c - c_clean).abs().max())
+            corrected += int(s["flag"][tile] == 1 and fix_err < 5e-3)
+            worst_fix = max(worst_fix, fix_err)
+        extras["abft_4096"].update({
+            "campaign_launches": args.ft_launches,
+            "detection_rate": detected / max(args.ft_launches, 1),
+            "location_rate": located / max(args.ft_launches, 1),
+            "correction_rate": corrected / max(args.ft_launches, 1),
+            "false_positive_tiles": false_pos,
+            "fault_free_flags": int(np.count_nonzero(clean["flag"])),
+            "fault_free_max_residual": float(clean["max_clean_residual"].max()),
+            "worst_abs_error_after_correction": worst_fix,
+            "campaign_seconds": round(time.perf_counter() - t0, 2),
+        })
+        del a, b, c, c_clean
+
+        # ---- SAXPY / SDOT at n = 2^28 (12 and 8 algorithmic bytes per element)
+        nv = 1 << 28
+        x = torch.empty(nv, device=dev)
+        y = torch.empty(nv, device=dev)
+        out = torch.zeros(1, device=dev)
+        blas.fill_uniform(x, 30)
+        blas.fill_uniform(y, 31)
+        ms = median_timed(lambda: blas.saxpy(nv, 2.5, x, y), 20, 3)
+        extras["saxpy_2p28"] = {"GBps": round(12.0 * nv / ms / 1e6, 1), "frac_hbm_peak": round(12.0 * nv / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                "us": round(ms * 1e3, 1)}
+        ms = median_timed(lambda: blas.sdot(nv, x, y, out), 20, 3)
+        extras["sdot_2p28"] = {"GBps": round(8.0 * nv / ms / 1e6, 1), "frac_hbm_peak": round(8.0 * nv / ms / 1e6 / PEAK_HBM_GBS, 4),
+                               "us": round(ms * 1e3, 1)}
+        z = torch.empty_like(x)
+        ms = median_timed(lambda: z.copy_(x), 20, 3)
+        extras["device_copy_2p28_GBps"] = round(8.0 * nv / ms / 1e6, 1)
+        del z
+        nt = (1 << 20) + 7
+        ms = median_timed(lambda: blas.saxpy(nt, 2.5, x, y), 50, 5)
+        extras["saxpy_2p20_plus_7_GBps"] = round(12.0 * nt / ms / 1e6, 1)
+        ms = median_timed(lambda: blas.sdot(nt, x, y, out), 50, 5)
+        extras["sdot_2p20_plus_7_GBps"] = round(8.0 * nt / ms / 1e6, 1)
+        del x, y
+        result["extras"] = extras
+
+    # ---------------- CPU baseline: the oracle's restatement of the reference's cpu_gemm, one thread, bounded sample
+    if not args.no_cpu:
+        import oracle
+
+        m = 1024
+        ha = oracle.fill_uniform_matrix(m, m, 1)
+        hb = oracle.fill_uniform_matrix(m, m, 2)
+        hc = np.zeros((m, m), dtype=np.float32)
+        t0 = time.perf_counter()
+        oracle.cpu_gemm(1.0, 0.0, ha, hb, m, hc)
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {
+            "value": round(2.0 * m ** 3 / dt / 1e9, 3),
+            "unit": "GFLOP/s",
+            "cores": 1,
+            "kind": "port",
+            "sample": f"oracle cpu_gemm (naive i-j-k, float accumulator, reference utils/utils.cu:93-103) at "
+                      f"M=N=K=1024 (the reference's CPU-runnable configuration), one run, {dt:.2f} s; "
+                      f"host has {os.cpu_count()} logical CPUs",
+        }
+        if not args.no_extras:
+            nv = 1 << 26
+            hx, hy = oracle.fill_uniform(nv, 3), oracle.fill_uniform(nv, 4)
+            t0 = time.perf_counter()
+            oracle.saxpy(2.5, hx, hy)
+            t1 = time.perf_counter()
+            oracle.sdot_f32(hx, hy)
+            t2 = time.perf_counter()
+            result["cpu_baseline"]["saxpy_GBps_1thread_2p26"] = round(12.0 * nv / (t1 - t0) / 1e9, 2)
+            result["cpu_baseline"]["sdot_GBps_1thread_2p26"] = round(8.0 * nv / (t2 - t1) / 1e9, 2)
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

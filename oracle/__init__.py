@@ -83,6 +83,12 @@ def _load():
     lib.oracle_sdot_f64.argtypes = [C.c_int64, fp, fp]
     lib.oracle_sdot_f32.restype = C.c_float
     lib.oracle_sdot_f32.argtypes = [C.c_int64, fp, fp]
+    lib.oracle_tile_acc.restype = None
+    lib.oracle_tile_acc.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp]
+    lib.oracle_abft_reference_checksums.restype = None
+    lib.oracle_abft_reference_checksums.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, dp, dp]
+    lib.oracle_abft_observe.restype = None
+    lib.oracle_abft_observe.argtypes = [C.c_int, C.c_int, fp, C.c_int, dp, dp, dp, dp]
     lib.oracle_abft_residuals.restype = None
     lib.oracle_abft_residuals.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, dp, dp]
     lib.oracle_abft_decide.restype = C.c_float
@@ -169,6 +175,28 @@ def sdot_f64(x: np.ndarray, y: np.ndarray) -> float:
 
 def sdot_f32(x: np.ndarray, y: np.ndarray) -> float:
     return float(_load().oracle_sdot_f32(x.size, _f(x), _f(y)))
+
+
+def tile_acc(a_tile, lda, b_tile, ldb, tm, tn, K) -> np.ndarray:
+    """Float-accumulated (k ascending, fused) product block of one tile, tm x tn packed."""
+    acc = np.empty((tm, tn), dtype=np.float32)
+    _load().oracle_tile_acc(tm, tn, K, _f(a_tile), lda, _f(b_tile), ldb, _f(acc))
+    return acc
+
+
+def abft_reference_checksums(a_tile, lda, b_tile, ldb, tm, tn, K):
+    cr = np.empty(tm, dtype=np.float64)
+    cc = np.empty(tn, dtype=np.float64)
+    _load().oracle_abft_reference_checksums(tm, tn, K, _f(a_tile), lda, _f(b_tile), ldb, _d(cr), _d(cc))
+    return cr, cc
+
+
+def abft_observe(acc, ldacc, cr_ref, cc_ref):
+    tm, tn = len(cr_ref), len(cc_ref)
+    dr = np.empty(tm, dtype=np.float64)
+    dc = np.empty(tn, dtype=np.float64)
+    _load().oracle_abft_observe(tm, tn, _f(acc), ldacc, _d(cr_ref), _d(cc_ref), _d(dr), _d(dc))
+    return dr, dc
 
 
 def abft_residuals(a_tile, lda, b_tile, ldb, acc, ldacc, tm, tn, K):

@@ -178,20 +178,33 @@ typedef struct {
     float max_clean_residual;/* largest |residual| among the lines judged clean */
 } oracle_ft_status;
 
-/* Steps 1-3 of the online-ABFT scheme for one output tile
- * (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:67-102,442-474 encode;
- * :147-171 observe; :200-262 residual; explicit form in
- * ft_sgemm_large.cuh:372-436).  acc is the tile's accumulator block
- * (tm x tn, row stride ldacc) BEFORE the alpha/beta epilogue; A and B point
- * at the tile's first row / first column.  Reference checksums are formed
- * from A and B only:
+/* Accumulator block of one output tile as the model sees it: float
+ * accumulator, one fused multiply-add per k, k ascending (the arithmetic of
+ * one reference thread's `tab` FMA chain, kernel_13.cuh:55-81).  acc is
+ * tm x tn packed. */
+void oracle_tile_acc(int tm, int tn, int K, const float* A, int lda, const float* B, int ldb, float* acc) {
+    #pragma omp parallel for schedule(static)
+    for (int m = 0; m < tm; ++m) {
+        float* arow = acc + (size_t)m * tn;
+        for (int n = 0; n < tn; ++n) arow[n] = 0.0f;
+        for (int k = 0; k < K; ++k) {
+            float a = A[(size_t)m * lda + k];
+            const float* brow = B + (size_t)k * ldb;
+            for (int n = 0; n < tn; ++n) arow[n] = fmaf(a, brow[n], arow[n]);
+        }
+    }
+}
+
+/* Step 1 (encode) of the online-ABFT scheme for one output tile
+ * (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:67-102,442-474; explicit form in
+ * ft_sgemm_large.cuh:372-436): reference checksums formed from A and B only,
  *     cc_ref[n] = sum_k (sum_m A[m,k]) * B[k,n]      (= e^T A B)
  *     cr_ref[m] = sum_k A[m,k] * (sum_n B[k,n])      (= A B e)
- * and the residuals are reference minus observed line sums of acc. */
-void oracle_abft_residuals(int tm, int tn, int K, const float* A, int lda, const float* B, int ldb,
-                           const float* acc, int ldacc, double* dr, double* dc) {
-    double* cc_ref = (double*)calloc((size_t)tn, sizeof(double));
-    double* cr_ref = (double*)calloc((size_t)tm, sizeof(double));
+ * A and B point at the tile's first row / first column. */
+void oracle_abft_reference_checksums(int tm, int tn, int K, const float* A, int lda, const float* B,
+                                     int ldb, double* cr_ref, double* cc_ref) {
+    for (int m = 0; m < tm; ++m) cr_ref[m] = 0.0;
+    for (int n = 0; n < tn; ++n) cc_ref[n] = 0.0;
     for (int k = 0; k < K; ++k) {
         double a_c = 0.0, b_r = 0.0;
         for (int m = 0; m < tm; ++m) a_c += (double)A[(size_t)m * lda + k];
@@ -199,6 +212,13 @@ void oracle_abft_residuals(int tm, int tn, int K, const float* A, int lda, const
         for (int n = 0; n < tn; ++n) cc_ref[n] += a_c * (double)B[(size_t)k * ldb + n];
         for (int m = 0; m < tm; ++m) cr_ref[m] += (double)A[(size_t)m * lda + k] * b_r;
     }
+}
+
+/* Steps 2-3 (observe, residual; ft_sgemm_huge.cuh:147-171, :200-262):
+ * residual = reference checksum minus the line sum of the accumulator block
+ * acc (tm x tn, row stride ldacc) taken BEFORE the alpha/beta epilogue. */
+void oracle_abft_observe(int tm, int tn, const float* acc, int ldacc, const double* cr_ref,
+                         const double* cc_ref, double* dr, double* dc) {
     for (int m = 0; m < tm; ++m) {
         double s = 0.0;
         for (int n = 0; n < tn; ++n) s += (double)acc[(size_t)m * ldacc + n];
@@ -209,7 +229,15 @@ void oracle_abft_residuals(int tm, int tn, int K, const float* A, int lda, const
         for (int m = 0; m < tm; ++m) s += (double)acc[(size_t)m * ldacc + n];
         dc[n] = cc_ref[n] - s;
     }
-    free(cc_ref);
+}
+
+/* Steps 1-3 in one call. */
+void oracle_abft_residuals(int tm, int tn, int K, const float* A, int lda, const float* B, int ldb,
+                           const float* acc, int ldacc, double* dr, double* dc) {
+    double* cr_ref = (double*)malloc(sizeof(double) * (size_t)(tm + tn));
+    double* cc_ref = cr_ref + tm;
+    oracle_abft_reference_checksums(tm, tn, K, A, lda, B, ldb, cr_ref, cc_ref);
+    oracle_abft_observe(tm, tn, acc, ldacc, cr_ref, cc_ref, dr, dc);
     free(cr_ref);
 }
 

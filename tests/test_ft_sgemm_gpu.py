@@ -1,0 +1,183 @@
+"""GPU parity of the fused ABFT SGEMM against the CPU model of the reference's checksum logic.
+
+Values: same 1e-5 componentwise criterion as plain SGEMM (after correction).  Decisions (flag, located row and
+column, number of flagged lines) must equal the CPU model's exactly on the same seeded faults.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+DECISION_FIELDS = ("flag", "row", "col", "n_bad_rows", "n_bad_cols")
+
+
+def _run(blas, oracle_mod, M, N, K, alpha, beta, tau, fault, seed=400, lda=None, ldb=None, ldc=None):
+    lda, ldb, ldc = lda or K, ldb or N, ldc or N
+    a = oracle_mod.fill_uniform_matrix(M, K, seed, ld=lda)
+    b = oracle_mod.fill_uniform_matrix(K, N, seed + 1, ld=ldb)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, seed + 2, ld=ldc)
+    da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+    status = blas.ft_status_alloc(M, N)
+    blas.ft_sgemm(M, N, K, da, db, dc, alpha, beta, tau=tau, fault=fault, status=status)
+    st = blas.ft_status_numpy(status)
+    c = dc.cpu().numpy()
+    # model: a, b with zeroed padding so that the model never multiplies NaN padding (it indexes with ld too)
+    c_model = c0.copy()
+    st_model = oracle_mod.ft_sgemm(M, N, K, a, lda, b, ldb, c_model, ldc, alpha, beta, blas.FT_TILE_M, blas.FT_TILE_N,
+                                   tau, fault)
+    return a, b, c0, c, st, c_model, st_model
+
+
+def _assert_values(oracle_mod, M, N, K, a, b, c0, c, alpha, beta):
+    ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, a.shape[1], b, b.shape[1], c0, c0.shape[1], alpha, beta)
+    err = oracle_mod.gemm_max_err(N, c, c.shape[1], ref, den)
+    assert err <= TOL, err
+    assert np.all(np.isnan(c[:, N:]))
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 128, 64), (512, 384, 320), (300, 200, 100), (1, 1, 1), (257, 129, 17), (1024, 1024, 1024)])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, -1.5)])
+def test_fault_free_matches_model_and_oracle(blas, oracle_mod, M, N, K, alpha, beta):
+    tau = blas.ft_default_tau(K)
+    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, alpha, beta, tau, None)
+    _assert_values(oracle_mod, M, N, K, a, b, c0, c, alpha, beta)
+    for f in DECISION_FIELDS:
+        assert np.array_equal(st[f], st_model[f]), f
+    assert np.all(st["flag"] == 0) and np.all(st["row"] == -1) and np.all(st["col"] == -1)
+    # fault-free residuals are rounding noise, far below the threshold
+    assert st["max_clean_residual"].max() < 0.5 * tau
+
+
+def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod):
+    """The reference's only fault experiment: +1.0 into local element (m=0, n=1) of a tile, threshold 0.1
+    (ft_sgemm_huge.cuh:30,40,145) -> row 0 / column 1 located, 1.0 removed."""
+    M, N, K = 512, 256, 256
+    for tile in range(4):
+        a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, 0.1, (tile, 0, 1, 1.0))
+        exp = [0, 0, 0, 0]
+        exp[tile] = 1
+        assert st["flag"].tolist() == exp
+        assert (st["row"][tile], st["col"][tile]) == (0, 1)
+        assert round(-float(st["row_residual"][tile])) == 1 and abs(st["row_residual"][tile] + 1.0) < 1e-3
+        assert abs(st["col_residual"][tile] + 1.0) < 1e-3
+        _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 0.0)
+
+
+def test_seeded_faults_decisions_equal_cpu_model(blas, oracle_mod):
+    # ragged problem: 3 x 3 tiles, last row/column of tiles clipped; padded leading dimensions
+    M, N, K = 600, 300, 512
+    tau = blas.ft_default_tau(K)
+    rng = np.random.default_rng(7)
+    ntiles = blas.ft_num_tiles(M, N)
+    assert ntiles == 9
+    for trial in range(24):
+        tile = int(rng.integers(ntiles))
+        tm = min(blas.FT_TILE_M, M - (tile // 3) * blas.FT_TILE_M)
+        tn = min(blas.FT_TILE_N, N - (tile % 3) * blas.FT_TILE_N)
+        i, j = int(rng.integers(tm)), int(rng.integers(tn))
+        delta = float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-2, 2)))
+        fault = (tile, i, j, delta)
+        a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 1.0, tau, fault,
+                                                  seed=500 + trial, lda=K + 4, ldb=N + 4, ldc=N + 8)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (fault, f, st[f], st_model[f])
+        assert st["flag"][tile] == 1 and (st["row"][tile], st["col"][tile]) == (i, j), fault
+        assert abs(st["row_residual"][tile] + delta) < 2e-3 and abs(st["col_residual"][tile] + delta) < 2e-3
+        assert np.allclose(st["row_residual"], st_model["row_residual"], atol=2e-3)
+        _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 1.0)
+
+
+def test_fault_below_threshold_or_outside_matrix_is_not_flagged(blas, oracle_mod):
+    M, N, K = 300, 200, 256
+    tau = blas.ft_default_tau(K)
+    # far below the threshold: stays in C (documented behaviour), nothing flagged
+    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, tau, (0, 3, 5, tau * 0.1))
+    assert np.all(st["flag"] == 0) and np.array_equal(st["flag"], st_model["flag"])
+    # a fault aimed at a clipped-away element of an edge tile lands in zero padding that is never stored:
+    # it is detected and removed by both the device and the model, or ignored by both
+    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, tau, (3, 200, 100, 5.0))
+    _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 0.0)
+
+
+def test_many_flagged_lines_are_reported_uncorrectable(blas, oracle_mod):
+    """More than one faulty row or column cannot be located by row x column intersection: a threshold below the
+    rounding noise flags many lines, and the kernel must report flag 2 and leave the accumulators alone."""
+    M, N, K = 256, 128, 512
+    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, 1e-9, None)
+    assert st["flag"][0] == 2 and st["n_bad_rows"][0] > 1 and st["n_bad_cols"][0] > 1
+    assert (st["row"][0], st["col"][0]) == (-1, -1)
+    _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 0.0)
+
+
+class _TileModel:
+    """CPU model of one 256x128 tile at full K, cached so that each further fault on the tile costs O(tile)."""
+
+    def __init__(self, oracle_mod, a, b, K, N, tile, tm, tn, ntn):
+        m0, n0 = (tile // ntn) * tm, (tile % ntn) * tn
+        at, bt = a[m0:m0 + tm], b[:, n0:n0 + tn]
+        self.acc = oracle_mod.tile_acc(at, K, bt, N, tm, tn, K)
+        self.cr, self.cc = oracle_mod.abft_reference_checksums(at, K, bt, N, tm, tn, K)
+        self.oracle = oracle_mod
+
+    def decide(self, i, j, delta, tau):
+        acc = self.acc.copy()
+        acc[i, j] += np.float32(delta)
+        dr, dc = self.oracle.abft_observe(acc, acc.shape[1], self.cr, self.cc)
+        return self.oracle.abft_decide(dr, dc, tau)
+
+
+def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod):
+    """BASELINE config 4: M=N=K=4096, alpha=1, beta=0, one seeded fault (tile, i, j, magnitude in [1e-2, 1e2],
+    random sign) per launch.  Every launch: detected, located at the injected element, corrected, no other tile
+    flagged; decisions equal the CPU model's for every launch (the model is evaluated on the faulted tile)."""
+    M = N = K = 4096
+    launches = 1000
+    dev = "cuda"
+    da, db = torch.empty(M, K, device=dev), torch.empty(K, N, device=dev)
+    dc = torch.zeros(M, N, device=dev)
+    blas.fill_uniform_matrix(da, M, K, 20)
+    blas.fill_uniform_matrix(db, K, N, 21)
+    a = oracle_mod.fill_uniform_matrix(M, K, 20)
+    b = oracle_mod.fill_uniform_matrix(K, N, 21)
+    tau = blas.ft_default_tau(K)
+    status = blas.ft_status_alloc(M, N)
+    ntiles, ntn = blas.ft_num_tiles(M, N), N // blas.FT_TILE_N
+    assert ntiles == 512
+
+    blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=tau, status=status)
+    clean = blas.ft_status_numpy(status)
+    assert np.count_nonzero(clean["flag"]) == 0          # no false positives on the fault-free run
+    assert clean["max_clean_residual"].max() < 0.6 * tau
+    c_clean = dc.clone()
+    plain = torch.zeros(M, N, device=dev)
+    blas.sgemm(M, N, K, da, db, plain, 1.0, 0.0, tile=0, split_k=1)
+    assert torch.equal(plain, c_clean)                   # fault-free ABFT output is bit-identical to plain SGEMM
+
+    rng = np.random.default_rng(2024)
+    models = {}
+    worst_err = 0.0
+    for launch in range(launches):
+        tile = int(rng.integers(ntiles))
+        i, j = int(rng.integers(blas.FT_TILE_M)), int(rng.integers(blas.FT_TILE_N))
+        delta = float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-2, 2)))
+        blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=tau, fault=(tile, i, j, delta), status=status)
+        st = blas.ft_status_numpy(status)
+        assert st["flag"][tile] == 1, (launch, tile, i, j, delta, st[tile])
+        assert (st["row"][tile], st["col"][tile]) == (i, j), (launch, tile, i, j, delta, st[tile])
+        assert np.count_nonzero(st["flag"]) == 1, (launch, "false positive elsewhere")
+        # correction restores the fault-free result to within the checksum noise (<< 1e-5 * (|A||B|)_ij ~ 1e-2)
+        diff = (dc - c_clean).abs()
+        err = float(diff.max())
+        worst_err = max(worst_err, err)
+        assert err < 4e-3, (launch, err)
+        assert int(torch.count_nonzero(diff)) <= 1
+        if tile not in models:
+            models[tile] = _TileModel(oracle_mod, a, b, K, N, tile, blas.FT_TILE_M, blas.FT_TILE_N, ntn)
+        st_model, fix_model = models[tile].decide(i, j, delta, tau)
+        for f in DECISION_FIELDS:
+            assert st[f][tile] == st_model[f], (launch, f, st[tile], st_model)
+        assert abs(float(st["row_residual"][tile]) - fix_model) < 3e-3
+    print(f"campaign: {launches} launches, worst |C - C_clean| after correction {worst_err:.3e}, "
+          f"fault-free max residual {clean['max_clean_residual'].max():.3e}, tau {tau:.1e}")
