@@ -14,31 +14,33 @@ struct TileConfig {
     float rel_speed;  // measured steady-state throughput relative to the best configuration
 };
 
-#define HPCDNN_TILE(BM, BN, BK, WGM, WGN, STAGES, OCC, SPEED)                                   \
-    {                                                                                            \
-        BM, BN, BK, OCC, gemm_lds_bytes<BM, BN, BK, STAGES>(),                                   \
-            sgemm_kernel<BM, BN, BK, WGM, WGN, STAGES, false, false, OCC>,                       \
-            sgemm_kernel<BM, BN, BK, WGM, WGN, STAGES, true, false, OCC>, SPEED                  \
+#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, RESIDENT, SPEED)                                              \
+    {                                                                                                    \
+        BM, BN, kGemmBK, RESIDENT, gemm_lds_bytes<BM, BN>(), sgemm_kernel<BM, BN, WGM, WGN, false, false, OCC>, \
+            sgemm_kernel<BM, BN, WGM, WGN, true, false, OCC>, SPEED                                       \
     }
 
 // The counterpart of the reference's small/medium/large/tall/wide/huge shape
 // table (kernel/ft_sgemm/code_gen/main.py:8-16), re-derived for 32x32 MFMA
-// blocks and four 64-lane waves per workgroup.
+// blocks and four 64-lane waves per workgroup.  RESIDENT = workgroups that fit
+// on one CU (registers and LDS); SPEED = measured steady-state fraction of the
+// FP32 MFMA peak.
 static const TileConfig kTiles[] = {
-    HPCDNN_TILE(256, 128, 16, 2, 2, 2, 2, 1.00f),  // 0 huge
-    HPCDNN_TILE(128, 128, 16, 2, 2, 2, 2, 0.90f),  // 1 large
-    HPCDNN_TILE(128, 64, 16, 2, 2, 2, 2, 0.75f),   // 2 tall
-    HPCDNN_TILE(64, 128, 16, 2, 2, 2, 2, 0.75f),   // 3 wide
-    HPCDNN_TILE(64, 64, 16, 2, 2, 2, 4, 0.55f),    // 4 medium
-    HPCDNN_TILE(256, 128, 32, 2, 2, 2, 1, 1.00f),  // 5 huge, deep K step
-    HPCDNN_TILE(256, 256, 16, 2, 2, 2, 1, 1.00f),  // 6 giant
-    HPCDNN_TILE(192, 256, 16, 2, 2, 2, 1, 1.00f),  // 7 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
+    HPCDNN_TILE(256, 128, 2, 2, 2, 2, 0.93f),  // 0 huge (the ABFT tile)
+    HPCDNN_TILE(128, 128, 2, 2, 2, 3, 0.90f),  // 1 large
+    HPCDNN_TILE(128, 64, 2, 2, 2, 4, 0.80f),   // 2 tall
+    HPCDNN_TILE(64, 128, 2, 2, 2, 4, 0.80f),   // 3 wide
+    HPCDNN_TILE(64, 64, 2, 2, 4, 8, 0.65f),    // 4 medium
+    HPCDNN_TILE(256, 256, 2, 2, 1, 1, 0.945f), // 5 giant
+    HPCDNN_TILE(192, 256, 2, 2, 1, 1, 0.94f),  // 6 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
+    HPCDNN_TILE(256, 192, 2, 2, 1, 1, 0.93f),  // 7
+    HPCDNN_TILE(128, 256, 2, 2, 2, 2, 0.93f),  // 8
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 constexpr int kFtTile = 0;  // 256 x 128, matches HPCDNN_FT_TILE_M/N
-static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, 16, 2, 2, 2, false, true, 2>;
-static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, 16, 2, 2, 2, true, true, 2>;
+static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, 2, 2, false, true, 2>;
+static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, 2, 2, true, true, 2>;
 
 static int device_cus() {
     static int cus = 0;
@@ -105,6 +107,9 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes) 
     return best;
 }
 
+constexpr int kMaxLda = (1 << 21) - 64;   // 256 * lda * 4 < 2^31
+constexpr int kMaxLdb = (1 << 25) - 1024;  // 16 * ldb * 4 + row < 2^31
+
 static int check_gemm_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
     if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
     if (lda < (K > 1 ? K : 1) || ldb < (N > 1 ? N : 1) || ldc < (N > 1 ? N : 1)) return HPCDNN_ERR_INVALID_VALUE;
@@ -112,6 +117,8 @@ static int check_gemm_args(int M, int N, int K, const float* A, int lda, const f
     if (M > 0 && N > 0 && K > 0 && (!A || !B)) return HPCDNN_ERR_INVALID_VALUE;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) & 3u)
         return HPCDNN_ERR_INVALID_VALUE;
+    // byte offsets inside one tile are 32-bit: 256 rows of A, 16 rows of B
+    if (lda > kMaxLda || ldb > kMaxLdb) return HPCDNN_ERR_INVALID_VALUE;
     return HPCDNN_OK;
 }
 
@@ -125,14 +132,14 @@ static GemmArgs make_args(int M, int N, int K, const float* A, int lda, const fl
     a.tiles_n = static_cast<int>(ceil_div(N, cfg.bn));
     a.k_chunk = static_cast<int>(ceil_div(K > 0 ? K : 1, cfg.bk)) * cfg.bk;
     a.partial = nullptr;
-    a.vec_a = ((reinterpret_cast<uintptr_t>(A) & 15u) == 0 && lda % 4 == 0) ? 1 : 0;
-    a.vec_b = ((reinterpret_cast<uintptr_t>(B) & 15u) == 0 && ldb % 4 == 0) ? 1 : 0;
     a.fault_tile = -1;
     return a;
 }
 
-static bool needs_edge(const GemmArgs& a, const TileConfig& cfg, int k_slice_len_multiple_of_bk) {
-    return !(a.M % cfg.bm == 0 && a.N % cfg.bn == 0 && a.K % cfg.bk == 0 && k_slice_len_multiple_of_bk && a.vec_a && a.vec_b);
+// The ragged-tile kernel masks the K tail and the columns past N; full tiles with K a multiple of the K step
+// (per slice, which k_chunk guarantees for all but the last) skip that work.
+static bool needs_edge(const GemmArgs& a, const TileConfig& cfg) {
+    return !(a.M % cfg.bm == 0 && a.N % cfg.bn == 0 && a.K % cfg.bk == 0);
 }
 
 static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
@@ -163,7 +170,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         split = static_cast<int>(ceil_div(K, a.k_chunk));  // drop empty slices
         if (split > 1) a.partial = static_cast<float*>(ws);
     }
-    const bool edge = needs_edge(a, cfg, 1);
+    const bool edge = needs_edge(a, cfg);
     void (*fn)(const GemmArgs) = edge ? cfg.edge : cfg.plain;
     rc = enable_lds(fn, cfg.lds_bytes);
     if (rc != HPCDNN_OK) return rc;
@@ -235,7 +242,7 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
         a.fault_col = inject->col;
         a.fault_delta = inject->delta;
     }
-    const bool edge = needs_edge(a, cfg, 1);
+    const bool edge = needs_edge(a, cfg);
     void (*fn)(const GemmArgs) = edge ? kFtEdge : kFtPlain;
     rc = enable_lds(fn, cfg.lds_bytes);
     if (rc != HPCDNN_OK) return rc;

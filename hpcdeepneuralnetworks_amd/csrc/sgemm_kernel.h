@@ -2,16 +2,21 @@
 //
 // One workgroup of 256 threads (4 waves) owns a BM x BN tile of C; wave w owns
 // a (BM/WGM) x (BN/WGN) sub-tile made of 32x32 MFMA blocks whose accumulators
-// stay in registers for the whole K loop.  Per K step of BK the A tile
-// (BM x BK) and B tile (BK x BN) go HBM/L2 -> VGPR (16-byte loads, issued one
-// K step ahead) -> LDS -> MFMA operands.
+// stay in registers for the whole K loop.  K advances in steps of 16.
+//
+// Data path per K step: HBM/L2 -> VGPR with buffer_load_dwordx4 (the hardware
+// range check of the buffer descriptor returns 0 for rows past the end of the
+// matrix, so ragged tiles need no branches) -> LDS (ds_write_b128) -> operand
+// fragments (ds_read) -> MFMA.  Global loads run two K steps ahead of the
+// MFMAs that consume them, LDS is double buffered, fragments are double
+// buffered in registers.
 //
 // LDS layout (floats):
-//   A stage: [BM][BK + 4]   k contiguous, as in memory.  Lane (row r, half h)
+//   A stage: [BM][20]       k contiguous, as in memory.  Lane (row r, half h)
 //            reads 16 bytes = k {8g+4h .. 8g+4h+3}: one ds_read_b128 feeds four
-//            MFMA k-steps.  Row stride BK+4 spreads 16 consecutive rows over
-//            all banks.
-//   B stage: [BK][BN + 8]   n contiguous, as in memory; lane (col c, half h)
+//            MFMA k-steps.  Row stride 20 spreads 8 consecutive rows over all
+//            banks for that read.
+//   B stage: [16][BN + 8]   n contiguous, as in memory; lane (col c, half h)
 //            reads B[8g+4h+q][c] with ds_read_b32.  Stride BN+8 puts the two
 //            half-waves (rows 4 apart) on disjoint banks.
 // The MFMA k index is a permutation of the memory k index (lane half h of
@@ -21,9 +26,17 @@
 // Accumulator layout of one 32x32 block (16 VGPRs): register v of lane l holds
 // element (row 8*(v/4) + 4*(l/32) + v%4, col l%32).
 //
-// With FT = true the kernel is the fused online-ABFT variant: see the comment
-// at "Online ABFT encode" in the main loop and "ABFT verification" after it.
+// Instruction order in the main loop is fixed by hand: the MFMA pipe takes 64
+// cycles per instruction, and "side" instructions (fragment reads, global
+// loads, LDS writes, a few checksum VALU ops) are placed one group behind each
+// MFMA so that they issue while the matrix core is busy.  sched_barrier fences
+// keep the compiler from regrouping them.
+//
+// With FT = true the kernel is the fused online-ABFT variant: see "ABFT
+// encode" in the main loop and "ABFT verification" after it.
 #pragma once
+
+#include <type_traits>
 
 #include "common.h"
 
@@ -39,10 +52,8 @@ struct GemmArgs {
     int ldc;
     float alpha, beta;
     int tiles_m, tiles_n;
-    int k_chunk;     // K range of one grid.z slice, a multiple of BK (>= K when not split)
+    int k_chunk;     // K range of one grid.z slice, a multiple of 16 (>= K when not split)
     float* partial;  // split-K: [gridDim.z][M][N] raw accumulators; nullptr = write C directly
-    int vec_a;       // every in-range 4-float group of A is 16-byte aligned
-    int vec_b;
     // ABFT
     float tau;
     int fault_tile, fault_row, fault_col;
@@ -51,12 +62,21 @@ struct GemmArgs {
 };
 
 constexpr int kGemmThreads = 256;
+constexpr int kGemmBK = 16;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tiles share A and B panels
 
-template <int BM, int BN, int BK, int STAGES>
+template <int BM, int BN>
 constexpr size_t gemm_lds_bytes() {
-    return sizeof(float) * STAGES * (static_cast<size_t>(BM) * (BK + 4) + static_cast<size_t>(BK) * (BN + 8));
+    return sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8));
+}
+
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
 }
 
 // Workgroup id -> tile.  The hardware deals consecutive workgroup ids round-
@@ -78,10 +98,22 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
     tn = in_group / gsz;
 }
 
-template <int BM, int BN, int BK, int WGM, int WGN, int STAGES, bool EDGE, bool FT, int MIN_BLOCKS>
+// Raw buffer descriptor over [base, base + bytes): loads past the end return 0.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* base, int64_t bytes) {
+    const int64_t clipped = bytes < 0 ? 0 : (bytes > 0xFFFFFFFFll ? 0xFFFFFFFFll : bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, static_cast<int>(clipped), 0x00020000);
+}
+
+__device__ __forceinline__ v4f buffer_load_v4f(__amdgpu_buffer_rsrc_t rsrc, int byte_offset) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0);
+    return __builtin_bit_cast(v4f, v);
+}
+
+template <int BM, int BN, int WGM, int WGN, bool EDGE, bool FT, int MIN_BLOCKS>
 __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
+    constexpr int BK = kGemmBK;
     static_assert(WGM * WGN == kGemmThreads / kWave, "four waves per workgroup");
-    static_assert(BK % 8 == 0, "K step is consumed in groups of 8");
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 32, TN = WN / 32;
     static_assert(TM >= 1 && TN >= 1 && WM % 32 == 0 && WN % 32 == 0, "wave tile is made of 32x32 blocks");
@@ -90,11 +122,15 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
     constexpr int A_V4_PER_ROW = BK / 4, B_V4_PER_ROW = BN / 4;
     constexpr int A_SLOTS = BM * BK / 4 / kGemmThreads, B_SLOTS = BK * BN / 4 / kGemmThreads;
     static_assert(A_SLOTS >= 1 && B_SLOTS >= 1, "every thread stages at least one 16-byte group of A and of B");
-    static_assert(STAGES == 1 || STAGES == 2, "single or double buffered LDS");
+    static_assert((BM * BK) % (4 * kGemmThreads) == 0 && (BN * BK) % (4 * kGemmThreads) == 0,
+                  "tiles split evenly over the threads");
+    constexpr int NGL = A_SLOTS + B_SLOTS;  // global loads (and LDS writes) per thread per K step
+    constexpr int NRD = TM + TN;            // fragment read groups per half K step
+    constexpr int NMG = 4 * TM * TN;        // MFMAs per half K step (8 k values)
 
     extern __shared__ __align__(16) float smem[];
     float* const As = smem;
-    float* const Bs = smem + STAGES * A_STAGE;
+    float* const Bs = smem + 2 * A_STAGE;
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1), wave = tid / kWave;
@@ -108,81 +144,83 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
     const int kend = (p.K - kbeg < p.k_chunk) ? p.K : kbeg + p.k_chunk;
     const int nkt = (kend - kbeg + BK - 1) / BK;
 
-    // ---- staging slots: which 16-byte groups of the A and B tiles this thread moves
-    int a_row[A_SLOTS], a_kc[A_SLOTS], b_row[B_SLOTS], b_nc[B_SLOTS];
-    const float* a_ptr[A_SLOTS];
-    const float* b_ptr[B_SLOTS];
+    // ---- global -> register staging: which 16-byte groups of the A and B tiles this thread moves.
+    // Descriptors start at the tile's first element of the current K step and end with the matrix, so that
+    // rows m >= M of A and rows k >= K of B read as 0; the base moves forward by one K step per load.
+    const float* a_base = p.A + static_cast<int64_t>(m0) * p.lda + kbeg;
+    const float* b_base = p.B + static_cast<int64_t>(kbeg) * p.ldb + n0;
+    int64_t a_left = (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - kbeg)) * 4;  // bytes from a_base to the end of A
+    int64_t b_left = (static_cast<int64_t>(p.K - 1 - kbeg) * p.ldb + (p.N - n0)) * 4;
+    const int64_t b_step = static_cast<int64_t>(BK) * p.ldb;
+
+    int a_voff[A_SLOTS], a_lds[A_SLOTS], a_kc[A_SLOTS];
+    int b_voff[B_SLOTS], b_lds[B_SLOTS], b_row[B_SLOTS], b_nvalid[B_SLOTS];
 #pragma unroll
     for (int s = 0; s < A_SLOTS; ++s) {
         const int idx = tid + s * kGemmThreads;
-        a_row[s] = idx / A_V4_PER_ROW;
+        const int row = idx / A_V4_PER_ROW;
         a_kc[s] = (idx % A_V4_PER_ROW) * 4;
-        a_ptr[s] = p.A + static_cast<size_t>(m0 + a_row[s]) * p.lda + (kbeg + a_kc[s]);
+        a_voff[s] = (row * p.lda + a_kc[s]) * 4;
+        a_lds[s] = row * AS + a_kc[s];
     }
 #pragma unroll
     for (int s = 0; s < B_SLOTS; ++s) {
         const int idx = tid + s * kGemmThreads;
         b_row[s] = idx / B_V4_PER_ROW;
-        b_nc[s] = (idx % B_V4_PER_ROW) * 4;
-        b_ptr[s] = p.B + static_cast<size_t>(kbeg + b_row[s]) * p.ldb + (n0 + b_nc[s]);
+        const int nc = (idx % B_V4_PER_ROW) * 4;
+        b_voff[s] = (b_row[s] * p.ldb + nc) * 4;
+        b_lds[s] = b_row[s] * BS + nc;
+        b_nvalid[s] = p.N - (n0 + nc);  // columns of this group inside the matrix (may be <= 0 or >= 4)
     }
 
-    v4f ra[A_SLOTS], rb[B_SLOTS];
+    v4f ra[2][A_SLOTS], rb[2][B_SLOTS];  // two staging slots: K steps t+1 and t+2 are in flight while t is multiplied
+    int k_loaded = kbeg;                 // absolute k of the K step the next load call fetches
 
-    auto load_tile = [&](int k0) {  // k0: absolute k of the tile's first column; never touches memory outside A/B
-#pragma unroll
-        for (int s = 0; s < A_SLOTS; ++s) {
-            if (!EDGE) {
-                ra[s] = *reinterpret_cast<const v4f*>(a_ptr[s]);
-            } else {
-                v4f v = {0.f, 0.f, 0.f, 0.f};
-                const int gk = k0 + a_kc[s];
-                if (m0 + a_row[s] < p.M && gk < kend) {
-                    if (p.vec_a && gk + 4 <= kend) {
-                        v = *reinterpret_cast<const v4f*>(a_ptr[s]);
-                    } else {
-                        v.x = a_ptr[s][0];
-                        if (gk + 1 < kend) v.y = a_ptr[s][1];
-                        if (gk + 2 < kend) v.z = a_ptr[s][2];
-                        if (gk + 3 < kend) v.w = a_ptr[s][3];
-                    }
-                }
-                ra[s] = v;
+    // One staging load (part P of the K step at a_base/b_base) into slot S.
+    auto gload1 = [&](auto slot, auto part) {
+        constexpr int S = decltype(slot)::value, P = decltype(part)::value;
+        if constexpr (P < A_SLOTS) {
+            v4f v = buffer_load_v4f(make_rsrc(a_base, a_left), a_voff[P]);
+            if constexpr (EDGE) {  // columns k >= kend hold padding, the next slice, or the next row: force 0
+                const int left = kend - (k_loaded + a_kc[P]);
+                v.x = left > 0 ? v.x : 0.f;
+                v.y = left > 1 ? v.y : 0.f;
+                v.z = left > 2 ? v.z : 0.f;
+                v.w = left > 3 ? v.w : 0.f;
             }
-            a_ptr[s] += BK;
-        }
-#pragma unroll
-        for (int s = 0; s < B_SLOTS; ++s) {
-            if (!EDGE) {
-                rb[s] = *reinterpret_cast<const v4f*>(b_ptr[s]);
-            } else {
-                v4f v = {0.f, 0.f, 0.f, 0.f};
-                const int gn = n0 + b_nc[s];
-                if (k0 + b_row[s] < kend && gn < p.N) {
-                    if (p.vec_b && gn + 4 <= p.N) {
-                        v = *reinterpret_cast<const v4f*>(b_ptr[s]);
-                    } else {
-                        v.x = b_ptr[s][0];
-                        if (gn + 1 < p.N) v.y = b_ptr[s][1];
-                        if (gn + 2 < p.N) v.z = b_ptr[s][2];
-                        if (gn + 3 < p.N) v.w = b_ptr[s][3];
-                    }
-                }
-                rb[s] = v;
+            ra[S][P] = v;
+        } else {
+            constexpr int Q = P - A_SLOTS;
+            v4f v = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[Q]);
+            if constexpr (EDGE) {
+                const bool row_ok = k_loaded + b_row[Q] < kend;
+                v.x = (row_ok && b_nvalid[Q] > 0) ? v.x : 0.f;
+                v.y = (row_ok && b_nvalid[Q] > 1) ? v.y : 0.f;
+                v.z = (row_ok && b_nvalid[Q] > 2) ? v.z : 0.f;
+                v.w = (row_ok && b_nvalid[Q] > 3) ? v.w : 0.f;
             }
-            b_ptr[s] += static_cast<size_t>(BK) * p.ldb;
+            rb[S][Q] = v;
         }
     };
-
-    auto store_tile = [&](int stage) {
-        float* as = As + stage * A_STAGE;
-        float* bs = Bs + stage * B_STAGE;
-#pragma unroll
-        for (int s = 0; s < A_SLOTS; ++s) *reinterpret_cast<v4f*>(as + a_row[s] * AS + a_kc[s]) = ra[s];
-#pragma unroll
-        for (int s = 0; s < B_SLOTS; ++s) *reinterpret_cast<v4f*>(bs + b_row[s] * BS + b_nc[s]) = rb[s];
+    // After the last part of a K step: move to the next one, unless that would leave the slice (then the same
+    // step is simply fetched again; its data is never multiplied).
+    auto gload_advance = [&]() {
+        const bool more = k_loaded + BK < kend;
+        a_base += more ? BK : 0;
+        a_left -= more ? BK * 4 : 0;
+        b_base += more ? b_step : 0;
+        b_left -= more ? b_step * 4 : 0;
+        k_loaded += more ? BK : 0;
+    };
+    auto lstore1 = [&](auto slot, auto part, int stage) {
+        constexpr int S = decltype(slot)::value, P = decltype(part)::value;
+        if constexpr (P < A_SLOTS)
+            *reinterpret_cast<v4f*>(As + stage * A_STAGE + a_lds[P]) = ra[S][P];
+        else
+            *reinterpret_cast<v4f*>(Bs + stage * B_STAGE + b_lds[P - A_SLOTS]) = rb[S][P - A_SLOTS];
     };
 
+    // ---- LDS -> fragment registers -> MFMA
     v16f acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -191,108 +229,173 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // ABFT reference checksums (see abft comment below); dead code when !FT.
+    v4f fa[2][TM];  // fragment buffer b holds the operands of half K step g = b
+    float fb[2][TN][4];
+    const int a_frag_off = (wm * WM + lr) * AS + lh * 4;
+    const int b_frag_off = (lh * 4) * BS + wn * WN + lr;
+
+    auto fread1 = [&](auto buf, auto part, int stage, int g) {  // part < TM: A block `part`; else B block `part - TM`
+        constexpr int Bf = decltype(buf)::value, P = decltype(part)::value;
+        if constexpr (P < TM) {
+            fa[Bf][P] = *reinterpret_cast<const v4f*>(As + stage * A_STAGE + a_frag_off + g * 8 + P * 32 * AS);
+        } else {
+            constexpr int j = P - TM;
+            const float* bs = Bs + stage * B_STAGE + b_frag_off + g * 8 * BS + j * 32;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) fb[Bf][j][q] = bs[q * BS];
+        }
+    };
+    auto mfma1 = [&](auto buf, auto idx) {
+        constexpr int Bf = decltype(buf)::value, I = decltype(idx)::value;
+        constexpr int q = I / (TM * TN), i = (I / TN) % TM, j = I % TN;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[Bf][i][q], fb[Bf][j][q], acc[i][j], 0, 0, 0);
+    };
+
+    // ---- ABFT encode (dead code when !FT).
+    // The reference forms e^T A and B e on its global->shared staging registers with warp shuffles and adds the
+    // rank-1 products into spare shared memory (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:442-474).  Here each
+    // wave works on the operand fragments it already holds: for its WM rows, its WN columns and the 4 k values of
+    // its lane half,
+    //     acs[q] = sum over the wave's rows of A[., k]      (e^T A)
+    //     brs[q] = sum over the wave's columns of B[k, .]   (B e)
+    // then cc += acs * B[k, n] (column n = lane) and cr += A[m, k] * brs (row m = lane).  The 4-term partial is
+    // formed in FP32 and added to an FP64 running sum, so the reference checksums carry no drift of their own
+    // over a long K.  The work is cut into pieces of a few VALU instructions, one piece behind an MFMA.
     double cc_ref[TN], cr_ref[TM];
 #pragma unroll
     for (int j = 0; j < TN; ++j) cc_ref[j] = 0.0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) cr_ref[i] = 0.0;
-
-    const int a_frag_off = (wm * WM + lr) * AS + lh * 4;
-    const int b_frag_off = (lh * 4) * BS + wn * WN + lr;
-
-    auto compute_tile = [&](int stage) {
-        const float* as = As + stage * A_STAGE + a_frag_off;
-        const float* bs = Bs + stage * B_STAGE + b_frag_off;
+    float e_acs[4], e_brs[4], e_sa[4], e_sb[4], cc_lo[TN], cr_lo[TM];
+    constexpr int NENC = FT ? (4 * 5 + 1) : 0;  // pieces per half K step: 5 per k value + the FP64 flush
+    auto encode1 = [&](auto buf, auto piece) {
+        constexpr int Bf = decltype(buf)::value, E = decltype(piece)::value;
+        if constexpr (E < 20) {
+            constexpr int q = E / 5, ph = E % 5;
+            if constexpr (ph == 0) {  // in-lane sums over the wave tile's blocks
+                float a = fa[Bf][0][q], b = fb[Bf][0][q];
 #pragma unroll
-        for (int g = 0; g < BK / 8; ++g) {
-            v4f a[TM];
-            float b[TN][4];
+                for (int i = 1; i < TM; ++i) a += fa[Bf][i][q];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const v4f*>(as + i * 32 * AS + g * 8);
+                for (int j = 1; j < TN; ++j) b += fb[Bf][j][q];
+                e_acs[q] = a;
+                e_brs[q] = b;
+            } else if constexpr (ph == 1) {  // butterfly inside quads
+                e_acs[q] += dpp_mov<kDppXor1>(e_acs[q]);
+                e_brs[q] += dpp_mov<kDppXor1>(e_brs[q]);
+                e_acs[q] += dpp_mov<kDppXor2>(e_acs[q]);
+                e_brs[q] += dpp_mov<kDppXor2>(e_brs[q]);
+            } else if constexpr (ph == 2) {  // inside rows of 16, then fetch the partner row's sum
+                e_acs[q] += dpp_mov<kDppHalfMirror>(e_acs[q]);
+                e_brs[q] += dpp_mov<kDppHalfMirror>(e_brs[q]);
+                e_acs[q] += dpp_mov<kDppMirror>(e_acs[q]);
+                e_brs[q] += dpp_mov<kDppMirror>(e_brs[q]);
+                e_sa[q] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_acs[q]), 0x401F));
+                e_sb[q] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_brs[q]), 0x401F));
+            } else if constexpr (ph == 3) {  // every lane of the half now holds the sum over 32 lanes
+                e_acs[q] += e_sa[q];
+                e_brs[q] += e_sb[q];
+            } else {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) b[j][q] = bs[(g * 8 + q) * BS + j * 32];
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
+                for (int j = 0; j < TN; ++j)
+                    cc_lo[j] = (q == 0) ? e_acs[q] * fb[Bf][j][q] : __builtin_fmaf(e_acs[q], fb[Bf][j][q], cc_lo[j]);
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][q], b[j][q], acc[i][j], 0, 0, 0);
-
-            if constexpr (FT) {
-                // Online ABFT encode (the reference forms e^T A and B e on its
-                // global->shared staging registers with warp shuffles and adds
-                // the rank-1 products into spare shared memory,
-                // kernel/ft_sgemm/include/ft_sgemm_huge.cuh:442-474).  Here each
-                // wave works on the operand fragments it already holds: for
-                // its WM rows and WN columns and the 4 k values of its lane half,
-                //   acs[q] = sum over the wave's rows of A[., k]     (e^T A)
-                //   brs[q] = sum over the wave's columns of B[k, .]  (B e)
-                // then cc += acs*B[k, n] (column n = lane) and cr += A[m, k]*brs
-                // (row m = lane).  The 4-term partial is formed in FP32 and
-                // added to an FP64 running sum so that the reference checksums
-                // carry no drift of their own over a long K.
-                float cc_lo[TN], cr_lo[TM];
-#pragma unroll
-                for (int j = 0; j < TN; ++j) cc_lo[j] = 0.f;
-#pragma unroll
-                for (int i = 0; i < TM; ++i) cr_lo[i] = 0.f;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    float acs = a[0][q], brs = b[0][q];
-#pragma unroll
-                    for (int i = 1; i < TM; ++i) acs += a[i][q];
-#pragma unroll
-                    for (int j = 1; j < TN; ++j) brs += b[j][q];
-                    acs = half32_allsum(acs);
-                    brs = half32_allsum(brs);
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) cc_lo[j] = __builtin_fmaf(acs, b[j][q], cc_lo[j]);
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) cr_lo[i] = __builtin_fmaf(a[i][q], brs, cr_lo[i]);
-                }
-#pragma unroll
-                for (int j = 0; j < TN; ++j) cc_ref[j] += static_cast<double>(cc_lo[j]);
-#pragma unroll
-                for (int i = 0; i < TM; ++i) cr_ref[i] += static_cast<double>(cr_lo[i]);
+                    cr_lo[i] = (q == 0) ? fa[Bf][i][q] * e_brs[q] : __builtin_fmaf(fa[Bf][i][q], e_brs[q], cr_lo[i]);
             }
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) cc_ref[j] += static_cast<double>(cc_lo[j]);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) cr_ref[i] += static_cast<double>(cr_lo[i]);
         }
     };
 
-    // ---- main loop: global loads run one K step ahead of the MFMAs
-    if (nkt > 0) {
-        load_tile(kbeg);
-        store_tile(0);
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+
+    // One K step.  On entry: LDS stage kt&1 holds step kt, fragment buffer 0 holds its first half, staging slot
+    // `sl_next` holds step kt+1 (possibly still in flight), slot `sl_free` is free.
+    //   first half : MFMAs on buffer 0 | read second-half fragments into buffer 1, fetch step kt+2 into sl_free,
+    //                write step kt+1 from sl_next into the other LDS stage
+    //   barrier    : the other stage is complete; nobody reads this stage's fragments any more
+    //   second half: MFMAs on buffer 1 | read the first-half fragments of step kt+1 into buffer 0
+    // Work past the end of the slice (kt+1, kt+2 >= nkt) moves duplicate data that is never multiplied, which
+    // keeps the loop free of branches (and lets the loads stay two steps ahead).
+    auto step = [&](auto sl_next, auto sl_free, int kt) {
+        const int st = kt & 1;
+        constexpr int MEM0 = NRD + 2 * NGL;  // memory side ops of the first half
+        constexpr int NS0 = MEM0 + NENC;
+        constexpr int NS1 = NRD + NENC;
+        static_for<NMG>([&](auto m) {
+            constexpr int Mi = decltype(m)::value;
+            mfma1(S0{}, m);
+            // side ops k_lo .. k_hi-1 of NS0 go behind MFMA Mi; memory ops and checksum pieces are spread evenly
+            constexpr int k_lo = (Mi * NS0 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS0 + NMG - 1) / NMG;
+            static_for<k_hi - k_lo>([&](auto d) {
+                constexpr int k = k_lo + decltype(d)::value;
+                constexpr int mem_before = (k * MEM0 + NS0 - 1) / NS0, mem_after = ((k + 1) * MEM0 + NS0 - 1) / NS0;
+                if constexpr (mem_after > mem_before) {
+                    constexpr int o = mem_before;  // fragment reads first (needed soonest), then loads, then LDS writes
+                    if constexpr (o < NRD) {
+                        fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
+                    } else if constexpr (o < NRD + NGL) {
+                        gload1(sl_free, std::integral_constant<int, o - NRD>{});
+                        if constexpr (o == NRD + NGL - 1) gload_advance();
+                    } else {
+                        lstore1(sl_next, std::integral_constant<int, o - NRD - NGL>{}, st ^ 1);
+                    }
+                } else {
+                    encode1(S0{}, std::integral_constant<int, k - mem_before>{});
+                }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
         __syncthreads();
-    }
-    for (int kt = 0; kt < nkt; ++kt) {
-        const bool more = (kt + 1 < nkt);
-        if (more) load_tile(kbeg + (kt + 1) * BK);
-        if (STAGES == 2) {
-            compute_tile(kt & 1);
-            if (more) store_tile((kt + 1) & 1);
-            __syncthreads();
-        } else {
-            compute_tile(0);
-            __syncthreads();
-            if (more) store_tile(0);
-            __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<NMG>([&](auto m) {
+            constexpr int Mi = decltype(m)::value;
+            mfma1(S1{}, m);
+            constexpr int k_lo = (Mi * NS1 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS1 + NMG - 1) / NMG;
+            static_for<k_hi - k_lo>([&](auto d) {
+                constexpr int k = k_lo + decltype(d)::value;
+                constexpr int mem_before = (k * NRD + NS1 - 1) / NS1, mem_after = ((k + 1) * NRD + NS1 - 1) / NS1;
+                if constexpr (mem_after > mem_before)
+                    fread1(S0{}, std::integral_constant<int, mem_before>{}, st ^ 1, 0);
+                else
+                    encode1(S1{}, std::integral_constant<int, k - mem_before>{});
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    if (nkt > 0) {
+        // prologue: step 0 -> LDS stage 0, step 1 -> staging slot 1, first-half fragments of step 0 -> buffer 0
+        static_for<NGL>([&](auto s) { gload1(S0{}, s); });
+        gload_advance();
+        static_for<NGL>([&](auto s) { lstore1(S0{}, s, 0); });
+        static_for<NGL>([&](auto s) { gload1(S1{}, s); });
+        gload_advance();
+        __syncthreads();
+        static_for<NRD>([&](auto s) { fread1(S0{}, s, 0, 0); });
+        int kt = 0;
+        for (; kt + 1 < nkt; kt += 2) {
+            step(S1{}, S0{}, kt);
+            step(S0{}, S1{}, kt + 1);
         }
+        if (kt < nkt) step(S1{}, S0{}, kt);
+        __syncthreads();  // every wave is done with the staging buffers (the verification below reuses them)
     }
 
     // ---- ABFT verification: inject (testing aid), observe, compare, locate, correct
     if constexpr (FT) {
-        // The staging buffers are free after the loop's last barrier; reuse them.
         double* const s_ccref = reinterpret_cast<double*>(smem);    // [WGM][BN] reference column checksums per wave row
         double* const s_crref = s_ccref + WGM * BN;                 // [WGN][BM] reference row checksums per wave column
         float* const s_ccobs = reinterpret_cast<float*>(s_crref + WGN * BM);  // [WGM][BN] observed column sums
         float* const s_crobs = s_ccobs + WGM * BN;                  // [WGN][BM] observed row sums
         float* const s_dr = s_crobs + WGN * BM;                     // [BM] row residuals, then [BN] column residuals
         int* const s_meta = reinterpret_cast<int*>(s_dr + BM + BN); // nbr, nbc, bad row, bad col, max clean (float bits)
-        static_assert(gemm_lds_bytes<BM, BN, BK, STAGES>() >=
+        static_assert(gemm_lds_bytes<BM, BN>() >=
                           sizeof(double) * (WGM * BN + WGN * BM) + sizeof(float) * (WGM * BN + WGN * BM + BM + BN) + 32,
                       "verification scratch fits in the staging buffers");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
@@ -376,8 +479,7 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
             } else {
                 atomicMax(&s_meta[4], __float_as_int(static_cast<float>(fabs(d))));
             }
-            if (is_row) s_dr[idx] = static_cast<float>(d);
-            else s_dr[BM + idx] = static_cast<float>(d);   // column residuals follow the row residuals
+            s_dr[line] = static_cast<float>(d);  // column residuals follow the row residuals
         }
         __syncthreads();
 
