@@ -39,8 +39,8 @@ static const TileConfig kTiles[] = {
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 constexpr int kFtTile = 0;  // 256 x 128, matches HPCDNN_FT_TILE_M/N
-static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, 2, 2, false, true, 2>;
-static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, 2, 2, true, true, 2>;
+static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, 2, 2, false, true, 1>;
+static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, 2, 2, true, true, 1>;
 
 static int device_cus() {
     static int cus = 0;
@@ -244,10 +244,11 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
     }
     const bool edge = needs_edge(a, cfg);
     void (*fn)(const GemmArgs) = edge ? kFtEdge : kFtPlain;
-    rc = enable_lds(fn, cfg.lds_bytes);
+    constexpr size_t ft_lds = gemm_lds_bytes<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N, true>();
+    rc = enable_lds(fn, ft_lds);
     if (rc != HPCDNN_OK) return rc;
     dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
-    hipLaunchKernelGGL(fn, grid, dim3(kGemmThreads), cfg.lds_bytes, stream ? static_cast<hipStream_t>(stream) : nullptr, a);
+    hipLaunchKernelGGL(fn, grid, dim3(kGemmThreads), ft_lds, stream ? static_cast<hipStream_t>(stream) : nullptr, a);
     return launch_status();
 }
 

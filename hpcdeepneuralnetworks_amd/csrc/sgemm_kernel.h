@@ -66,9 +66,12 @@ constexpr int kGemmBK = 16;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tiles share A and B panels
 
-template <int BM, int BN>
+template <int BM, int BN, bool FT = false>
 constexpr size_t gemm_lds_bytes() {
-    return sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8));
+    // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x 8 half
+    // waves of column sums, 16 row sums)
+    return sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8)) +
+           (FT ? sizeof(float) * 2 * (kGemmBK * 8 + kGemmBK) : 0);
 }
 
 template <int N, class F>
@@ -252,62 +255,138 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
     };
 
     // ---- ABFT encode (dead code when !FT).
-    // The reference forms e^T A and B e on its global->shared staging registers with warp shuffles and adds the
-    // rank-1 products into spare shared memory (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:442-474).  Here each
-    // wave works on the operand fragments it already holds: for its WM rows, its WN columns and the 4 k values of
-    // its lane half,
-    //     acs[q] = sum over the wave's rows of A[., k]      (e^T A)
-    //     brs[q] = sum over the wave's columns of B[k, .]   (B e)
-    // then cc += acs * B[k, n] (column n = lane) and cr += A[m, k] * brs (row m = lane).  The 4-term partial is
-    // formed in FP32 and added to an FP64 running sum, so the reference checksums carry no drift of their own
-    // over a long K.  The work is cut into pieces of a few VALU instructions, one piece behind an MFMA.
-    double cc_ref[TN], cr_ref[TM];
+    // Like the reference, which forms e^T A and B e on its global->shared staging registers with warp shuffles
+    // and adds the rank-1 products into spare shared memory (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:442-474),
+    // the checksums are encoded from the staging registers of K step t+1 while step t is being multiplied:
+    //   before the barrier ("produce"): this thread holds 4 k values of A_SLOTS rows and 4 columns of B_SLOTS k
+    //     rows.  Column sums of A over the tile's rows: in-thread over the slots, then over the 16 lanes of a
+    //     half wave that hold the same k group (row_ror 4, 8; swap with lane^16) -> one partial per half wave in
+    //     LDS.  Row sums of B over the tile's columns: in-thread over the 4 columns, then over the 32 lanes of
+    //     the half wave (which holds whole k rows) -> b_r[k] in LDS.
+    //   after the barrier ("consume"): a_c[k] = sum of the 8 half-wave partials for the thread's own k rows,
+    //     cc[n] += a_c[k] * B[k, n] on its B registers; b_r[k] for its own 4 k values, cr[m] += A[m, k] * b_r[k]
+    //     on its A registers.  Partial sums are FP32 over two K steps, then added to FP64 running sums, so the
+    //     reference checksums carry no drift of their own over a long K.
+    // Per thread the running sums cover columns nc..nc+3 over the k rows it stages (8 threads share a column)
+    // and rows row(s) over the k group it stages (4 threads share a row); the verification step adds them up.
+    constexpr int kHalfWaves = 2 * kGemmThreads / kWave;  // 8
+    static_assert(!FT || (A_V4_PER_ROW == 4 && B_V4_PER_ROW == 32), "ABFT encode is laid out for a 128-column tile");
+    float* const s_apart = smem + 2 * (A_STAGE + B_STAGE);          // [2][16 k][8 half waves]
+    float* const s_br = s_apart + 2 * BK * kHalfWaves;              // [2][16 k]
+    double cc_ref[4], cr_ref[A_SLOTS];
+    float cc_lo[4], cr_lo[A_SLOTS];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) cc_ref[j] = 0.0;
+    for (int e = 0; e < 4; ++e) { cc_ref[e] = 0.0; cc_lo[e] = 0.f; }
 #pragma unroll
-    for (int i = 0; i < TM; ++i) cr_ref[i] = 0.0;
-    float e_acs[4], e_brs[4], e_sa[4], e_sb[4], cc_lo[TN], cr_lo[TM];
-    constexpr int NENC = FT ? (4 * 5 + 1) : 0;  // pieces per half K step: 5 per k value + the FP64 flush
-    auto encode1 = [&](auto buf, auto piece) {
-        constexpr int Bf = decltype(buf)::value, E = decltype(piece)::value;
-        if constexpr (E < 20) {
-            constexpr int q = E / 5, ph = E % 5;
-            if constexpr (ph == 0) {  // in-lane sums over the wave tile's blocks
-                float a = fa[Bf][0][q], b = fb[Bf][0][q];
+    for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] = 0.0; cr_lo[sl] = 0.f; }
+    float e_pa[4], e_sw[4];
+    v4f e_t[2 * B_SLOTS], e_brv;
+    float e_pb[B_SLOTS], e_swb[B_SLOTS], e_ac[B_SLOTS];
+    const int e_hw = tid >> 5;           // half wave 0..7 = first k row this thread stages of B
+    const int e_class = tid & 3;         // k group (4 k values) this thread stages of A
+    constexpr int NPROD = FT ? 10 : 0;   // pieces before the barrier
+    constexpr int NCONS = FT ? 6 : 0;    // pieces after the barrier
+    constexpr int kDppRor4 = 0x124, kDppRor8 = 0x128;  // rotate right inside each row of 16 lanes
+
+    auto produce1 = [&](auto slot, auto piece, int par) {
+        constexpr int S = decltype(slot)::value, E = decltype(piece)::value;
+        if constexpr (E == 0) {
+            v4f t = ra[S][0];
 #pragma unroll
-                for (int i = 1; i < TM; ++i) a += fa[Bf][i][q];
+            for (int sl = 1; sl < A_SLOTS; ++sl) t += ra[S][sl];
+            e_pa[0] = t.x; e_pa[1] = t.y; e_pa[2] = t.z; e_pa[3] = t.w;
+        } else if constexpr (E == 1) {
 #pragma unroll
-                for (int j = 1; j < TN; ++j) b += fb[Bf][j][q];
-                e_acs[q] = a;
-                e_brs[q] = b;
-            } else if constexpr (ph == 1) {  // butterfly inside quads
-                e_acs[q] += dpp_mov<kDppXor1>(e_acs[q]);
-                e_brs[q] += dpp_mov<kDppXor1>(e_brs[q]);
-                e_acs[q] += dpp_mov<kDppXor2>(e_acs[q]);
-                e_brs[q] += dpp_mov<kDppXor2>(e_brs[q]);
-            } else if constexpr (ph == 2) {  // inside rows of 16, then fetch the partner row's sum
-                e_acs[q] += dpp_mov<kDppHalfMirror>(e_acs[q]);
-                e_brs[q] += dpp_mov<kDppHalfMirror>(e_brs[q]);
-                e_acs[q] += dpp_mov<kDppMirror>(e_acs[q]);
-                e_brs[q] += dpp_mov<kDppMirror>(e_brs[q]);
-                e_sa[q] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_acs[q]), 0x401F));
-                e_sb[q] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_brs[q]), 0x401F));
-            } else if constexpr (ph == 3) {  // every lane of the half now holds the sum over 32 lanes
-                e_acs[q] += e_sa[q];
-                e_brs[q] += e_sb[q];
-            } else {
+            for (int e = 0; e < 4; ++e) e_pa[e] += dpp_mov<kDppRor4>(e_pa[e]);
+        } else if constexpr (E == 2) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    cc_lo[j] = (q == 0) ? e_acs[q] * fb[Bf][j][q] : __builtin_fmaf(e_acs[q], fb[Bf][j][q], cc_lo[j]);
+            for (int e = 0; e < 4; ++e) e_pa[e] += dpp_mov<kDppRor8>(e_pa[e]);
+        } else if constexpr (E == 3) {
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    cr_lo[i] = (q == 0) ? fa[Bf][i][q] * e_brs[q] : __builtin_fmaf(fa[Bf][i][q], e_brs[q], cr_lo[i]);
+            for (int e = 0; e < 4; ++e)
+                e_sw[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pa[e]), 0x401F));
+        } else if constexpr (E == 4) {
+#pragma unroll
+            for (int sl = 0; sl < B_SLOTS; ++sl) e_pb[sl] = (rb[S][sl].x + rb[S][sl].y) + (rb[S][sl].z + rb[S][sl].w);
+        } else if constexpr (E == 5) {
+#pragma unroll
+            for (int sl = 0; sl < B_SLOTS; ++sl) {
+                e_pb[sl] += dpp_mov<kDppXor1>(e_pb[sl]);
+                e_pb[sl] += dpp_mov<kDppXor2>(e_pb[sl]);
             }
+        } else if constexpr (E == 6) {
+#pragma unroll
+            for (int sl = 0; sl < B_SLOTS; ++sl) {
+                e_pb[sl] += dpp_mov<kDppHalfMirror>(e_pb[sl]);
+                e_pb[sl] += dpp_mov<kDppMirror>(e_pb[sl]);
+            }
+        } else if constexpr (E == 7) {
+#pragma unroll
+            for (int sl = 0; sl < B_SLOTS; ++sl)
+                e_swb[sl] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pb[sl]), 0x401F));
+        } else if constexpr (E == 8) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) e_pa[e] += e_sw[e];
+#pragma unroll
+            for (int sl = 0; sl < B_SLOTS; ++sl) e_pb[sl] += e_swb[sl];
         } else {
+            float* ap = s_apart + par * BK * kHalfWaves;
+            float* br = s_br + par * BK;
+            if (lr < 4) {  // lanes 0..3 of each half wave publish the four k groups
 #pragma unroll
-            for (int j = 0; j < TN; ++j) cc_ref[j] += static_cast<double>(cc_lo[j]);
+                for (int e = 0; e < 4; ++e) ap[(4 * e_class + e) * kHalfWaves + e_hw] = e_pa[e];
+            }
+            if (lr == 0) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) cr_ref[i] += static_cast<double>(cr_lo[i]);
+                for (int sl = 0; sl < B_SLOTS; ++sl) br[e_hw + kHalfWaves * sl] = e_pb[sl];
+            }
+        }
+    };
+    // `live` is false for the duplicate K step fetched past the end of the slice: it must not be counted.
+    auto consume1 = [&](auto slot, auto piece, int par, bool live, auto flush) {
+        constexpr int S = decltype(slot)::value, E = decltype(piece)::value;
+        constexpr bool kFlush = decltype(flush)::value;
+        const float* ap = s_apart + par * BK * kHalfWaves;
+        const float* br = s_br + par * BK;
+        if constexpr (E == 0) {
+#pragma unroll
+            for (int sl = 0; sl < B_SLOTS; ++sl) {
+                const float* row = ap + (e_hw + kHalfWaves * sl) * kHalfWaves;
+                e_t[2 * sl] = *reinterpret_cast<const v4f*>(row);
+                e_t[2 * sl + 1] = *reinterpret_cast<const v4f*>(row + 4);
+            }
+            e_brv = *reinterpret_cast<const v4f*>(br + 4 * e_class);
+        } else if constexpr (E == 1) {
+#pragma unroll
+            for (int sl = 0; sl < B_SLOTS; ++sl) {
+                const v4f u = e_t[2 * sl] + e_t[2 * sl + 1];
+                const float a = (u.x + u.y) + (u.z + u.w);
+                e_ac[sl] = live ? a : 0.f;
+            }
+            e_brv.x = live ? e_brv.x : 0.f; e_brv.y = live ? e_brv.y : 0.f;
+            e_brv.z = live ? e_brv.z : 0.f; e_brv.w = live ? e_brv.w : 0.f;
+        } else if constexpr (E == 2) {
+#pragma unroll
+            for (int sl = 0; sl < B_SLOTS; ++sl) {
+                cc_lo[0] = __builtin_fmaf(e_ac[sl], rb[S][sl].x, cc_lo[0]);
+                cc_lo[1] = __builtin_fmaf(e_ac[sl], rb[S][sl].y, cc_lo[1]);
+                cc_lo[2] = __builtin_fmaf(e_ac[sl], rb[S][sl].z, cc_lo[2]);
+                cc_lo[3] = __builtin_fmaf(e_ac[sl], rb[S][sl].w, cc_lo[3]);
+            }
+        } else if constexpr (E == 3 || E == 4) {
+            constexpr int lo = (E == 3) ? 0 : A_SLOTS / 2, hi = (E == 3) ? A_SLOTS / 2 : A_SLOTS;
+#pragma unroll
+            for (int sl = lo; sl < hi; ++sl) {
+                float t = __builtin_fmaf(ra[S][sl].x, e_brv.x, cr_lo[sl]);
+                t = __builtin_fmaf(ra[S][sl].y, e_brv.y, t);
+                t = __builtin_fmaf(ra[S][sl].z, e_brv.z, t);
+                cr_lo[sl] = __builtin_fmaf(ra[S][sl].w, e_brv.w, t);
+            }
+        } else if constexpr (kFlush) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { cc_ref[e] += static_cast<double>(cc_lo[e]); cc_lo[e] = 0.f; }
+#pragma unroll
+            for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] += static_cast<double>(cr_lo[sl]); cr_lo[sl] = 0.f; }
         }
     };
 
@@ -317,36 +396,35 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
     // One K step.  On entry: LDS stage kt&1 holds step kt, fragment buffer 0 holds its first half, staging slot
     // `sl_next` holds step kt+1 (possibly still in flight), slot `sl_free` is free.
     //   first half : MFMAs on buffer 0 | read second-half fragments into buffer 1, fetch step kt+2 into sl_free,
-    //                write step kt+1 from sl_next into the other LDS stage
+    //                write step kt+1 from sl_next into the other LDS stage (+ produce its checksum partials)
     //   barrier    : the other stage is complete; nobody reads this stage's fragments any more
     //   second half: MFMAs on buffer 1 | read the first-half fragments of step kt+1 into buffer 0
+    //                (+ consume the checksum partials of step kt+1)
     // Work past the end of the slice (kt+1, kt+2 >= nkt) moves duplicate data that is never multiplied, which
     // keeps the loop free of branches (and lets the loads stay two steps ahead).
-    auto step = [&](auto sl_next, auto sl_free, int kt) {
+    auto step = [&](auto sl_next, auto sl_free, int kt, auto flush) {
         const int st = kt & 1;
+        const bool next_live = kt + 1 < nkt;
         constexpr int MEM0 = NRD + 2 * NGL;  // memory side ops of the first half
-        constexpr int NS0 = MEM0 + NENC;
-        constexpr int NS1 = NRD + NENC;
+        constexpr int NS0 = MEM0 + NPROD;
+        constexpr int NS1 = NRD + NCONS;
         static_for<NMG>([&](auto m) {
             constexpr int Mi = decltype(m)::value;
             mfma1(S0{}, m);
-            // side ops k_lo .. k_hi-1 of NS0 go behind MFMA Mi; memory ops and checksum pieces are spread evenly
+            // side ops k_lo .. k_hi-1 of NS0 go behind MFMA Mi: fragment reads first (needed soonest), then
+            // loads, LDS writes, and last the checksum pieces (they need the same staged data as the LDS writes)
             constexpr int k_lo = (Mi * NS0 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS0 + NMG - 1) / NMG;
             static_for<k_hi - k_lo>([&](auto d) {
-                constexpr int k = k_lo + decltype(d)::value;
-                constexpr int mem_before = (k * MEM0 + NS0 - 1) / NS0, mem_after = ((k + 1) * MEM0 + NS0 - 1) / NS0;
-                if constexpr (mem_after > mem_before) {
-                    constexpr int o = mem_before;  // fragment reads first (needed soonest), then loads, then LDS writes
-                    if constexpr (o < NRD) {
-                        fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
-                    } else if constexpr (o < NRD + NGL) {
-                        gload1(sl_free, std::integral_constant<int, o - NRD>{});
-                        if constexpr (o == NRD + NGL - 1) gload_advance();
-                    } else {
-                        lstore1(sl_next, std::integral_constant<int, o - NRD - NGL>{}, st ^ 1);
-                    }
+                constexpr int o = k_lo + decltype(d)::value;
+                if constexpr (o < NRD) {
+                    fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
+                } else if constexpr (o < NRD + NGL) {
+                    gload1(sl_free, std::integral_constant<int, o - NRD>{});
+                    if constexpr (o == NRD + NGL - 1) gload_advance();
+                } else if constexpr (o < MEM0) {
+                    lstore1(sl_next, std::integral_constant<int, o - NRD - NGL>{}, st ^ 1);
                 } else {
-                    encode1(S0{}, std::integral_constant<int, k - mem_before>{});
+                    produce1(sl_next, std::integral_constant<int, o - MEM0>{}, st ^ 1);
                 }
             });
             __builtin_amdgcn_sched_barrier(0);
@@ -358,12 +436,11 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
             mfma1(S1{}, m);
             constexpr int k_lo = (Mi * NS1 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS1 + NMG - 1) / NMG;
             static_for<k_hi - k_lo>([&](auto d) {
-                constexpr int k = k_lo + decltype(d)::value;
-                constexpr int mem_before = (k * NRD + NS1 - 1) / NS1, mem_after = ((k + 1) * NRD + NS1 - 1) / NS1;
-                if constexpr (mem_after > mem_before)
-                    fread1(S0{}, std::integral_constant<int, mem_before>{}, st ^ 1, 0);
-                else
-                    encode1(S1{}, std::integral_constant<int, k - mem_before>{});
+                constexpr int o = k_lo + decltype(d)::value;
+                // checksum reads go first so that their latency is covered before the sums need them
+                if constexpr (FT && o == 0) consume1(sl_next, std::integral_constant<int, 0>{}, st ^ 1, next_live, flush);
+                else if constexpr (o < NRD + (FT ? 1 : 0)) fread1(S0{}, std::integral_constant<int, o - (FT ? 1 : 0)>{}, st ^ 1, 0);
+                else consume1(sl_next, std::integral_constant<int, o - NRD>{}, st ^ 1, next_live, flush);
             });
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -374,29 +451,32 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
         static_for<NGL>([&](auto s) { gload1(S0{}, s); });
         gload_advance();
         static_for<NGL>([&](auto s) { lstore1(S0{}, s, 0); });
+        static_for<NPROD>([&](auto e) { produce1(S0{}, e, 0); });
         static_for<NGL>([&](auto s) { gload1(S1{}, s); });
         gload_advance();
         __syncthreads();
+        static_for<NCONS>([&](auto e) { consume1(S0{}, e, 0, true, std::true_type{}); });
         static_for<NRD>([&](auto s) { fread1(S0{}, s, 0, 0); });
         int kt = 0;
         for (; kt + 1 < nkt; kt += 2) {
-            step(S1{}, S0{}, kt);
-            step(S0{}, S1{}, kt + 1);
+            step(S1{}, S0{}, kt, std::false_type{});
+            step(S0{}, S1{}, kt + 1, std::true_type{});
         }
-        if (kt < nkt) step(S1{}, S0{}, kt);
+        if (kt < nkt) step(S1{}, S0{}, kt, std::true_type{});
         __syncthreads();  // every wave is done with the staging buffers (the verification below reuses them)
     }
 
     // ---- ABFT verification: inject (testing aid), observe, compare, locate, correct
     if constexpr (FT) {
-        double* const s_ccref = reinterpret_cast<double*>(smem);    // [WGM][BN] reference column checksums per wave row
-        double* const s_crref = s_ccref + WGM * BN;                 // [WGN][BM] reference row checksums per wave column
-        float* const s_ccobs = reinterpret_cast<float*>(s_crref + WGN * BM);  // [WGM][BN] observed column sums
-        float* const s_crobs = s_ccobs + WGM * BN;                  // [WGN][BM] observed row sums
-        float* const s_dr = s_crobs + WGN * BM;                     // [BM] row residuals, then [BN] column residuals
-        int* const s_meta = reinterpret_cast<int*>(s_dr + BM + BN); // nbr, nbc, bad row, bad col, max clean (float bits)
+        constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;             // partials per column / per row checksum
+        double* const s_ccref = reinterpret_cast<double*>(smem);        // [CCP][BN] reference column checksum partials
+        double* const s_crref = s_ccref + CCP * BN;                     // [CRP][BM] reference row checksum partials
+        float* const s_ccobs = reinterpret_cast<float*>(s_crref + CRP * BM);  // [WGM][BN] observed column sums
+        float* const s_crobs = s_ccobs + WGM * BN;                      // [WGN][BM] observed row sums
+        float* const s_dr = s_crobs + WGN * BM;                         // [BM] row residuals, then [BN] column residuals
+        int* const s_meta = reinterpret_cast<int*>(s_dr + BM + BN);     // nbr, nbc, bad row, bad col, max clean (float bits)
         static_assert(gemm_lds_bytes<BM, BN>() >=
-                          sizeof(double) * (WGM * BN + WGN * BM) + sizeof(float) * (WGM * BN + WGN * BM + BM + BN) + 32,
+                          sizeof(double) * (CCP * BN + CRP * BM) + sizeof(float) * (WGM * BN + WGN * BM + BM + BN) + 32,
                       "verification scratch fits in the staging buffers");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
 
@@ -421,17 +501,12 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
 
         if (tid == 0) { s_meta[0] = 0; s_meta[1] = 0; s_meta[2] = -1; s_meta[3] = -1; s_meta[4] = 0; }
 
-        // reference checksums: fold the two lane halves (disjoint k subsets), publish per wave
+        // reference checksums: every thread publishes its partial sums (columns nc..nc+3 over its k rows, its
+        // rows over its k group); the residual step below adds the partials in a fixed order
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const double t = cc_ref[j] + __shfl_xor(cc_ref[j], 32, kWave);
-            if (lh == 0) s_ccref[wm * BN + wn * WN + j * 32 + lr] = t;
-        }
+        for (int e = 0; e < 4; ++e) s_ccref[e_hw * BN + (tid & 31) * 4 + e] = cc_ref[e];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const double t = cr_ref[i] + __shfl_xor(cr_ref[i], 32, kWave);
-            if (lh == 0) s_crref[wn * BM + wm * WM + i * 32 + lr] = t;
-        }
+        for (int sl = 0; sl < A_SLOTS; ++sl) s_crref[e_class * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = cr_ref[sl];
         // observed column sums of the accumulators (ft_sgemm_huge.cuh:147-154): lane = column
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
@@ -467,10 +542,14 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
             double ref = 0.0, obs = 0.0;
             if (is_row) {
 #pragma unroll
-                for (int w = 0; w < WGN; ++w) { ref += s_crref[w * BM + idx]; obs += static_cast<double>(s_crobs[w * BM + idx]); }
+                for (int w = 0; w < CRP; ++w) ref += s_crref[w * BM + idx];
+#pragma unroll
+                for (int w = 0; w < WGN; ++w) obs += static_cast<double>(s_crobs[w * BM + idx]);
             } else {
 #pragma unroll
-                for (int w = 0; w < WGM; ++w) { ref += s_ccref[w * BN + idx]; obs += static_cast<double>(s_ccobs[w * BN + idx]); }
+                for (int w = 0; w < CCP; ++w) ref += s_ccref[w * BN + idx];
+#pragma unroll
+                for (int w = 0; w < WGM; ++w) obs += static_cast<double>(s_ccobs[w * BN + idx]);
             }
             const double d = ref - obs;
             if (fabs(d) > tau) {
