@@ -69,9 +69,9 @@ constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tile
 template <int BM, int BN, bool FT = false>
 constexpr size_t gemm_lds_bytes() {
     // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x 8 half
-    // waves of column sums, 16 row sums)
+    // waves of column sums, 16 row sums) and one dump word per thread for its branch-free predicated writes
     return sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8)) +
-           (FT ? sizeof(float) * 2 * (kGemmBK * 8 + kGemmBK) : 0);
+           (FT ? sizeof(float) * (2 * (kGemmBK * 8 + kGemmBK) + kGemmThreads) : 0);
 }
 
 template <int N, class F>
@@ -81,6 +81,11 @@ __device__ __forceinline__ void static_for(F&& f) {
         f(std::integral_constant<int, N - 1>{});
     }
 }
+
+// Pins a value at this point of the instruction stream: the compiler may neither sink the computation that
+// produces it below this point nor hoist its uses above it (it would otherwise gather the checksum arithmetic,
+// which has no side effects, into one block and stall the matrix core behind it).
+#define HPCDNN_PIN(x) asm volatile("" : "+v"(x))
 
 // Workgroup id -> tile.  The hardware deals consecutive workgroup ids round-
 // robin to the 8 XCDs (each with a private L2), so id -> (xcd = id % 8,
@@ -273,6 +278,7 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
     static_assert(!FT || (A_V4_PER_ROW == 4 && B_V4_PER_ROW == 32), "ABFT encode is laid out for a 128-column tile");
     float* const s_apart = smem + 2 * (A_STAGE + B_STAGE);          // [2][16 k][8 half waves]
     float* const s_br = s_apart + 2 * BK * kHalfWaves;              // [2][16 k]
+    float* const s_dump = s_br + 2 * BK + tid;                      // where the lanes that publish nothing write
     double cc_ref[4], cr_ref[A_SLOTS];
     float cc_lo[4], cr_lo[A_SLOTS];
 #pragma unroll
@@ -295,30 +301,41 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
 #pragma unroll
             for (int sl = 1; sl < A_SLOTS; ++sl) t += ra[S][sl];
             e_pa[0] = t.x; e_pa[1] = t.y; e_pa[2] = t.z; e_pa[3] = t.w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) HPCDNN_PIN(e_pa[e]);
         } else if constexpr (E == 1) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) e_pa[e] += dpp_mov<kDppRor4>(e_pa[e]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) HPCDNN_PIN(e_pa[e]);
         } else if constexpr (E == 2) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) e_pa[e] += dpp_mov<kDppRor8>(e_pa[e]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) HPCDNN_PIN(e_pa[e]);
         } else if constexpr (E == 3) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 e_sw[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pa[e]), 0x401F));
         } else if constexpr (E == 4) {
 #pragma unroll
-            for (int sl = 0; sl < B_SLOTS; ++sl) e_pb[sl] = (rb[S][sl].x + rb[S][sl].y) + (rb[S][sl].z + rb[S][sl].w);
+            for (int sl = 0; sl < B_SLOTS; ++sl) {
+                e_pb[sl] = (rb[S][sl].x + rb[S][sl].y) + (rb[S][sl].z + rb[S][sl].w);
+                HPCDNN_PIN(e_pb[sl]);
+            }
         } else if constexpr (E == 5) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
                 e_pb[sl] += dpp_mov<kDppXor1>(e_pb[sl]);
                 e_pb[sl] += dpp_mov<kDppXor2>(e_pb[sl]);
+                HPCDNN_PIN(e_pb[sl]);
             }
         } else if constexpr (E == 6) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
                 e_pb[sl] += dpp_mov<kDppHalfMirror>(e_pb[sl]);
                 e_pb[sl] += dpp_mov<kDppMirror>(e_pb[sl]);
+                HPCDNN_PIN(e_pb[sl]);
             }
         } else if constexpr (E == 7) {
 #pragma unroll
@@ -326,19 +343,23 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
                 e_swb[sl] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pb[sl]), 0x401F));
         } else if constexpr (E == 8) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) e_pa[e] += e_sw[e];
+            for (int e = 0; e < 4; ++e) { e_pa[e] += e_sw[e]; HPCDNN_PIN(e_pa[e]); }
 #pragma unroll
-            for (int sl = 0; sl < B_SLOTS; ++sl) e_pb[sl] += e_swb[sl];
+            for (int sl = 0; sl < B_SLOTS; ++sl) { e_pb[sl] += e_swb[sl]; HPCDNN_PIN(e_pb[sl]); }
         } else {
+            // lanes 0..3 of each half wave publish the four k groups, lane 0 the row sums; the other lanes write
+            // the same values to their dump word, which keeps the loop free of branches
             float* ap = s_apart + par * BK * kHalfWaves;
             float* br = s_br + par * BK;
-            if (lr < 4) {  // lanes 0..3 of each half wave publish the four k groups
 #pragma unroll
-                for (int e = 0; e < 4; ++e) ap[(4 * e_class + e) * kHalfWaves + e_hw] = e_pa[e];
+            for (int e = 0; e < 4; ++e) {
+                float* dst = (lr < 4) ? ap + (4 * e_class + e) * kHalfWaves + e_hw : s_dump;
+                *dst = e_pa[e];
             }
-            if (lr == 0) {
 #pragma unroll
-                for (int sl = 0; sl < B_SLOTS; ++sl) br[e_hw + kHalfWaves * sl] = e_pb[sl];
+            for (int sl = 0; sl < B_SLOTS; ++sl) {
+                float* dst = (lr == 0) ? br + e_hw + kHalfWaves * sl : s_dump;
+                *dst = e_pb[sl];
             }
         }
     };
@@ -362,9 +383,11 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
                 const v4f u = e_t[2 * sl] + e_t[2 * sl + 1];
                 const float a = (u.x + u.y) + (u.z + u.w);
                 e_ac[sl] = live ? a : 0.f;
+                HPCDNN_PIN(e_ac[sl]);
             }
             e_brv.x = live ? e_brv.x : 0.f; e_brv.y = live ? e_brv.y : 0.f;
             e_brv.z = live ? e_brv.z : 0.f; e_brv.w = live ? e_brv.w : 0.f;
+            HPCDNN_PIN(e_brv);
         } else if constexpr (E == 2) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
@@ -373,6 +396,8 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
                 cc_lo[2] = __builtin_fmaf(e_ac[sl], rb[S][sl].z, cc_lo[2]);
                 cc_lo[3] = __builtin_fmaf(e_ac[sl], rb[S][sl].w, cc_lo[3]);
             }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) HPCDNN_PIN(cc_lo[e]);
         } else if constexpr (E == 3 || E == 4) {
             constexpr int lo = (E == 3) ? 0 : A_SLOTS / 2, hi = (E == 3) ? A_SLOTS / 2 : A_SLOTS;
 #pragma unroll
@@ -381,12 +406,13 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
                 t = __builtin_fmaf(ra[S][sl].y, e_brv.y, t);
                 t = __builtin_fmaf(ra[S][sl].z, e_brv.z, t);
                 cr_lo[sl] = __builtin_fmaf(ra[S][sl].w, e_brv.w, t);
+                HPCDNN_PIN(cr_lo[sl]);
             }
         } else if constexpr (kFlush) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { cc_ref[e] += static_cast<double>(cc_lo[e]); cc_lo[e] = 0.f; }
+            for (int e = 0; e < 4; ++e) { cc_ref[e] += static_cast<double>(cc_lo[e]); cc_lo[e] = 0.f; HPCDNN_PIN(cc_ref[e]); }
 #pragma unroll
-            for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] += static_cast<double>(cr_lo[sl]); cr_lo[sl] = 0.f; }
+            for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] += static_cast<double>(cr_lo[sl]); cr_lo[sl] = 0.f; HPCDNN_PIN(cr_ref[sl]); }
         }
     };
 
@@ -416,15 +442,17 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
             constexpr int k_lo = (Mi * NS0 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS0 + NMG - 1) / NMG;
             static_for<k_hi - k_lo>([&](auto d) {
                 constexpr int o = k_lo + decltype(d)::value;
+                // order: fragment reads (needed soonest), checksum pieces of step kt+1 (its staged data arrived a
+                // step ago; their cross-lane chain must be finished well before the barrier), global loads, LDS writes
                 if constexpr (o < NRD) {
                     fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
-                } else if constexpr (o < NRD + NGL) {
-                    gload1(sl_free, std::integral_constant<int, o - NRD>{});
-                    if constexpr (o == NRD + NGL - 1) gload_advance();
-                } else if constexpr (o < MEM0) {
-                    lstore1(sl_next, std::integral_constant<int, o - NRD - NGL>{}, st ^ 1);
+                } else if constexpr (o < NRD + NPROD) {
+                    produce1(sl_next, std::integral_constant<int, o - NRD>{}, st ^ 1);
+                } else if constexpr (o < NRD + NPROD + NGL) {
+                    gload1(sl_free, std::integral_constant<int, o - NRD - NPROD>{});
+                    if constexpr (o == NRD + NPROD + NGL - 1) gload_advance();
                 } else {
-                    produce1(sl_next, std::integral_constant<int, o - MEM0>{}, st ^ 1);
+                    lstore1(sl_next, std::integral_constant<int, o - NRD - NPROD - NGL>{}, st ^ 1);
                 }
             });
             __builtin_amdgcn_sched_barrier(0);
@@ -437,9 +465,8 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
             constexpr int k_lo = (Mi * NS1 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS1 + NMG - 1) / NMG;
             static_for<k_hi - k_lo>([&](auto d) {
                 constexpr int o = k_lo + decltype(d)::value;
-                // checksum reads go first so that their latency is covered before the sums need them
-                if constexpr (FT && o == 0) consume1(sl_next, std::integral_constant<int, 0>{}, st ^ 1, next_live, flush);
-                else if constexpr (o < NRD + (FT ? 1 : 0)) fread1(S0{}, std::integral_constant<int, o - (FT ? 1 : 0)>{}, st ^ 1, 0);
+                // fragment reads first (the next step's first MFMAs wait for them), then the checksum pieces
+                if constexpr (o < NRD) fread1(S0{}, std::integral_constant<int, o>{}, st ^ 1, 0);
                 else consume1(sl_next, std::integral_constant<int, o - NRD>{}, st ^ 1, next_live, flush);
             });
             __builtin_amdgcn_sched_barrier(0);
