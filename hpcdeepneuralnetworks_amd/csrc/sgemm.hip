@@ -7,6 +7,7 @@ namespace hpcdnn {
 
 struct TileConfig {
     int bm, bn, bk;
+    int threads;
     int blocks_per_cu;  // resident workgroups per CU the kernel is built for
     size_t lds_bytes;
     void (*plain)(const GemmArgs);
@@ -16,7 +17,8 @@ struct TileConfig {
 
 #define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, RESIDENT, SPEED)                                              \
     {                                                                                                    \
-        BM, BN, kGemmBK, RESIDENT, gemm_lds_bytes<BM, BN>(), sgemm_kernel<BM, BN, WGM, WGN, false, false, OCC>, \
+        BM, BN, kGemmBK, WGM * WGN * kWave, RESIDENT, gemm_lds_bytes<BM, BN>(),                            \
+            sgemm_kernel<BM, BN, WGM, WGN, false, false, OCC>,                                           \
             sgemm_kernel<BM, BN, WGM, WGN, true, false, OCC>, SPEED                                       \
     }
 
@@ -35,12 +37,19 @@ static const TileConfig kTiles[] = {
     HPCDNN_TILE(192, 256, 2, 2, 1, 1, 0.94f),  // 6 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
     HPCDNN_TILE(256, 192, 2, 2, 1, 1, 0.93f),  // 7
     HPCDNN_TILE(128, 256, 2, 2, 2, 2, 0.93f),  // 8
+    HPCDNN_TILE(256, 256, 2, 4, 1, 1, 0.95f),  // 9 giant, eight waves
+    HPCDNN_TILE(256, 128, 4, 2, 1, 1, 0.93f),  // 10 huge, eight waves
+    HPCDNN_TILE(256, 256, 4, 2, 1, 1, 0.95f),  // 11 giant, eight waves (4 x 2)
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 constexpr int kFtTile = 0;  // 256 x 128, matches HPCDNN_FT_TILE_M/N
-static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, 2, 2, false, true, 1>;
-static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, 2, 2, true, true, 1>;
+// Four waves: on this part every VALU instruction takes its issue cycles away from the FP32 matrix pipe of the
+// same SIMD, whichever wave it comes from, so more waves do not hide the checksum arithmetic; fewer, fatter
+// threads need the fewest VALU instructions per K step.
+constexpr int kFtWavesM = 2, kFtWavesN = 2, kFtThreads = kFtWavesM * kFtWavesN * kWave;
+static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, false, true, 1>;
+static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, true, true, 1>;
 
 static int device_cus() {
     static int cus = 0;
@@ -176,7 +185,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     if (rc != HPCDNN_OK) return rc;
 
     dim3 grid(a.tiles_m * a.tiles_n, 1, split);
-    hipLaunchKernelGGL(fn, grid, dim3(kGemmThreads), cfg.lds_bytes, stream, a);
+    hipLaunchKernelGGL(fn, grid, dim3(cfg.threads), cfg.lds_bytes, stream, a);
     rc = launch_status();
     if (rc != HPCDNN_OK || split == 1) return rc;
 
@@ -244,11 +253,11 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
     }
     const bool edge = needs_edge(a, cfg);
     void (*fn)(const GemmArgs) = edge ? kFtEdge : kFtPlain;
-    constexpr size_t ft_lds = gemm_lds_bytes<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N, true>();
+    constexpr size_t ft_lds = gemm_lds_bytes<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N, true, kFtThreads>();
     rc = enable_lds(fn, ft_lds);
     if (rc != HPCDNN_OK) return rc;
     dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
-    hipLaunchKernelGGL(fn, grid, dim3(kGemmThreads), ft_lds, stream ? static_cast<hipStream_t>(stream) : nullptr, a);
+    hipLaunchKernelGGL(fn, grid, dim3(kFtThreads), ft_lds, stream ? static_cast<hipStream_t>(stream) : nullptr, a);
     return launch_status();
 }
 

@@ -1,6 +1,6 @@
 // Row-major FP32 GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32).
 //
-// One workgroup of 256 threads (4 waves) owns a BM x BN tile of C; wave w owns
+// One workgroup of WGM x WGN waves (4 or 8) owns a BM x BN tile of C; wave w owns
 // a (BM/WGM) x (BN/WGN) sub-tile made of 32x32 MFMA blocks whose accumulators
 // stay in registers for the whole K loop.  K advances in steps of 16.
 //
@@ -61,17 +61,16 @@ struct GemmArgs {
     hpcdnn_ft_status* status;
 };
 
-constexpr int kGemmThreads = 256;
 constexpr int kGemmBK = 16;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tiles share A and B panels
 
-template <int BM, int BN, bool FT = false>
+template <int BM, int BN, bool FT = false, int THREADS = 256>
 constexpr size_t gemm_lds_bytes() {
-    // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x 8 half
-    // waves of column sums, 16 row sums) and one dump word per thread for its branch-free predicated writes
+    // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x one column
+    // sum per half wave, 16 row sums) and one dump word per thread for its branch-free predicated writes
     return sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8)) +
-           (FT ? sizeof(float) * (2 * (kGemmBK * 8 + kGemmBK) + kGemmThreads) : 0);
+           (FT ? sizeof(float) * (2 * (kGemmBK * (THREADS / 32) + kGemmBK) + THREADS) : 0);
 }
 
 template <int N, class F>
@@ -119,9 +118,10 @@ __device__ __forceinline__ v4f buffer_load_v4f(__amdgpu_buffer_rsrc_t rsrc, int 
 }
 
 template <int BM, int BN, int WGM, int WGN, bool EDGE, bool FT, int MIN_BLOCKS>
-__global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
+__global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
-    static_assert(WGM * WGN == kGemmThreads / kWave, "four waves per workgroup");
+    constexpr int kGemmThreads = WGM * WGN * kWave;
+    static_assert(WGM * WGN == 4 || WGM * WGN == 8, "four or eight waves per workgroup");
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 32, TN = WN / 32;
     static_assert(TM >= 1 && TN >= 1 && WM % 32 == 0 && WN % 32 == 0, "wave tile is made of 32x32 blocks");
@@ -210,14 +210,15 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
             rb[S][Q] = v;
         }
     };
-    // After the last part of a K step: move to the next one, unless that would leave the slice (then the same
-    // step is simply fetched again; its data is never multiplied).
+    // After the last part of a K step: move to the next one, unless that would leave the slice; then the
+    // descriptors are emptied, so the fetches that run ahead past the end all return 0 (never multiplied, and
+    // neutral for the checksums).
     auto gload_advance = [&]() {
         const bool more = k_loaded + BK < kend;
         a_base += more ? BK : 0;
-        a_left -= more ? BK * 4 : 0;
+        a_left = more ? a_left - BK * 4 : 0;
         b_base += more ? b_step : 0;
-        b_left -= more ? b_step * 4 : 0;
+        b_left = more ? b_left - b_step * 4 : 0;
         k_loaded += more ? BK : 0;
     };
     auto lstore1 = [&](auto slot, auto part, int stage) {
@@ -274,11 +275,16 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
     //     reference checksums carry no drift of their own over a long K.
     // Per thread the running sums cover columns nc..nc+3 over the k rows it stages (8 threads share a column)
     // and rows row(s) over the k group it stages (4 threads share a row); the verification step adds them up.
-    constexpr int kHalfWaves = 2 * kGemmThreads / kWave;  // 8
+    constexpr int kHalfWaves = 2 * kGemmThreads / kWave;  // 8 or 16
+    constexpr int kPartV4 = kHalfWaves / 4;               // 16-byte groups of column-sum partials per k
     static_assert(!FT || (A_V4_PER_ROW == 4 && B_V4_PER_ROW == 32), "ABFT encode is laid out for a 128-column tile");
-    float* const s_apart = smem + 2 * (A_STAGE + B_STAGE);          // [2][16 k][8 half waves]
+    float* const s_apart = smem + 2 * (A_STAGE + B_STAGE);          // [2][16 k][half waves]
     float* const s_br = s_apart + 2 * BK * kHalfWaves;              // [2][16 k]
     float* const s_dump = s_br + 2 * BK + tid;                      // where the lanes that publish nothing write
+    // parity-0 destinations of this lane's publishes (parity 1 is a fixed distance further)
+    float* const pub_a = (lr < 4) ? s_apart + (4 * (tid & 3)) * kHalfWaves + (tid >> 5) : s_dump;
+    float* const pub_b = (lr < B_SLOTS) ? s_br + (tid >> 5) + kHalfWaves * lr : s_dump;
+    const int pub_a_step = (lr < 4) ? kHalfWaves : 0, pub_a_par = (lr < 4) ? BK * kHalfWaves : 0, pub_b_par = (lr < B_SLOTS) ? BK : 0;
     double cc_ref[4], cr_ref[A_SLOTS];
     float cc_lo[4], cr_lo[A_SLOTS];
 #pragma unroll
@@ -286,9 +292,9 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
 #pragma unroll
     for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] = 0.0; cr_lo[sl] = 0.f; }
     float e_pa[4], e_sw[4];
-    v4f e_t[2 * B_SLOTS], e_brv;
-    float e_pb[B_SLOTS], e_swb[B_SLOTS], e_ac[B_SLOTS];
-    const int e_hw = tid >> 5;           // half wave 0..7 = first k row this thread stages of B
+    v4f e_t[kPartV4 * B_SLOTS], e_brv;
+    float e_pb0, e_pb1, e_pk, e_swb, e_ac[B_SLOTS];
+    const int e_hw = tid >> 5;           // half wave = first k row this thread stages of B
     const int e_class = tid & 3;         // k group (4 k values) this thread stages of A
     constexpr int NPROD = FT ? 10 : 0;   // pieces before the barrier
     constexpr int NCONS = FT ? 6 : 0;    // pieces after the barrier
@@ -318,53 +324,45 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
             for (int e = 0; e < 4; ++e)
                 e_sw[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pa[e]), 0x401F));
         } else if constexpr (E == 4) {
-#pragma unroll
-            for (int sl = 0; sl < B_SLOTS; ++sl) {
-                e_pb[sl] = (rb[S][sl].x + rb[S][sl].y) + (rb[S][sl].z + rb[S][sl].w);
-                HPCDNN_PIN(e_pb[sl]);
+            // row sums of B: in-thread over the 4 columns, first butterfly step for each staged k row ...
+            e_pb0 = (rb[S][0].x + rb[S][0].y) + (rb[S][0].z + rb[S][0].w);
+            e_pb0 += dpp_mov<kDppXor1>(e_pb0);
+            HPCDNN_PIN(e_pb0);
+            if constexpr (B_SLOTS == 2) {
+                e_pb1 = (rb[S][B_SLOTS - 1].x + rb[S][B_SLOTS - 1].y) + (rb[S][B_SLOTS - 1].z + rb[S][B_SLOTS - 1].w);
+                e_pb1 += dpp_mov<kDppXor1>(e_pb1);
+                HPCDNN_PIN(e_pb1);
             }
         } else if constexpr (E == 5) {
-#pragma unroll
-            for (int sl = 0; sl < B_SLOTS; ++sl) {
-                e_pb[sl] += dpp_mov<kDppXor1>(e_pb[sl]);
-                e_pb[sl] += dpp_mov<kDppXor2>(e_pb[sl]);
-                HPCDNN_PIN(e_pb[sl]);
-            }
+            // ... then the two k rows share one register (even lanes carry row 0, odd lanes row 1) and the
+            // remaining steps, which keep lane parity, reduce both at once
+            static_assert(B_SLOTS <= 2, "two staged k rows are packed by lane parity");
+            e_pk = e_pb0;
+            if constexpr (B_SLOTS == 2) e_pk = (lane & 1) ? e_pb1 : e_pb0;
+            e_pk += dpp_mov<kDppXor2>(e_pk);
+            HPCDNN_PIN(e_pk);
         } else if constexpr (E == 6) {
-#pragma unroll
-            for (int sl = 0; sl < B_SLOTS; ++sl) {
-                e_pb[sl] += dpp_mov<kDppHalfMirror>(e_pb[sl]);
-                e_pb[sl] += dpp_mov<kDppMirror>(e_pb[sl]);
-                HPCDNN_PIN(e_pb[sl]);
-            }
+            e_pk += dpp_mov<kDppRor4>(e_pk);
+            e_pk += dpp_mov<kDppRor8>(e_pk);
+            HPCDNN_PIN(e_pk);
         } else if constexpr (E == 7) {
-#pragma unroll
-            for (int sl = 0; sl < B_SLOTS; ++sl)
-                e_swb[sl] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pb[sl]), 0x401F));
+            e_swb = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pk), 0x401F));
         } else if constexpr (E == 8) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) { e_pa[e] += e_sw[e]; HPCDNN_PIN(e_pa[e]); }
-#pragma unroll
-            for (int sl = 0; sl < B_SLOTS; ++sl) { e_pb[sl] += e_swb[sl]; HPCDNN_PIN(e_pb[sl]); }
+            e_pk += e_swb;
+            HPCDNN_PIN(e_pk);
         } else {
-            // lanes 0..3 of each half wave publish the four k groups, lane 0 the row sums; the other lanes write
-            // the same values to their dump word, which keeps the loop free of branches
-            float* ap = s_apart + par * BK * kHalfWaves;
-            float* br = s_br + par * BK;
+            // lanes 0..3 of each half wave publish the four k groups, lanes 0 (and 1) the row sums; the other
+            // lanes write to their dump word, which keeps the loop free of branches
+            float* da = pub_a + par * pub_a_par;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float* dst = (lr < 4) ? ap + (4 * e_class + e) * kHalfWaves + e_hw : s_dump;
-                *dst = e_pa[e];
-            }
-#pragma unroll
-            for (int sl = 0; sl < B_SLOTS; ++sl) {
-                float* dst = (lr == 0) ? br + e_hw + kHalfWaves * sl : s_dump;
-                *dst = e_pb[sl];
-            }
+            for (int e = 0; e < 4; ++e) da[e * pub_a_step] = e_pa[e];
+            *(pub_b + par * pub_b_par) = e_pk;
         }
     };
-    // `live` is false for the duplicate K step fetched past the end of the slice: it must not be counted.
-    auto consume1 = [&](auto slot, auto piece, int par, bool live, auto flush) {
+    bool flush_now = true;  // uniform; set by the main loop before each K step that may flush
+    auto consume1 = [&](auto slot, auto piece, int par, auto flush) {
         constexpr int S = decltype(slot)::value, E = decltype(piece)::value;
         constexpr bool kFlush = decltype(flush)::value;
         const float* ap = s_apart + par * BK * kHalfWaves;
@@ -373,21 +371,19 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
                 const float* row = ap + (e_hw + kHalfWaves * sl) * kHalfWaves;
-                e_t[2 * sl] = *reinterpret_cast<const v4f*>(row);
-                e_t[2 * sl + 1] = *reinterpret_cast<const v4f*>(row + 4);
+#pragma unroll
+                for (int v = 0; v < kPartV4; ++v) e_t[kPartV4 * sl + v] = *reinterpret_cast<const v4f*>(row + 4 * v);
             }
             e_brv = *reinterpret_cast<const v4f*>(br + 4 * e_class);
         } else if constexpr (E == 1) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
-                const v4f u = e_t[2 * sl] + e_t[2 * sl + 1];
-                const float a = (u.x + u.y) + (u.z + u.w);
-                e_ac[sl] = live ? a : 0.f;
+                v4f u = e_t[kPartV4 * sl];
+#pragma unroll
+                for (int v = 1; v < kPartV4; ++v) u += e_t[kPartV4 * sl + v];
+                e_ac[sl] = (u.x + u.y) + (u.z + u.w);
                 HPCDNN_PIN(e_ac[sl]);
             }
-            e_brv.x = live ? e_brv.x : 0.f; e_brv.y = live ? e_brv.y : 0.f;
-            e_brv.z = live ? e_brv.z : 0.f; e_brv.w = live ? e_brv.w : 0.f;
-            HPCDNN_PIN(e_brv);
         } else if constexpr (E == 2) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
@@ -409,10 +405,14 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
                 HPCDNN_PIN(cr_lo[sl]);
             }
         } else if constexpr (kFlush) {
+            // every 16th K step (and after the last one): FP32 partial -> FP64 running sum.  FP64 VALU
+            // instructions are twice as expensive as FP32 ones, so this is kept rare.
+            if (flush_now) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { cc_ref[e] += static_cast<double>(cc_lo[e]); cc_lo[e] = 0.f; HPCDNN_PIN(cc_ref[e]); }
+                for (int e = 0; e < 4; ++e) { cc_ref[e] += static_cast<double>(cc_lo[e]); cc_lo[e] = 0.f; }
 #pragma unroll
-            for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] += static_cast<double>(cr_lo[sl]); cr_lo[sl] = 0.f; HPCDNN_PIN(cr_ref[sl]); }
+                for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] += static_cast<double>(cr_lo[sl]); cr_lo[sl] = 0.f; }
+            }
         }
     };
 
@@ -430,7 +430,6 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
     // keeps the loop free of branches (and lets the loads stay two steps ahead).
     auto step = [&](auto sl_next, auto sl_free, int kt, auto flush) {
         const int st = kt & 1;
-        const bool next_live = kt + 1 < nkt;
         constexpr int MEM0 = NRD + 2 * NGL;  // memory side ops of the first half
         constexpr int NS0 = MEM0 + NPROD;
         constexpr int NS1 = NRD + NCONS;
@@ -467,7 +466,7 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
                 constexpr int o = k_lo + decltype(d)::value;
                 // fragment reads first (the next step's first MFMAs wait for them), then the checksum pieces
                 if constexpr (o < NRD) fread1(S0{}, std::integral_constant<int, o>{}, st ^ 1, 0);
-                else consume1(sl_next, std::integral_constant<int, o - NRD>{}, st ^ 1, next_live, flush);
+                else consume1(sl_next, std::integral_constant<int, o - NRD>{}, st ^ 1, flush);
             });
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -482,13 +481,15 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
         static_for<NGL>([&](auto s) { gload1(S1{}, s); });
         gload_advance();
         __syncthreads();
-        static_for<NCONS>([&](auto e) { consume1(S0{}, e, 0, true, std::true_type{}); });
+        static_for<NCONS>([&](auto e) { consume1(S0{}, e, 0, std::true_type{}); });
         static_for<NRD>([&](auto s) { fread1(S0{}, s, 0, 0); });
         int kt = 0;
         for (; kt + 1 < nkt; kt += 2) {
             step(S1{}, S0{}, kt, std::false_type{});
+            flush_now = ((kt & 14) == 14) || (kt + 2 >= nkt);
             step(S0{}, S1{}, kt + 1, std::true_type{});
         }
+        flush_now = true;
         if (kt < nkt) step(S1{}, S0{}, kt, std::true_type{});
         __syncthreads();  // every wave is done with the staging buffers (the verification below reuses them)
     }
@@ -502,7 +503,7 @@ __global__ __launch_bounds__(kGemmThreads, MIN_BLOCKS) void sgemm_kernel(const G
         float* const s_crobs = s_ccobs + WGM * BN;                      // [WGN][BM] observed row sums
         float* const s_dr = s_crobs + WGN * BM;                         // [BM] row residuals, then [BN] column residuals
         int* const s_meta = reinterpret_cast<int*>(s_dr + BM + BN);     // nbr, nbc, bad row, bad col, max clean (float bits)
-        static_assert(gemm_lds_bytes<BM, BN>() >=
+        static_assert(gemm_lds_bytes<BM, BN, true, kGemmThreads>() >=
                           sizeof(double) * (CCP * BN + CRP * BM) + sizeof(float) * (WGM * BN + WGN * BM + BM + BN) + 32,
                       "verification scratch fits in the staging buffers");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
