@@ -68,9 +68,10 @@ constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tile
 template <int BM, int BN, bool FT = false, int THREADS = 256>
 constexpr size_t gemm_lds_bytes() {
     // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x one column
-    // sum per half wave, 16 row sums) and one dump word per thread for its branch-free predicated writes
+    // sum per wave, 16 row sums) and a dump area for the branch-free predicated writes of the lanes that
+    // publish nothing (one word per thread plus the reach of the strided writes)
     return sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8)) +
-           (FT ? sizeof(float) * (2 * (kGemmBK * (THREADS / 32) + kGemmBK) + THREADS) : 0);
+           (FT ? sizeof(float) * (2 * (kGemmBK * (THREADS / 64) + kGemmBK) + THREADS + 2 * kGemmBK * (THREADS / 64)) : 0);
 }
 
 template <int N, class F>
@@ -276,15 +277,17 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // Per thread the running sums cover columns nc..nc+3 over the k rows it stages (8 threads share a column)
     // and rows row(s) over the k group it stages (4 threads share a row); the verification step adds them up.
     constexpr int kHalfWaves = 2 * kGemmThreads / kWave;  // 8 or 16
-    constexpr int kPartV4 = kHalfWaves / 4;               // 16-byte groups of column-sum partials per k
+    constexpr int kParts = kGemmThreads / kWave;          // column-sum partials per k: one per wave
+    constexpr int kPartV4 = kParts / 4;                   // 16-byte groups of them
     static_assert(!FT || (A_V4_PER_ROW == 4 && B_V4_PER_ROW == 32), "ABFT encode is laid out for a 128-column tile");
-    float* const s_apart = smem + 2 * (A_STAGE + B_STAGE);          // [2][16 k][half waves]
-    float* const s_br = s_apart + 2 * BK * kHalfWaves;              // [2][16 k]
+    float* const s_apart = smem + 2 * (A_STAGE + B_STAGE);          // [2][16 k][waves]
+    float* const s_br = s_apart + 2 * BK * kParts;                  // [2][16 k]
     float* const s_dump = s_br + 2 * BK + tid;                      // where the lanes that publish nothing write
-    // parity-0 destinations of this lane's publishes (parity 1 is a fixed distance further)
-    float* const pub_a = (lr < 4) ? s_apart + (4 * (tid & 3)) * kHalfWaves + (tid >> 5) : s_dump;
+    // destinations of this lane's publishes (parity 0); strides and the parity distance are the same for the
+    // publishing lanes and the dump, so every write is base + immediate offset
+    float* const pub_a = (lane < 4) ? s_apart + (4 * (tid & 3)) * kParts + wave : s_dump;
     float* const pub_b = (lr < B_SLOTS) ? s_br + (tid >> 5) + kHalfWaves * lr : s_dump;
-    const int pub_a_step = (lr < 4) ? kHalfWaves : 0, pub_a_par = (lr < 4) ? BK * kHalfWaves : 0, pub_b_par = (lr < B_SLOTS) ? BK : 0;
+    const int x32_addr = (lane ^ 32) * 4;  // ds_bpermute address of the partner lane in the other half wave
     double cc_ref[4], cr_ref[A_SLOTS];
     float cc_lo[4], cr_lo[A_SLOTS];
 #pragma unroll
@@ -296,7 +299,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     float e_pb0, e_pb1, e_pk, e_swb, e_ac[B_SLOTS];
     const int e_hw = tid >> 5;           // half wave = first k row this thread stages of B
     const int e_class = tid & 3;         // k group (4 k values) this thread stages of A
-    constexpr int NPROD = FT ? 10 : 0;   // pieces before the barrier
+    constexpr int NPROD = FT ? 11 : 0;   // pieces before the barrier
     constexpr int NCONS = FT ? 6 : 0;    // pieces after the barrier
     constexpr int kDppRor4 = 0x124, kDppRor8 = 0x128;  // rotate right inside each row of 16 lanes
 
@@ -349,28 +352,34 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             e_swb = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pk), 0x401F));
         } else if constexpr (E == 8) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { e_pa[e] += e_sw[e]; HPCDNN_PIN(e_pa[e]); }
+            for (int e = 0; e < 4; ++e) {
+                e_pa[e] += e_sw[e];
+                e_sw[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(x32_addr, __builtin_bit_cast(int, e_pa[e])));
+            }
             e_pk += e_swb;
             HPCDNN_PIN(e_pk);
-        } else {
-            // lanes 0..3 of each half wave publish the four k groups, lanes 0 (and 1) the row sums; the other
-            // lanes write to their dump word, which keeps the loop free of branches
-            float* da = pub_a + par * pub_a_par;
+        } else if constexpr (E == 9) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) da[e * pub_a_step] = e_pa[e];
-            *(pub_b + par * pub_b_par) = e_pk;
+            for (int e = 0; e < 4; ++e) { e_pa[e] += e_sw[e]; HPCDNN_PIN(e_pa[e]); }  // sum over the whole wave
+        } else {
+            // lanes 0..3 of each wave publish the four k groups, lanes 0 (and 1) of each half wave the row sums; the other
+            // lanes write to their dump word, which keeps the loop free of branches
+            float* da = pub_a + par * (BK * kParts);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) da[e * kParts] = e_pa[e];
+            *(pub_b + par * BK) = e_pk;
         }
     };
     bool flush_now = true;  // uniform; set by the main loop before each K step that may flush
     auto consume1 = [&](auto slot, auto piece, int par, auto flush) {
         constexpr int S = decltype(slot)::value, E = decltype(piece)::value;
         constexpr bool kFlush = decltype(flush)::value;
-        const float* ap = s_apart + par * BK * kHalfWaves;
+        const float* ap = s_apart + par * BK * kParts;
         const float* br = s_br + par * BK;
         if constexpr (E == 0) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
-                const float* row = ap + (e_hw + kHalfWaves * sl) * kHalfWaves;
+                const float* row = ap + (e_hw + kHalfWaves * sl) * kParts;
 #pragma unroll
                 for (int v = 0; v < kPartV4; ++v) e_t[kPartV4 * sl + v] = *reinterpret_cast<const v4f*>(row + 4 * v);
             }
@@ -428,8 +437,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     //                (+ consume the checksum partials of step kt+1)
     // Work past the end of the slice (kt+1, kt+2 >= nkt) moves duplicate data that is never multiplied, which
     // keeps the loop free of branches (and lets the loads stay two steps ahead).
-    auto step = [&](auto sl_next, auto sl_free, int kt, auto flush) {
-        const int st = kt & 1;
+    auto step = [&](auto sl_next, auto sl_free, auto flush) {
+        // steps alternate between (next = slot 1, LDS stage 0) and (next = slot 0, LDS stage 1)
+        constexpr int st = (decltype(sl_next)::value == 1) ? 0 : 1;
         constexpr int MEM0 = NRD + 2 * NGL;  // memory side ops of the first half
         constexpr int NS0 = MEM0 + NPROD;
         constexpr int NS1 = NRD + NCONS;
@@ -485,12 +495,12 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         static_for<NRD>([&](auto s) { fread1(S0{}, s, 0, 0); });
         int kt = 0;
         for (; kt + 1 < nkt; kt += 2) {
-            step(S1{}, S0{}, kt, std::false_type{});
+            step(S1{}, S0{}, std::false_type{});
             flush_now = ((kt & 14) == 14) || (kt + 2 >= nkt);
-            step(S0{}, S1{}, kt + 1, std::true_type{});
+            step(S0{}, S1{}, std::true_type{});
         }
         flush_now = true;
-        if (kt < nkt) step(S1{}, S0{}, kt, std::true_type{});
+        if (kt < nkt) step(S1{}, S0{}, std::true_type{});
         __syncthreads();  // every wave is done with the staging buffers (the verification below reuses them)
     }
 
