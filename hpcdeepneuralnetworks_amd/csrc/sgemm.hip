@@ -12,34 +12,35 @@ struct TileConfig {
     size_t lds_bytes;
     void (*plain)(const GemmArgs);
     void (*edge)(const GemmArgs);
-    float rel_speed;  // measured steady-state throughput relative to the best configuration
+    float eff;       // measured steady-state fraction of the FP32 MFMA peak of one CU
+    float fixed_us;  // measured per-tile prologue + epilogue time
 };
 
-#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, RESIDENT, SPEED)                                              \
+#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, RESIDENT, EFF, FIXED)                                             \
     {                                                                                                    \
         BM, BN, kGemmBK, WGM * WGN * kWave, RESIDENT, gemm_lds_bytes<BM, BN>(),                            \
             sgemm_kernel<BM, BN, WGM, WGN, false, false, OCC>,                                           \
-            sgemm_kernel<BM, BN, WGM, WGN, true, false, OCC>, SPEED                                       \
+            sgemm_kernel<BM, BN, WGM, WGN, true, false, OCC>, EFF, FIXED                                  \
     }
 
 // The counterpart of the reference's small/medium/large/tall/wide/huge shape
 // table (kernel/ft_sgemm/code_gen/main.py:8-16), re-derived for 32x32 MFMA
-// blocks and four 64-lane waves per workgroup.  RESIDENT = workgroups that fit
-// on one CU (registers and LDS); SPEED = measured steady-state fraction of the
-// FP32 MFMA peak.
+// blocks and four or eight 64-lane waves per workgroup.  RESIDENT = workgroups
+// that fit on one CU (registers and LDS); EFF and FIXED are least-squares fits
+// of t = rounds * (BM*BN*K / (EFF * peak per CU) + FIXED) to measured times over
+// square sizes 256..6144 on an MI355X.
 static const TileConfig kTiles[] = {
-    HPCDNN_TILE(256, 128, 2, 2, 2, 2, 0.93f),  // 0 huge (the ABFT tile)
-    HPCDNN_TILE(128, 128, 2, 2, 2, 3, 0.90f),  // 1 large
-    HPCDNN_TILE(128, 64, 2, 2, 2, 4, 0.80f),   // 2 tall
-    HPCDNN_TILE(64, 128, 2, 2, 2, 4, 0.80f),   // 3 wide
-    HPCDNN_TILE(64, 64, 2, 2, 4, 8, 0.65f),    // 4 medium
-    HPCDNN_TILE(256, 256, 2, 2, 1, 1, 0.945f), // 5 giant
-    HPCDNN_TILE(192, 256, 2, 2, 1, 1, 0.94f),  // 6 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
-    HPCDNN_TILE(256, 192, 2, 2, 1, 1, 0.93f),  // 7
-    HPCDNN_TILE(128, 256, 2, 2, 2, 2, 0.93f),  // 8
-    HPCDNN_TILE(256, 256, 2, 4, 1, 1, 0.95f),  // 9 giant, eight waves
-    HPCDNN_TILE(256, 128, 4, 2, 1, 1, 0.93f),  // 10 huge, eight waves
-    HPCDNN_TILE(256, 256, 4, 2, 1, 1, 0.95f),  // 11 giant, eight waves (4 x 2)
+    HPCDNN_TILE(256, 128, 2, 2, 2, 2, 0.940f, 6.2f),   // 0 huge (the ABFT tile)
+    HPCDNN_TILE(128, 128, 2, 2, 2, 3, 0.919f, 4.1f),   // 1 large
+    HPCDNN_TILE(128, 64, 2, 2, 2, 4, 0.864f, 3.1f),    // 2 tall
+    HPCDNN_TILE(64, 128, 2, 2, 2, 4, 0.892f, 3.4f),    // 3 wide
+    HPCDNN_TILE(64, 64, 2, 2, 4, 8, 0.816f, 2.3f),     // 4 medium
+    HPCDNN_TILE(192, 256, 2, 2, 1, 1, 0.954f, 7.3f),   // 5 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
+    HPCDNN_TILE(256, 192, 2, 2, 1, 1, 0.935f, 7.4f),   // 6
+    HPCDNN_TILE(128, 256, 2, 2, 2, 2, 0.937f, 6.3f),   // 7
+    HPCDNN_TILE(256, 256, 2, 4, 1, 1, 0.971f, 10.8f),  // 8 giant, eight waves
+    HPCDNN_TILE(256, 128, 4, 2, 1, 1, 0.927f, 4.7f),   // 9 huge, eight waves
+    HPCDNN_TILE(256, 256, 4, 2, 1, 1, 0.968f, 9.0f),   // 10 giant, eight waves (4 x 2)
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
@@ -85,15 +86,23 @@ struct Plan {
     int split;
 };
 
+// Predicted run time in seconds.  Workgroups are dealt evenly to the CUs, so a launch takes as long as the CU
+// with the most tiles: ceil(tiles / CUs) tile times (co-resident workgroups share the CU's matrix cores, which
+// changes the overlap of prologues, not the throughput).
+constexpr double kPeakFlopsPerCu = 157.3e12 / 256.0;
+constexpr double kEdgePenalty = 1.10;        // ragged-tile kernel: mask instructions compete with the MFMAs
+constexpr double kReduceFixed = 8e-6;        // second launch of split-K
+constexpr double kReduceBytesPerSec = 3e12;  // partials written once and read once, C written once
+
 static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int cus) {
     const double tiles = static_cast<double>(ceil_div(M, t.bm)) * ceil_div(N, t.bn) * split;
-    const double slots = static_cast<double>(cus) * t.blocks_per_cu;
-    const double rounds = ceil(tiles / slots);
-    // time of one round: a resident set of blocks_per_cu workgroups shares the CU's matrix cores
+    const double rounds = ceil(tiles / cus);
     const double k_slice = ceil(static_cast<double>(ceil_div(K, split)) / t.bk) * t.bk;
-    const double per_tile = static_cast<double>(t.bm) * t.bn * (k_slice + 64.0);  // + prologue/epilogue in k-equivalents
-    double cost = rounds * per_tile * t.blocks_per_cu / t.rel_speed;
-    if (split > 1) cost += 3.0 * M * static_cast<double>(N) * split / cus * 8.0;  // partial write + ordered re-read
+    const bool edge = (M % t.bm) || (N % t.bn) || (K % t.bk);
+    const double per_tile = 2.0 * t.bm * t.bn * k_slice / (kPeakFlopsPerCu * t.eff) * (edge ? kEdgePenalty : 1.0) +
+                            t.fixed_us * 1e-6;
+    double cost = rounds * per_tile;
+    if (split > 1) cost += kReduceFixed + (2.0 * split + 1.0) * M * static_cast<double>(N) * 4.0 / kReduceBytesPerSec;
     return cost;
 }
 
@@ -106,7 +115,7 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes) 
         for (int split = 1; split <= 64; split *= 2) {
             if (split > 1) {
                 if (!allow_split) break;
-                if (ceil_div(K, split) < 4 * cfg.bk) break;
+                if (ceil_div(K, split) < 8 * cfg.bk) break;
                 if (static_cast<size_t>(M) * N * split * sizeof(float) > ws_bytes) break;
             }
             const double c = plan_cost(cfg, M, N, K, split, cus);

@@ -185,29 +185,36 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     v4f ra[2][A_SLOTS], rb[2][B_SLOTS];  // two staging slots: K steps t+1 and t+2 are in flight while t is multiplied
     int k_loaded = kbeg;                 // absolute k of the K step the next load call fetches
 
-    // One staging load (part P of the K step at a_base/b_base) into slot S.
+    // One staging load (part P of the K step at a_base/b_base) into slot S.  Nothing here touches the loaded
+    // value, so the load stays in flight until the slot is consumed a K step later.
+    int k_slot[2] = {kbeg, kbeg};  // absolute k of the K step held by each staging slot
     auto gload1 = [&](auto slot, auto part) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
+        if constexpr (P == 0) k_slot[S] = k_loaded;
+        if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc(a_base, a_left), a_voff[P]);
+        else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[P - A_SLOTS]);
+    };
+    // Ragged tiles only, applied when the slot is consumed: columns k >= kend of A hold padding, the next K
+    // slice or the next row, and columns n >= N / rows k >= kend of B likewise: force them to 0 (rows m >= M
+    // of A and k >= K of B already read as 0 through the descriptor).
+    auto gmask1 = [&](auto slot, auto part) {
+        constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P < A_SLOTS) {
-            v4f v = buffer_load_v4f(make_rsrc(a_base, a_left), a_voff[P]);
-            if constexpr (EDGE) {  // columns k >= kend hold padding, the next slice, or the next row: force 0
-                const int left = kend - (k_loaded + a_kc[P]);
-                v.x = left > 0 ? v.x : 0.f;
-                v.y = left > 1 ? v.y : 0.f;
-                v.z = left > 2 ? v.z : 0.f;
-                v.w = left > 3 ? v.w : 0.f;
-            }
+            const int left = kend - (k_slot[S] + a_kc[P]);
+            v4f v = ra[S][P];
+            v.x = left > 0 ? v.x : 0.f;
+            v.y = left > 1 ? v.y : 0.f;
+            v.z = left > 2 ? v.z : 0.f;
+            v.w = left > 3 ? v.w : 0.f;
             ra[S][P] = v;
         } else {
             constexpr int Q = P - A_SLOTS;
-            v4f v = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[Q]);
-            if constexpr (EDGE) {
-                const bool row_ok = k_loaded + b_row[Q] < kend;
-                v.x = (row_ok && b_nvalid[Q] > 0) ? v.x : 0.f;
-                v.y = (row_ok && b_nvalid[Q] > 1) ? v.y : 0.f;
-                v.z = (row_ok && b_nvalid[Q] > 2) ? v.z : 0.f;
-                v.w = (row_ok && b_nvalid[Q] > 3) ? v.w : 0.f;
-            }
+            const int nv = (k_slot[S] + b_row[Q] < kend) ? b_nvalid[Q] : 0;
+            v4f v = rb[S][Q];
+            v.x = nv > 0 ? v.x : 0.f;
+            v.y = nv > 1 ? v.y : 0.f;
+            v.z = nv > 2 ? v.z : 0.f;
+            v.w = nv > 3 ? v.w : 0.f;
             rb[S][Q] = v;
         }
     };
@@ -440,8 +447,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     auto step = [&](auto sl_next, auto sl_free, auto flush) {
         // steps alternate between (next = slot 1, LDS stage 0) and (next = slot 0, LDS stage 1)
         constexpr int st = (decltype(sl_next)::value == 1) ? 0 : 1;
-        constexpr int MEM0 = NRD + 2 * NGL;  // memory side ops of the first half
-        constexpr int NS0 = MEM0 + NPROD;
+        constexpr int NMASK = EDGE ? NGL : 0;
+        constexpr int NS0 = NRD + NMASK + NPROD + 2 * NGL;
         constexpr int NS1 = NRD + NCONS;
         static_for<NMG>([&](auto m) {
             constexpr int Mi = decltype(m)::value;
@@ -451,17 +458,20 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             constexpr int k_lo = (Mi * NS0 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS0 + NMG - 1) / NMG;
             static_for<k_hi - k_lo>([&](auto d) {
                 constexpr int o = k_lo + decltype(d)::value;
-                // order: fragment reads (needed soonest), checksum pieces of step kt+1 (its staged data arrived a
-                // step ago; their cross-lane chain must be finished well before the barrier), global loads, LDS writes
+                // order: fragment reads (needed soonest); ragged-tile masks and checksum pieces of step kt+1 (its
+                // staged data arrived a step ago; the cross-lane chain must be finished well before the barrier);
+                // global loads of step kt+2; LDS writes of step kt+1
                 if constexpr (o < NRD) {
                     fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
-                } else if constexpr (o < NRD + NPROD) {
-                    produce1(sl_next, std::integral_constant<int, o - NRD>{}, st ^ 1);
-                } else if constexpr (o < NRD + NPROD + NGL) {
-                    gload1(sl_free, std::integral_constant<int, o - NRD - NPROD>{});
-                    if constexpr (o == NRD + NPROD + NGL - 1) gload_advance();
+                } else if constexpr (o < NRD + NMASK) {
+                    gmask1(sl_next, std::integral_constant<int, o - NRD>{});
+                } else if constexpr (o < NRD + NMASK + NPROD) {
+                    produce1(sl_next, std::integral_constant<int, o - NRD - NMASK>{}, st ^ 1);
+                } else if constexpr (o < NRD + NMASK + NPROD + NGL) {
+                    gload1(sl_free, std::integral_constant<int, o - NRD - NMASK - NPROD>{});
+                    if constexpr (o == NRD + NMASK + NPROD + NGL - 1) gload_advance();
                 } else {
-                    lstore1(sl_next, std::integral_constant<int, o - NRD - NPROD - NGL>{}, st ^ 1);
+                    lstore1(sl_next, std::integral_constant<int, o - NRD - NMASK - NPROD - NGL>{}, st ^ 1);
                 }
             });
             __builtin_amdgcn_sched_barrier(0);
@@ -486,6 +496,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         // prologue: step 0 -> LDS stage 0, step 1 -> staging slot 1, first-half fragments of step 0 -> buffer 0
         static_for<NGL>([&](auto s) { gload1(S0{}, s); });
         gload_advance();
+        if constexpr (EDGE) static_for<NGL>([&](auto s) { gmask1(S0{}, s); });
         static_for<NGL>([&](auto s) { lstore1(S0{}, s, 0); });
         static_for<NPROD>([&](auto e) { produce1(S0{}, e, 0); });
         static_for<NGL>([&](auto s) { gload1(S1{}, s); });
