@@ -34,6 +34,8 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline SGEMM line only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--ft-launches", type=int, default=1000, help="launches of the ABFT fault campaign")
+    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "ft_sgemm", "saxpy", "sdot", "copy"],
+                    help="run one kernel only for --steps launches (for profiling with rocprofv3) and print a short line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is a single-GPU library (no collectives); run with --gpus 1", file=sys.stderr)
@@ -72,6 +74,36 @@ def main() -> int:
         blas.fill_uniform_matrix(b, K, N, seed + 1)
         blas.fill_uniform_matrix(c, M, N, seed + 2)
         return a, b, c
+
+    if args.kernel not in ("all", "sgemm"):
+        # single-kernel mode for the profiler: same shapes as the full run
+        if args.kernel == "ft_sgemm":
+            m = 4096
+            a, b, c = operands(m, m, m, 20)
+            status = blas.ft_status_alloc(m, m)
+            fn = lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=blas.ft_default_tau(m), status=status)
+            work, unit = 2.0 * m ** 3, "GFLOP/s"
+        else:
+            nv = 1 << 28
+            x = torch.empty(nv, device=dev)
+            y = torch.empty(nv, device=dev)
+            out = torch.zeros(1, device=dev)
+            blas.fill_uniform(x, 30)
+            blas.fill_uniform(y, 31)
+            if args.kernel == "saxpy":
+                fn, work = (lambda: blas.saxpy(nv, 2.5, x, y)), 12.0 * nv
+            elif args.kernel == "sdot":
+                fn, work = (lambda: blas.sdot(nv, x, y, out)), 8.0 * nv
+            else:
+                z = torch.empty_like(x)
+                fn, work = (lambda: z.copy_(x)), 8.0 * nv
+            unit = "GB/s"
+        ms = timed(fn, args.steps, args.warmup)
+        print(json.dumps({"kernel": args.kernel, "steps": args.steps, "ms_per_step": round(ms, 4),
+                          "value": round(work / ms / 1e6, 1), "unit": unit}))
+        return 0
+    if args.kernel == "sgemm":
+        args.no_extras = args.no_cpu = True
 
     # ---------------- headline: SGEMM 6144^3, exactly K timed steps between two synchronisations
     n = 6144
@@ -146,13 +178,23 @@ def main() -> int:
             sweep[str(m)] = round(2.0 * m ** 3 / ms / 1e6, 1)
         extras["sgemm_square_gflops"] = sweep
 
+        # irregular / skinny shapes (split-K with a caller-provided workspace where the library chooses it)
+        irregular = {}
+        for (M, N, K) in ((8192, 8192, 256), (16384, 64, 4096), (128, 128, 65536), (6000, 6000, 6000), (3001, 3001, 3001)):
+            a, b, c = operands(M, N, K, 15)
+            ws = blas.workspace(max(blas.sgemm_workspace_bytes(M, N, K), 4))
+            ms = median_timed(lambda: blas.sgemm(M, N, K, a, b, c, 1.0, 0.0, ws=ws), st, wu)
+            irregular[f"{M}x{N}x{K}"] = round(2.0 * M * N * K / ms / 1e6, 1)
+            del a, b, c, ws
+        extras["sgemm_irregular_gflops"] = irregular
+
         # ---- ABFT at 4096^3: overhead vs plain SGEMM and the seeded single-fault campaign
         m = 4096
         a, b, c = operands(m, m, m, 20)
         status = blas.ft_status_alloc(m, m)
         tau = blas.ft_default_tau(m)
         ms_plain = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0), st, wu)
-        ms_plain_same_tile = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0, tile=0, split_k=1), st, wu)
+        ms_plain_same_tile = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0, tile=0, split_k=1), st, wu)  # 256x128, the ABFT tile
         ms_ft = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status), st, wu)
         extras["abft_4096"] = {
             "sgemm_gflops": round(2.0 * m ** 3 / ms_plain / 1e6, 1),

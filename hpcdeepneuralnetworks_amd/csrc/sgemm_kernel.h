@@ -654,21 +654,33 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         return;
     }
 
+    // C = alpha*acc + beta*C.  With beta != 0 the 16 old values of a 32x32 block are fetched together before the
+    // first store, so that their latencies overlap instead of queueing behind each other.
     const float alpha = p.alpha, beta = p.beta;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j) {
+            const int col = col_base + j * 32;
+            float* cbase = p.C + static_cast<size_t>(row_base + i * 32) * p.ldc + col;
+            float old[16];
+            if (beta != 0.f) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
-                const int col = col_base + j * 32;
-                if (!EDGE || (row < p.M && col < p.N)) {
-                    float* c = p.C + static_cast<size_t>(row) * p.ldc + col;
-                    const float t = alpha * acc[i][j][v];
-                    *c = (beta == 0.f) ? t : __builtin_fmaf(beta, *c, t);
+                for (int v = 0; v < 16; ++v) {
+                    const int r = 8 * (v / 4) + (v % 4);
+                    const bool ok = !EDGE || (row_base + i * 32 + r < p.M && col < p.N);
+                    old[v] = ok ? cbase[static_cast<size_t>(r) * p.ldc] : 0.f;
                 }
             }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = 8 * (v / 4) + (v % 4);
+                if (!EDGE || (row_base + i * 32 + r < p.M && col < p.N)) {
+                    const float t = alpha * acc[i][j][v];
+                    cbase[static_cast<size_t>(r) * p.ldc] = (beta == 0.f) ? t : __builtin_fmaf(beta, old[v], t);
+                }
+            }
+        }
 }
 
 // Fixed-order second phase of split-K: C = alpha * (ws[0] + ws[1] + ...) + beta*C.

@@ -1,0 +1,57 @@
+// C++ convenience layer over the C ABI (hpcdnn.h): the reference's spellings and argument order.
+//
+// The reference drivers launch `sgemm_k<<<...>>>(N, A, B, C, alpha, beta)` (kernel/sgemm/sgemm.cu:120-141),
+// `[ft_]sgemm_<shape><<<...>>>(M, N, K, A, B, C, alpha, beta)` (kernel/ft_sgemm/sgemm.cu:114-165),
+// `saxpy<<<...>>>(N, alpha, x, y)` (kernel/saxpy/saxpy.cu:110) and `_sdot<<<...>>>(N, x, y, out)`
+// (kernel/sdot/sdot.cu:156), and call `cpu_gemm(alpha, beta, A, B, n, C)` (utils/utils.cuh:97) on the host.
+// The overloads below take the same arguments on device pointers (row-major, packed leading dimensions),
+// enqueue on the null stream and return the library's status code instead of nothing.
+#pragma once
+
+#include <chrono>
+
+#include "hpcdnn.h"
+
+namespace hpcdnn {
+
+// kernel/sgemm series: square, ld = N
+inline int sgemm(int N, const float* A, const float* B, float* C, float alpha, float beta) {
+    return hpcdnn_sgemm(N, N, N, A, N, B, N, C, N, alpha, beta, nullptr, 0, nullptr);
+}
+// kernel/ft_sgemm family: general M, N, K (row-major here: lda = K, ldb = N, ldc = N)
+inline int sgemm(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta) {
+    return hpcdnn_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, nullptr, 0, nullptr);
+}
+inline int ft_sgemm(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta,
+                    hpcdnn_ft_status* status = nullptr, const hpcdnn_fault* inject = nullptr) {
+    return hpcdnn_ft_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, 0.0f, inject, status, nullptr);
+}
+inline int saxpy(int N, float alpha, const float* x, float* y) { return hpcdnn_saxpy(N, alpha, x, y, nullptr); }
+// `ws` from hpcdnn_workspace_bytes(HPCDNN_OP_SDOT, ...) / hpcdnn_workspace_init
+inline int sdot(int N, const float* x, const float* y, float* out, void* ws, size_t ws_bytes) {
+    return hpcdnn_sdot(N, x, y, out, ws, ws_bytes, nullptr);
+}
+inline void cpu_gemm(float alpha, float beta, const float* mat1, const float* mat2, int n, float* mat3) {
+    hpcdnn_cpu_gemm(alpha, beta, mat1, mat2, n, mat3);
+}
+
+// utils/utils.cuh:53 and :56-77
+constexpr long ceil_div(long m, long n) { return (m + n - 1) / n; }
+
+class timer {
+public:
+    timer() { reset(); }
+    void reset() { t0_ = std::chrono::high_resolution_clock::now(); }
+    double elapsed(bool reset_timer = false) {
+        const auto t = std::chrono::high_resolution_clock::now();
+        const double s = std::chrono::duration<double>(t - t0_).count();
+        if (reset_timer) reset();
+        return s;
+    }
+    double elapsed_msec(bool reset_timer = false) { return elapsed(reset_timer) * 1000.0; }
+
+private:
+    std::chrono::high_resolution_clock::time_point t0_;
+};
+
+}  // namespace hpcdnn
