@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 4 SIMD x 64 flop/clk x 2.4 GHz
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per 6144^3 SGEMM launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by what the same
+# counters read for a device copy of known size): the figures and commands are in profiles/sgemm_kernel_6144cube.md
+SGEMM_6144_TRAFFIC_BYTES = 1.812e9
 
 
 def main() -> int:
@@ -148,7 +151,7 @@ def main() -> int:
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
-            "traffic": None,
+            "traffic": SGEMM_6144_TRAFFIC_BYTES,
             "kernel": "sgemm_kernel (one launch = 2*6144^3 flop)",
             "kernel_ms": round(kern_ms, 4),
         },
