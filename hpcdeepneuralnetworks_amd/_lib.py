@@ -15,6 +15,7 @@ CSRC = os.path.join(_PKG, "csrc")
 
 OP_SGEMM = 0
 OP_SDOT = 1
+OP_FT_SGEMM = 2
 FT_TILE_M = 256
 FT_TILE_N = 128
 
@@ -81,7 +82,7 @@ def lib():
     L.hpcdnn_sgemm_tile_info.restype = i
     L.hpcdnn_sgemm_tile_info.argtypes = [i, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.hpcdnn_ft_sgemm.restype = i
-    L.hpcdnn_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp]
+    L.hpcdnn_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, vp]
     L.hpcdnn_ft_num_tiles.restype = i
     L.hpcdnn_ft_num_tiles.argtypes = [i, i]
     L.hpcdnn_ft_default_tau.restype = f

@@ -95,8 +95,10 @@ def sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Te
 
 
 def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
-             tau: float = 0.0, fault=None, status: torch.Tensor | None = None) -> None:
-    """ABFT GEMM; ``fault`` = (tile, row, col, delta) or None; ``status`` = int32 tensor of 8*ft_num_tiles words.
+             tau: float = 0.0, fault=None, status: torch.Tensor | None = None, ws: torch.Tensor | None = None) -> None:
+    """ABFT GEMM; ``fault`` = (tile, row, col, delta) or None; ``status`` = int32 tensor of 8*ft_num_tiles words;
+    ``ws`` = optional scratch tensor of ``ft_workspace_bytes(M, N, K)`` bytes (checksum vectors are then formed
+    by a pre-pass instead of inside the main loop).
 
     Counterpart of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)`` (kernel/ft_sgemm/sgemm.cu:159-165).
     """
@@ -113,7 +115,13 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
     f = None
     if fault is not None:
         f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
-    check(L.hpcdnn_ft_sgemm(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, f, sp, _stream()), "hpcdnn_ft_sgemm")
+    wp, wb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
+    check(L.hpcdnn_ft_sgemm(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, f, sp, wp, wb, _stream()),
+          "hpcdnn_ft_sgemm")
+
+
+def ft_workspace_bytes(M: int, N: int, K: int) -> int:
+    return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_FT_SGEMM, M, N, K))
 
 
 def ft_num_tiles(M: int, N: int) -> int:

@@ -7,6 +7,7 @@
 namespace hpcdnn {
 size_t sdot_workspace_bytes();
 size_t sgemm_workspace_bytes(int M, int N, int K);
+size_t ft_workspace_bytes(int M, int N, int K);
 }  // namespace hpcdnn
 
 extern "C" const char* hpcdnn_version(void) { return "hpcdnn 0.1 (gfx950)"; }
@@ -24,6 +25,7 @@ extern "C" size_t hpcdnn_workspace_bytes(int op, int M, int N, int K) {
     switch (op) {
         case HPCDNN_OP_SGEMM: return hpcdnn::sgemm_workspace_bytes(M, N, K);
         case HPCDNN_OP_SDOT: return hpcdnn::sdot_workspace_bytes();
+        case HPCDNN_OP_FT_SGEMM: return hpcdnn::ft_workspace_bytes(M, N, K);
         default: return 0;
     }
 }

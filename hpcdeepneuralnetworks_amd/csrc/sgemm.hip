@@ -45,12 +45,19 @@ static const TileConfig kTiles[] = {
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 constexpr int kFtTile = 0;  // 256 x 128, matches HPCDNN_FT_TILE_M/N
+// row length of the pre-encoded checksum vectors: K rounded up to the K step, plus two K steps of zeros for the
+// fetches that run ahead of the main loop
+static int ft_enc_ld(int K) { return (static_cast<int>(ceil_div(K, kGemmBK)) + 2) * kGemmBK; }
+size_t ft_workspace_bytes(int M, int N, int K);
 // Four waves: on this part every VALU instruction takes its issue cycles away from the FP32 matrix pipe of the
 // same SIMD, whichever wave it comes from, so more waves do not hide the checksum arithmetic; fewer, fatter
 // threads need the fewest VALU instructions per K step.
 constexpr int kFtWavesM = 2, kFtWavesN = 2, kFtThreads = kFtWavesM * kFtWavesN * kWave;
-static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, false, true, 1>;
-static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, true, true, 1>;
+static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, false, 1, 1>;
+static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, true, 1, 1>;
+// the same with the operands' checksum vectors read from a workspace (filled by the pre-encode kernels)
+static void (*const kFtPrePlain)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, false, 2, 1>;
+static void (*const kFtPreEdge)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, true, 2, 1>;
 
 static int device_cus() {
     static int cus = 0;
@@ -243,7 +250,7 @@ extern "C" float hpcdnn_ft_default_tau(int K) {
 
 extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                                float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
-                               void* stream) {
+                               void* ws, size_t ws_bytes, void* stream) {
     int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
     if (rc != HPCDNN_OK) return rc;
     if (M == 0 || N == 0) return HPCDNN_OK;
@@ -261,16 +268,44 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
         a.fault_delta = inject->delta;
     }
     const bool edge = needs_edge(a, cfg);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
+    // With a workspace the checksum vectors of A and B are formed once per tile row / tile column by two small
+    // bandwidth-bound kernels and the main loop only reads them; without one every workgroup forms them itself.
+    const size_t need = ft_workspace_bytes(M, N, K);
+    if (ws && K > 0) {
+        if (ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 15u)) return HPCDNN_ERR_WORKSPACE;
+        a.enc_ld = ft_enc_ld(K);
+        float* enc_a = static_cast<float*>(ws);
+        float* enc_b = enc_a + static_cast<size_t>(a.tiles_m) * a.enc_ld;
+        a.enc_a = enc_a;
+        a.enc_b = enc_b;
+        abft_encode_a_kernel<HPCDNN_FT_TILE_M><<<dim3(static_cast<unsigned>(ceil_div(a.enc_ld, 256)), a.tiles_m), 1024, 0, s>>>(
+            M, K, A, lda, enc_a, a.enc_ld);
+        abft_encode_b_kernel<HPCDNN_FT_TILE_N><<<dim3(static_cast<unsigned>(ceil_div(a.enc_ld, 64)), a.tiles_n), 256, 0, s>>>(
+            K, N, B, ldb, enc_b, a.enc_ld);
+        rc = launch_status();
+        if (rc != HPCDNN_OK) return rc;
+        void (*fn)(const GemmArgs) = edge ? kFtPreEdge : kFtPrePlain;
+        constexpr size_t lds = gemm_lds_bytes<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N, 2, kFtThreads>();
+        rc = enable_lds(fn, lds);
+        if (rc != HPCDNN_OK) return rc;
+        hipLaunchKernelGGL(fn, grid, dim3(kFtThreads), lds, s, a);
+        return launch_status();
+    }
     void (*fn)(const GemmArgs) = edge ? kFtEdge : kFtPlain;
-    constexpr size_t ft_lds = gemm_lds_bytes<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N, true, kFtThreads>();
+    constexpr size_t ft_lds = gemm_lds_bytes<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N, 1, kFtThreads>();
     rc = enable_lds(fn, ft_lds);
     if (rc != HPCDNN_OK) return rc;
-    dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
-    hipLaunchKernelGGL(fn, grid, dim3(kFtThreads), ft_lds, stream ? static_cast<hipStream_t>(stream) : nullptr, a);
+    hipLaunchKernelGGL(fn, grid, dim3(kFtThreads), ft_lds, s, a);
     return launch_status();
 }
 
 namespace hpcdnn {
+size_t ft_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return static_cast<size_t>(ceil_div(M, HPCDNN_FT_TILE_M) + ceil_div(N, HPCDNN_FT_TILE_N)) * ft_enc_ld(K) * sizeof(float);
+}
 size_t sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     Plan plan = choose_plan(M, N, K, true, static_cast<size_t>(-1));

@@ -32,14 +32,17 @@
 // MFMA so that they issue while the matrix core is busy.  sched_barrier fences
 // keep the compiler from regrouping them.
 //
-// With FT = true the kernel is the fused online-ABFT variant: see "ABFT
-// encode" in the main loop and "ABFT verification" after it.
+// With FT != 0 the kernel is the online-ABFT variant: see "ABFT encode" in the
+// main loop and "ABFT verification" after it.
 #pragma once
 
 #include <type_traits>
 
 #include "common.h"
 
+#ifndef HPCDNN_ABL
+#define HPCDNN_ABL 0
+#endif
 namespace hpcdnn {
 
 struct GemmArgs {
@@ -59,19 +62,22 @@ struct GemmArgs {
     int fault_tile, fault_row, fault_col;
     float fault_delta;
     hpcdnn_ft_status* status;
+    const float* enc_a;  // FT == 2: [tiles_m][enc_ld] column sums of A over each tile's rows
+    const float* enc_b;  // FT == 2: [tiles_n][enc_ld] row sums of B over each tile's columns
+    int enc_ld;          // row length: K rounded up to the K step, plus two K steps of zeros
 };
 
 constexpr int kGemmBK = 16;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tiles share A and B panels
 
-template <int BM, int BN, bool FT = false, int THREADS = 256>
+template <int BM, int BN, int FT = 0, int THREADS = 256>
 constexpr size_t gemm_lds_bytes() {
     // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x one column
     // sum per wave, 16 row sums) and a dump area for the branch-free predicated writes of the lanes that
     // publish nothing (one word per thread plus the reach of the strided writes)
     return sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8)) +
-           (FT ? sizeof(float) * (2 * (kGemmBK * (THREADS / 64) + kGemmBK) + THREADS + 2 * kGemmBK * (THREADS / 64)) : 0);
+           (FT == 1 ? sizeof(float) * (2 * (kGemmBK * (THREADS / 64) + kGemmBK) + THREADS + 2 * kGemmBK * (THREADS / 64)) : 0);
 }
 
 template <int N, class F>
@@ -106,9 +112,13 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
     tn = in_group / gsz;
 }
 
-// Raw buffer descriptor over [base, base + bytes): loads past the end return 0.
+// Raw buffer descriptor over [base, base + bytes), bytes >= 0: loads past the end return 0.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* base, int64_t bytes) {
-    const int64_t clipped = bytes < 0 ? 0 : (bytes > 0xFFFFFFFFll ? 0xFFFFFFFFll : bytes);
+    // bytes >= 0.  Clamped to 2^32 - 1 by looking at the upper half only: the value is wave-uniform, and a 32-bit
+    // compare stays on the scalar unit (a 64-bit signed one would occupy the vector unit the MFMAs need).
+    const unsigned hi = static_cast<unsigned>(static_cast<uint64_t>(bytes) >> 32);
+    const unsigned lo = static_cast<unsigned>(bytes);
+    const unsigned clipped = hi != 0u ? 0xFFFFFFFFu : lo;
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, static_cast<int>(clipped), 0x00020000);
 }
 
@@ -118,7 +128,9 @@ __device__ __forceinline__ v4f buffer_load_v4f(__amdgpu_buffer_rsrc_t rsrc, int 
     return __builtin_bit_cast(v4f, v);
 }
 
-template <int BM, int BN, int WGM, int WGN, bool EDGE, bool FT, int MIN_BLOCKS>
+// FT: 0 = plain SGEMM; 1 = ABFT, checksum vectors e^T A and B e formed inside the main loop; 2 = ABFT, checksum
+// vectors read from a workspace filled by abft_encode_a/b_kernel (fewer VALU instructions in the main loop).
+template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS>
 __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
     constexpr int kGemmThreads = WGM * WGN * kWave;
@@ -188,11 +200,34 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // One staging load (part P of the K step at a_base/b_base) into slot S.  Nothing here touches the loaded
     // value, so the load stays in flight until the slot is consumed a K step later.
     int k_slot[2] = {kbeg, kbeg};  // absolute k of the K step held by each staging slot
+    // FT == 2: the K step's slice of the pre-encoded checksum vectors travels with it (same run-ahead, same
+    // slots).  The rows of enc_a / enc_b end with two K steps of zeros, so the fetches that run ahead past the
+    // end need no bounds: one descriptor per row, a per-thread offset, and a scalar offset that moves on by one
+    // K step per fetch.
+    const __amdgpu_buffer_rsrc_t enc_a_rsrc =
+        make_rsrc(FT == 2 ? p.enc_a + static_cast<int64_t>(tile_m) * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * 4);
+    const __amdgpu_buffer_rsrc_t enc_b_rsrc =
+        make_rsrc(FT == 2 ? p.enc_b + static_cast<int64_t>(tile_n) * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * 4);
+    const int enc_a_voff = (tid >> 5) * 8;  // a_c of the two k rows of B this thread stages (stored side by side)
+    const int enc_b_voff = (tid & 3) * 16;  // b_r of the four k values of A this thread stages
+    int enc_off = kbeg * 4;
+    float g_ac[2][B_SLOTS];
+    v4f g_br[2];
     auto gload1 = [&](auto slot, auto part) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P == 0) k_slot[S] = k_loaded;
         if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc(a_base, a_left), a_voff[P]);
         else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[P - A_SLOTS]);
+        if constexpr (FT == 2 && P == NGL - 1) {
+            static_assert(FT != 2 || B_SLOTS == 2, "enc_a pairs the two k rows a thread stages");
+            typedef unsigned v2u __attribute__((ext_vector_type(2)));
+            typedef float v2f __attribute__((ext_vector_type(2)));
+            const v2f t = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(enc_a_rsrc, enc_a_voff, enc_off, 0));
+            g_ac[S][0] = t[0];
+            g_ac[S][B_SLOTS - 1] = t[1];
+            typedef unsigned v4u __attribute__((ext_vector_type(4)));
+            g_br[S] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_b_rsrc, enc_b_voff, enc_off, 0));
+        }
     };
     // Ragged tiles only, applied when the slot is consumed: columns k >= kend of A hold padding, the next K
     // slice or the next row, and columns n >= N / rows k >= kend of B likewise: force them to 0 (rows m >= M
@@ -228,6 +263,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         b_base += more ? b_step : 0;
         b_left = more ? b_left - b_step * 4 : 0;
         k_loaded += more ? BK : 0;
+        if constexpr (FT == 2) enc_off += BK * 4;
     };
     auto lstore1 = [&](auto slot, auto part, int stage) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
@@ -296,18 +332,26 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     float* const pub_b = (lr < B_SLOTS) ? s_br + (tid >> 5) + kHalfWaves * lr : s_dump;
     const int x32_addr = (lane ^ 32) * 4;  // ds_bpermute address of the partner lane in the other half wave
     double cc_ref[4], cr_ref[A_SLOTS];
-    float cc_lo[4], cr_lo[A_SLOTS];
+    float cc_lo[B_SLOTS][4], cr_lo[A_SLOTS][4];  // FP32 partials of the running sums, one per staged element
 #pragma unroll
-    for (int e = 0; e < 4; ++e) { cc_ref[e] = 0.0; cc_lo[e] = 0.f; }
+    for (int e = 0; e < 4; ++e) cc_ref[e] = 0.0;
 #pragma unroll
-    for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] = 0.0; cr_lo[sl] = 0.f; }
+    for (int sl = 0; sl < A_SLOTS; ++sl) cr_ref[sl] = 0.0;
+#pragma unroll
+    for (int sl = 0; sl < B_SLOTS; ++sl)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cc_lo[sl][e] = 0.f;
+#pragma unroll
+    for (int sl = 0; sl < A_SLOTS; ++sl)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cr_lo[sl][e] = 0.f;
     float e_pa[4], e_sw[4];
     v4f e_t[kPartV4 * B_SLOTS], e_brv;
     float e_pb0, e_pb1, e_pk, e_swb, e_ac[B_SLOTS];
     const int e_hw = tid >> 5;           // half wave = first k row this thread stages of B
     const int e_class = tid & 3;         // k group (4 k values) this thread stages of A
-    constexpr int NPROD = FT ? 11 : 0;   // pieces before the barrier
-    constexpr int NCONS = FT ? 6 : 0;    // pieces after the barrier
+    constexpr int NPROD = (FT == 1) ? 11 : 0;  // pieces before the barrier
+    constexpr int NCONS = FT ? 6 : 0;          // pieces after the barrier
     constexpr int kDppRor4 = 0x124, kDppRor8 = 0x128;  // rotate right inside each row of 16 lanes
 
     auto produce1 = [&](auto slot, auto piece, int par) {
@@ -383,7 +427,13 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         constexpr bool kFlush = decltype(flush)::value;
         const float* ap = s_apart + par * BK * kParts;
         const float* br = s_br + par * BK;
-        if constexpr (E == 0) {
+        if constexpr (FT == 2 && E <= 1) {
+            if constexpr (E == 0) {
+#pragma unroll
+                for (int sl = 0; sl < B_SLOTS; ++sl) e_ac[sl] = g_ac[S][sl];
+                e_brv = g_br[S];
+            }
+        } else if constexpr (E == 0) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
                 const float* row = ap + (e_hw + kHalfWaves * sl) * kParts;
@@ -400,34 +450,58 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 e_ac[sl] = (u.x + u.y) + (u.z + u.w);
                 HPCDNN_PIN(e_ac[sl]);
             }
+        } else if constexpr ((HPCDNN_ABL & 3) && E >= 2 && E <= 4) {
+            if constexpr ((HPCDNN_ABL & 1) && E == 2) {
+#pragma unroll
+                for (int sl = 0; sl < B_SLOTS; ++sl) asm volatile("" ::"v"(e_ac[sl]));
+                asm volatile("" ::"v"(e_brv));
+            }
         } else if constexpr (E == 2) {
+            // independent accumulators: a wave alone on its SIMD cannot hide the latency of dependent VALU
+            // instructions behind other waves
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
-                cc_lo[0] = __builtin_fmaf(e_ac[sl], rb[S][sl].x, cc_lo[0]);
-                cc_lo[1] = __builtin_fmaf(e_ac[sl], rb[S][sl].y, cc_lo[1]);
-                cc_lo[2] = __builtin_fmaf(e_ac[sl], rb[S][sl].z, cc_lo[2]);
-                cc_lo[3] = __builtin_fmaf(e_ac[sl], rb[S][sl].w, cc_lo[3]);
+                cc_lo[sl][0] = __builtin_fmaf(e_ac[sl], rb[S][sl].x, cc_lo[sl][0]);
+                cc_lo[sl][1] = __builtin_fmaf(e_ac[sl], rb[S][sl].y, cc_lo[sl][1]);
+                cc_lo[sl][2] = __builtin_fmaf(e_ac[sl], rb[S][sl].z, cc_lo[sl][2]);
+                cc_lo[sl][3] = __builtin_fmaf(e_ac[sl], rb[S][sl].w, cc_lo[sl][3]);
             }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) HPCDNN_PIN(cc_lo[e]);
+            for (int sl = 0; sl < B_SLOTS; ++sl)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) HPCDNN_PIN(cc_lo[sl][e]);
         } else if constexpr (E == 3 || E == 4) {
             constexpr int lo = (E == 3) ? 0 : A_SLOTS / 2, hi = (E == 3) ? A_SLOTS / 2 : A_SLOTS;
 #pragma unroll
             for (int sl = lo; sl < hi; ++sl) {
-                float t = __builtin_fmaf(ra[S][sl].x, e_brv.x, cr_lo[sl]);
-                t = __builtin_fmaf(ra[S][sl].y, e_brv.y, t);
-                t = __builtin_fmaf(ra[S][sl].z, e_brv.z, t);
-                cr_lo[sl] = __builtin_fmaf(ra[S][sl].w, e_brv.w, t);
-                HPCDNN_PIN(cr_lo[sl]);
+                cr_lo[sl][0] = __builtin_fmaf(ra[S][sl].x, e_brv.x, cr_lo[sl][0]);
+                cr_lo[sl][1] = __builtin_fmaf(ra[S][sl].y, e_brv.y, cr_lo[sl][1]);
+                cr_lo[sl][2] = __builtin_fmaf(ra[S][sl].z, e_brv.z, cr_lo[sl][2]);
+                cr_lo[sl][3] = __builtin_fmaf(ra[S][sl].w, e_brv.w, cr_lo[sl][3]);
             }
+#pragma unroll
+            for (int sl = lo; sl < hi; ++sl)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) HPCDNN_PIN(cr_lo[sl][e]);
         } else if constexpr (kFlush) {
-            // every 16th K step (and after the last one): FP32 partial -> FP64 running sum.  FP64 VALU
+            // every 16th K step (and after the last one): FP32 partials -> FP64 running sums.  FP64 VALU
             // instructions are twice as expensive as FP32 ones, so this is kept rare.
             if (flush_now) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { cc_ref[e] += static_cast<double>(cc_lo[e]); cc_lo[e] = 0.f; }
+                for (int e = 0; e < 4; ++e) {
+                    float t = cc_lo[0][e];
 #pragma unroll
-                for (int sl = 0; sl < A_SLOTS; ++sl) { cr_ref[sl] += static_cast<double>(cr_lo[sl]); cr_lo[sl] = 0.f; }
+                    for (int sl = 1; sl < B_SLOTS; ++sl) t += cc_lo[sl][e];
+                    cc_ref[e] += static_cast<double>(t);
+#pragma unroll
+                    for (int sl = 0; sl < B_SLOTS; ++sl) cc_lo[sl][e] = 0.f;
+                }
+#pragma unroll
+                for (int sl = 0; sl < A_SLOTS; ++sl) {
+                    cr_ref[sl] += static_cast<double>((cr_lo[sl][0] + cr_lo[sl][1]) + (cr_lo[sl][2] + cr_lo[sl][3]));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) cr_lo[sl][e] = 0.f;
+                }
             }
         }
     };
@@ -516,7 +590,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     }
 
     // ---- ABFT verification: inject (testing aid), observe, compare, locate, correct
-    if constexpr (FT) {
+    if constexpr (FT && !(HPCDNN_ABL & 4)) {
         constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;             // partials per column / per row checksum
         double* const s_ccref = reinterpret_cast<double*>(smem);        // [CCP][BN] reference column checksum partials
         double* const s_crref = s_ccref + CCP * BN;                     // [CRP][BM] reference row checksum partials
@@ -524,7 +598,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         float* const s_crobs = s_ccobs + WGM * BN;                      // [WGN][BM] observed row sums
         float* const s_dr = s_crobs + WGN * BM;                         // [BM] row residuals, then [BN] column residuals
         int* const s_meta = reinterpret_cast<int*>(s_dr + BM + BN);     // nbr, nbc, bad row, bad col, max clean (float bits)
-        static_assert(gemm_lds_bytes<BM, BN, true, kGemmThreads>() >=
+        static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads>() >=
                           sizeof(double) * (CCP * BN + CRP * BM) + sizeof(float) * (WGM * BN + WGN * BM + BM + BN) + 32,
                       "verification scratch fits in the staging buffers");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
@@ -695,6 +769,85 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
         float* dst = C + r * ldc + c;
         const float t = alpha * s;
         *dst = (beta == 0.f) ? t : __builtin_fmaf(beta, *dst, t);
+    }
+}
+
+// ---- ABFT pre-encode: the checksum vectors of the operands, one per tile row / tile column.
+// enc_a[tm][k'] = sum over the rows m of tile row tm (m < M) of A[m][k]; zero for K <= k < enc_ld; k' is k with
+// the order inside each group of 16 changed to 0, 8, 1, 9, ...
+// Block = 1024 threads: lane group q (64 of them) owns 4 consecutive k, wave w (16 of them) owns 16 of the
+// tile's 256 rows; the 16 partials are added in wave order, so the result does not depend on timing.
+template <int BM>
+__global__ __launch_bounds__(1024) void abft_encode_a_kernel(int M, int K, const float* __restrict__ A, int lda,
+                                                             float* __restrict__ enc_a, int enc_ld) {
+    constexpr int kWaves = 16, kRows = BM / kWaves;
+    __shared__ v4f part[kWaves][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int tile_m = blockIdx.y, m0 = tile_m * BM;
+    const int k = (blockIdx.x * kWave + lane) * 4;
+    const float* base = A + static_cast<int64_t>(m0) * lda;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base, (static_cast<int64_t>(M - 1 - m0) * lda + K) * 4);
+    v4f s = {0.f, 0.f, 0.f, 0.f};
+    if (k < K) {
+        v4f v[kRows];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) v[r] = buffer_load_v4f(rsrc, ((wave * kRows + r) * lda + k) * 4);
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) s += v[r];
+        // the group's tail beyond K holds the next row's first elements
+        s.y = (k + 1 < K) ? s.y : 0.f;
+        s.z = (k + 2 < K) ? s.z : 0.f;
+        s.w = (k + 3 < K) ? s.w : 0.f;
+    }
+    part[wave][lane] = s;
+    __syncthreads();
+    if (wave == 0 && k < enc_ld) {
+        v4f t = part[0][lane];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) t += part[w][lane];
+        // within each K step of 16, k and k + 8 sit side by side: the GEMM thread that stages rows k and k + 8 of
+        // the B tile fetches both with one 8-byte load
+        float* dst = enc_a + static_cast<int64_t>(tile_m) * enc_ld + (k & ~15);
+        const int q = k & 15, pos = (q & 7) * 2 + (q >> 3);
+        dst[pos] = t.x;
+        dst[pos + 2] = t.y;
+        dst[pos + 4] = t.z;
+        dst[pos + 6] = t.w;
+    }
+}
+
+// enc_b[tn][k] = sum over the columns n of tile column tn (n < N) of B[k][n]; zero for K <= k < enc_ld.
+// Block = 256 threads = 8 half waves; a half wave reads one k row of the tile (32 lanes x 4 columns) and owns
+// 8 rows of the block's 64.
+template <int BN>
+__global__ __launch_bounds__(256) void abft_encode_b_kernel(int K, int N, const float* __restrict__ B, int ldb,
+                                                            float* __restrict__ enc_b, int enc_ld) {
+    static_assert(BN == 128, "a half wave covers the tile's columns with one 16-byte load per lane");
+    constexpr int kRowsPerHalf = 8, kHalves = 8;
+    const int lr = threadIdx.x & 31, half = threadIdx.x >> 5;
+    const int tile_n = blockIdx.y, n0 = tile_n * BN;
+    const int kb = blockIdx.x * (kRowsPerHalf * kHalves);
+    float s[kRowsPerHalf];
+    v4f v[kRowsPerHalf];
+#pragma unroll
+    for (int i = 0; i < kRowsPerHalf; ++i) {
+        const int k = kb + half + kHalves * i;
+        const int kc = k < K ? k : K - 1;
+        const float* base = B + static_cast<int64_t>(kc) * ldb + n0;
+        v[i] = buffer_load_v4f(make_rsrc(base, static_cast<int64_t>(N - n0) * 4), lr * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < kRowsPerHalf; ++i) {
+        const int k = kb + half + kHalves * i;
+        float t = (v[i].x + v[i].y) + (v[i].z + v[i].w);
+        s[i] = half32_allsum(k < K ? t : 0.f);
+    }
+    if (lr < kRowsPerHalf) {
+        float out = s[0];
+#pragma unroll
+        for (int i = 1; i < kRowsPerHalf; ++i) out = (lr == i) ? s[i] : out;
+        const int k = kb + half + kHalves * lr;
+        if (k < enc_ld) enc_b[static_cast<int64_t>(tile_n) * enc_ld + k] = out;
     }
 }
 

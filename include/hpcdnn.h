@@ -43,6 +43,7 @@ extern "C" {
 /* Operation selectors for hpcdnn_workspace_bytes(). */
 #define HPCDNN_OP_SGEMM 0
 #define HPCDNN_OP_SDOT 1
+#define HPCDNN_OP_FT_SGEMM 2
 
 /* One soft error to inject: `delta` is added to the accumulator of element
  * (row, col) of output tile `tile` after the K loop and before verification.
@@ -103,11 +104,17 @@ int hpcdnn_sgemm_tile_info(int tile, int* bm, int* bn, int* bk);
  * (<= 0 selects the default for inputs of magnitude <= 1); `inject` is a HOST
  * pointer to one fault or NULL; `status` is DEVICE memory for
  * hpcdnn_ft_num_tiles(M,N) records or NULL.
+ * `ws`/`ws_bytes`: optional DEVICE scratch of
+ * hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM,M,N,K) bytes, 16-byte aligned, no
+ * initialisation needed.  With it the checksum vectors of A and B are formed
+ * once per tile row / tile column by two small kernels ahead of the GEMM
+ * (faster); with ws == NULL each workgroup forms them in its main loop, as the
+ * reference does.  Detection, location and correction are the same in both.
  * Replaces ft_sgemm_huge <<<dim3(M/128,N/128),256>>>(M,N,K,A,B,C,alpha,beta)
  * (kernel/ft_sgemm/sgemm.cu:159-165, kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21). */
 int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                     float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
-                    void* stream);
+                    void* ws, size_t ws_bytes, void* stream);
 int hpcdnn_ft_num_tiles(int M, int N);
 /* Threshold hpcdnn_ft_sgemm uses when tau <= 0. */
 float hpcdnn_ft_default_tau(int K);

@@ -23,8 +23,9 @@ inline int sgemm(int M, int N, int K, const float* A, const float* B, float* C, 
     return hpcdnn_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, nullptr, 0, nullptr);
 }
 inline int ft_sgemm(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta,
-                    hpcdnn_ft_status* status = nullptr, const hpcdnn_fault* inject = nullptr) {
-    return hpcdnn_ft_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, 0.0f, inject, status, nullptr);
+                    hpcdnn_ft_status* status = nullptr, const hpcdnn_fault* inject = nullptr, void* ws = nullptr,
+                    size_t ws_bytes = 0) {
+    return hpcdnn_ft_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, 0.0f, inject, status, ws, ws_bytes, nullptr);
 }
 inline int saxpy(int N, float alpha, const float* x, float* y) { return hpcdnn_saxpy(N, alpha, x, y, nullptr); }
 // `ws` from hpcdnn_workspace_bytes(HPCDNN_OP_SDOT, ...) / hpcdnn_workspace_init

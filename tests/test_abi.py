@@ -71,9 +71,9 @@ def test_bad_arguments_are_rejected_without_a_gpu(L):
     from hpcdeepneuralnetworks_amd._lib import Fault
 
     bad = Fault(5, 0, 0, 1.0)  # only one tile exists
-    assert L.hpcdnn_ft_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, 0.0, C.byref(bad), None, None) == INVALID
+    assert L.hpcdnn_ft_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, 0.0, C.byref(bad), None, None, 0, None) == INVALID
     bad = Fault(0, 256, 0, 1.0)
-    assert L.hpcdnn_ft_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, 0.0, C.byref(bad), None, None) == INVALID
+    assert L.hpcdnn_ft_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, 0.0, C.byref(bad), None, None, 0, None) == INVALID
 
 
 def test_tile_table_and_workspace_sizes(L):

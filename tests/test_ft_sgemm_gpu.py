@@ -1,4 +1,5 @@
-"""GPU parity of the fused ABFT SGEMM against the CPU model of the reference's checksum logic.
+"""GPU parity of the ABFT SGEMM against the CPU model of the reference's checksum logic, in both of its modes:
+checksum vectors formed inside the main loop (no workspace) and by the pre-pass kernels (with workspace).
 
 Values: same 1e-5 componentwise criterion as plain SGEMM (after correction).  Decisions (flag, located row and
 column, number of flagged lines) must equal the CPU model's exactly on the same seeded faults.
@@ -13,14 +14,28 @@ TOL = 1e-5
 DECISION_FIELDS = ("flag", "row", "col", "n_bad_rows", "n_bad_cols")
 
 
-def _run(blas, oracle_mod, M, N, K, alpha, beta, tau, fault, seed=400, lda=None, ldb=None, ldc=None):
+@pytest.fixture(params=["fused", "workspace"])
+def ft_mode(request):
+    return request.param
+
+
+def _ws(blas, mode, M, N, K):
+    if mode == "fused":
+        return None
+    nbytes = blas.ft_workspace_bytes(M, N, K)
+    assert nbytes == 4 * (-(-M // blas.FT_TILE_M) + -(-N // blas.FT_TILE_N)) * ((-(-K // 16) + 2) * 16)
+    # poisoned: the library must not rely on the workspace's previous contents
+    return torch.full((max(nbytes // 4, 4),), float("nan"), dtype=torch.float32, device="cuda")
+
+
+def _run(blas, oracle_mod, mode, M, N, K, alpha, beta, tau, fault, seed=400, lda=None, ldb=None, ldc=None):
     lda, ldb, ldc = lda or K, ldb or N, ldc or N
     a = oracle_mod.fill_uniform_matrix(M, K, seed, ld=lda)
     b = oracle_mod.fill_uniform_matrix(K, N, seed + 1, ld=ldb)
     c0 = oracle_mod.fill_uniform_matrix(M, N, seed + 2, ld=ldc)
     da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
     status = blas.ft_status_alloc(M, N)
-    blas.ft_sgemm(M, N, K, da, db, dc, alpha, beta, tau=tau, fault=fault, status=status)
+    blas.ft_sgemm(M, N, K, da, db, dc, alpha, beta, tau=tau, fault=fault, status=status, ws=_ws(blas, mode, M, N, K))
     st = blas.ft_status_numpy(status)
     c = dc.cpu().numpy()
     # model: a, b with zeroed padding so that the model never multiplies NaN padding (it indexes with ld too)
@@ -39,9 +54,9 @@ def _assert_values(oracle_mod, M, N, K, a, b, c0, c, alpha, beta):
 
 @pytest.mark.parametrize("M,N,K", [(256, 128, 64), (512, 384, 320), (300, 200, 100), (1, 1, 1), (257, 129, 17), (1024, 1024, 1024)])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, -1.5)])
-def test_fault_free_matches_model_and_oracle(blas, oracle_mod, M, N, K, alpha, beta):
+def test_fault_free_matches_model_and_oracle(blas, oracle_mod, ft_mode, M, N, K, alpha, beta):
     tau = blas.ft_default_tau(K)
-    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, alpha, beta, tau, None)
+    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, ft_mode, M, N, K, alpha, beta, tau, None)
     _assert_values(oracle_mod, M, N, K, a, b, c0, c, alpha, beta)
     for f in DECISION_FIELDS:
         assert np.array_equal(st[f], st_model[f]), f
@@ -50,12 +65,12 @@ def test_fault_free_matches_model_and_oracle(blas, oracle_mod, M, N, K, alpha, b
     assert st["max_clean_residual"].max() < 0.5 * tau
 
 
-def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod):
+def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod, ft_mode):
     """The reference's only fault experiment: +1.0 into local element (m=0, n=1) of a tile, threshold 0.1
     (ft_sgemm_huge.cuh:30,40,145) -> row 0 / column 1 located, 1.0 removed."""
     M, N, K = 512, 256, 256
     for tile in range(4):
-        a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, 0.1, (tile, 0, 1, 1.0))
+        a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, ft_mode, M, N, K, 1.0, 0.0, 0.1, (tile, 0, 1, 1.0))
         exp = [0, 0, 0, 0]
         exp[tile] = 1
         assert st["flag"].tolist() == exp
@@ -65,7 +80,7 @@ def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod):
         _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 0.0)
 
 
-def test_seeded_faults_decisions_equal_cpu_model(blas, oracle_mod):
+def test_seeded_faults_decisions_equal_cpu_model(blas, oracle_mod, ft_mode):
     # ragged problem: 3 x 3 tiles, last row/column of tiles clipped; padded leading dimensions
     M, N, K = 600, 300, 512
     tau = blas.ft_default_tau(K)
@@ -79,7 +94,7 @@ def test_seeded_faults_decisions_equal_cpu_model(blas, oracle_mod):
         i, j = int(rng.integers(tm)), int(rng.integers(tn))
         delta = float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-2, 2)))
         fault = (tile, i, j, delta)
-        a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 1.0, tau, fault,
+        a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, ft_mode, M, N, K, 1.0, 1.0, tau, fault,
                                                   seed=500 + trial, lda=K + 4, ldb=N + 4, ldc=N + 8)
         for f in DECISION_FIELDS:
             assert np.array_equal(st[f], st_model[f]), (fault, f, st[f], st_model[f])
@@ -89,23 +104,23 @@ def test_seeded_faults_decisions_equal_cpu_model(blas, oracle_mod):
         _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 1.0)
 
 
-def test_fault_below_threshold_or_outside_matrix_is_not_flagged(blas, oracle_mod):
+def test_fault_below_threshold_or_outside_matrix_is_not_flagged(blas, oracle_mod, ft_mode):
     M, N, K = 300, 200, 256
     tau = blas.ft_default_tau(K)
     # far below the threshold: stays in C (documented behaviour), nothing flagged
-    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, tau, (0, 3, 5, tau * 0.1))
+    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, ft_mode, M, N, K, 1.0, 0.0, tau, (0, 3, 5, tau * 0.1))
     assert np.all(st["flag"] == 0) and np.array_equal(st["flag"], st_model["flag"])
     # a fault aimed at a clipped-away element of an edge tile lands in zero padding that is never stored:
     # it is detected and removed by both the device and the model, or ignored by both
-    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, tau, (3, 200, 100, 5.0))
+    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, ft_mode, M, N, K, 1.0, 0.0, tau, (3, 200, 100, 5.0))
     _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 0.0)
 
 
-def test_many_flagged_lines_are_reported_uncorrectable(blas, oracle_mod):
+def test_many_flagged_lines_are_reported_uncorrectable(blas, oracle_mod, ft_mode):
     """More than one faulty row or column cannot be located by row x column intersection: a threshold below the
     rounding noise flags many lines, and the kernel must report flag 2 and leave the accumulators alone."""
     M, N, K = 256, 128, 512
-    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, 1e-9, None)
+    a, b, c0, c, st, c_model, st_model = _run(blas, oracle_mod, ft_mode, M, N, K, 1.0, 0.0, 1e-9, None)
     assert st["flag"][0] == 2 and st["n_bad_rows"][0] > 1 and st["n_bad_cols"][0] > 1
     assert (st["row"][0], st["col"][0]) == (-1, -1)
     _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 0.0)
@@ -128,7 +143,7 @@ class _TileModel:
         return self.oracle.abft_decide(dr, dc, tau)
 
 
-def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod):
+def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod, ft_mode):
     """BASELINE config 4: M=N=K=4096, alpha=1, beta=0, one seeded fault (tile, i, j, magnitude in [1e-2, 1e2],
     random sign) per launch.  Every launch: detected, located at the injected element, corrected, no other tile
     flagged; decisions equal the CPU model's for every launch (the model is evaluated on the faulted tile)."""
@@ -143,10 +158,11 @@ def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod):
     b = oracle_mod.fill_uniform_matrix(K, N, 21)
     tau = blas.ft_default_tau(K)
     status = blas.ft_status_alloc(M, N)
+    ws = _ws(blas, ft_mode, M, N, K)
     ntiles, ntn = blas.ft_num_tiles(M, N), N // blas.FT_TILE_N
     assert ntiles == 512
 
-    blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=tau, status=status)
+    blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=tau, status=status, ws=ws)
     clean = blas.ft_status_numpy(status)
     assert np.count_nonzero(clean["flag"]) == 0          # no false positives on the fault-free run
     assert clean["max_clean_residual"].max() < 0.6 * tau
@@ -162,7 +178,7 @@ def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod):
         tile = int(rng.integers(ntiles))
         i, j = int(rng.integers(blas.FT_TILE_M)), int(rng.integers(blas.FT_TILE_N))
         delta = float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-2, 2)))
-        blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=tau, fault=(tile, i, j, delta), status=status)
+        blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=tau, fault=(tile, i, j, delta), status=status, ws=ws)
         st = blas.ft_status_numpy(status)
         assert st["flag"][tile] == 1, (launch, tile, i, j, delta, st[tile])
         assert (st["row"][tile], st["col"][tile]) == (i, j), (launch, tile, i, j, delta, st[tile])
@@ -179,5 +195,5 @@ def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod):
         for f in DECISION_FIELDS:
             assert st[f][tile] == st_model[f], (launch, f, st[tile], st_model)
         assert abs(float(st["row_residual"][tile]) - fix_model) < 3e-3
-    print(f"campaign: {launches} launches, worst |C - C_clean| after correction {worst_err:.3e}, "
+    print(f"campaign ({ft_mode}): {launches} launches, worst |C - C_clean| after correction {worst_err:.3e}, "
           f"fault-free max residual {clean['max_clean_residual'].max():.3e}, tau {tau:.1e}")
