@@ -84,7 +84,8 @@ def main() -> int:
             m = 4096
             a, b, c = operands(m, m, m, 20)
             status = blas.ft_status_alloc(m, m)
-            fn = lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=blas.ft_default_tau(m), status=status)
+            ft_ws = blas.workspace(blas.ft_workspace_bytes(m, m, m))
+            fn = lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=blas.ft_default_tau(m), status=status, ws=ft_ws)
             work, unit = 2.0 * m ** 3, "GFLOP/s"
         else:
             nv = 1 << 28
@@ -198,17 +199,23 @@ def main() -> int:
         tau = blas.ft_default_tau(m)
         ms_plain = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0), st, wu)
         ms_plain_same_tile = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0, tile=0, split_k=1), st, wu)  # 256x128, the ABFT tile
-        ms_ft = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status), st, wu)
+        ft_ws = blas.workspace(blas.ft_workspace_bytes(m, m, m))
+        # with the workspace: checksum vectors pre-encoded by one small kernel (timed as part of the call)
+        ms_ft = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ft_ws), st, wu)
+        # without: every workgroup encodes them in its main loop
+        ms_ft_fused = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status), st, wu)
         extras["abft_4096"] = {
             "sgemm_gflops": round(2.0 * m ** 3 / ms_plain / 1e6, 1),
             "sgemm_same_tile_gflops": round(2.0 * m ** 3 / ms_plain_same_tile / 1e6, 1),
             "ft_sgemm_gflops": round(2.0 * m ** 3 / ms_ft / 1e6, 1),
             "overhead_pct_vs_sgemm": round((ms_ft - ms_plain) / ms_plain * 100.0, 2),
             "overhead_pct_vs_same_tile_sgemm": round((ms_ft - ms_plain_same_tile) / ms_plain_same_tile * 100.0, 2),
+            "no_workspace_ft_sgemm_gflops": round(2.0 * m ** 3 / ms_ft_fused / 1e6, 1),
+            "no_workspace_overhead_pct_vs_sgemm": round((ms_ft_fused - ms_plain) / ms_plain * 100.0, 2),
             "tau": tau,
         }
         ntiles = blas.ft_num_tiles(m, m)
-        blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status)
+        blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ft_ws)
         clean = blas.ft_status_numpy(status)
         c_clean = c.clone()
         rng = np.random.default_rng(2024)
@@ -218,7 +225,7 @@ def main() -> int:
         for _ in range(args.ft_launches):
             tile, i, j = int(rng.integers(ntiles)), int(rng.integers(blas.FT_TILE_M)), int(rng.integers(blas.FT_TILE_N))
             delta = float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-2, 2)))
-            blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, fault=(tile, i, j, delta), status=status)
+            blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, fault=(tile, i, j, delta), status=status, ws=ft_ws)
             s = blas.ft_status_numpy(status)
             hit = s["flag"][tile] != 0
             detected += int(hit)

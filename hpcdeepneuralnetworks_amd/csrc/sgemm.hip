@@ -280,10 +280,9 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
         float* enc_b = enc_a + static_cast<size_t>(a.tiles_m) * a.enc_ld;
         a.enc_a = enc_a;
         a.enc_b = enc_b;
-        abft_encode_a_kernel<HPCDNN_FT_TILE_M><<<dim3(static_cast<unsigned>(ceil_div(a.enc_ld, 256)), a.tiles_m), 1024, 0, s>>>(
-            M, K, A, lda, enc_a, a.enc_ld);
-        abft_encode_b_kernel<HPCDNN_FT_TILE_N><<<dim3(static_cast<unsigned>(ceil_div(a.enc_ld, 64)), a.tiles_n), 256, 0, s>>>(
-            K, N, B, ldb, enc_b, a.enc_ld);
+        const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
+        abft_encode_kernel<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N><<<k_blocks * (a.tiles_m + a.tiles_n), 1024, 0, s>>>(
+            M, N, K, A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, a.tiles_m);
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;
         void (*fn)(const GemmArgs) = edge ? kFtPreEdge : kFtPrePlain;

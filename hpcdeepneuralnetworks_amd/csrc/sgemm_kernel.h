@@ -772,82 +772,86 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
     }
 }
 
-// ---- ABFT pre-encode: the checksum vectors of the operands, one per tile row / tile column.
+// ---- ABFT pre-encode: the checksum vectors of the operands, one per tile row / tile column, in one launch of
+// 1024-thread blocks that each cover 256 values of k: the first k_blocks * tiles_m blocks encode A, the rest B.
+//
 // enc_a[tm][k'] = sum over the rows m of tile row tm (m < M) of A[m][k]; zero for K <= k < enc_ld; k' is k with
-// the order inside each group of 16 changed to 0, 8, 1, 9, ...
-// Block = 1024 threads: lane group q (64 of them) owns 4 consecutive k, wave w (16 of them) owns 16 of the
-// tile's 256 rows; the 16 partials are added in wave order, so the result does not depend on timing.
-template <int BM>
-__global__ __launch_bounds__(1024) void abft_encode_a_kernel(int M, int K, const float* __restrict__ A, int lda,
-                                                             float* __restrict__ enc_a, int enc_ld) {
-    constexpr int kWaves = 16, kRows = BM / kWaves;
-    __shared__ v4f part[kWaves][kWave];
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    const int tile_m = blockIdx.y, m0 = tile_m * BM;
-    const int k = (blockIdx.x * kWave + lane) * 4;
-    const float* base = A + static_cast<int64_t>(m0) * lda;
-    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base, (static_cast<int64_t>(M - 1 - m0) * lda + K) * 4);
-    v4f s = {0.f, 0.f, 0.f, 0.f};
-    if (k < K) {
-        v4f v[kRows];
-#pragma unroll
-        for (int r = 0; r < kRows; ++r) v[r] = buffer_load_v4f(rsrc, ((wave * kRows + r) * lda + k) * 4);
-#pragma unroll
-        for (int r = 0; r < kRows; ++r) s += v[r];
-        // the group's tail beyond K holds the next row's first elements
-        s.y = (k + 1 < K) ? s.y : 0.f;
-        s.z = (k + 2 < K) ? s.z : 0.f;
-        s.w = (k + 3 < K) ? s.w : 0.f;
-    }
-    part[wave][lane] = s;
-    __syncthreads();
-    if (wave == 0 && k < enc_ld) {
-        v4f t = part[0][lane];
-#pragma unroll
-        for (int w = 1; w < kWaves; ++w) t += part[w][lane];
-        // within each K step of 16, k and k + 8 sit side by side: the GEMM thread that stages rows k and k + 8 of
-        // the B tile fetches both with one 8-byte load
-        float* dst = enc_a + static_cast<int64_t>(tile_m) * enc_ld + (k & ~15);
-        const int q = k & 15, pos = (q & 7) * 2 + (q >> 3);
-        dst[pos] = t.x;
-        dst[pos + 2] = t.y;
-        dst[pos + 4] = t.z;
-        dst[pos + 6] = t.w;
-    }
-}
-
-// enc_b[tn][k] = sum over the columns n of tile column tn (n < N) of B[k][n]; zero for K <= k < enc_ld.
-// Block = 256 threads = 8 half waves; a half wave reads one k row of the tile (32 lanes x 4 columns) and owns
-// 8 rows of the block's 64.
-template <int BN>
-__global__ __launch_bounds__(256) void abft_encode_b_kernel(int K, int N, const float* __restrict__ B, int ldb,
-                                                            float* __restrict__ enc_b, int enc_ld) {
+// the order inside each group of 16 changed to 0, 8, 1, 9, ...  Lane q of a wave owns 4 consecutive k, wave w (16
+// of them) owns 16 of the tile's 256 rows; the 16 partials are added in wave order, so the result does not depend
+// on timing.
+//
+// enc_b[tn][k] = sum over the columns n of tile column tn (n < N) of B[k][n]; zero for K <= k < enc_ld.  A half
+// wave reads one k row of the tile (32 lanes x 4 columns) and owns 8 of the block's 256 rows.
+template <int BM, int BN>
+__global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
+                                                           const float* __restrict__ B, int ldb,
+                                                           float* __restrict__ enc_a, float* __restrict__ enc_b,
+                                                           int enc_ld, int k_blocks, int tiles_m) {
     static_assert(BN == 128, "a half wave covers the tile's columns with one 16-byte load per lane");
-    constexpr int kRowsPerHalf = 8, kHalves = 8;
-    const int lr = threadIdx.x & 31, half = threadIdx.x >> 5;
-    const int tile_n = blockIdx.y, n0 = tile_n * BN;
-    const int kb = blockIdx.x * (kRowsPerHalf * kHalves);
-    float s[kRowsPerHalf];
-    v4f v[kRowsPerHalf];
+    constexpr int kWaves = 16, kRows = BM / kWaves;
+    constexpr int kHalves = 2 * kWaves, kRowsPerHalf = 256 / kHalves;
+    __shared__ v4f part[kWaves][kWave];
+    const int a_blocks = k_blocks * tiles_m;
+    if (static_cast<int>(blockIdx.x) < a_blocks) {
+        const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+        const int tile_m = blockIdx.x / k_blocks, m0 = tile_m * BM;
+        const int k = ((blockIdx.x % k_blocks) * kWave + lane) * 4;
+        const float* base = A + static_cast<int64_t>(m0) * lda;
+        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base, (static_cast<int64_t>(M - 1 - m0) * lda + K) * 4);
+        v4f s = {0.f, 0.f, 0.f, 0.f};
+        if (k < K) {
+            v4f v[kRows];
 #pragma unroll
-    for (int i = 0; i < kRowsPerHalf; ++i) {
-        const int k = kb + half + kHalves * i;
-        const int kc = k < K ? k : K - 1;
-        const float* base = B + static_cast<int64_t>(kc) * ldb + n0;
-        v[i] = buffer_load_v4f(make_rsrc(base, static_cast<int64_t>(N - n0) * 4), lr * 16);
-    }
+            for (int r = 0; r < kRows; ++r) v[r] = buffer_load_v4f(rsrc, ((wave * kRows + r) * lda + k) * 4);
 #pragma unroll
-    for (int i = 0; i < kRowsPerHalf; ++i) {
-        const int k = kb + half + kHalves * i;
-        float t = (v[i].x + v[i].y) + (v[i].z + v[i].w);
-        s[i] = half32_allsum(k < K ? t : 0.f);
-    }
-    if (lr < kRowsPerHalf) {
-        float out = s[0];
+            for (int r = 0; r < kRows; ++r) s += v[r];
+            // the group's tail beyond K holds the next row's first elements
+            s.y = (k + 1 < K) ? s.y : 0.f;
+            s.z = (k + 2 < K) ? s.z : 0.f;
+            s.w = (k + 3 < K) ? s.w : 0.f;
+        }
+        part[wave][lane] = s;
+        __syncthreads();
+        if (wave == 0 && k < enc_ld) {
+            v4f t = part[0][lane];
 #pragma unroll
-        for (int i = 1; i < kRowsPerHalf; ++i) out = (lr == i) ? s[i] : out;
-        const int k = kb + half + kHalves * lr;
-        if (k < enc_ld) enc_b[static_cast<int64_t>(tile_n) * enc_ld + k] = out;
+            for (int w = 1; w < kWaves; ++w) t += part[w][lane];
+            // within each K step of 16, k and k + 8 sit side by side: the GEMM thread that stages rows k and
+            // k + 8 of the B tile fetches both with one 8-byte load
+            float* dst = enc_a + static_cast<int64_t>(tile_m) * enc_ld + (k & ~15);
+            const int q = k & 15, pos = (q & 7) * 2 + (q >> 3);
+            dst[pos] = t.x;
+            dst[pos + 2] = t.y;
+            dst[pos + 4] = t.z;
+            dst[pos + 6] = t.w;
+        }
+    } else {
+        const int bid = blockIdx.x - a_blocks;
+        const int lr = threadIdx.x & 31, half = threadIdx.x >> 5;
+        const int tile_n = bid / k_blocks, n0 = tile_n * BN;
+        const int kb = (bid % k_blocks) * 256;
+        float s[kRowsPerHalf];
+        v4f v[kRowsPerHalf];
+#pragma unroll
+        for (int i = 0; i < kRowsPerHalf; ++i) {
+            const int k = kb + half + kHalves * i;
+            const int kc = k < K ? k : K - 1;
+            const float* base = B + static_cast<int64_t>(kc) * ldb + n0;
+            v[i] = buffer_load_v4f(make_rsrc(base, static_cast<int64_t>(N - n0) * 4), lr * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < kRowsPerHalf; ++i) {
+            const int k = kb + half + kHalves * i;
+            const float t = (v[i].x + v[i].y) + (v[i].z + v[i].w);
+            s[i] = half32_allsum(k < K ? t : 0.f);
+        }
+        if (lr < kRowsPerHalf) {
+            float out = s[0];
+#pragma unroll
+            for (int i = 1; i < kRowsPerHalf; ++i) out = (lr == i) ? s[i] : out;
+            const int k = kb + half + kHalves * lr;
+            if (k < enc_ld) enc_b[static_cast<int64_t>(tile_n) * enc_ld + k] = out;
+        }
     }
 }
 
