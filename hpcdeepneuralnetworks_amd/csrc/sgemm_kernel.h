@@ -116,7 +116,8 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* base, int64_t bytes) {
     // bytes >= 0.  Clamped to 2^32 - 1 by looking at the upper half only: the value is wave-uniform, and a 32-bit
     // compare stays on the scalar unit (a 64-bit signed one would occupy the vector unit the MFMAs need).
-    const unsigned hi = static_cast<unsigned>(static_cast<uint64_t>(bytes) >> 32);
+    unsigned hi = static_cast<unsigned>(static_cast<uint64_t>(bytes) >> 32);
+    asm volatile("" : "+s"(hi));  // keeps the compiler from fusing the test below back into a 64-bit compare
     const unsigned lo = static_cast<unsigned>(bytes);
     const unsigned clipped = hi != 0u ? 0xFFFFFFFFu : lo;
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, static_cast<int>(clipped), 0x00020000);
