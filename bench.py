@@ -271,6 +271,31 @@ def main() -> int:
         ms = median_timed(lambda: blas.sdot(nt, x, y, out), 50, 5)
         extras["sdot_2p20_plus_7_GBps"] = round(8.0 * nt / ms / 1e6, 1)
         del x, y
+
+        # ---- SGEMV (4 algorithmic bytes per matrix element) and the offline ABFT baseline built from it
+        mv = 16384
+        am = torch.empty(mv, mv, device=dev)
+        blas.fill_uniform_matrix(am, mv, mv, 40)
+        xv = torch.empty(mv, device=dev)
+        yv = torch.empty(mv, device=dev)
+        blas.fill_uniform(xv, 41)
+        gws = blas.workspace(max(blas.sgemv_workspace_bytes(mv, mv), 4))
+        ms_n = median_timed(lambda: blas.sgemv(False, mv, mv, 1.0, am, xv, 0.0, yv), 20, 3)
+        ms_t = median_timed(lambda: blas.sgemv(True, mv, mv, 1.0, am, xv, 0.0, yv, ws=gws), 20, 3)
+        extras["sgemv_16384"] = {"n_GBps": round(4.0 * mv * mv / ms_n / 1e6, 1), "t_GBps": round(4.0 * mv * mv / ms_t / 1e6, 1),
+                                 "n_frac_hbm_peak": round(4.0 * mv * mv / ms_n / 1e6 / PEAK_HBM_GBS, 4),
+                                 "t_frac_hbm_peak": round(4.0 * mv * mv / ms_t / 1e6 / PEAK_HBM_GBS, 4)}
+        del am, xv, yv, gws
+        m = 4096
+        a, b, c = operands(m, m, m, 20)
+        ows = blas.workspace(blas.offline_ft_workspace_bytes(m, m, m))
+        res = torch.zeros(2 * (m // 256), device=dev)
+        ms_plain = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0), st, wu)
+        ms_off = median_timed(lambda: blas.offline_ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, res, ows), st, wu)
+        extras["offline_abft_4096"] = {"gflops": round(2.0 * m ** 3 / ms_off / 1e6, 1),
+                                       "overhead_pct_vs_sgemm": round((ms_off - ms_plain) / ms_plain * 100.0, 2),
+                                       "max_abs_residual_sum": float(res.abs().max())}
+        del a, b, c, ows
         result["extras"] = extras
 
     # ---------------- CPU baseline: the oracle's restatement of the reference's cpu_gemm, one thread, bounded sample

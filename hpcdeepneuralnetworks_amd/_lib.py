@@ -16,6 +16,9 @@ CSRC = os.path.join(_PKG, "csrc")
 OP_SGEMM = 0
 OP_SDOT = 1
 OP_FT_SGEMM = 2
+OP_SGEMV = 3
+OP_OFFLINE_FT_SGEMM = 4
+OFFLINE_FT_PANEL_K = 256
 FT_TILE_M = 256
 FT_TILE_N = 128
 
@@ -30,6 +33,8 @@ EXPORTS = (
     "hpcdnn_ft_sgemm",
     "hpcdnn_ft_num_tiles",
     "hpcdnn_ft_default_tau",
+    "hpcdnn_sgemv",
+    "hpcdnn_offline_ft_sgemm",
     "hpcdnn_saxpy",
     "hpcdnn_sdot",
     "hpcdnn_workspace_bytes",
@@ -87,6 +92,10 @@ def lib():
     L.hpcdnn_ft_num_tiles.argtypes = [i, i]
     L.hpcdnn_ft_default_tau.restype = f
     L.hpcdnn_ft_default_tau.argtypes = [i]
+    L.hpcdnn_sgemv.restype = i
+    L.hpcdnn_sgemv.argtypes = [i, i, i, f, fp, i, fp, f, fp, vp, sz, vp]
+    L.hpcdnn_offline_ft_sgemm.restype = i
+    L.hpcdnn_offline_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, C.POINTER(Fault), fp, vp, sz, vp]
     L.hpcdnn_saxpy.restype = i
     L.hpcdnn_saxpy.argtypes = [i64, f, fp, fp, vp]
     L.hpcdnn_sdot.restype = i

@@ -124,6 +124,49 @@ def ft_workspace_bytes(M: int, N: int, K: int) -> int:
     return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_FT_SGEMM, M, N, K))
 
 
+def sgemv(trans: bool, M: int, N: int, alpha: float, A: torch.Tensor, x: torch.Tensor, beta: float, y: torch.Tensor,
+          ws: torch.Tensor | None = None) -> None:
+    """Row-major SGEMV on an ``M x N`` matrix: ``y = alpha*A*x + beta*y`` or, with ``trans``, ``alpha*A^T*x + beta*y``.
+
+    Counterpart of the cublasSgemv calls in kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:8-23.
+    """
+    pa, lda = _matrix(A, M, N, "A")
+    px, py = _dev(x, "x"), _dev(y, "y")
+    if x.numel() < (M if trans else N) or y.numel() < (N if trans else M):
+        raise HpcdnnError("x or y shorter than the matrix dimension it pairs with")
+    wp, wb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
+    check(_lib.lib().hpcdnn_sgemv(1 if trans else 0, M, N, alpha, pa, lda, px, beta, py, wp, wb, _stream()), "hpcdnn_sgemv")
+
+
+def sgemv_workspace_bytes(M: int, N: int) -> int:
+    return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_SGEMV, M, N, 0))
+
+
+def offline_ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float,
+                     beta: float, residuals: torch.Tensor, ws: torch.Tensor, fault=None) -> None:
+    """Panel-wise (offline) ABFT GEMM; ``residuals`` = float32 tensor of ``2*ceil(K/256)`` elements (column-side and
+    row-side residual sums per panel); ``fault`` = (panel, row, col, delta) with global row/col, or None.
+
+    Counterpart of ``baseline_ft_sgemm(...)`` (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:1-34).
+    """
+    pa, lda = _matrix(A, M, K, "A")
+    pb, ldb = _matrix(B, K, N, "B")
+    pc, ldc = _matrix(Cm, M, N, "C")
+    panels = -(-K // _lib.OFFLINE_FT_PANEL_K)
+    pr = _dev(residuals, "residuals")
+    if residuals.numel() < 2 * panels or not residuals.is_contiguous():
+        raise HpcdnnError(f"residuals must be a contiguous float32 GPU tensor with >= {2 * panels} elements")
+    f = None
+    if fault is not None:
+        f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
+    check(_lib.lib().hpcdnn_offline_ft_sgemm(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, f, pr, ws.data_ptr(),
+                                             ws.numel() * ws.element_size(), _stream()), "hpcdnn_offline_ft_sgemm")
+
+
+def offline_ft_workspace_bytes(M: int, N: int, K: int) -> int:
+    return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_OFFLINE_FT_SGEMM, M, N, K))
+
+
 def ft_num_tiles(M: int, N: int) -> int:
     return int(_lib.lib().hpcdnn_ft_num_tiles(M, N))
 

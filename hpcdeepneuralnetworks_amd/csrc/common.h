@@ -72,4 +72,22 @@ __device__ __forceinline__ float wave_sum_lane63(float v) {
     return v;
 }
 
+// ---- buffer addressing --------------------------------------------------
+// Raw buffer descriptor over [base, base + bytes), bytes >= 0: loads past the end return 0.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* base, int64_t bytes) {
+    // bytes >= 0.  Clamped to 2^32 - 1 by looking at the upper half only: the value is wave-uniform, and a 32-bit
+    // compare stays on the scalar unit (a 64-bit signed one would occupy the vector unit the MFMAs need).
+    unsigned hi = static_cast<unsigned>(static_cast<uint64_t>(bytes) >> 32);
+    asm volatile("" : "+s"(hi));  // keeps the compiler from fusing the test below back into a 64-bit compare
+    const unsigned lo = static_cast<unsigned>(bytes);
+    const unsigned clipped = hi != 0u ? 0xFFFFFFFFu : lo;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, static_cast<int>(clipped), 0x00020000);
+}
+
+__device__ __forceinline__ v4f buffer_load_v4f(__amdgpu_buffer_rsrc_t rsrc, int byte_offset) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0);
+    return __builtin_bit_cast(v4f, v);
+}
+
 }  // namespace hpcdnn

@@ -112,23 +112,6 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
     tn = in_group / gsz;
 }
 
-// Raw buffer descriptor over [base, base + bytes), bytes >= 0: loads past the end return 0.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* base, int64_t bytes) {
-    // bytes >= 0.  Clamped to 2^32 - 1 by looking at the upper half only: the value is wave-uniform, and a 32-bit
-    // compare stays on the scalar unit (a 64-bit signed one would occupy the vector unit the MFMAs need).
-    unsigned hi = static_cast<unsigned>(static_cast<uint64_t>(bytes) >> 32);
-    asm volatile("" : "+s"(hi));  // keeps the compiler from fusing the test below back into a 64-bit compare
-    const unsigned lo = static_cast<unsigned>(bytes);
-    const unsigned clipped = hi != 0u ? 0xFFFFFFFFu : lo;
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, static_cast<int>(clipped), 0x00020000);
-}
-
-__device__ __forceinline__ v4f buffer_load_v4f(__amdgpu_buffer_rsrc_t rsrc, int byte_offset) {
-    typedef unsigned v4u __attribute__((ext_vector_type(4)));
-    const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0);
-    return __builtin_bit_cast(v4f, v);
-}
-
 // FT: 0 = plain SGEMM; 1 = ABFT, checksum vectors e^T A and B e formed inside the main loop; 2 = ABFT, checksum
 // vectors read from a workspace filled by abft_encode_a/b_kernel (fewer VALU instructions in the main loop).
 template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS>
@@ -221,12 +204,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[P - A_SLOTS]);
         if constexpr (FT == 2 && P == NGL - 1) {
             static_assert(FT != 2 || B_SLOTS == 2, "enc_a pairs the two k rows a thread stages");
-            typedef unsigned v2u __attribute__((ext_vector_type(2)));
             typedef float v2f __attribute__((ext_vector_type(2)));
             const v2f t = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(enc_a_rsrc, enc_a_voff, enc_off, 0));
             g_ac[S][0] = t[0];
             g_ac[S][B_SLOTS - 1] = t[1];
-            typedef unsigned v4u __attribute__((ext_vector_type(4)));
             g_br[S] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_b_rsrc, enc_b_voff, enc_off, 0));
         }
     };

@@ -44,6 +44,12 @@ extern "C" {
 #define HPCDNN_OP_SGEMM 0
 #define HPCDNN_OP_SDOT 1
 #define HPCDNN_OP_FT_SGEMM 2
+#define HPCDNN_OP_SGEMV 3            /* M, N as passed to hpcdnn_sgemv; only trans = 1 uses a workspace */
+#define HPCDNN_OP_OFFLINE_FT_SGEMM 4
+
+/* K panel of hpcdnn_offline_ft_sgemm (the reference checks every 256 columns,
+ * kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:3). */
+#define HPCDNN_OFFLINE_FT_PANEL_K 256
 
 /* One soft error to inject: `delta` is added to the accumulator of element
  * (row, col) of output tile `tile` after the K loop and before verification.
@@ -118,6 +124,42 @@ int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B
 int hpcdnn_ft_num_tiles(int M, int N);
 /* Threshold hpcdnn_ft_sgemm uses when tau <= 0. */
 float hpcdnn_ft_default_tau(int K);
+
+/* Row-major SGEMV, A is M x N with leading dimension lda >= N:
+ *   trans = 0:  y[M] = alpha * A   * x[N] + beta * y
+ *   trans = 1:  y[N] = alpha * A^T * x[M] + beta * y
+ * beta == 0 never reads y.  `ws`/`ws_bytes`: optional scratch of
+ * hpcdnn_workspace_bytes(HPCDNN_OP_SGEMV, M, N, 0) bytes for trans = 1 (rows
+ * are then split over more workgroups; the partial sums are added in a fixed
+ * order, so results do not depend on timing either way).
+ * Stands in for the cublasSgemv calls of the reference's offline ABFT baseline
+ * (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:8-23), which are column-major:
+ * its CUBLAS_OP_N on an M x N column-major matrix is trans = 1 on the same
+ * memory read as an N x M row-major one. */
+int hpcdnn_sgemv(int trans, int M, int N, float alpha, const float* A, int lda, const float* x, float beta, float* y,
+                 void* ws, size_t ws_bytes, void* stream);
+
+/* Offline (panel-wise) ABFT SGEMM composed from hpcdnn_sgemm, hpcdnn_sgemv,
+ * hpcdnn_saxpy and hpcdnn_sdot: C = alpha*A*B + beta*C is formed one K panel of
+ * HPCDNN_OFFLINE_FT_PANEL_K at a time, and after every panel the row and
+ * column sums of C are compared with checksums carried through the operands
+ * (e^T A_p) B_p and A_p (B_p e), accumulated over the panels.
+ * `residuals`: DEVICE array of 2*ceil(K/panel) floats; [2p] = sum over the
+ * columns of (column sums of C - reference), [2p+1] = the same over the rows,
+ * after panel p.  Fault-free both are rounding noise; a soft error of size d
+ * in C shows up as d in both from its panel on.  Detection only: like the
+ * reference baseline it neither locates nor corrects.
+ * `inject`: HOST pointer or NULL; `tile` = panel after whose product `delta`
+ * is added to C[row][col] (row, col global).
+ * `ws`: DEVICE scratch of hpcdnn_workspace_bytes(HPCDNN_OP_OFFLINE_FT_SGEMM,
+ * M,N,K) bytes, 16-byte aligned, no initialisation needed.
+ * Replaces baseline_ft_sgemm(num_tests, M, N, K, handle, dA, dB, dC, dE, dRes,
+ * dcheck_*..., alpha, beta, negative_1)
+ * (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:1-34; call site
+ * kernel/ft_sgemm/sgemm.cu:306), whose scratch vectors are the workspace here. */
+int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                            float alpha, float beta, const hpcdnn_fault* inject, float* residuals, void* ws,
+                            size_t ws_bytes, void* stream);
 
 /* y = alpha*x + y, one fused multiply-add per element, any n >= 0, any 4-byte
  * aligned x and y.  Replaces saxpy/saxpy3/_saxpy <<<ceil(n/4/tpb),tpb>>>

@@ -97,6 +97,11 @@ def _load():
     lib.oracle_ft_sgemm.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
                                     C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int, C.c_int, C.c_float,
                                     C.c_void_p]
+    lib.oracle_sgemv_f64.restype = None
+    lib.oracle_sgemv_f64.argtypes = [C.c_int, C.c_int, C.c_int, C.c_float, fp, C.c_int, fp, C.c_float, fp, dp, dp]
+    lib.oracle_offline_ft_sgemm.restype = None
+    lib.oracle_offline_ft_sgemm.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
+                                            C.c_float, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, dp]
     _lib = lib
     return lib
 
@@ -223,3 +228,23 @@ def ft_sgemm(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, tile_m, tile_n, tau, 
     _load().oracle_ft_sgemm(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, tile_m, tile_n, tau,
                             int(ft), int(fi), int(fj), float(fd), status.ctypes.data_as(C.c_void_p))
     return status
+
+
+def sgemv_f64(trans: bool, M: int, N: int, alpha: float, a: np.ndarray, lda: int, x: np.ndarray, beta: float,
+              y: np.ndarray | None):
+    """FP64 row-major SGEMV and its absolute-value scale: (out, den), both float64 of length N if trans else M."""
+    ylen = N if trans else M
+    out, den = np.empty(ylen, np.float64), np.empty(ylen, np.float64)
+    yp = _f(y) if (y is not None and beta != 0.0) else None
+    _load().oracle_sgemv_f64(int(bool(trans)), M, N, alpha, _f(a), lda, _f(x), beta, yp, _d(out), _d(den))
+    return out, den
+
+
+def offline_ft_sgemm(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, panel, fault=None) -> np.ndarray:
+    """FP64 model of the panel-wise ABFT GEMM; updates ``c`` in place and returns the 2*ceil(K/panel) residual sums."""
+    panels = -(-K // panel)
+    res = np.zeros(2 * max(panels, 1), np.float64)
+    fp_, fr, fc, fd = (-1, 0, 0, 0.0) if fault is None else fault
+    _load().oracle_offline_ft_sgemm(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, panel, int(fp_), int(fr),
+                                    int(fc), float(fd), _d(res))
+    return res[:2 * panels]

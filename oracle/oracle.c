@@ -13,6 +13,14 @@
  *
  * Parity status:
  *   oracle_cpu_gemm, oracle_gemm_f64, oracle_saxpy, oracle_sdot_*: pinned.
+ *   oracle_sgemv_f64: pinned (numpy float64 matrix-vector products, both
+ *     orientations, padded leading dimension).
+ *   oracle_offline_ft_sgemm: pinned to the closed form (residual sums are 0
+ *     before the faulted panel and delta from it on, for any alpha, beta and
+ *     panel width; final C equals the FP64 product plus the uncorrected
+ *     fault).  The reference computes these sums and never checks or prints
+ *     them (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:26-30), so it holds
+ *     no expected values: bit-level agreement with cuBLAS is parity unpinned.
  *   oracle_abft_*: pinned to the checksum algebra (e^T(AB) = (e^T A)B,
  *     (AB)e = A(Be)) and to the one known-answer case the reference holds
  *     (+1.0 at tile-local (0,1), threshold 0.1 -> row 0, col 1, magnitude 1;
@@ -315,4 +323,107 @@ void oracle_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         free(acc);
         free(dr);
     }
+}
+
+/* ----------------------------------------------- SGEMV / offline ABFT -- */
+
+/* Row-major SGEMV in FP64 on an M x N matrix: trans = 0: out[m] = alpha *
+ * sum_n A[m][n] x[n] + beta * y[m]; trans = 1: out[n] = alpha * sum_m A[m][n]
+ * x[m] + beta * y[n]; den = the same with absolute values (the scale the
+ * componentwise error criterion divides by).  y may be NULL when beta == 0.
+ * Restates what the reference asks of cublasSgemv in its offline ABFT baseline
+ * (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:8-23), in row-major terms. */
+void oracle_sgemv_f64(int trans, int M, int N, float alpha, const float* A, int lda, const float* x,
+                      float beta, const float* y, double* out, double* den) {
+    int ylen = trans ? N : M;
+    for (int i = 0; i < ylen; ++i) {
+        double s = 0.0, a = 0.0;
+        if (!trans)
+            for (int n = 0; n < N; ++n) {
+                double p = (double)A[(size_t)i * lda + n] * (double)x[n];
+                s += p; a += fabs(p);
+            }
+        else
+            for (int m = 0; m < M; ++m) {
+                double p = (double)A[(size_t)m * lda + i] * (double)x[m];
+                s += p; a += fabs(p);
+            }
+        double yv = (beta != 0.0f && y) ? (double)y[i] : 0.0;
+        out[i] = (double)alpha * s + (double)beta * yv;
+        den[i] = fabs((double)alpha) * a + fabs((double)beta) * fabs(yv);
+    }
+}
+
+/* Offline (panel-wise) ABFT in FP64: C is formed one K panel at a time; after
+ * panel p, res[2p] = sum_n (colsum(C)[n] - ref_col[n]) and res[2p+1] =
+ * sum_m (rowsum(C)[m] - ref_row[m]), where the references are carried through
+ * the operands: ref_col += alpha * (e^T A_p) B_p, ref_row += alpha * A_p (B_p e),
+ * starting from beta * colsum / rowsum of the initial C.  One fault: delta is
+ * added to C[row][col] right after panel fault_panel's product (fault_panel
+ * < 0: none).  C (float, M x N, ldc) receives the final result rounded to
+ * FP32.  Restates the call sequence of baseline_ft_sgemm
+ * (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:3-31: gemm, two gemv over C,
+ * two gemv over the panels, two gemv carrying them through, two axpy, two
+ * dot), with references that accumulate over the panels. */
+void oracle_offline_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb,
+                             float* C, int ldc, float alpha, float beta, int panel, int fault_panel,
+                             int fault_row, int fault_col, float fault_delta, double* res) {
+    double* acc = (double*)calloc((size_t)M * N, sizeof(double));
+    double* ref_row = (double*)calloc((size_t)M, sizeof(double));
+    double* ref_col = (double*)calloc((size_t)N, sizeof(double));
+    double* a_col = (double*)malloc(sizeof(double) * (size_t)panel);
+    double* b_row = (double*)malloc(sizeof(double) * (size_t)panel);
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            double c0 = (beta != 0.0f) ? (double)beta * (double)C[(size_t)m * ldc + n] : 0.0;
+            acc[(size_t)m * N + n] = c0;
+            ref_row[m] += c0;
+            ref_col[n] += c0;
+        }
+    int panels = (K + panel - 1) / panel;
+    for (int p = 0; p < panels; ++p) {
+        int k0 = p * panel, kp = (K - k0 < panel) ? K - k0 : panel;
+        #pragma omp parallel for schedule(static)
+        for (int m = 0; m < M; ++m)
+            for (int k = 0; k < kp; ++k) {
+                double a = (double)alpha * (double)A[(size_t)m * lda + k0 + k];
+                const float* brow = B + (size_t)(k0 + k) * ldb;
+                double* crow = acc + (size_t)m * N;
+                for (int n = 0; n < N; ++n) crow[n] += a * (double)brow[n];
+            }
+        if (p == fault_panel) acc[(size_t)fault_row * N + fault_col] += (double)fault_delta;
+        for (int k = 0; k < kp; ++k) {
+            double s = 0.0, t = 0.0;
+            for (int m = 0; m < M; ++m) s += (double)A[(size_t)m * lda + k0 + k];
+            for (int n = 0; n < N; ++n) t += (double)B[(size_t)(k0 + k) * ldb + n];
+            a_col[k] = s;
+            b_row[k] = t;
+        }
+        for (int n = 0; n < N; ++n) {
+            double s = 0.0;
+            for (int k = 0; k < kp; ++k) s += a_col[k] * (double)B[(size_t)(k0 + k) * ldb + n];
+            ref_col[n] += (double)alpha * s;
+        }
+        for (int m = 0; m < M; ++m) {
+            double s = 0.0;
+            for (int k = 0; k < kp; ++k) s += (double)A[(size_t)m * lda + k0 + k] * b_row[k];
+            ref_row[m] += (double)alpha * s;
+        }
+        double rc = 0.0, rr = 0.0;
+        for (int n = 0; n < N; ++n) {
+            double s = 0.0;
+            for (int m = 0; m < M; ++m) s += acc[(size_t)m * N + n];
+            rc += s - ref_col[n];
+        }
+        for (int m = 0; m < M; ++m) {
+            double s = 0.0;
+            for (int n = 0; n < N; ++n) s += acc[(size_t)m * N + n];
+            rr += s - ref_row[m];
+        }
+        res[2 * p] = rc;
+        res[2 * p + 1] = rr;
+    }
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) C[(size_t)m * ldc + n] = (float)acc[(size_t)m * N + n];
+    free(acc); free(ref_row); free(ref_col); free(a_col); free(b_row);
 }

@@ -251,3 +251,46 @@ def test_ft_sgemm_model_detects_and_corrects(oracle_mod, fault):
         assert flags == exp
         assert (st["row"][fault[0]], st["col"][fault[0]]) == (fault[1], fault[2])
         assert st["row_residual"][fault[0]] == pytest.approx(-fault[3], abs=1e-4)
+
+
+@pytest.mark.parametrize("trans", [False, True])
+def test_sgemv_f64_matches_numpy_and_is_not_transposed(oracle_mod, trans):
+    M, N, lda = 13, 29, 37
+    a = oracle_mod.fill_uniform_matrix(M, N, 71, ld=lda)
+    x = oracle_mod.fill_uniform(M if trans else N, 72)
+    y = oracle_mod.fill_uniform(N if trans else M, 73)
+    a64 = a[:, :N].astype(np.float64)
+    out, den = oracle_mod.sgemv_f64(trans, M, N, 1.25, a, lda, x, -0.75, y)
+    mat = a64.T if trans else a64
+    assert np.allclose(out, 1.25 * (mat @ x.astype(np.float64)) - 0.75 * y.astype(np.float64), rtol=0, atol=1e-12)
+    assert np.allclose(den, 1.25 * (np.abs(mat) @ np.abs(x).astype(np.float64)) + 0.75 * np.abs(y).astype(np.float64), rtol=0, atol=1e-12)
+    # a non-square matrix with the wrong orientation would not even have matching lengths: check one known entry
+    e = np.zeros(M if trans else N, np.float32)
+    e[2] = 1.0
+    out, _ = oracle_mod.sgemv_f64(trans, M, N, 1.0, a, lda, e, 0.0, None)
+    assert np.array_equal(out, (a64[2, :] if trans else a64[:, 2]))
+
+
+@pytest.mark.parametrize("alpha,beta,panel", [(1.0, 0.0, 256), (1.5, -0.5, 256), (1.0, 1.0, 100)])
+def test_offline_ft_model_closed_form(oracle_mod, alpha, beta, panel):
+    """Row and column sums of alpha*A*B + beta*C0 equal the checksums carried through the operands, so every
+    residual sum is 0 until a fault of size delta enters C and delta from that panel on; C keeps the fault."""
+    M, N, K = 37, 23, 700
+    a = oracle_mod.fill_uniform_matrix(M, K, 81)
+    b = oracle_mod.fill_uniform_matrix(K, N, 82)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, 83)
+    ref = alpha * (a.astype(np.float64) @ b.astype(np.float64)) + beta * c0
+    panels = -(-K // panel)
+    c = c0.copy()
+    res = oracle_mod.offline_ft_sgemm(M, N, K, a, K, b, N, c, N, alpha, beta, panel)
+    assert res.shape == (2 * panels,) and np.abs(res).max() < 1e-9
+    assert np.abs(c - ref).max() < 1e-5
+    for fault_panel in (0, panels - 1):
+        c = c0.copy()
+        res = oracle_mod.offline_ft_sgemm(M, N, K, a, K, b, N, c, N, alpha, beta, panel, (fault_panel, 5, 7, -3.5))
+        expect = np.repeat(np.where(np.arange(panels) >= fault_panel, -3.5, 0.0), 2)
+        assert np.abs(res - expect).max() < 1e-9
+        diff = c - ref
+        assert abs(diff[5, 7] + 3.5) < 1e-5
+        diff[5, 7] = 0.0
+        assert np.abs(diff).max() < 1e-5
