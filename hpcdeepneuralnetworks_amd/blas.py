@@ -65,6 +65,13 @@ def sgemm_workspace_bytes(M: int, N: int, K: int) -> int:
     return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_SGEMM, M, N, K))
 
 
+def sgemm_plan(M: int, N: int, K: int, ws_bytes: int = 0):
+    """(tile, split_k) the library picks for this shape."""
+    t, sp = C.c_int(), C.c_int()
+    check(_lib.lib().hpcdnn_sgemm_plan(M, N, K, ws_bytes, C.byref(t), C.byref(sp)), "hpcdnn_sgemm_plan")
+    return t.value, sp.value
+
+
 def tile_table():
     L = _lib.lib()
     out = []

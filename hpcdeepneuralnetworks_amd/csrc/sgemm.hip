@@ -8,39 +8,35 @@ namespace hpcdnn {
 struct TileConfig {
     int bm, bn, bk;
     int threads;
-    int blocks_per_cu;  // resident workgroups per CU the kernel is built for
+    int blocks_per_cu;  // resident workgroups per CU the kernel is built for (its launch bound)
     size_t lds_bytes;
     void (*plain)(const GemmArgs);
     void (*edge)(const GemmArgs);
-    float eff;       // measured steady-state fraction of the FP32 MFMA peak of one CU
-    float fixed_us;  // measured per-tile prologue + epilogue time
+    float eff;  // fitted steady-state fraction of the FP32 MFMA peak of one CU
 };
 
-#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, RESIDENT, EFF, FIXED)                                             \
+#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, EFF)                                                          \
     {                                                                                                    \
-        BM, BN, kGemmBK, WGM * WGN * kWave, RESIDENT, gemm_lds_bytes<BM, BN>(),                            \
-            sgemm_kernel<BM, BN, WGM, WGN, false, false, OCC>,                                           \
-            sgemm_kernel<BM, BN, WGM, WGN, true, false, OCC>, EFF, FIXED                                  \
+        BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
+            sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC>, EFF \
     }
 
-// The counterpart of the reference's small/medium/large/tall/wide/huge shape
-// table (kernel/ft_sgemm/code_gen/main.py:8-16), re-derived for 32x32 MFMA
-// blocks and four or eight 64-lane waves per workgroup.  RESIDENT = workgroups
-// that fit on one CU (registers and LDS); EFF and FIXED are least-squares fits
-// of t = rounds * (BM*BN*K / (EFF * peak per CU) + FIXED) to measured times over
-// square sizes 256..6144 on an MI355X.
+// The counterpart of the reference's small/medium/large/tall/wide/huge shape table
+// (kernel/ft_sgemm/code_gen/main.py:8-16), re-derived for 32x32 MFMA blocks and four or eight 64-lane waves per
+// workgroup.  EFF comes from a least-squares fit of plan_cost() below to measured times of every tile over
+// squares 256..6144 with K = n, 1024 and 256 and a set of skinny shapes on an MI355X.
 static const TileConfig kTiles[] = {
-    HPCDNN_TILE(256, 128, 2, 2, 2, 2, 0.940f, 6.2f),   // 0 huge (the ABFT tile)
-    HPCDNN_TILE(128, 128, 2, 2, 2, 3, 0.919f, 4.1f),   // 1 large
-    HPCDNN_TILE(128, 64, 2, 2, 2, 4, 0.864f, 3.1f),    // 2 tall
-    HPCDNN_TILE(64, 128, 2, 2, 2, 4, 0.892f, 3.4f),    // 3 wide
-    HPCDNN_TILE(64, 64, 2, 2, 4, 8, 0.816f, 2.3f),     // 4 medium
-    HPCDNN_TILE(192, 256, 2, 2, 1, 1, 0.954f, 7.3f),   // 5 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
-    HPCDNN_TILE(256, 192, 2, 2, 1, 1, 0.935f, 7.4f),   // 6
-    HPCDNN_TILE(128, 256, 2, 2, 2, 2, 0.937f, 6.3f),   // 7
-    HPCDNN_TILE(256, 256, 2, 4, 1, 1, 0.971f, 10.8f),  // 8 giant, eight waves
-    HPCDNN_TILE(256, 128, 4, 2, 1, 1, 0.927f, 4.7f),   // 9 huge, eight waves
-    HPCDNN_TILE(256, 256, 4, 2, 1, 1, 0.968f, 9.0f),   // 10 giant, eight waves (4 x 2)
+    HPCDNN_TILE(256, 128, 2, 2, 2, 0.978f),  // 0 huge (the ABFT tile)
+    HPCDNN_TILE(128, 128, 2, 2, 2, 0.970f),  // 1 large
+    HPCDNN_TILE(128, 64, 2, 2, 2, 0.945f),   // 2 tall
+    HPCDNN_TILE(64, 128, 2, 2, 2, 0.939f),   // 3 wide
+    HPCDNN_TILE(64, 64, 2, 2, 4, 0.929f),    // 4 medium
+    HPCDNN_TILE(192, 256, 2, 2, 1, 0.964f),  // 5 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
+    HPCDNN_TILE(256, 192, 2, 2, 1, 0.946f),  // 6
+    HPCDNN_TILE(128, 256, 2, 2, 2, 0.987f),  // 7
+    HPCDNN_TILE(256, 256, 2, 4, 1, 1.000f),  // 8 giant, eight waves
+    HPCDNN_TILE(256, 128, 4, 2, 1, 1.000f),  // 9 huge, eight waves
+    HPCDNN_TILE(256, 256, 4, 2, 1, 1.000f),  // 10 giant, eight waves (4 x 2)
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
@@ -93,22 +89,33 @@ struct Plan {
     int split;
 };
 
-// Predicted run time in seconds.  Workgroups are dealt evenly to the CUs, so a launch takes as long as the CU
-// with the most tiles: ceil(tiles / CUs) tile times (co-resident workgroups share the CU's matrix cores, which
-// changes the overlap of prologues, not the throughput).
+// Predicted run time in seconds (up to a constant per launch).  Workgroups are dealt evenly to the CUs, so a launch
+// takes as long as the CU with the most tiles: n = ceil(tiles / CUs) tile times on its matrix cores (co-resident
+// workgroups share them), plus the part of each tile's prologue and epilogue that nothing overlaps: all of it when
+// one workgroup owns the CU, a fraction of it (after the first) when co-resident workgroups cover for each other.
+// The epilogue grows with the tile's area (C is written at the CU's share of HBM bandwidth).  A four-per-CU tile
+// running with fewer co-residents loses efficiency: one wave per SIMD cannot hide its own barriers.
 constexpr double kPeakFlopsPerCu = 157.3e12 / 256.0;
-constexpr double kEdgePenalty = 1.10;        // ragged-tile kernel: mask instructions compete with the MFMAs
-constexpr double kReduceFixed = 8e-6;        // second launch of split-K
-constexpr double kReduceBytesPerSec = 3e12;  // partials written once and read once, C written once
+constexpr double kEdgePenalty = 1.10;          // ragged-tile kernel: mask instructions compete with the MFMAs
+constexpr double kFixedBase = 2.133e-6;        // prologue + epilogue of a tile: base ...
+constexpr double kFixedPer32K = 2.31e-6;       // ... plus this per 32768 elements of tile area
+constexpr double kCoveredFraction = 0.209;     // exposed share of the fixed part behind a co-resident workgroup
+constexpr double kThinPenalty = 0.253;         // efficiency lost by a 4-per-CU tile per missing co-resident (x 1/4)
+constexpr double kReduceFixed = 2.5e-6;        // second launch of split-K
+constexpr double kReduceBytesPerSec = 8e12;    // partials written once and read once, C written once
 
 static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int cus) {
     const double tiles = static_cast<double>(ceil_div(M, t.bm)) * ceil_div(N, t.bn) * split;
-    const double rounds = ceil(tiles / cus);
+    const double n = ceil(tiles / cus);
     const double k_slice = ceil(static_cast<double>(ceil_div(K, split)) / t.bk) * t.bk;
     const bool edge = (M % t.bm) || (N % t.bn) || (K % t.bk);
-    const double per_tile = 2.0 * t.bm * t.bn * k_slice / (kPeakFlopsPerCu * t.eff) * (edge ? kEdgePenalty : 1.0) +
-                            t.fixed_us * 1e-6;
-    double cost = rounds * per_tile;
+    double eff = t.eff;
+    const double resident = t.blocks_per_cu < n ? t.blocks_per_cu : n;
+    if (t.blocks_per_cu >= 4) eff *= 1.0 - kThinPenalty * (t.blocks_per_cu - resident) / t.blocks_per_cu;
+    const double per_tile = 2.0 * t.bm * t.bn * k_slice / (kPeakFlopsPerCu * eff) * (edge ? kEdgePenalty : 1.0);
+    const double fixed = kFixedBase + kFixedPer32K * t.bm * t.bn / 32768.0;
+    const double exposed = t.blocks_per_cu == 1 ? n : 1.0 + kCoveredFraction * (n - 1.0);
+    double cost = n * per_tile + exposed * fixed;
     if (split > 1) cost += kReduceFixed + (2.0 * split + 1.0) * M * static_cast<double>(N) * 4.0 / kReduceBytesPerSec;
     return cost;
 }
@@ -235,6 +242,14 @@ extern "C" int hpcdnn_sgemm_tile_info(int tile, int* bm, int* bn, int* bk) {
     if (bm) *bm = kTiles[tile].bm;
     if (bn) *bn = kTiles[tile].bn;
     if (bk) *bk = kTiles[tile].bk;
+    return HPCDNN_OK;
+}
+
+extern "C" int hpcdnn_sgemm_plan(int M, int N, int K, size_t ws_bytes, int* tile, int* split_k) {
+    if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
+    const Plan plan = choose_plan(M, N, K, ws_bytes > 0, ws_bytes);
+    if (tile) *tile = plan.tile;
+    if (split_k) *split_k = plan.split;
     return HPCDNN_OK;
 }
 

@@ -101,6 +101,9 @@ int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B
  * shape table (kernel/ft_sgemm/code_gen/main.py:8-16). */
 int hpcdnn_sgemm_num_tiles(void);
 int hpcdnn_sgemm_tile_info(int tile, int* bm, int* bn, int* bk);
+/* The (tile, split_k) hpcdnn_sgemm picks for a shape when given a workspace of
+ * ws_bytes (0 = none): a function of the shape and the device's CU count only. */
+int hpcdnn_sgemm_plan(int M, int N, int K, size_t ws_bytes, int* tile, int* split_k);
 
 /* SGEMM with fused online ABFT: row/column checksums of each 256x128 output
  * tile are accumulated from A and B inside the main loop, compared with the
