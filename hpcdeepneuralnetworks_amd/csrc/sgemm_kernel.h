@@ -40,9 +40,6 @@
 
 #include "common.h"
 
-#ifndef HPCDNN_ABL
-#define HPCDNN_ABL 0
-#endif
 namespace hpcdnn {
 
 struct GemmArgs {
@@ -432,12 +429,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 e_ac[sl] = (u.x + u.y) + (u.z + u.w);
                 HPCDNN_PIN(e_ac[sl]);
             }
-        } else if constexpr ((HPCDNN_ABL & 3) && E >= 2 && E <= 4) {
-            if constexpr ((HPCDNN_ABL & 1) && E == 2) {
-#pragma unroll
-                for (int sl = 0; sl < B_SLOTS; ++sl) asm volatile("" ::"v"(e_ac[sl]));
-                asm volatile("" ::"v"(e_brv));
-            }
         } else if constexpr (E == 2) {
             // independent accumulators: a wave alone on its SIMD cannot hide the latency of dependent VALU
             // instructions behind other waves
@@ -572,7 +563,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     }
 
     // ---- ABFT verification: inject (testing aid), observe, compare, locate, correct
-    if constexpr (FT && !(HPCDNN_ABL & 4)) {
+    if constexpr (FT) {
         constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;             // partials per column / per row checksum
         double* const s_ccref = reinterpret_cast<double*>(smem);        // [CCP][BN] reference column checksum partials
         double* const s_crref = s_ccref + CCP * BN;                     // [CRP][BM] reference row checksum partials
