@@ -175,11 +175,18 @@ def main() -> int:
         extras["rocblas_via_torch_6144_gflops"] = round(flop / ms / 1e6, 1)
         del a, b, c
 
+        # square sizes of the sweep: without a workspace (no split of any kind) and with the optional workspace
+        # (the tiles left over after the last full round of CUs are then split along K), hipBLASLt beside them
         sweep = {}
         for m in (1024, 2048, 3072, 4096, 5120):
             a, b, c = operands(m, m, m, 10)
+            ws = blas.workspace(max(blas.sgemm_workspace_bytes(m, m, m), 4))
             ms = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0), st, wu)
-            sweep[str(m)] = round(2.0 * m ** 3 / ms / 1e6, 1)
+            ms_ws = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0, ws=ws), st, wu)
+            ms_lt = median_timed(lambda: torch.matmul(a, b, out=c), st, wu)
+            sweep[str(m)] = {"no_workspace": round(2.0 * m ** 3 / ms / 1e6, 1), "workspace": round(2.0 * m ** 3 / ms_ws / 1e6, 1),
+                             "hipblaslt_via_torch": round(2.0 * m ** 3 / ms_lt / 1e6, 1)}
+            del a, b, c, ws
         extras["sgemm_square_gflops"] = sweep
 
         # irregular / skinny shapes (split-K with a caller-provided workspace where the library chooses it)

@@ -86,7 +86,8 @@ static int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {
 
 struct Plan {
     int tile;
-    int split;
+    int split;  // > 1: every tile split this many ways along K; < -1: only the tiles after the last full round of CUs
+                // are split (-split ways); 1: no split
 };
 
 // Predicted run time in seconds (up to a constant per launch).  Workgroups are dealt evenly to the CUs, so a launch
@@ -120,6 +121,32 @@ static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int
     return cost;
 }
 
+// Tail split: with T tiles on `cus` CUs the last T % cus tiles keep only some CUs busy for a whole tile time.
+// Splitting just those tiles s ways along K turns that round into ceil(r*s/cus) rounds of 1/s tile time each, at the
+// price of writing and re-reading r*s raw tiles.  Returns the cost, and the chosen s through *ways (0 = no gain).
+static double tail_plan_cost(const TileConfig& t, int M, int N, int K, int cus, size_t ws_bytes, int* ways) {
+    *ways = 0;
+    const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+    const int64_t r = tiles % cus, full = tiles - r;
+    if (full == 0 || r == 0 || 2 * r > cus) return 1e300;
+    int64_t s = cus / r;
+    const int64_t most = K / (8 * t.bk);  // at least 8 K steps per slice
+    if (s > most) s = most;
+    if (s > 16) s = 16;
+    const size_t tile_bytes = static_cast<size_t>(t.bm) * t.bn * sizeof(float);
+    while (s >= 2 && static_cast<size_t>(r * s) * tile_bytes > ws_bytes) --s;
+    if (s < 2) return 1e300;
+    const bool edge = (M % t.bm) || (N % t.bn) || (K % t.bk);
+    const double per_tile = 2.0 * t.bm * t.bn * K / (kPeakFlopsPerCu * t.eff) * (edge ? kEdgePenalty : 1.0);
+    const double n_full = static_cast<double>(full / cus);
+    const double fixed = kFixedBase + kFixedPer32K * t.bm * t.bn / 32768.0;
+    const double n = n_full + 1.0;
+    const double exposed = t.blocks_per_cu == 1 ? n : 1.0 + kCoveredFraction * (n - 1.0);
+    *ways = static_cast<int>(s);
+    return n_full * per_tile + ceil(static_cast<double>(r * s) / cus) * per_tile / s + exposed * fixed + kReduceFixed +
+           (2.0 * s + 1.0) * r * static_cast<double>(tile_bytes) / kReduceBytesPerSec;
+}
+
 static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes) {
     const int cus = device_cus();
     Plan best{0, 1};
@@ -134,6 +161,11 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes) 
             }
             const double c = plan_cost(cfg, M, N, K, split, cus);
             if (c < best_cost) { best_cost = c; best = Plan{t, split}; }
+        }
+        if (allow_split) {
+            int ways = 0;
+            const double c = tail_plan_cost(cfg, M, N, K, cus, ws_bytes, &ways);
+            if (ways >= 2 && c < best_cost) { best_cost = c; best = Plan{t, -ways}; }
         }
     }
     return best;
@@ -178,7 +210,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
                      float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split, hipStream_t stream) {
     int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
     if (rc != HPCDNN_OK) return rc;
-    if (tile >= kNumTiles || split < 0) return HPCDNN_ERR_INVALID_VALUE;
+    if (tile >= kNumTiles || split == -1) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
 
     if (tile < 0 || split == 0) {
@@ -191,13 +223,33 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         }
     }
     const TileConfig& cfg = kTiles[tile];
+    GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
+    const int tiles = a.tiles_m * a.tiles_n;
+    a.full_tiles = tiles;
+    a.tail_split = 1;
+    int tail_tiles = 0;
+    if (split < -1) {
+        // tail split: the tiles after the last full round of CUs, -split ways (fewer if K is short)
+        const int cus = device_cus();
+        tail_tiles = tiles % cus;
+        int ways = -split;
+        a.tail_k_chunk = static_cast<int>(ceil_div(ceil_div(K, ways), cfg.bk)) * cfg.bk;
+        ways = K > 0 ? static_cast<int>(ceil_div(K, a.tail_k_chunk)) : 1;  // drop empty slices
+        if (tail_tiles == 0 || tail_tiles == tiles || ways < 2) {
+            tail_tiles = 0;  // nothing to gain: plain launch
+        } else {
+            const size_t need = static_cast<size_t>(tail_tiles) * ways * cfg.bm * cfg.bn * sizeof(float);
+            if (!ws || need > ws_bytes) return HPCDNN_ERR_WORKSPACE;
+            if (reinterpret_cast<uintptr_t>(ws) & 15u) return HPCDNN_ERR_INVALID_VALUE;
+            a.full_tiles = tiles - tail_tiles;
+            a.tail_split = ways;
+            a.tail_partial = static_cast<float*>(ws);
+        }
+        split = 1;
+    }
     if (split > 1) {
         if (!ws || static_cast<size_t>(M) * N * split * sizeof(float) > ws_bytes) return HPCDNN_ERR_WORKSPACE;
         if (reinterpret_cast<uintptr_t>(ws) & 3u) return HPCDNN_ERR_INVALID_VALUE;
-    }
-
-    GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
-    if (split > 1) {
         a.k_chunk = static_cast<int>(ceil_div(ceil_div(K, split), cfg.bk)) * cfg.bk;
         split = static_cast<int>(ceil_div(K, a.k_chunk));  // drop empty slices
         if (split > 1) a.partial = static_cast<float*>(ws);
@@ -207,10 +259,17 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     rc = enable_lds(fn, cfg.lds_bytes);
     if (rc != HPCDNN_OK) return rc;
 
-    dim3 grid(a.tiles_m * a.tiles_n, 1, split);
+    dim3 grid(a.full_tiles + tail_tiles * a.tail_split, 1, split);
     hipLaunchKernelGGL(fn, grid, dim3(cfg.threads), cfg.lds_bytes, stream, a);
     rc = launch_status();
-    if (rc != HPCDNN_OK || split == 1) return rc;
+    if (rc != HPCDNN_OK) return rc;
+    if (tail_tiles > 0) {
+        tail_reduce_kernel<<<dim3(tail_tiles, cfg.bm / 32), 256, 0, stream>>>(M, N, cfg.bm, cfg.bn, a.tiles_m, a.tiles_n,
+                                                                             a.full_tiles, a.tail_split, a.tail_partial, C,
+                                                                             ldc, alpha, beta);
+        return launch_status();
+    }
+    if (split == 1) return rc;
 
     const int64_t total = static_cast<int64_t>(M) * N;
     int rgrid = static_cast<int>(ceil_div(total, 256));
@@ -322,7 +381,13 @@ size_t ft_workspace_bytes(int M, int N, int K) {
 }
 size_t sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    Plan plan = choose_plan(M, N, K, true, static_cast<size_t>(-1));
-    return plan.split > 1 ? static_cast<size_t>(M) * N * plan.split * sizeof(float) : 0;
+    const Plan plan = choose_plan(M, N, K, true, static_cast<size_t>(-1));
+    if (plan.split > 1) return static_cast<size_t>(M) * N * plan.split * sizeof(float);
+    if (plan.split < -1) {
+        const TileConfig& cfg = kTiles[plan.tile];
+        const int64_t tail = (ceil_div(M, cfg.bm) * ceil_div(N, cfg.bn)) % device_cus();
+        return static_cast<size_t>(tail) * (-plan.split) * cfg.bm * cfg.bn * sizeof(float);
+    }
+    return 0;
 }
 }  // namespace hpcdnn

@@ -54,6 +54,10 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     int k_chunk;     // K range of one grid.z slice, a multiple of 16 (>= K when not split)
     float* partial;  // split-K: [gridDim.z][M][N] raw accumulators; nullptr = write C directly
+    // tail split: workgroups 0 .. full_tiles-1 compute whole tiles; the tiles after them are each split tail_split
+    // ways along K (tail_k_chunk per slice) and write raw accumulators to tail_partial[tile - full_tiles][slice][BM*BN]
+    int full_tiles, tail_split, tail_k_chunk;
+    float* tail_partial;
     // ABFT
     float tau;
     int fault_tile, fault_row, fault_col;
@@ -140,10 +144,19 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int wm = wave / WGN, wn = wave % WGN;
 
     int tile_m, tile_n;
-    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    int tile_id = blockIdx.x, k_slice = blockIdx.z, k_chunk = p.k_chunk;
+    float* tail_out = nullptr;
+    if (FT == 0 && p.tail_split > 1 && tile_id >= p.full_tiles) {
+        const int r = tile_id - p.full_tiles;
+        tile_id = p.full_tiles + r / p.tail_split;
+        k_slice = r % p.tail_split;
+        k_chunk = p.tail_k_chunk;
+        tail_out = p.tail_partial + static_cast<size_t>(r) * (BM * BN);
+    }
+    tile_of_block(tile_id, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int kbeg = blockIdx.z * p.k_chunk;
-    const int kend = (p.K - kbeg < p.k_chunk) ? p.K : kbeg + p.k_chunk;
+    const int kbeg = k_slice * k_chunk;
+    const int kend = (p.K - kbeg < k_chunk) ? p.K : kbeg + k_chunk;
     const int nkt = (kend - kbeg + BK - 1) / BK;
 
     // ---- global -> register staging: which 16-byte groups of the A and B tiles this thread moves.
@@ -686,6 +699,17 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int row_base = m0 + wm * WM + lh * 4;  // + i*32 + 8*(v/4) + v%4
     const int col_base = n0 + wn * WN + lr;      // + j*32
 
+    if (FT == 0 && tail_out) {
+        // whole tile, no bounds: rows and columns past the matrix hold zeros (their operands read as zeros)
+        float* out = tail_out + (wm * WM + lh * 4) * BN + wn * WN + lr;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) out[(i * 32 + 8 * (v / 4) + (v % 4)) * BN + j * 32] = acc[i][j][v];
+        return;
+    }
     if (p.partial) {
         float* out = p.partial + static_cast<size_t>(blockIdx.z) * p.M * p.N;
 #pragma unroll
@@ -742,6 +766,35 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
         float* dst = C + r * ldc + c;
         const float t = alpha * s;
         *dst = (beta == 0.f) ? t : __builtin_fmaf(beta, *dst, t);
+    }
+}
+
+// Fixed-order second phase of the tail split: for the tiles after the first full_tiles, C = alpha * (slice 0 +
+// slice 1 + ...) + beta*C.  grid = (tail tiles, bm / 32): one block adds 32 rows of one tile, 4 columns per thread.
+__global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, int bn, int tiles_m, int tiles_n,
+                                                          int full_tiles, int splits, const float* __restrict__ partial,
+                                                          float* __restrict__ C, int ldc, float alpha, float beta) {
+    int tile_m, tile_n;
+    tile_of_block(full_tiles + blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * bm, n0 = tile_n * bn;
+    const size_t tile_elems = static_cast<size_t>(bm) * bn;
+    const float* src = partial + static_cast<size_t>(blockIdx.x) * splits * tile_elems;
+    const int groups_per_row = bn / 4;
+    for (int g = threadIdx.x; g < 32 * groups_per_row; g += 256) {
+        const int r = blockIdx.y * 32 + g / groups_per_row, c = (g % groups_per_row) * 4;
+        const int row = m0 + r, col = n0 + c;
+        if (row >= M || col >= N) continue;
+        const size_t off = static_cast<size_t>(r) * bn + c;
+        v4f s = *reinterpret_cast<const v4f*>(src + off);
+        for (int z = 1; z < splits; ++z) s += *reinterpret_cast<const v4f*>(src + z * tile_elems + off);
+        const float sv[4] = {s.x, s.y, s.z, s.w};
+        float* dst = C + static_cast<size_t>(row) * ldc + col;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (col + e < N) {
+                const float t = alpha * sv[e];
+                dst[e] = (beta == 0.f) ? t : __builtin_fmaf(beta, dst[e], t);
+            }
     }
 }
 

@@ -92,7 +92,10 @@ int hpcdnn_sgemm(int M, int N, int K, const float* A, int lda, const float* B, i
 /* Same contract with the kernel choice pinned, for tests and sweeps:
  * `tile` indexes the built-in tile table (hpcdnn_sgemm_tile_info), -1 = pick
  * as hpcdnn_sgemm does; `split_k` >= 1 forces that many K slices (needs a
- * workspace of M*N*split_k floats when > 1), 0 = pick. */
+ * workspace of M*N*split_k floats when > 1), 0 = pick; `split_k` = -s (s >= 2)
+ * splits only the tiles left over after the last full round of CUs, s ways
+ * (workspace: leftover tiles * s * tile size floats, 16-byte aligned).  Either
+ * way the slices are added in a fixed order. */
 int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                     float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split_k, void* stream);
 
@@ -102,7 +105,8 @@ int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B
 int hpcdnn_sgemm_num_tiles(void);
 int hpcdnn_sgemm_tile_info(int tile, int* bm, int* bn, int* bk);
 /* The (tile, split_k) hpcdnn_sgemm picks for a shape when given a workspace of
- * ws_bytes (0 = none): a function of the shape and the device's CU count only. */
+ * ws_bytes (0 = none), split_k with the meaning it has for hpcdnn_sgemm_ex: a
+ * function of the shape and the device's CU count only. */
 int hpcdnn_sgemm_plan(int M, int N, int K, size_t ws_bytes, int* tile, int* split_k);
 
 /* SGEMM with fused online ABFT: row/column checksums of each 256x128 output

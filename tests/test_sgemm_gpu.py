@@ -188,3 +188,33 @@ def test_split_k_forced_matches_and_is_deterministic(blas, oracle_mod):
         outs.append(_check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=1, split_k=split, ws=ws, ldc=144))
     again = _check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=1, split_k=8, ws=ws, ldc=144)
     assert np.array_equal(outs[-1][:, :N], again[:, :N])
+
+
+def test_tail_split_forced_matches_and_is_deterministic(blas, oracle_mod):
+    """Only the tiles left over after the last full round of CUs are split along K (split_k < -1)."""
+    M, N, K = 1088, 1024, 520  # 64x64 tiles: 17 x 16 = 272 = 256 + 16 leftover tiles; ragged K
+    ws = blas.workspace(16 * 8 * 64 * 64 * 4)
+    outs = []
+    for ways in (2, 3, 8):
+        outs.append(_check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=4, split_k=-ways, ws=ws, ldc=N + 8))
+    again = _check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=4, split_k=-8, ws=ws, ldc=N + 8)
+    assert np.array_equal(outs[-1][:, :N], again[:, :N])
+    # the full tiles do not depend on how the leftover ones are split
+    plain = _check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=4, split_k=1, ldc=N + 8)
+    same = (plain[:, :N] == outs[0][:, :N])
+    assert same.mean() > 0.9
+    # ragged M and N with a leftover round, and no leftover at all (falls back to a plain launch)
+    _check(oracle_mod, blas, 1085, 1001, 300, 1.0, 0.0, tile=4, split_k=-2, ws=ws)
+    _check(oracle_mod, blas, 1024, 1024, 256, 1.0, 0.0, tile=4, split_k=-4, ws=ws)
+    with pytest.raises(blas.HpcdnnError):
+        _check(oracle_mod, blas, M, N, K, 1.0, 0.0, tile=4, split_k=-8, ws=None)
+
+
+def test_plan_is_a_function_of_the_shape_and_runs(blas, oracle_mod):
+    for shape in [(3072, 3072, 3072), (5120, 5120, 1024), (4352, 4352, 4352)]:
+        need = blas.sgemm_workspace_bytes(*shape)
+        plan = blas.sgemm_plan(*shape, need)
+        assert plan == blas.sgemm_plan(*shape, need)
+        assert blas.sgemm_plan(*shape, 0)[1] == 1  # no workspace, no split of any kind
+        ws = blas.workspace(max(need, 4))
+        _sampled_check(oracle_mod, blas, *shape, 1.0, 1.0, nrows=12, ws=ws)
