@@ -147,7 +147,7 @@ static double tail_plan_cost(const TileConfig& t, int M, int N, int K, int cus, 
            (2.0 * s + 1.0) * r * static_cast<double>(tile_bytes) / kReduceBytesPerSec;
 }
 
-static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes) {
+static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, bool allow_tail = true) {
     const int cus = device_cus();
     Plan best{0, 1};
     double best_cost = 1e300;
@@ -162,7 +162,7 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes) 
             const double c = plan_cost(cfg, M, N, K, split, cus);
             if (c < best_cost) { best_cost = c; best = Plan{t, split}; }
         }
-        if (allow_split) {
+        if (allow_split && allow_tail) {
             int ways = 0;
             const double c = tail_plan_cost(cfg, M, N, K, cus, ws_bytes, &ways);
             if (ways >= 2 && c < best_cost) { best_cost = c; best = Plan{t, -ways}; }
@@ -214,7 +214,8 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     if (M == 0 || N == 0) return HPCDNN_OK;
 
     if (tile < 0 || split == 0) {
-        Plan plan = choose_plan(M, N, K, ws != nullptr, ws ? ws_bytes : 0);
+        // the tail split moves 16-byte groups through the workspace
+        Plan plan = choose_plan(M, N, K, ws != nullptr, ws ? ws_bytes : 0, (reinterpret_cast<uintptr_t>(ws) & 15u) == 0);
         if (tile < 0) {
             tile = plan.tile;
             if (split == 0) split = plan.split;

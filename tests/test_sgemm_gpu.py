@@ -218,3 +218,15 @@ def test_plan_is_a_function_of_the_shape_and_runs(blas, oracle_mod):
         assert blas.sgemm_plan(*shape, 0)[1] == 1  # no workspace, no split of any kind
         ws = blas.workspace(max(need, 4))
         _sampled_check(oracle_mod, blas, *shape, 1.0, 1.0, nrows=12, ws=ws)
+
+
+SWEEP = list(range(256, 6145, 256)) + [1000, 3001, 6000]
+
+
+@pytest.mark.parametrize("n", SWEEP)
+def test_config3_square_sweep_every_size(blas, oracle_mod, n):
+    """Every size of the square sweep (256..6144 step 256, plus 1000, 3001, 6000): beta = 0 with the optional
+    workspace (whatever split the library picks), beta = 1 without."""
+    ws = blas.workspace(max(blas.sgemm_workspace_bytes(n, n, n), 4))
+    _sampled_check(oracle_mod, blas, n, n, n, 1.0, 0.0, nrows=6, seed=900 + n, ws=ws)
+    _sampled_check(oracle_mod, blas, n, n, n, 1.0, 1.0, nrows=6, seed=901 + n)
