@@ -97,7 +97,7 @@ struct Plan {
 // The epilogue grows with the tile's area (C is written at the CU's share of HBM bandwidth).  A four-per-CU tile
 // running with fewer co-residents loses efficiency: one wave per SIMD cannot hide its own barriers.
 constexpr double kPeakFlopsPerCu = 157.3e12 / 256.0;
-constexpr double kEdgePenalty = 1.10;          // ragged-tile kernel: mask instructions compete with the MFMAs
+constexpr double kEdgePenalty = 1.03;          // ragged tiles: partly empty tiles are paid in full by tile counting; this is the rest
 constexpr double kFixedBase = 2.133e-6;        // prologue + epilogue of a tile: base ...
 constexpr double kFixedPer32K = 2.31e-6;       // ... plus this per 32768 elements of tile area
 constexpr double kCoveredFraction = 0.209;     // exposed share of the fixed part behind a co-resident workgroup

@@ -222,8 +222,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         }
     };
     // Ragged tiles only, applied when the slot is consumed: columns k >= kend of A hold padding, the next K
-    // slice or the next row, and columns n >= N / rows k >= kend of B likewise: force them to 0 (rows m >= M
-    // of A and k >= K of B already read as 0 through the descriptor).
+    // slice or the next row: force them to 0 (rows m >= M of A and k >= K of B already read as 0 through the
+    // descriptor).  Columns n >= N of B hold the next row or padding too, but they only ever reach accumulators of
+    // columns n >= N, which are never stored: plain SGEMM leaves them alone, the ABFT kernels (whose row sums of B
+    // run over the whole tile width) force them to 0 as well.
     auto gmask1 = [&](auto slot, auto part) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P < A_SLOTS) {
@@ -234,7 +236,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             v.z = left > 2 ? v.z : 0.f;
             v.w = left > 3 ? v.w : 0.f;
             ra[S][P] = v;
-        } else {
+        } else if constexpr (FT != 0) {
             constexpr int Q = P - A_SLOTS;
             const int nv = (k_slot[S] + b_row[Q] < kend) ? b_nvalid[Q] : 0;
             v4f v = rb[S][Q];
@@ -504,10 +506,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     //                (+ consume the checksum partials of step kt+1)
     // Work past the end of the slice (kt+1, kt+2 >= nkt) moves duplicate data that is never multiplied, which
     // keeps the loop free of branches (and lets the loads stay two steps ahead).
-    auto step = [&](auto sl_next, auto sl_free, auto flush) {
+    auto step = [&](auto sl_next, auto sl_free, auto flush, auto masked) {
         // steps alternate between (next = slot 1, LDS stage 0) and (next = slot 0, LDS stage 1)
         constexpr int st = (decltype(sl_next)::value == 1) ? 0 : 1;
-        constexpr int NMASK = EDGE ? NGL : 0;
+        constexpr int NMASK = (EDGE && decltype(masked)::value) ? (FT ? NGL : A_SLOTS) : 0;
         constexpr int NS0 = NRD + NMASK + NPROD + 2 * NGL;
         constexpr int NS1 = NRD + NCONS;
         static_for<NMG>([&](auto m) {
@@ -565,13 +567,21 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         static_for<NCONS>([&](auto e) { consume1(S0{}, e, 0, std::true_type{}); });
         static_for<NRD>([&](auto s) { fread1(S0{}, s, 0, 0); });
         int kt = 0;
+        if constexpr (EDGE && FT == 0) {
+            // plain SGEMM on a ragged tile: only the last K step can be partial, and step kt consumes the staged
+            // data of step kt+1, so every step before kt = nkt-2 runs without the masks
+            for (; kt + 3 < nkt; kt += 2) {
+                step(S1{}, S0{}, std::false_type{}, std::false_type{});
+                step(S0{}, S1{}, std::false_type{}, std::false_type{});
+            }
+        }
         for (; kt + 1 < nkt; kt += 2) {
-            step(S1{}, S0{}, std::false_type{});
+            step(S1{}, S0{}, std::false_type{}, std::true_type{});
             flush_now = ((kt & 14) == 14) || (kt + 2 >= nkt);
-            step(S0{}, S1{}, std::true_type{});
+            step(S0{}, S1{}, std::true_type{}, std::true_type{});
         }
         flush_now = true;
-        if (kt < nkt) step(S1{}, S0{}, std::true_type{});
+        if (kt < nkt) step(S1{}, S0{}, std::true_type{}, std::true_type{});
         __syncthreads();  // every wave is done with the staging buffers (the verification below reuses them)
     }
 
