@@ -42,9 +42,10 @@ __global__ __launch_bounds__(kGemvThreads) void sgemv_n_kernel(int M, int N, flo
 }
 
 // out[n] = sum over the rows m of one chunk of A[m][n] x[m], for the 256 columns of one block.  Wave w takes rows
-// first + w, first + w + 4, ...: every load is one 1 KiB piece of a row; the four wave partials are added in wave
+// first + w, first + w + 4, ... (U of them in flight): every load is one 1 KiB piece of a row; the four wave partials are added in wave
 // order.  With partial == nullptr (a single chunk) the block finishes y itself; otherwise it writes its chunk's
 // partial sums and sgemv_t_finish_kernel adds the chunks in order.
+template <int U>
 __global__ __launch_bounds__(kGemvThreads) void sgemv_t_kernel(int M, int N, int rows_per_chunk, float alpha,
                                                                const float* __restrict__ A, int lda,
                                                                const float* __restrict__ x, float beta,
@@ -57,11 +58,11 @@ __global__ __launch_bounds__(kGemvThreads) void sgemv_t_kernel(int M, int N, int
     const int last = (M - first < rows_per_chunk) ? M : first + rows_per_chunk;
     const int64_t row_bytes = static_cast<int64_t>(N - n0) * 4;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
-    for (int m = first + wave; m < last; m += 4 * kGemvWaves) {
-        v4f a[4];
-        float xm[4];
+    for (int m = first + wave; m < last; m += U * kGemvWaves) {
+        v4f a[U];
+        float xm[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int mm = m + u * kGemvWaves;
             const bool valid = mm < last;
             const int mc = valid ? mm : first;
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(kGemvThreads) void sgemv_t_kernel(int M, int N, int
             xm[u] = valid ? x[mc] : 0.f;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             acc.x = __builtin_fmaf(a[u].x, xm[u], acc.x);
             acc.y = __builtin_fmaf(a[u].y, xm[u], acc.y);
             acc.z = __builtin_fmaf(a[u].z, xm[u], acc.z);
@@ -127,7 +128,7 @@ static int device_cus() {
 // Row chunks of the transposed product: enough blocks to fill the device, at least 32 rows each.
 static int gemv_t_chunks(int M, int N) {
     const int64_t col_blocks = ceil_div(N, kGemvColsPerBlock);
-    int64_t want = ceil_div(4 * 256, col_blocks);  // about four blocks per CU of an MI355X; a function of the shape only
+    int64_t want = ceil_div(2 * 256, col_blocks);  // about two blocks per CU of an MI355X; a function of the shape only
     const int64_t most = ceil_div(M, 32);
     if (want > most) want = most;
     if (want > kGemvMaxChunks) want = kGemvMaxChunks;
@@ -162,7 +163,7 @@ static int run_sgemv(int trans, int M, int N, float alpha, const float* A, int l
     chunks = M > 0 ? static_cast<int>(ceil_div(M, rows_per_chunk)) : 1;
     const dim3 grid(static_cast<unsigned>(ceil_div(N, kGemvColsPerBlock)), chunks);
     float* partial = chunks > 1 ? static_cast<float*>(ws) : nullptr;
-    sgemv_t_kernel<<<grid, kGemvThreads, 0, s>>>(M, N, rows_per_chunk, alpha, A, lda, x, beta, y, partial);
+    sgemv_t_kernel<8><<<grid, kGemvThreads, 0, s>>>(M, N, rows_per_chunk, alpha, A, lda, x, beta, y, partial);
     if (chunks > 1)
         sgemv_t_finish_kernel<<<static_cast<int>(ceil_div(N, kGemvThreads)), kGemvThreads, 0, s>>>(N, chunks, alpha, partial,
                                                                                                   beta, y);
