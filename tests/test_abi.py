@@ -105,3 +105,32 @@ def test_host_cpu_gemm_matches_oracle_and_numpy(L, oracle_mod):
         assert np.array_equal(c_lib, c_orc)  # same order, same float accumulator -> same bits
         ref = alpha * (a.astype(np.float64) @ b.astype(np.float64)) + beta * c0
         assert np.max(np.abs(c_lib - ref)) < 5e-5
+
+
+def test_plan_query_without_a_gpu(L):
+    """Tile / split choice is host arithmetic on the shape (256 CUs assumed when no device is present)."""
+    def plan(M, N, K, ws):
+        t, s = C.c_int(-1), C.c_int(0)
+        assert L.hpcdnn_sgemm_plan(M, N, K, ws, C.byref(t), C.byref(s)) == 0
+        return t.value, s.value
+
+    n_tiles = L.hpcdnn_sgemm_num_tiles()
+    for shape in [(1024, 1024, 1024), (4096, 4096, 4096), (6144, 6144, 6144), (3072, 3072, 3072), (128, 128, 65536), (16384, 64, 4096)]:
+        t, s = plan(*shape, 0)
+        assert 0 <= t < n_tiles and s == 1                      # no workspace: nothing is split
+        need = L.hpcdnn_workspace_bytes(0, *shape)
+        t, s = plan(*shape, need)
+        assert 0 <= t < n_tiles and (s >= 1 or s <= -2)
+        if s == 1:
+            assert need == 0
+        elif s > 1:
+            assert need == shape[0] * shape[1] * s * 4           # split-K: one raw copy of C per slice
+        else:
+            bm, bn = C.c_int(), C.c_int()
+            assert L.hpcdnn_sgemm_tile_info(t, C.byref(bm), C.byref(bn), None) == 0
+            tiles = -(-shape[0] // bm.value) * -(-shape[1] // bn.value)
+            assert 0 < tiles % 256 <= 128 and need == (tiles % 256) * (-s) * bm.value * bn.value * 4
+    assert plan(128, 128, 65536, 1 << 30)[1] >= 16               # deep K: split-K
+    assert plan(3072, 3072, 3072, 1 << 30)[1] <= -2              # 3072^3: a partial last round, tail split
+    assert plan(4096, 4096, 4096, 1 << 30)[1] == 1               # 4096^3: whole rounds, nothing to split
+    assert L.hpcdnn_sgemm_plan(-1, 1, 1, 0, None, None) == 1
