@@ -149,7 +149,12 @@ static double tail_plan_cost(const TileConfig& t, int M, int N, int K, int cus, 
 
 static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, bool allow_tail = true) {
     const int cus = device_cus();
-    Plan best{0, 1};
+    struct Candidate {
+        Plan plan;
+        double cost;
+    };
+    Candidate cand[kNumTiles * 8];
+    int n_cand = 0;
     double best_cost = 1e300;
     for (int t = 0; t < kNumTiles; ++t) {
         const TileConfig& cfg = kTiles[t];
@@ -160,13 +165,27 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
                 if (static_cast<size_t>(M) * N * split * sizeof(float) > ws_bytes) break;
             }
             const double c = plan_cost(cfg, M, N, K, split, cus);
-            if (c < best_cost) { best_cost = c; best = Plan{t, split}; }
+            cand[n_cand++] = Candidate{Plan{t, split}, c};
+            if (c < best_cost) best_cost = c;
         }
         if (allow_split && allow_tail) {
             int ways = 0;
             const double c = tail_plan_cost(cfg, M, N, K, cus, ws_bytes, &ways);
-            if (ways >= 2 && c < best_cost) { best_cost = c; best = Plan{t, -ways}; }
+            if (ways >= 2) {
+                cand[n_cand++] = Candidate{Plan{t, -ways}, c};
+                if (c < best_cost) best_cost = c;
+            }
         }
+    }
+    // Among plans the model cannot tell apart (within 1 %), take the one that moves the least data: no split
+    // before a split, then the larger tile (A and B are re-read once per tile column / tile row).
+    Plan best{0, 1};
+    double best_key = -1.0;
+    for (int i = 0; i < n_cand; ++i) {
+        if (cand[i].cost > best_cost * 1.01) continue;
+        const TileConfig& cfg = kTiles[cand[i].plan.tile];
+        const double key = (cand[i].plan.split == 1 ? 1e12 : 0.0) + static_cast<double>(cfg.bm) * cfg.bn - cand[i].cost;
+        if (key > best_key) { best_key = key; best = cand[i].plan; }
     }
     return best;
 }
