@@ -114,7 +114,7 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
 }
 
 // FT: 0 = plain SGEMM; 1 = ABFT, checksum vectors e^T A and B e formed inside the main loop; 2 = ABFT, checksum
-// vectors read from a workspace filled by abft_encode_a/b_kernel (fewer VALU instructions in the main loop).
+// vectors read from a workspace filled by abft_encode_kernel (fewer VALU instructions in the main loop).
 template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS>
 __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
@@ -298,19 +298,20 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[Bf][i][q], fb[Bf][j][q], acc[i][j], 0, 0, 0);
     };
 
-    // ---- ABFT encode (dead code when !FT).
+    // ---- ABFT encode (dead code when FT == 0).
     // Like the reference, which forms e^T A and B e on its global->shared staging registers with warp shuffles
     // and adds the rank-1 products into spare shared memory (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:442-474),
     // the checksums are encoded from the staging registers of K step t+1 while step t is being multiplied:
-    //   before the barrier ("produce"): this thread holds 4 k values of A_SLOTS rows and 4 columns of B_SLOTS k
-    //     rows.  Column sums of A over the tile's rows: in-thread over the slots, then over the 16 lanes of a
-    //     half wave that hold the same k group (row_ror 4, 8; swap with lane^16) -> one partial per half wave in
-    //     LDS.  Row sums of B over the tile's columns: in-thread over the 4 columns, then over the 32 lanes of
-    //     the half wave (which holds whole k rows) -> b_r[k] in LDS.
-    //   after the barrier ("consume"): a_c[k] = sum of the 8 half-wave partials for the thread's own k rows,
-    //     cc[n] += a_c[k] * B[k, n] on its B registers; b_r[k] for its own 4 k values, cr[m] += A[m, k] * b_r[k]
-    //     on its A registers.  Partial sums are FP32 over two K steps, then added to FP64 running sums, so the
-    //     reference checksums carry no drift of their own over a long K.
+    //   before the barrier ("produce", FT == 1 only): this thread holds 4 k values of A_SLOTS rows and 4 columns
+    //     of B_SLOTS k rows.  Column sums of A over the tile's rows: in-thread over the slots, then over the 16
+    //     lanes of the wave that hold the same k group (row_ror 4, 8; swap with lane^16; swap with lane^32) ->
+    //     one partial per wave in LDS.  Row sums of B over the tile's columns: in-thread over the 4 columns, then
+    //     over the 32 lanes of the half wave (which holds whole k rows) -> b_r[k] in LDS.
+    //   after the barrier ("consume"): a_c[k] = sum of the per-wave partials for the thread's own k rows (FT == 2:
+    //     fetched from the pre-encoded vectors with the staged tile), cc[n] += a_c[k] * B[k, n] on its B
+    //     registers; b_r[k] for its own 4 k values, cr[m] += A[m, k] * b_r[k] on its A registers.  Partial sums
+    //     are FP32 over 16 K steps, then added to FP64 running sums, so the reference checksums carry no drift
+    //     of their own over a long K.
     // Per thread the running sums cover columns nc..nc+3 over the k rows it stages (8 threads share a column)
     // and rows row(s) over the k group it stages (4 threads share a row); the verification step adds them up.
     constexpr int kHalfWaves = 2 * kGemmThreads / kWave;  // 8 or 16
