@@ -129,7 +129,10 @@ int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B
                     float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
                     void* ws, size_t ws_bytes, void* stream);
 int hpcdnn_ft_num_tiles(int M, int N);
-/* Threshold hpcdnn_ft_sgemm uses when tau <= 0. */
+/* Threshold hpcdnn_ft_sgemm uses when tau <= 0: 1.1e-6 * max(K, 64), twice the
+ * largest fault-free residual measured for operands uniform in [-1, 1] (the
+ * rounding noise of the FP32 accumulators grows linearly with K).  Scale it by
+ * max|A| * max|B| for other data. */
 float hpcdnn_ft_default_tau(int K);
 
 /* Row-major SGEMV, A is M x N with leading dimension lda >= N:

