@@ -144,3 +144,34 @@ def test_sdot_full_size_2_pow_28(blas, oracle_mod):
     assert abs(float(xx) - oracle_mod.sdot_f64(x, x)) <= 1e-5 * float(xx)
     assert abs(float(xx) / n - 1.0 / 3.0) < 1e-3
     assert _sdot(blas, n, dy, dx).tobytes() == got.tobytes()
+
+
+def test_vectors_longer_than_2_pow_31_elements(blas, oracle_mod):
+    """Indices past 2^31 (64-bit indexing; the reference's `int N` stops at 2^31 - 1): SAXPY bit-exact on sampled
+    elements and on the n % 4 tail, untouched past n; SDOT against an FP64 sum formed chunk by chunk."""
+    n = (1 << 31) + (1 << 20) + 3
+    dx = torch.empty(n + 5, dtype=torch.float32, device="cuda")
+    dy = torch.empty(n + 5, dtype=torch.float32, device="cuda")
+    blas.fill_uniform(dx, 61)
+    blas.fill_uniform(dy, 62)
+    exact = 0.0
+    chunk = 1 << 28
+    for s in range(0, n, chunk):
+        e = min(n, s + chunk)
+        exact += float((dx[s:e].double() * dy[s:e].double()).sum())
+    got = float(_sdot(blas, n, dx, dy))
+    assert abs(got - exact) <= 1e-5 * abs(exact) + 1e-2, (got, exact)
+
+    blas.saxpy(n, 2.5, dx, dy)
+    rng = np.random.default_rng(5)
+    idx = np.unique(np.concatenate([rng.integers(0, n, 4000), np.arange(n - 8, n + 5), np.arange(0, 8),
+                                    np.arange((1 << 31) - 8, (1 << 31) + 8), np.arange((1 << 29) - 4, (1 << 29) + 4) * 4]))
+    got_y = dy[torch.from_numpy(idx).cuda()].cpu().numpy()
+    for i, g in zip(idx.tolist(), got_y.tolist()):
+        x0, y0 = np.float32(oracle_mod.uniform(61, i)), np.float32(oracle_mod.uniform(62, i))
+        if i < n:
+            xs, ys = np.array([x0], np.float32), np.array([y0], np.float32)
+            oracle_mod.saxpy(2.5, xs, ys)
+            assert np.float32(g) == ys[0], i
+        else:
+            assert np.float32(g) == y0, i  # past n: untouched
