@@ -230,3 +230,31 @@ def test_config3_square_sweep_every_size(blas, oracle_mod, n):
     ws = blas.workspace(max(blas.sgemm_workspace_bytes(n, n, n), 4))
     _sampled_check(oracle_mod, blas, n, n, n, 1.0, 0.0, nrows=6, seed=900 + n, ws=ws)
     _sampled_check(oracle_mod, blas, n, n, n, 1.0, 1.0, nrows=6, seed=901 + n)
+
+
+def test_operands_larger_than_4_gib(blas):
+    """A of 5.3 GB and C of 5.3 GB in two shapes: row offsets past 2^32 bytes in A, in C and in the split-K
+    workspace.  Checked with FP64 products of sampled rows and a Freivalds identity formed on the device."""
+    dev = "cuda"
+    for (M, N, K) in [(33000, 200, 40000), (40000, 33000, 96)]:
+        a = torch.empty(M, K, device=dev)
+        b = torch.empty(K, N, device=dev)
+        c = torch.empty(M, N, device=dev)
+        blas.fill_uniform_matrix(a, M, K, 71)
+        blas.fill_uniform_matrix(b, K, N, 72)
+        ws = blas.workspace(max(blas.sgemm_workspace_bytes(M, N, K), 4))
+        blas.sgemm(M, N, K, a, b, c, 1.0, 0.0, ws=ws)
+        rows = torch.tensor([0, 1, M // 2, M - 300, M - 2, M - 1], device=dev)
+        ref = a[rows].double() @ b.double()
+        den = a[rows].double().abs() @ b.double().abs()
+        assert torch.all((c[rows].double() - ref).abs() <= TOL * den), (M, N, K)
+        v = torch.randint(0, 2, (N,), device=dev, dtype=torch.float64) * 2 - 1
+        bv = b.double() @ v
+        babs = b.double().abs().sum(dim=1)
+        for s in range(0, M, 8192):
+            e = min(M, s + 8192)
+            lhs = c[s:e].double() @ v
+            rhs = a[s:e].double() @ bv
+            bound = a[s:e].double().abs() @ babs
+            assert torch.all((lhs - rhs).abs() <= TOL * bound), (M, N, K, s)
+        del a, b, c, ws
