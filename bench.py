@@ -265,6 +265,15 @@ def main() -> int:
         ms = median_timed(lambda: blas.saxpy(nv, 2.5, x, y), 20, 3)
         extras["saxpy_2p28"] = {"GBps": round(12.0 * nv / ms / 1e6, 1), "frac_hbm_peak": round(12.0 * nv / ms / 1e6 / PEAK_HBM_GBS, 4),
                                 "us": round(ms * 1e3, 1)}
+        # the same with y placed 1 MiB + 8 KiB further from x than the allocator put it (x and y otherwise sit exactly
+        # 1 GiB apart, the worst case for HBM channel/bank interleaving): placement, not the kernel, moves the rate
+        ybig = torch.empty(nv + (1 << 19), device=dev)
+        ysk = ybig[(1 << 18) + 2048:(1 << 18) + 2048 + nv]
+        ysk.copy_(y)
+        ms = median_timed(lambda: blas.saxpy(nv, 2.5, x, ysk), 20, 3)
+        extras["saxpy_2p28"]["GBps_y_skewed_by_1MiB_8KiB"] = round(12.0 * nv / ms / 1e6, 1)
+        extras["saxpy_2p28"]["x_y_distance_bytes"] = [int(y.data_ptr() - x.data_ptr()), int(ysk.data_ptr() - x.data_ptr())]
+        del ybig, ysk
         ms = median_timed(lambda: blas.sdot(nv, x, y, out), 20, 3)
         extras["sdot_2p28"] = {"GBps": round(8.0 * nv / ms / 1e6, 1), "frac_hbm_peak": round(8.0 * nv / ms / 1e6 / PEAK_HBM_GBS, 4),
                                "us": round(ms * 1e3, 1)}
