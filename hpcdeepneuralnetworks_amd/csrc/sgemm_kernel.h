@@ -202,7 +202,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         make_rsrc(FT == 2 ? p.enc_a + static_cast<int64_t>(tile_m) * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * 4);
     const __amdgpu_buffer_rsrc_t enc_b_rsrc =
         make_rsrc(FT == 2 ? p.enc_b + static_cast<int64_t>(tile_n) * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * 4);
-    const int enc_a_voff = (tid >> 5) * 8;  // a_c of the two k rows of B this thread stages (stored side by side)
+    // a_c of the k rows of B this thread stages: k = tid/32 (and k + 8 with four waves), which the pre-encode kernel
+    // stores side by side (order 0, 8, 1, 9, ... inside each K step)
+    const int enc_a_voff = B_SLOTS == 2 ? (tid >> 5) * 8 : ((((tid >> 5) & 7) * 2 + (tid >> 8)) * 4);
     const int enc_b_voff = (tid & 3) * 16;  // b_r of the four k values of A this thread stages
     int enc_off = kbeg * 4;
     float g_ac[2][B_SLOTS];
@@ -213,11 +215,15 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc(a_base, a_left), a_voff[P]);
         else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[P - A_SLOTS]);
         if constexpr (FT == 2 && P == NGL - 1) {
-            static_assert(FT != 2 || B_SLOTS == 2, "enc_a pairs the two k rows a thread stages");
-            typedef float v2f __attribute__((ext_vector_type(2)));
-            const v2f t = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(enc_a_rsrc, enc_a_voff, enc_off, 0));
-            g_ac[S][0] = t[0];
-            g_ac[S][B_SLOTS - 1] = t[1];
+            static_assert(FT != 2 || B_SLOTS <= 2, "a thread stages one or two k rows of B");
+            if constexpr (B_SLOTS == 2) {
+                typedef float v2f __attribute__((ext_vector_type(2)));
+                const v2f t = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(enc_a_rsrc, enc_a_voff, enc_off, 0));
+                g_ac[S][0] = t[0];
+                g_ac[S][B_SLOTS - 1] = t[1];
+            } else {
+                g_ac[S][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(enc_a_rsrc, enc_a_voff, enc_off, 0));
+            }
             g_br[S] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_b_rsrc, enc_b_voff, enc_off, 0));
         }
     };
