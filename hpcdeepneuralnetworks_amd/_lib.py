@@ -31,6 +31,7 @@ EXPORTS = (
     "hpcdnn_sgemm_num_tiles",
     "hpcdnn_sgemm_tile_info",
     "hpcdnn_sgemm_plan",
+    "hpcdnn_sgemm_row_split",
     "hpcdnn_ft_sgemm",
     "hpcdnn_ft_num_tiles",
     "hpcdnn_ft_default_tau",
@@ -89,6 +90,8 @@ def lib():
     L.hpcdnn_sgemm_tile_info.argtypes = [i, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.hpcdnn_sgemm_plan.restype = i
     L.hpcdnn_sgemm_plan.argtypes = [i, i, i, sz, C.POINTER(i), C.POINTER(i)]
+    L.hpcdnn_sgemm_row_split.restype = i
+    L.hpcdnn_sgemm_row_split.argtypes = [i, i, i, sz, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.hpcdnn_ft_sgemm.restype = i
     L.hpcdnn_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, vp]
     L.hpcdnn_ft_num_tiles.restype = i

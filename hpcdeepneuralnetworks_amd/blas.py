@@ -72,6 +72,13 @@ def sgemm_plan(M: int, N: int, K: int, ws_bytes: int = 0):
     return t.value, sp.value
 
 
+def sgemm_row_split(M: int, N: int, K: int, ws_bytes: int = 0):
+    """(rows_first, tile_first, tile_rest) when the library covers C with two launches, rows_first = 0 otherwise."""
+    r, t1, t2 = C.c_int(), C.c_int(), C.c_int()
+    check(_lib.lib().hpcdnn_sgemm_row_split(M, N, K, ws_bytes, C.byref(r), C.byref(t1), C.byref(t2)), "hpcdnn_sgemm_row_split")
+    return r.value, t1.value, t2.value
+
+
 def tile_table():
     L = _lib.lib()
     out = []

@@ -30,7 +30,7 @@ static const TileConfig kTiles[] = {
     HPCDNN_TILE(128, 128, 2, 2, 2, 0.970f),  // 1 large
     HPCDNN_TILE(128, 64, 2, 2, 2, 0.945f),   // 2 tall
     HPCDNN_TILE(64, 128, 2, 2, 2, 0.939f),   // 3 wide
-    HPCDNN_TILE(64, 64, 2, 2, 4, 0.929f),    // 4 medium
+    HPCDNN_TILE(64, 64, 2, 2, 4, 0.900f),    // 4 medium
     HPCDNN_TILE(192, 256, 2, 2, 1, 0.964f),  // 5 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
     HPCDNN_TILE(256, 192, 2, 2, 1, 0.946f),  // 6
     HPCDNN_TILE(128, 256, 2, 2, 2, 0.987f),  // 7
@@ -150,7 +150,8 @@ static double tail_plan_cost(const TileConfig& t, int M, int N, int K, int cus, 
            (2.0 * s + 1.0) * r * static_cast<double>(tile_bytes) / kReduceBytesPerSec;
 }
 
-static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, bool allow_tail = true) {
+static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, bool allow_tail = true,
+                        double* cost_out = nullptr) {
     const int cus = device_cus();
     struct Candidate {
         Plan plan;
@@ -188,7 +189,36 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
         if (cand[i].cost > best_cost * 1.01) continue;
         const TileConfig& cfg = kTiles[cand[i].plan.tile];
         const double key = (cand[i].plan.split == 1 ? 1e12 : 0.0) + static_cast<double>(cfg.bm) * cfg.bn - cand[i].cost;
-        if (key > best_key) { best_key = key; best = cand[i].plan; }
+        if (key > best_key) { best_key = key; best = cand[i].plan; if (cost_out) *cost_out = cand[i].cost; }
+    }
+    return best;
+}
+
+// Row split, the workspace-free answer to a partial last round: the first rows1 rows of C (whole rounds of big tiles)
+// go to one launch, the remaining rows to a second launch with whatever tile suits that thin strip.  Every element
+// of C still comes from one workgroup that walks all of K, so the result has the same bits as a single launch.
+struct RowSplit {
+    int tile1, rows1, tile2;
+    double cost;
+};
+constexpr double kSecondLaunch = 3e-6;
+
+static RowSplit choose_row_split(int M, int N, int K, int cus) {
+    RowSplit best{-1, 0, -1, 1e300};
+    for (int t = 0; t < kNumTiles; ++t) {
+        const TileConfig& cfg = kTiles[t];
+        const int64_t tiles_n = ceil_div(N, cfg.bn), tiles_m = ceil_div(M, cfg.bm);
+        const int64_t rounds = tiles_m * tiles_n / cus;
+        for (int64_t k = rounds; k >= 1 && k + 1 >= rounds; --k) {
+            const int64_t tile_rows = k * cus / tiles_n;
+            const int64_t rows1 = tile_rows * cfg.bm;
+            if (tile_rows < 1 || rows1 >= M) continue;
+            const double c1 = plan_cost(cfg, static_cast<int>(rows1), N, K, 1, cus);
+            double c2 = 0.0;
+            const Plan rest = choose_plan(M - static_cast<int>(rows1), N, K, false, 0, false, &c2);
+            const double c = c1 + c2 + kSecondLaunch;
+            if (c < best.cost) best = RowSplit{t, static_cast<int>(rows1), rest.tile, c};
+        }
     }
     return best;
 }
@@ -237,7 +267,17 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
 
     if (tile < 0 || split == 0) {
         // the tail split moves 16-byte groups through the workspace
-        Plan plan = choose_plan(M, N, K, ws != nullptr, ws ? ws_bytes : 0, (reinterpret_cast<uintptr_t>(ws) & 15u) == 0);
+        double cost = 0.0;
+        Plan plan = choose_plan(M, N, K, ws != nullptr, ws ? ws_bytes : 0, (reinterpret_cast<uintptr_t>(ws) & 15u) == 0, &cost);
+        if (tile < 0 && split == 0 && K > 0) {
+            const RowSplit rs = choose_row_split(M, N, K, device_cus());
+            if (rs.tile1 >= 0 && rs.cost < 0.97 * cost) {
+                rc = run_sgemm(rs.rows1, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, rs.tile1, 1, stream);
+                if (rc != HPCDNN_OK) return rc;
+                return run_sgemm(M - rs.rows1, N, K, A + static_cast<int64_t>(rs.rows1) * lda, lda, B, ldb,
+                                 C + static_cast<int64_t>(rs.rows1) * ldc, ldc, alpha, beta, nullptr, 0, rs.tile2, 1, stream);
+            }
+        }
         if (tile < 0) {
             tile = plan.tile;
             if (split == 0) split = plan.split;
@@ -332,6 +372,22 @@ extern "C" int hpcdnn_sgemm_plan(int M, int N, int K, size_t ws_bytes, int* tile
     const Plan plan = choose_plan(M, N, K, ws_bytes > 0, ws_bytes);
     if (tile) *tile = plan.tile;
     if (split_k) *split_k = plan.split;
+    return HPCDNN_OK;
+}
+
+extern "C" int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first, int* tile_first,
+                                      int* tile_rest) {
+    if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
+    int rows = 0, t1 = -1, t2 = -1;
+    if (M > 0 && N > 0 && K > 0) {
+        double cost = 0.0;
+        choose_plan(M, N, K, ws_bytes > 0, ws_bytes, true, &cost);
+        const RowSplit rs = choose_row_split(M, N, K, device_cus());
+        if (rs.tile1 >= 0 && rs.cost < 0.97 * cost) { rows = rs.rows1; t1 = rs.tile1; t2 = rs.tile2; }
+    }
+    if (rows_first) *rows_first = rows;
+    if (tile_first) *tile_first = t1;
+    if (tile_rest) *tile_rest = t2;
     return HPCDNN_OK;
 }
 

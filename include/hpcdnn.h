@@ -108,6 +108,12 @@ int hpcdnn_sgemm_tile_info(int tile, int* bm, int* bn, int* bk);
  * ws_bytes (0 = none), split_k with the meaning it has for hpcdnn_sgemm_ex: a
  * function of the shape and the device's CU count only. */
 int hpcdnn_sgemm_plan(int M, int N, int K, size_t ws_bytes, int* tile, int* split_k);
+/* hpcdnn_sgemm may instead cover C with two launches: the first *rows_first rows
+ * (whole rounds of tile *tile_first over the CUs) and the remaining rows (tile
+ * *tile_rest), when that beats the single plan above by more than 3 %; no
+ * workspace is involved and every element of C still sums K in one piece.
+ * *rows_first = 0 when it does not. */
+int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first, int* tile_first, int* tile_rest);
 
 /* SGEMM with fused online ABFT: row/column checksums of each 256x128 output
  * tile are accumulated from A and B inside the main loop, compared with the

@@ -258,3 +258,19 @@ def test_operands_larger_than_4_gib(blas):
             bound = a[s:e].double().abs() @ babs
             assert torch.all((lhs - rhs).abs() <= TOL * bound), (M, N, K, s)
         del a, b, c, ws
+
+
+def test_row_split_gives_the_same_bits_as_one_launch(blas, oracle_mod):
+    """Sizes where the library covers C with two launches (no workspace): same bits as one launch of the first
+    launch's tile, because every element still sums K in one workgroup and in the same order."""
+    found = 0
+    for n in (3584, 4608, 5120):
+        rows, t1, t2 = blas.sgemm_row_split(n, n, n, 0)
+        if rows == 0:
+            continue
+        found += 1
+        assert 0 < rows < n and t1 >= 0 and t2 >= 0
+        c_auto = _sampled_check(oracle_mod, blas, n, n, n, 1.0, 1.0, nrows=6, seed=950 + n)
+        c_one = _sampled_check(oracle_mod, blas, n, n, n, 1.0, 1.0, nrows=6, seed=950 + n, tile=t1, split_k=1)
+        assert torch.equal(c_auto, c_one), n
+    assert found >= 1
