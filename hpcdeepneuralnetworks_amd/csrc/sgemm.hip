@@ -266,17 +266,39 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     if (M == 0 || N == 0) return HPCDNN_OK;
 
     if (tile < 0 || split == 0) {
+        // The decision is a function of the shape and of what the workspace allows; callers tend to repeat shapes,
+        // so each thread remembers its last one instead of re-evaluating the cost model on every call.
+        struct Decision {
+            int M, N, K;
+            size_t ws_bytes;
+            bool ws_aligned, valid;
+            Plan plan;
+            RowSplit rows;
+        };
+        static thread_local Decision memo{};
         // the tail split moves 16-byte groups through the workspace
-        double cost = 0.0;
-        Plan plan = choose_plan(M, N, K, ws != nullptr, ws ? ws_bytes : 0, (reinterpret_cast<uintptr_t>(ws) & 15u) == 0, &cost);
-        if (tile < 0 && split == 0 && K > 0) {
-            const RowSplit rs = choose_row_split(M, N, K, device_cus());
-            if (rs.tile1 >= 0 && rs.cost < 0.97 * cost) {
-                rc = run_sgemm(rs.rows1, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, rs.tile1, 1, stream);
-                if (rc != HPCDNN_OK) return rc;
-                return run_sgemm(M - rs.rows1, N, K, A + static_cast<int64_t>(rs.rows1) * lda, lda, B, ldb,
-                                 C + static_cast<int64_t>(rs.rows1) * ldc, ldc, alpha, beta, nullptr, 0, rs.tile2, 1, stream);
+        const bool ws_aligned = (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
+        const size_t usable = ws ? ws_bytes : 0;
+        if (!(memo.valid && memo.M == M && memo.N == N && memo.K == K && memo.ws_bytes == usable && memo.ws_aligned == ws_aligned)) {
+            double cost = 0.0;
+            memo.plan = choose_plan(M, N, K, ws != nullptr, usable, ws_aligned, &cost);
+            memo.rows = RowSplit{-1, 0, -1, 1e300};
+            if (K > 0) {
+                const RowSplit rs = choose_row_split(M, N, K, device_cus());
+                if (rs.tile1 >= 0 && rs.cost < 0.97 * cost) memo.rows = rs;
             }
+            memo.M = M; memo.N = N; memo.K = K;
+            memo.ws_bytes = usable;
+            memo.ws_aligned = ws_aligned;
+            memo.valid = true;
+        }
+        const Plan plan = memo.plan;
+        const RowSplit rs = memo.rows;  // copied: the nested calls below do not touch the memo, but keep it simple
+        if (tile < 0 && split == 0 && rs.tile1 >= 0) {
+            rc = run_sgemm(rs.rows1, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, rs.tile1, 1, stream);
+            if (rc != HPCDNN_OK) return rc;
+            return run_sgemm(M - rs.rows1, N, K, A + static_cast<int64_t>(rs.rows1) * lda, lda, B, ldb,
+                             C + static_cast<int64_t>(rs.rows1) * ldc, ldc, alpha, beta, nullptr, 0, rs.tile2, 1, stream);
         }
         if (tile < 0) {
             tile = plan.tile;
