@@ -255,6 +255,25 @@ def main() -> int:
         })
         del a, b, c, c_clean
 
+        # ---- ABFT on a smaller problem: the tile class the library suggests (more, smaller checksum tiles)
+        m, kk = 2048, 1024
+        a, b, c = operands(m, m, kk, 25)
+        cls = blas.ft_pick_class(m, m, kk)
+        status_s = blas.ft_status_alloc(m, m, tile_class=cls)
+        status_0 = blas.ft_status_alloc(m, m)
+        ft_ws_s = blas.workspace(blas.ft_workspace_bytes(m, m, kk))
+        ms_plain = median_timed(lambda: blas.sgemm(m, m, kk, a, b, c, 1.0, 0.0), st, wu)
+        ms_cls = median_timed(lambda: blas.ft_sgemm(m, m, kk, a, b, c, 1.0, 0.0, status=status_s, ws=ft_ws_s, tile_class=cls), st, wu)
+        ms_c0 = median_timed(lambda: blas.ft_sgemm(m, m, kk, a, b, c, 1.0, 0.0, status=status_0, ws=ft_ws_s), st, wu)
+        extras["abft_2048x2048x1024"] = {
+            "picked_tile_class": cls, "picked_tile": list(blas.ft_tile(cls)),
+            "sgemm_gflops": round(2.0 * m * m * kk / ms_plain / 1e6, 1),
+            "ft_sgemm_gflops": round(2.0 * m * m * kk / ms_cls / 1e6, 1),
+            "overhead_pct_vs_sgemm": round((ms_cls - ms_plain) / ms_plain * 100.0, 2),
+            "class0_256x128_ft_sgemm_gflops": round(2.0 * m * m * kk / ms_c0 / 1e6, 1),
+        }
+        del a, b, c
+
         # ---- SAXPY / SDOT at n = 2^28 (12 and 8 algorithmic bytes per element)
         nv = 1 << 28
         x = torch.empty(nv, device=dev)

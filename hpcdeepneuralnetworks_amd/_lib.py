@@ -21,6 +21,7 @@ OP_OFFLINE_FT_SGEMM = 4
 OFFLINE_FT_PANEL_K = 256
 FT_TILE_M = 256
 FT_TILE_N = 128
+FT_NUM_CLASSES = 3
 
 # every symbol include/hpcdnn.h declares
 EXPORTS = (
@@ -34,6 +35,10 @@ EXPORTS = (
     "hpcdnn_sgemm_row_split",
     "hpcdnn_ft_sgemm",
     "hpcdnn_ft_num_tiles",
+    "hpcdnn_ft_sgemm_ex",
+    "hpcdnn_ft_tile_info",
+    "hpcdnn_ft_num_tiles_ex",
+    "hpcdnn_ft_pick_class",
     "hpcdnn_ft_default_tau",
     "hpcdnn_sgemv",
     "hpcdnn_offline_ft_sgemm",
@@ -94,6 +99,14 @@ def lib():
     L.hpcdnn_sgemm_row_split.argtypes = [i, i, i, sz, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.hpcdnn_ft_sgemm.restype = i
     L.hpcdnn_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, vp]
+    L.hpcdnn_ft_sgemm_ex.restype = i
+    L.hpcdnn_ft_sgemm_ex.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, i, vp]
+    L.hpcdnn_ft_tile_info.restype = i
+    L.hpcdnn_ft_tile_info.argtypes = [i, C.POINTER(i), C.POINTER(i)]
+    L.hpcdnn_ft_num_tiles_ex.restype = i
+    L.hpcdnn_ft_num_tiles_ex.argtypes = [i, i, i]
+    L.hpcdnn_ft_pick_class.restype = i
+    L.hpcdnn_ft_pick_class.argtypes = [i, i, i]
     L.hpcdnn_ft_num_tiles.restype = i
     L.hpcdnn_ft_num_tiles.argtypes = [i, i]
     L.hpcdnn_ft_default_tau.restype = f

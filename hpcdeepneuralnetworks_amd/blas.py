@@ -109,10 +109,12 @@ def sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Te
 
 
 def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
-             tau: float = 0.0, fault=None, status: torch.Tensor | None = None, ws: torch.Tensor | None = None) -> None:
+             tau: float = 0.0, fault=None, status: torch.Tensor | None = None, ws: torch.Tensor | None = None,
+             tile_class: int = 0) -> None:
     """ABFT GEMM; ``fault`` = (tile, row, col, delta) or None; ``status`` = int32 tensor of 8*ft_num_tiles words;
     ``ws`` = optional scratch tensor of ``ft_workspace_bytes(M, N, K)`` bytes (checksum vectors are then formed
-    by a pre-pass instead of inside the main loop).
+    by a pre-pass instead of inside the main loop); ``tile_class`` selects the ABFT tile (0 = 256x128, 1 = 128x128,
+    2 = 64x128: tiles, status records and fault coordinates are per tile of that class).
 
     Counterpart of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)`` (kernel/ft_sgemm/sgemm.cu:159-165).
     """
@@ -122,7 +124,7 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
     L = _lib.lib()
     sp = None
     if status is not None:
-        need = 8 * L.hpcdnn_ft_num_tiles(M, N)
+        need = 8 * L.hpcdnn_ft_num_tiles_ex(tile_class, M, N)
         if not (status.is_cuda and status.dtype == torch.int32 and status.numel() >= need and status.is_contiguous()):
             raise HpcdnnError(f"status must be a contiguous int32 GPU tensor with >= {need} elements")
         sp = status.data_ptr()
@@ -130,7 +132,7 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
     if fault is not None:
         f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
     wp, wb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
-    check(L.hpcdnn_ft_sgemm(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, f, sp, wp, wb, _stream()),
+    check(L.hpcdnn_ft_sgemm_ex(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, f, sp, wp, wb, tile_class, _stream()),
           "hpcdnn_ft_sgemm")
 
 
@@ -181,16 +183,26 @@ def offline_ft_workspace_bytes(M: int, N: int, K: int) -> int:
     return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_OFFLINE_FT_SGEMM, M, N, K))
 
 
-def ft_num_tiles(M: int, N: int) -> int:
-    return int(_lib.lib().hpcdnn_ft_num_tiles(M, N))
+def ft_num_tiles(M: int, N: int, tile_class: int = 0) -> int:
+    return int(_lib.lib().hpcdnn_ft_num_tiles_ex(tile_class, M, N))
+
+
+def ft_tile(tile_class: int = 0):
+    bm, bn = C.c_int(), C.c_int()
+    check(_lib.lib().hpcdnn_ft_tile_info(tile_class, C.byref(bm), C.byref(bn)), "hpcdnn_ft_tile_info")
+    return bm.value, bn.value
+
+
+def ft_pick_class(M: int, N: int, K: int) -> int:
+    return int(_lib.lib().hpcdnn_ft_pick_class(M, N, K))
 
 
 def ft_default_tau(K: int) -> float:
     return float(_lib.lib().hpcdnn_ft_default_tau(K))
 
 
-def ft_status_alloc(M: int, N: int, device=None) -> torch.Tensor:
-    return torch.zeros(8 * ft_num_tiles(M, N), dtype=torch.int32, device=device or "cuda")
+def ft_status_alloc(M: int, N: int, device=None, tile_class: int = 0) -> torch.Tensor:
+    return torch.zeros(8 * ft_num_tiles(M, N, tile_class), dtype=torch.int32, device=device or "cuda")
 
 
 def ft_status_numpy(status: torch.Tensor) -> np.ndarray:

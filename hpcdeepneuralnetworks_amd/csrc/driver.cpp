@@ -118,7 +118,7 @@ struct Series {
     int number;        // the reference's kernel_number (kernel/ft_sgemm/sgemm.cu:186)
     const char* name;  // the reference's series name (:187-188) where a counterpart exists
     int kind;          // 0 plain SGEMM, 1 offline ABFT, 2 ABFT without workspace, 3 ABFT with workspace
-    int tile;          // plain SGEMM: row of the tile table, -1 = chosen by the library
+    int tile;          // plain SGEMM: row of the tile table, -1 = chosen by the library; ABFT: tile class
 };
 
 // The reference's 16x16 ... 128x128 thread-tile classes map to the MFMA tile classes in the same order of size.
@@ -131,8 +131,13 @@ const Series kSeries[] = {
     {5, "kernel_sgemm_wide", 0, 3},    // 64 x 128
     {6, "kernel_sgemm_huge", 0, 8},    // 256 x 256
     {10, "abft_baseline", 1, -1},
-    {16, "abft_kernel_huge", 2, -1},
-    {19, "abft_kernel_huge_workspace", 3, -1},  // no reference counterpart: checksum vectors from the pre-pass
+    {13, "abft_kernel_large", 2, 1},  // 128 x 128
+    {15, "abft_kernel_wide", 2, 2},   // 64 x 128
+    {16, "abft_kernel_huge", 2, 0},   // 256 x 128
+    // no reference counterpart: checksum vectors from the pre-pass
+    {19, "abft_kernel_huge_workspace", 3, 0},
+    {20, "abft_kernel_large_workspace", 3, 1},
+    {21, "abft_kernel_wide_workspace", 3, 2},
 };
 
 int run_ft_sgemm(int start, int end, int gap, int first, int last) {
@@ -199,11 +204,13 @@ int run_ft_sgemm(int start, int end, int gap, int first, int last) {
                     });
                     break;
                 case 2:
-                    perf = timed_gflops(flop, kNumTests, [&] { LIB_OK(hpcdnn::ft_sgemm(n, n, K, a, b, c, alpha, beta)); });
+                    perf = timed_gflops(flop, kNumTests, [&] {
+                        LIB_OK(hpcdnn_ft_sgemm_ex(n, n, K, a, K, b, n, c, n, alpha, beta, 0.f, nullptr, nullptr, nullptr, 0, sr.tile, nullptr));
+                    });
                     break;
                 default:
                     perf = timed_gflops(flop, kNumTests, [&] {
-                        LIB_OK(hpcdnn::ft_sgemm(n, n, K, a, b, c, alpha, beta, nullptr, nullptr, ft_ws, ft_ws_bytes));
+                        LIB_OK(hpcdnn_ft_sgemm_ex(n, n, K, a, K, b, n, c, n, alpha, beta, 0.f, nullptr, nullptr, ft_ws, ft_ws_bytes, sr.tile, nullptr));
                     });
             }
             std::printf("%8.2f,", perf);

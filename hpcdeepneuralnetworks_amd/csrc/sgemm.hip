@@ -40,23 +40,43 @@ static const TileConfig kTiles[] = {
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
-constexpr int kFtTile = 0;  // 256 x 128, matches HPCDNN_FT_TILE_M/N
 // row length of the pre-encoded checksum vectors: K rounded up to the K step, plus two K steps of zeros for the
 // fetches that run ahead of the main loop
 static int ft_enc_ld(int K) { return (static_cast<int>(ceil_div(K, kGemmBK)) + 2) * kGemmBK; }
 size_t ft_workspace_bytes(int M, int N, int K);
-// Four waves: on this part every VALU instruction takes its issue cycles away from the FP32 matrix pipe of the
-// same SIMD, whichever wave it comes from, so more waves do not hide the checksum arithmetic; fewer, fatter
-// threads need the fewest VALU instructions per K step.
-constexpr int kFtWavesM = 2, kFtWavesN = 2, kFtThreads = kFtWavesM * kFtWavesN * kWave;
-static void (*const kFtPlain)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, false, 1, 1>;
-static void (*const kFtEdge)(const GemmArgs) = sgemm_kernel<256, 128, kFtWavesM, kFtWavesN, true, 1, 1>;
-// The same with the operands' checksum vectors read from a workspace (filled by the pre-encode kernel).  No
-// cross-lane reductions are left in that loop, so the thread count no longer changes the VALU work per SIMD, and
-// eight waves (two per SIMD) hide each other's barriers and LDS latency: measured 2 % faster than four.
-constexpr int kFtPreWavesM = 2, kFtPreWavesN = 4, kFtPreThreads = kFtPreWavesM * kFtPreWavesN * kWave;
-static void (*const kFtPrePlain)(const GemmArgs) = sgemm_kernel<256, 128, kFtPreWavesM, kFtPreWavesN, false, 2, 1>;
-static void (*const kFtPreEdge)(const GemmArgs) = sgemm_kernel<256, 128, kFtPreWavesM, kFtPreWavesN, true, 2, 1>;
+// ABFT tile classes (the counterpart of the reference's abft_kernel_{huge,large,wide,...} family,
+// kernel/ft_sgemm/sgemm.cu:187-188): class 0 is the 256 x 128 tile of HPCDNN_FT_TILE_M/N; the smaller classes keep
+// more CUs busy on smaller problems.  The encode is laid out for 128-column tiles, so the classes differ in height.
+//
+// Without a workspace (FT = 1) four waves: on this part every VALU instruction takes its issue cycles away from the
+// FP32 matrix pipe of the same SIMD, whichever wave it comes from, so more waves do not hide the checksum arithmetic;
+// fewer, fatter threads need the fewest VALU instructions per K step.  With the operands' checksum vectors read from
+// a workspace (FT = 2) no cross-lane reductions are left in the loop, the thread count no longer changes the VALU
+// work per SIMD, and eight waves (two per SIMD) hide each other's barriers and LDS latency: measured 2 % faster.
+struct FtClass {
+    int bm, bn;
+    int threads_fused, threads_pre;
+    size_t lds_fused, lds_pre;
+    void (*fused_plain)(const GemmArgs);
+    void (*fused_edge)(const GemmArgs);
+    void (*pre_plain)(const GemmArgs);
+    void (*pre_edge)(const GemmArgs);
+    void (*encode)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int);
+};
+
+#define HPCDNN_FT_CLASS(BM, FM, FN, PM, PN)                                                                      \
+    {                                                                                                            \
+        BM, 128, FM * FN * kWave, PM * PN * kWave, gemm_lds_bytes<BM, 128, 1, FM * FN * kWave>(),                \
+            gemm_lds_bytes<BM, 128, 2, PM * PN * kWave>(), sgemm_kernel<BM, 128, FM, FN, false, 1, 1>,           \
+            sgemm_kernel<BM, 128, FM, FN, true, 1, 1>, sgemm_kernel<BM, 128, PM, PN, false, 2, 1>,               \
+            sgemm_kernel<BM, 128, PM, PN, true, 2, 1>, abft_encode_kernel<BM, 128>                               \
+    }
+
+static const FtClass kFtClasses[HPCDNN_FT_NUM_CLASSES] = {
+    HPCDNN_FT_CLASS(256, 2, 2, 2, 4),  // 0 huge
+    HPCDNN_FT_CLASS(128, 2, 2, 2, 2),  // 1 large
+    HPCDNN_FT_CLASS(64, 2, 2, 2, 2),   // 2 wide
+};
 
 static int device_cus() {
     static int cus = 0;
@@ -75,7 +95,7 @@ static int device_cus() {
 static int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {
     if (bytes <= 64 * 1024) return HPCDNN_OK;
     static std::mutex mu;
-    static const void* done[4 * kNumTiles] = {};
+    static const void* done[8 * kNumTiles] = {};
     std::lock_guard<std::mutex> lock(mu);
     const void* key = reinterpret_cast<const void*>(fn);
     for (const void* d : done)
@@ -413,9 +433,27 @@ extern "C" int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int*
     return HPCDNN_OK;
 }
 
-extern "C" int hpcdnn_ft_num_tiles(int M, int N) {
-    if (M < 0 || N < 0) return 0;
-    return static_cast<int>(ceil_div(M, HPCDNN_FT_TILE_M) * ceil_div(N, HPCDNN_FT_TILE_N));
+extern "C" int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn) {
+    if (tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
+    if (bm) *bm = kFtClasses[tile_class].bm;
+    if (bn) *bn = kFtClasses[tile_class].bn;
+    return HPCDNN_OK;
+}
+
+extern "C" int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N) {
+    if (M < 0 || N < 0 || tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return 0;
+    return static_cast<int>(ceil_div(M, kFtClasses[tile_class].bm) * ceil_div(N, kFtClasses[tile_class].bn));
+}
+
+extern "C" int hpcdnn_ft_num_tiles(int M, int N) { return hpcdnn_ft_num_tiles_ex(0, M, N); }
+
+// The largest class that still gives every CU a tile; the smallest one when even that cannot.
+extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
+    (void)K;
+    const int cus = device_cus();
+    for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c)
+        if (hpcdnn_ft_num_tiles_ex(c, M, N) >= cus) return c;
+    return HPCDNN_FT_NUM_CLASSES - 1;
 }
 
 // Fault-free residuals are the FP32 rounding of the accumulators added over a tile line; for operands uniform in
@@ -426,19 +464,30 @@ extern "C" float hpcdnn_ft_default_tau(int K) {
     return 1.1e-6f * static_cast<float>(k);
 }
 
-extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
-                               float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
-                               void* ws, size_t ws_bytes, void* stream) {
+static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const FtClass& fc = kFtClasses[tile_class];
+    return static_cast<size_t>(ceil_div(M, fc.bm) + ceil_div(N, fc.bn)) * ft_enc_ld(K) * sizeof(float);
+}
+
+extern "C" int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                                  float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
+                                  void* ws, size_t ws_bytes, int tile_class, void* stream) {
     int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
     if (rc != HPCDNN_OK) return rc;
+    if (tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
-    const TileConfig& cfg = kTiles[kFtTile];
+    const FtClass& fc = kFtClasses[tile_class];
+    TileConfig cfg{};
+    cfg.bm = fc.bm;
+    cfg.bn = fc.bn;
+    cfg.bk = kGemmBK;
     GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
     a.tau = (tau > 0.f) ? tau : hpcdnn_ft_default_tau(K);
     a.status = status;
     if (inject) {
-        if (inject->tile < 0 || inject->tile >= a.tiles_m * a.tiles_n || inject->row < 0 ||
-            inject->row >= HPCDNN_FT_TILE_M || inject->col < 0 || inject->col >= HPCDNN_FT_TILE_N)
+        if (inject->tile < 0 || inject->tile >= a.tiles_m * a.tiles_n || inject->row < 0 || inject->row >= fc.bm ||
+            inject->col < 0 || inject->col >= fc.bn)
             return HPCDNN_ERR_INVALID_VALUE;
         a.fault_tile = inject->tile;
         a.fault_row = inject->row;
@@ -448,40 +497,49 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
     const bool edge = needs_edge(a, cfg);
     hipStream_t s = static_cast<hipStream_t>(stream);
     dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
-    // With a workspace the checksum vectors of A and B are formed once per tile row / tile column by two small
-    // bandwidth-bound kernels and the main loop only reads them; without one every workgroup forms them itself.
-    const size_t need = ft_workspace_bytes(M, N, K);
+    // With a workspace the checksum vectors of A and B are formed once per tile row / tile column by a small
+    // bandwidth-bound kernel and the main loop only reads them; without one every workgroup forms them itself.
     if (ws && K > 0) {
-        if (ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 15u)) return HPCDNN_ERR_WORKSPACE;
+        if (ws_bytes < ft_class_workspace_bytes(tile_class, M, N, K) || (reinterpret_cast<uintptr_t>(ws) & 15u))
+            return HPCDNN_ERR_WORKSPACE;
         a.enc_ld = ft_enc_ld(K);
         float* enc_a = static_cast<float*>(ws);
         float* enc_b = enc_a + static_cast<size_t>(a.tiles_m) * a.enc_ld;
         a.enc_a = enc_a;
         a.enc_b = enc_b;
         const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
-        abft_encode_kernel<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N><<<k_blocks * (a.tiles_m + a.tiles_n), 1024, 0, s>>>(
-            M, N, K, A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, a.tiles_m);
+        hipLaunchKernelGGL(fc.encode, dim3(k_blocks * (a.tiles_m + a.tiles_n)), dim3(1024), 0, s, M, N, K, A, lda, B, ldb,
+                           enc_a, enc_b, a.enc_ld, k_blocks, a.tiles_m);
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;
-        void (*fn)(const GemmArgs) = edge ? kFtPreEdge : kFtPrePlain;
-        constexpr size_t lds = gemm_lds_bytes<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N, 2, kFtPreThreads>();
-        rc = enable_lds(fn, lds);
+        void (*fn)(const GemmArgs) = edge ? fc.pre_edge : fc.pre_plain;
+        rc = enable_lds(fn, fc.lds_pre);
         if (rc != HPCDNN_OK) return rc;
-        hipLaunchKernelGGL(fn, grid, dim3(kFtPreThreads), lds, s, a);
+        hipLaunchKernelGGL(fn, grid, dim3(fc.threads_pre), fc.lds_pre, s, a);
         return launch_status();
     }
-    void (*fn)(const GemmArgs) = edge ? kFtEdge : kFtPlain;
-    constexpr size_t ft_lds = gemm_lds_bytes<HPCDNN_FT_TILE_M, HPCDNN_FT_TILE_N, 1, kFtThreads>();
-    rc = enable_lds(fn, ft_lds);
+    void (*fn)(const GemmArgs) = edge ? fc.fused_edge : fc.fused_plain;
+    rc = enable_lds(fn, fc.lds_fused);
     if (rc != HPCDNN_OK) return rc;
-    hipLaunchKernelGGL(fn, grid, dim3(kFtThreads), ft_lds, s, a);
+    hipLaunchKernelGGL(fn, grid, dim3(fc.threads_fused), fc.lds_fused, s, a);
     return launch_status();
 }
 
+extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                               float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
+                               void* ws, size_t ws_bytes, void* stream) {
+    return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws, ws_bytes, 0, stream);
+}
+
 namespace hpcdnn {
+// enough for any tile class (the lowest class has the most tile rows)
 size_t ft_workspace_bytes(int M, int N, int K) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return static_cast<size_t>(ceil_div(M, HPCDNN_FT_TILE_M) + ceil_div(N, HPCDNN_FT_TILE_N)) * ft_enc_ld(K) * sizeof(float);
+    size_t most = 0;
+    for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
+        const size_t b = ft_class_workspace_bytes(c, M, N, K);
+        if (b > most) most = b;
+    }
+    return most;
 }
 size_t sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;

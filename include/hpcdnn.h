@@ -39,6 +39,8 @@ extern "C" {
  * tile = (i / 256) * ceil(N / 128) + (j / 128). */
 #define HPCDNN_FT_TILE_M 256
 #define HPCDNN_FT_TILE_N 128
+/* ABFT tile classes: 0 = 256x128 (above), 1 = 128x128, 2 = 64x128. */
+#define HPCDNN_FT_NUM_CLASSES 3
 
 /* Operation selectors for hpcdnn_workspace_bytes(). */
 #define HPCDNN_OP_SGEMM 0
@@ -135,6 +137,21 @@ int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B
                     float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
                     void* ws, size_t ws_bytes, void* stream);
 int hpcdnn_ft_num_tiles(int M, int N);
+
+/* The same on another tile class (hpcdnn_ft_sgemm is class 0): checksums,
+ * verification, status records and `inject` coordinates are per tile of that
+ * class, so `status` holds hpcdnn_ft_num_tiles_ex(tile_class, M, N) records.
+ * Smaller tiles keep more CUs busy on smaller problems; hpcdnn_ft_pick_class
+ * returns the largest class that still gives every CU a tile.  The workspace
+ * size of HPCDNN_OP_FT_SGEMM covers every class.  Counterpart of the reference's
+ * abft_kernel_{huge,large,wide} series (kernel/ft_sgemm/sgemm.cu:187-188,
+ * kernel/ft_sgemm/code_gen/main.py:8-16). */
+int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                       float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
+                       void* ws, size_t ws_bytes, int tile_class, void* stream);
+int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
+int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N);
+int hpcdnn_ft_pick_class(int M, int N, int K);
 /* Threshold hpcdnn_ft_sgemm uses when tau <= 0: 1.1e-6 * max(K, 64), twice the
  * largest fault-free residual measured for operands uniform in [-1, 1] (the
  * rounding noise of the FP32 accumulators grows linearly with K).  Scale it by

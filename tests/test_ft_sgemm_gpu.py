@@ -23,7 +23,7 @@ def _ws(blas, mode, M, N, K):
     if mode == "fused":
         return None
     nbytes = blas.ft_workspace_bytes(M, N, K)
-    assert nbytes == 4 * (-(-M // blas.FT_TILE_M) + -(-N // blas.FT_TILE_N)) * ((-(-K // 16) + 2) * 16)
+    assert nbytes == 4 * (-(-M // 64) + -(-N // 128)) * ((-(-K // 16) + 2) * 16)  # covers the class with the most tile rows
     # poisoned: the library must not rely on the workspace's previous contents
     return torch.full((max(nbytes // 4, 4),), float("nan"), dtype=torch.float32, device="cuda")
 
@@ -197,3 +197,47 @@ def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod, ft_mode):
         assert abs(float(st["row_residual"][tile]) - fix_model) < 3e-3
     print(f"campaign ({ft_mode}): {launches} launches, worst |C - C_clean| after correction {worst_err:.3e}, "
           f"fault-free max residual {clean['max_clean_residual'].max():.3e}, tau {tau:.1e}")
+
+
+@pytest.mark.parametrize("tile_class", [1, 2])
+def test_smaller_tile_classes_match_the_model(blas, oracle_mod, ft_mode, tile_class):
+    """The 128x128 and 64x128 ABFT tiles: tiles, status records and fault coordinates are per tile of the class."""
+    bm, bn = blas.ft_tile(tile_class)
+    assert (bm, bn) == {1: (128, 128), 2: (64, 128)}[tile_class]
+    M, N, K = 333, 300, 520  # ragged in every dimension
+    tau = blas.ft_default_tau(K)
+    ntm, ntn = -(-M // bm), -(-N // bn)
+    assert blas.ft_num_tiles(M, N, tile_class) == ntm * ntn
+    rng = np.random.default_rng(40 + tile_class)
+    for trial in range(8):
+        a = oracle_mod.fill_uniform_matrix(M, K, 600 + trial, ld=K + 4)
+        b = oracle_mod.fill_uniform_matrix(K, N, 700 + trial, ld=N + 4)
+        c0 = oracle_mod.fill_uniform_matrix(M, N, 800 + trial, ld=N + 8)
+        fault = None
+        if trial:
+            tile = int(rng.integers(ntm * ntn))
+            tm = min(bm, M - (tile // ntn) * bm)
+            tn = min(bn, N - (tile % ntn) * bn)
+            fault = (tile, int(rng.integers(tm)), int(rng.integers(tn)),
+                     float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-2, 2))))
+        da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+        status = blas.ft_status_alloc(M, N, tile_class=tile_class)
+        blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 1.0, tau=tau, fault=fault, status=status, ws=_ws(blas, ft_mode, M, N, K),
+                      tile_class=tile_class)
+        st = blas.ft_status_numpy(status)
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.0, 1.0, bm, bn, tau, fault)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (tile_class, fault, f, st[f], st_model[f])
+        if fault is not None:
+            assert st["flag"][fault[0]] == 1 and (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3]
+        _assert_values(oracle_mod, M, N, K, a, b, c0, dc.cpu().numpy(), 1.0, 1.0)
+
+
+def test_pick_class_and_bad_class(blas):
+    assert blas.ft_pick_class(4096, 4096, 4096) == 0      # 512 tiles of 256x128: every CU has one
+    assert blas.ft_pick_class(2048, 2048, 1024) == 1      # 128 tiles of 256x128, 256 of 128x128
+    assert blas.ft_pick_class(512, 512, 512) == 2
+    t = torch.zeros(64, 64, device="cuda")
+    with pytest.raises(blas.HpcdnnError):
+        blas.ft_sgemm(64, 64, 64, t, t, t.clone(), 1.0, 0.0, tile_class=3)
