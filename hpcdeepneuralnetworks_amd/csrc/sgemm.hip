@@ -447,13 +447,20 @@ extern "C" int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N) {
 
 extern "C" int hpcdnn_ft_num_tiles(int M, int N) { return hpcdnn_ft_num_tiles_ex(0, M, N); }
 
-// The largest class that still gives every CU a tile; the smallest one when even that cannot.
+// The class with the shortest predicted run: rounds of tiles over the CUs times the tile height (all classes are
+// 128 columns wide), with the measured efficiency of the smaller tiles relative to the 256-row one.
 extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
     (void)K;
+    static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 0.97, 0.90};
     const int cus = device_cus();
-    for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c)
-        if (hpcdnn_ft_num_tiles_ex(c, M, N) >= cus) return c;
-    return HPCDNN_FT_NUM_CLASSES - 1;
+    int best = 0;
+    double best_cost = 1e300;
+    for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
+        const int64_t tiles = hpcdnn_ft_num_tiles_ex(c, M, N);
+        const double cost = static_cast<double>(ceil_div(tiles > 0 ? tiles : 1, cus)) * kFtClasses[c].bm / rel_eff[c];
+        if (cost < best_cost) { best_cost = cost; best = c; }
+    }
+    return best;
 }
 
 // Fault-free residuals are the FP32 rounding of the accumulators added over a tile line; for operands uniform in

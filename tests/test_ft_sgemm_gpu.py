@@ -238,6 +238,7 @@ def test_pick_class_and_bad_class(blas):
     assert blas.ft_pick_class(4096, 4096, 4096) == 0      # 512 tiles of 256x128: every CU has one
     assert blas.ft_pick_class(2048, 2048, 1024) == 1      # 128 tiles of 256x128, 256 of 128x128
     assert blas.ft_pick_class(512, 512, 512) == 2
+    assert blas.ft_pick_class(3072, 3072, 3072) == 2      # 288 tiles of 256x128 would leave a nearly empty second round
     t = torch.zeros(64, 64, device="cuda")
     with pytest.raises(blas.HpcdnnError):
         blas.ft_sgemm(64, 64, 64, t, t, t.clone(), 1.0, 0.0, tile_class=3)
