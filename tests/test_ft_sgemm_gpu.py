@@ -242,3 +242,17 @@ def test_pick_class_and_bad_class(blas):
     t = torch.zeros(64, 64, device="cuda")
     with pytest.raises(blas.HpcdnnError):
         blas.ft_sgemm(64, 64, 64, t, t, t.clone(), 1.0, 0.0, tile_class=3)
+
+
+def test_k_zero_scales_c_and_flags_nothing(blas, ft_mode):
+    M, N = 300, 200
+    c0 = torch.rand(M, N, device="cuda")
+    c = c0.clone()
+    a = torch.zeros(M, 1, device="cuda")
+    b = torch.zeros(1, N, device="cuda")
+    status = blas.ft_status_alloc(M, N)
+    ws = None if ft_mode == "fused" else torch.zeros(64, device="cuda")
+    blas.ft_sgemm(M, N, 0, a[:, :0], b[:0, :], c, 1.0, 0.5, status=status, ws=ws)
+    assert torch.equal(c, c0 * 0.5)
+    st = blas.ft_status_numpy(status)
+    assert np.all(st["flag"] == 0) and np.all(st["max_clean_residual"] == 0.0)
