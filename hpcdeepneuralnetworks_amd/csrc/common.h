@@ -20,6 +20,20 @@ inline int launch_status() {
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Compute units of the current device (256 on an MI355X); 256 when no device can be queried.
+inline int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            return 256;
+    }
+    return cus;
+}
+
 // ---- counter-based RNG: splitmix64 finaliser of seed*golden + index ------
 __host__ __device__ inline uint64_t mix64(uint64_t z) {
     z ^= z >> 30; z *= 0xBF58476D1CE4E5B9ull;

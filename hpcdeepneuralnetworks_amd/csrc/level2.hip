@@ -112,19 +112,6 @@ __global__ __launch_bounds__(kGemvThreads) void fill_const_kernel(float* __restr
 
 __global__ void add_to_element_kernel(float* __restrict__ p, float delta) { *p += delta; }
 
-static int device_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            return 256;
-    }
-    return cus;
-}
-
 // Row chunks of the transposed product: enough blocks to fill the device, at least 32 rows each.
 static int gemv_t_chunks(int M, int N) {
     const int64_t col_blocks = ceil_div(N, kGemvColsPerBlock);

@@ -78,19 +78,6 @@ static const FtClass kFtClasses[HPCDNN_FT_NUM_CLASSES] = {
     HPCDNN_FT_CLASS(64, 2, 2, 2, 2),   // 2 wide
 };
 
-static int device_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-            cus = v;
-        else
-            return 256;
-    }
-    return cus;
-}
-
 // Kernels that use more than the default 64 KiB of LDS must opt in once.
 static int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {
     if (bytes <= 64 * 1024) return HPCDNN_OK;

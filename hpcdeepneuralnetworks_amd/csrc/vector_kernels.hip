@@ -188,19 +188,6 @@ __global__ __launch_bounds__(kVecThreads) void zero_words_kernel(uint32_t* __res
 }
 
 // ------------------------------------------------------------- launch glue --
-static int device_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-            cus = v;
-        else
-            return 256;
-    }
-    return cus;
-}
-
 static int stream_grid(int64_t work_items, int blocks_per_cu) {
     int64_t want = ceil_div(work_items, kVecThreads);
     int64_t cap = static_cast<int64_t>(device_cus()) * blocks_per_cu;
