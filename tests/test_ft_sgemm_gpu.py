@@ -144,7 +144,7 @@ class _TileModel:
 
 
 def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod, ft_mode):
-    """BASELINE config 4: M=N=K=4096, alpha=1, beta=0, one seeded fault (tile, i, j, magnitude in [1e-2, 1e2],
+    """The 4096-cube fault campaign: M=N=K=4096, alpha=1, beta=0, one seeded fault (tile, i, j, magnitude in [1e-2, 1e2],
     random sign) per launch.  Every launch: detected, located at the injected element, corrected, no other tile
     flagged; decisions equal the CPU model's for every launch (the model is evaluated on the faulted tile)."""
     M = N = K = 4096

@@ -36,7 +36,7 @@ def _check(oracle_mod, blas, M, N, K, alpha, beta, lda=None, ldb=None, ldc=None,
 
 
 def test_config1_1024_cube_against_reference_cpu_gemm(blas, oracle_mod):
-    """BASELINE config 1: M=N=K=1024, alpha=1, beta=0, C zero-initialised, validated against the reference's
+    """The reference's own CPU-checkable case: M=N=K=1024, alpha=1, beta=0, C zero-initialised, validated against the reference's
     CPU triple loop (utils/utils.cu:93-103) and against the FP64 criterion."""
     n = 1024
     a = oracle_mod.fill_uniform_matrix(n, n, 1)
