@@ -37,7 +37,7 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline SGEMM line only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--ft-launches", type=int, default=1000, help="launches of the ABFT fault campaign")
-    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "ft_sgemm", "saxpy", "sdot", "copy"],
+    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "ft_sgemm", "saxpy", "sdot", "copy", "sgemv_n", "sgemv_t"],
                     help="run one kernel only for --steps launches (for profiling with rocprofv3) and print a short line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -87,6 +87,17 @@ def main() -> int:
             ft_ws = blas.workspace(blas.ft_workspace_bytes(m, m, m))
             fn = lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=blas.ft_default_tau(m), status=status, ws=ft_ws)
             work, unit = 2.0 * m ** 3, "GFLOP/s"
+        elif args.kernel in ("sgemv_n", "sgemv_t"):
+            mv = 16384
+            am = torch.empty(mv, mv, device=dev)
+            blas.fill_uniform_matrix(am, mv, mv, 40)
+            xv = torch.empty(mv, device=dev)
+            yv = torch.empty(mv, device=dev)
+            blas.fill_uniform(xv, 41)
+            gws = blas.workspace(max(blas.sgemv_workspace_bytes(mv, mv), 4))
+            trans = args.kernel == "sgemv_t"
+            fn = lambda: blas.sgemv(trans, mv, mv, 1.0, am, xv, 0.0, yv, ws=gws)
+            work, unit = 4.0 * mv * mv, "GB/s"
         else:
             nv = 1 << 28
             x = torch.empty(nv, device=dev)
