@@ -10,34 +10,52 @@ constexpr int kGemvWaves = kGemvThreads / kWave;
 constexpr int kGemvColsPerBlock = 4 * kWave;  // one 16-byte load per lane
 constexpr int kGemvMaxChunks = 64;
 
-// y[m] = alpha * sum_n A[m][n] x[n] + beta * y[m].  One wave per row: the row is read in 1 KiB pieces (one
-// 16-byte load per lane), four pieces in flight; columns >= N read as 0 through the descriptors.  The lane
-// partials are added in a fixed order, so the result does not depend on timing.
+// y[m] = alpha * sum_n A[m][n] x[n] + beta * y[m].  One wave per group of kGemvRows rows: the rows are read in 1 KiB
+// pieces (one 16-byte load per lane), 8 / kGemvRows pieces of each row in flight, against the same two pieces of x, so x is
+// fetched once per four rows; columns >= N read as 0 through the descriptors.  The lane partials are added in a fixed
+// order, so the result does not depend on timing.  kGemvRows = 1 (one row per wave, more waves) suits matrices with
+// few or short rows.
+template <int kGemvRows>
 __global__ __launch_bounds__(kGemvThreads) void sgemv_n_kernel(int M, int N, float alpha, const float* __restrict__ A,
                                                                int lda, const float* __restrict__ x, float beta,
                                                                float* __restrict__ y) {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const __amdgpu_buffer_rsrc_t xr = make_rsrc(x, static_cast<int64_t>(N) * 4);
-    for (int m = blockIdx.x * kGemvWaves + wave; m < M; m += gridDim.x * kGemvWaves) {
-        const __amdgpu_buffer_rsrc_t ar = make_rsrc(A + static_cast<int64_t>(m) * lda, static_cast<int64_t>(N) * 4);
-        v4f acc = {0.f, 0.f, 0.f, 0.f};
-        for (int n0 = 0; n0 < N; n0 += 4 * kGemvColsPerBlock) {
-            v4f a[4], xv[4];
+    for (int m = kGemvRows * (blockIdx.x * kGemvWaves + wave); m < M; m += kGemvRows * gridDim.x * kGemvWaves) {
+        __amdgpu_buffer_rsrc_t ar[kGemvRows];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) a[u] = buffer_load_v4f(ar, (n0 + u * kGemvColsPerBlock + lane * 4) * 4);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) xv[u] = buffer_load_v4f(xr, (n0 + u * kGemvColsPerBlock + lane * 4) * 4);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                acc.x = __builtin_fmaf(a[u].x, xv[u].x, acc.x);
-                acc.y = __builtin_fmaf(a[u].y, xv[u].y, acc.y);
-                acc.z = __builtin_fmaf(a[u].z, xv[u].z, acc.z);
-                acc.w = __builtin_fmaf(a[u].w, xv[u].w, acc.w);
-            }
+        for (int r = 0; r < kGemvRows; ++r) {
+            const bool valid = m + r < M;
+            ar[r] = make_rsrc(A + static_cast<int64_t>(valid ? m + r : m) * lda, valid ? static_cast<int64_t>(N) * 4 : 0);
         }
-        const float s = wave_sum_lane63((acc.x + acc.y) + (acc.z + acc.w));
-        if (lane == kWave - 1) y[m] = (beta == 0.f) ? alpha * s : __builtin_fmaf(beta, y[m], alpha * s);
+        v4f acc[kGemvRows];
+#pragma unroll
+        for (int r = 0; r < kGemvRows; ++r) acc[r] = v4f{0.f, 0.f, 0.f, 0.f};
+        constexpr int kPieces = 8 / kGemvRows < 4 ? 8 / kGemvRows : 4;
+        for (int n0 = 0; n0 < N; n0 += kPieces * kGemvColsPerBlock) {
+            v4f a[kGemvRows][kPieces], xv[kPieces];
+#pragma unroll
+            for (int r = 0; r < kGemvRows; ++r)
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) a[r][u] = buffer_load_v4f(ar[r], (n0 + u * kGemvColsPerBlock + lane * 4) * 4);
+#pragma unroll
+            for (int u = 0; u < kPieces; ++u) xv[u] = buffer_load_v4f(xr, (n0 + u * kGemvColsPerBlock + lane * 4) * 4);
+#pragma unroll
+            for (int r = 0; r < kGemvRows; ++r)
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) {
+                    acc[r].x = __builtin_fmaf(a[r][u].x, xv[u].x, acc[r].x);
+                    acc[r].y = __builtin_fmaf(a[r][u].y, xv[u].y, acc[r].y);
+                    acc[r].z = __builtin_fmaf(a[r][u].z, xv[u].z, acc[r].z);
+                    acc[r].w = __builtin_fmaf(a[r][u].w, xv[u].w, acc[r].w);
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < kGemvRows; ++r) {
+            const float s = wave_sum_lane63((acc[r].x + acc[r].y) + (acc[r].z + acc[r].w));
+            if (lane == kWave - 1 && m + r < M) y[m + r] = (beta == 0.f) ? alpha * s : __builtin_fmaf(beta, y[m + r], alpha * s);
+        }
     }
 }
 
@@ -137,10 +155,14 @@ static int run_sgemv(int trans, int M, int N, float alpha, const float* A, int l
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3u)
         return HPCDNN_ERR_INVALID_VALUE;
     if (!trans) {
-        int64_t grid = ceil_div(M, kGemvWaves);
+        const bool grouped = N >= 4096 && M >= 8192;  // long rows and enough of them: share x between four rows
+        int64_t grid = ceil_div(M, (grouped ? 4 : 1) * kGemvWaves);
         const int64_t cap = static_cast<int64_t>(device_cus()) * 16;
         if (grid > cap) grid = cap;
-        sgemv_n_kernel<<<static_cast<int>(grid), kGemvThreads, 0, s>>>(M, N, alpha, A, lda, x, beta, y);
+        if (grouped)
+            sgemv_n_kernel<4><<<static_cast<int>(grid), kGemvThreads, 0, s>>>(M, N, alpha, A, lda, x, beta, y);
+        else
+            sgemv_n_kernel<1><<<static_cast<int>(grid), kGemvThreads, 0, s>>>(M, N, alpha, A, lda, x, beta, y);
         return launch_status();
     }
     int chunks = gemv_t_chunks(M, N);

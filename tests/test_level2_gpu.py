@@ -33,7 +33,7 @@ def _gemv_case(blas, oracle_mod, trans, M, N, alpha, beta, lda=None, use_ws=True
 
 
 @pytest.mark.parametrize("trans", [False, True])
-@pytest.mark.parametrize("M,N", [(1, 1), (3, 5), (64, 256), (257, 1023), (1000, 37), (37, 1000), (2048, 2048), (4096, 256), (256, 4096)])
+@pytest.mark.parametrize("M,N", [(1, 1), (3, 5), (64, 256), (257, 1023), (1000, 37), (37, 1000), (2048, 2048), (4096, 256), (256, 4096), (8195, 4100)])
 def test_sgemv_shapes(blas, oracle_mod, trans, M, N):
     _gemv_case(blas, oracle_mod, trans, M, N, 1.0, 0.0)
 
