@@ -59,7 +59,8 @@ struct GemmArgs {
     int full_tiles, tail_split, tail_k_chunk;
     float* tail_partial;
     // ABFT
-    float tau;
+    float tau;      // absolute residual threshold; 0 = relative mode
+    float tau_rel;  // relative mode: threshold of a line = tau_rel * sum |accumulators of the line| / sqrt(elements in it)
     int fault_tile, fault_row, fault_col;
     float fault_delta;
     hpcdnn_ft_status* status;
@@ -599,10 +600,12 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         double* const s_crref = s_ccref + CCP * BN;                     // [CRP][BM] reference row checksum partials
         float* const s_ccobs = reinterpret_cast<float*>(s_crref + CRP * BM);  // [WGM][BN] observed column sums
         float* const s_crobs = s_ccobs + WGM * BN;                      // [WGN][BM] observed row sums
-        float* const s_dr = s_crobs + WGN * BM;                         // [BM] row residuals, then [BN] column residuals
+        float* const s_ccabs = s_crobs + WGN * BM;                      // [WGM][BN] column sums of |accumulators|
+        float* const s_crabs = s_ccabs + WGM * BN;                      // [WGN][BM] row sums of |accumulators|
+        float* const s_dr = s_crabs + WGN * BM;                         // [BM] row residuals, then [BN] column residuals
         int* const s_meta = reinterpret_cast<int*>(s_dr + BM + BN);     // nbr, nbc, bad row, bad col, max clean (float bits)
         static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads>() >=
-                          sizeof(double) * (CCP * BN + CRP * BM) + sizeof(float) * (WGM * BN + WGN * BM + BM + BN) + 32,
+                          sizeof(double) * (CCP * BN + CRP * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + BM + BN) + 32,
                       "verification scratch fits in the staging buffers");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
 
@@ -633,10 +636,12 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         for (int e = 0; e < 4; ++e) s_ccref[e_hw * BN + (tid & 31) * 4 + e] = cc_ref[e];
 #pragma unroll
         for (int sl = 0; sl < A_SLOTS; ++sl) s_crref[e_class * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = cr_ref[sl];
-        // observed column sums of the accumulators (ft_sgemm_huge.cuh:147-154): lane = column
+        // observed column sums of the accumulators (ft_sgemm_huge.cuh:147-154): lane = column.  In relative mode the
+        // sums of absolute values go with them: they scale the threshold to the data.
+        const bool relative = p.tau <= 0.f;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            float s = 0.f;
+            float s = 0.f, sa = 0.f;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 float si = 0.f;
@@ -645,38 +650,66 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 s += si;
             }
             s += __shfl_xor(s, 32, kWave);
-            if (lh == 0) s_ccobs[wm * BN + wn * WN + j * 32 + lr] = s;
+            if (relative) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) sa += __builtin_fabsf(acc[i][j][v]);
+                sa += __shfl_xor(sa, 32, kWave);
+            }
+            if (lh == 0) {
+                s_ccobs[wm * BN + wn * WN + j * 32 + lr] = s;
+                s_ccabs[wm * BN + wn * WN + j * 32 + lr] = sa;
+            }
         }
         // observed row sums (ft_sgemm_huge.cuh:156-171): register = row, summed over the 32 column lanes
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                float s = acc[i][0][v];
+                float s = acc[i][0][v], sa = 0.f;
 #pragma unroll
                 for (int j = 1; j < TN; ++j) s += acc[i][j][v];
                 s = half32_allsum(s);
-                if (lr == 0) s_crobs[wn * BM + wm * WM + i * 32 + 8 * (v / 4) + 4 * lh + (v % 4)] = s;
+                if (relative) {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) sa += __builtin_fabsf(acc[i][j][v]);
+                    sa = half32_allsum(sa);
+                }
+                if (lr == 0) {
+                    s_crobs[wn * BM + wm * WM + i * 32 + 8 * (v / 4) + 4 * lh + (v % 4)] = s;
+                    s_crabs[wn * BM + wm * WM + i * 32 + 8 * (v / 4) + 4 * lh + (v % 4)] = sa;
+                }
             }
         __syncthreads();
 
-        // residual = reference - observed per line; |d| > tau marks the line (ft_sgemm_huge.cuh:200-271)
-        const double tau = static_cast<double>(p.tau);
+        // residual = reference - observed per line; |d| > tau marks the line (ft_sgemm_huge.cuh:200-271).  Relative
+        // mode: tau of a line = tau_rel * sum |acc| / sqrt(n), n = elements of the line inside the matrix (rounding
+        // noise of a sum of n accumulators grows like sqrt(n) times their magnitude).
+        const int rows_in = (p.M - m0 < BM) ? p.M - m0 : BM, cols_in = (p.N - n0 < BN) ? p.N - n0 : BN;
+        const float row_scale = p.tau_rel / __builtin_sqrtf(static_cast<float>(cols_in));
+        const float col_scale = p.tau_rel / __builtin_sqrtf(static_cast<float>(rows_in));
         for (int line = tid; line < BM + BN; line += kGemmThreads) {
             const bool is_row = line < BM;
             const int idx = is_row ? line : line - BM;
             double ref = 0.0, obs = 0.0;
+            float mag = 0.f;
             if (is_row) {
 #pragma unroll
                 for (int w = 0; w < CRP; ++w) ref += s_crref[w * BM + idx];
 #pragma unroll
                 for (int w = 0; w < WGN; ++w) obs += static_cast<double>(s_crobs[w * BM + idx]);
+#pragma unroll
+                for (int w = 0; w < WGN; ++w) mag += s_crabs[w * BM + idx];
             } else {
 #pragma unroll
                 for (int w = 0; w < CCP; ++w) ref += s_ccref[w * BN + idx];
 #pragma unroll
                 for (int w = 0; w < WGM; ++w) obs += static_cast<double>(s_ccobs[w * BN + idx]);
+#pragma unroll
+                for (int w = 0; w < WGM; ++w) mag += s_ccabs[w * BN + idx];
             }
+            const double tau = relative ? static_cast<double>(mag * (is_row ? row_scale : col_scale)) : static_cast<double>(p.tau);
             const double d = ref - obs;
             if (fabs(d) > tau) {
                 atomicAdd(&s_meta[is_row ? 0 : 1], 1);

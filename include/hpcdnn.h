@@ -121,8 +121,12 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * tile are accumulated from A and B inside the main loop, compared with the
  * line sums of the accumulators in the epilogue, and a single faulty element
  * per tile is located (faulty row x faulty column) and corrected before
- * alpha/beta are applied.  `tau` is the absolute residual threshold
- * (<= 0 selects the default for inputs of magnitude <= 1); `inject` is a HOST
+ * alpha/beta are applied.  `tau` > 0 is an absolute residual threshold, 0
+ * selects the default for inputs of magnitude <= 1 (hpcdnn_ft_default_tau),
+ * and `tau` < 0 scales the threshold to the data: a line is flagged when its
+ * residual exceeds -tau * 2.56e-7 * sqrt(K) * (sum of |accumulators| over the
+ * line) / sqrt(elements of the line), -1 being calibrated to twice the
+ * largest fault-free residual of uniform operands; `inject` is a HOST
  * pointer to one fault or NULL; `status` is DEVICE memory for
  * hpcdnn_ft_num_tiles(M,N) records or NULL.
  * `ws`/`ws_bytes`: optional DEVICE scratch of

@@ -256,16 +256,17 @@ void oracle_abft_residuals(int tm, int tn, int K, const float* A, int lda, const
  * for its +1.0 test fault; the sound value for any magnitude is the signed
  * row residual, added back to the accumulator (acc += dr[row]).
  * Returns the correction (0 when nothing is corrected). */
-float oracle_abft_decide(int tm, int tn, const double* dr, const double* dc, float tau,
-                         oracle_ft_status* st) {
+/* Per-line thresholds: tau_r[m] for row m, tau_c[n] for column n. */
+float oracle_abft_decide_lines(int tm, int tn, const double* dr, const double* dc, const double* tau_r,
+                               const double* tau_c, oracle_ft_status* st) {
     int nbr = 0, nbc = 0, r = -1, c = -1;
     double clean = 0.0;
     for (int m = 0; m < tm; ++m) {
-        if (fabs(dr[m]) > (double)tau) { ++nbr; r = m; }
+        if (fabs(dr[m]) > tau_r[m]) { ++nbr; r = m; }
         else if (fabs(dr[m]) > clean) clean = fabs(dr[m]);
     }
     for (int n = 0; n < tn; ++n) {
-        if (fabs(dc[n]) > (double)tau) { ++nbc; c = n; }
+        if (fabs(dc[n]) > tau_c[n]) { ++nbc; c = n; }
         else if (fabs(dc[n]) > clean) clean = fabs(dc[n]);
     }
     st->n_bad_rows = nbr;
@@ -283,10 +284,42 @@ float oracle_abft_decide(int tm, int tn, const double* dr, const double* dc, flo
     return 0.0f;
 }
 
+/* One absolute threshold for every line (the reference's scheme: 0.1, kernel/ft_sgemm/include/ft_sgemm_huge.cuh:30,263). */
+float oracle_abft_decide(int tm, int tn, const double* dr, const double* dc, float tau,
+                         oracle_ft_status* st) {
+    double* t = (double*)malloc(sizeof(double) * (size_t)(tm + tn));
+    for (int i = 0; i < tm + tn; ++i) t[i] = (double)tau;
+    float fix = oracle_abft_decide_lines(tm, tn, dr, dc, t, t + tm, st);
+    free(t);
+    return fix;
+}
+
+/* Data-scaled thresholds (no reference counterpart; the reference's thresholds are constants): a line's threshold
+ * is rel * sum |acc| over the line / sqrt(elements in the line), with rel = factor * 2.56e-7 * sqrt(K) (4.3 units of
+ * FP32 rounding per sqrt(K)): the rounding noise of a sum of n accumulators grows like sqrt(n) times their
+ * magnitude, and that of one accumulator like sqrt(K) times the rounding unit. */
+void oracle_abft_relative_thresholds(int tm, int tn, int K, const float* acc, int ldacc, float factor,
+                                     double* tau_r, double* tau_c) {
+    float rel = factor * 2.56e-7f * sqrtf((float)K);
+    float rs = rel / sqrtf((float)tn), cs = rel / sqrtf((float)tm);
+    for (int n = 0; n < tn; ++n) tau_c[n] = 0.0;
+    for (int m = 0; m < tm; ++m) {
+        double s = 0.0;
+        for (int n = 0; n < tn; ++n) {
+            double v = fabs((double)acc[(size_t)m * ldacc + n]);
+            s += v;
+            tau_c[n] += v;
+        }
+        tau_r[m] = (double)((float)s * rs);
+    }
+    for (int n = 0; n < tn; ++n) tau_c[n] = (double)((float)tau_c[n] * cs);
+}
+
 /* Whole-matrix model: C = alpha*acc + beta*C with acc = A*B accumulated in
  * float (k ascending), one fault (tile index in row-major tile order,
  * tile-local i, j, delta added to acc before verification) or none
- * (fault_tile < 0), tiles of tile_m x tile_n (edge tiles are clipped), one
+ * (fault_tile < 0), tiles of tile_m x tile_n (edge tiles are clipped), tau > 0
+ * absolute or tau < 0 data-scaled with factor -tau, one
  * status record per tile.  Mirrors the device entry point's contract; used on
  * sizes the CPU finishes in seconds. */
 void oracle_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
@@ -312,7 +345,15 @@ void oracle_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* 
             }
         if (t == fault_tile && fault_i < tm && fault_j < tn) acc[(size_t)fault_i * tn + fault_j] += fault_delta;
         oracle_abft_residuals(tm, tn, K, A + (size_t)m0 * lda, lda, B + n0, ldb, acc, tn, dr, dc);
-        float fix = oracle_abft_decide(tm, tn, dr, dc, tau, &status[t]);
+        float fix;
+        if (tau < 0.0f) {
+            double* thr = (double*)malloc(sizeof(double) * (size_t)(tm + tn));
+            oracle_abft_relative_thresholds(tm, tn, K, acc, tn, -tau, thr, thr + tm);
+            fix = oracle_abft_decide_lines(tm, tn, dr, dc, thr, thr + tm, &status[t]);
+            free(thr);
+        } else {
+            fix = oracle_abft_decide(tm, tn, dr, dc, tau, &status[t]);
+        }
         if (status[t].flag == 1) acc[(size_t)status[t].row * tn + status[t].col] += fix;
         for (int m = 0; m < tm; ++m)
             for (int n = 0; n < tn; ++n) {

@@ -256,3 +256,30 @@ def test_k_zero_scales_c_and_flags_nothing(blas, ft_mode):
     assert torch.equal(c, c0 * 0.5)
     st = blas.ft_status_numpy(status)
     assert np.all(st["flag"] == 0) and np.all(st["max_clean_residual"] == 0.0)
+
+
+@pytest.mark.parametrize("scale_a,scale_b,shift", [(1.0, 1.0, 0.0), (250.0, 0.004, 0.0), (1e-3, 1e-3, 0.0), (1.0, 1.0, 0.5)])
+def test_data_scaled_threshold(blas, oracle_mod, ft_mode, scale_a, scale_b, shift):
+    """tau < 0: thresholds follow the magnitude of the accumulators, so the same call works for operands of any scale
+    and for operands with a non-zero mean (where the absolute default for unit data would flag rounding noise or miss
+    small faults).  Decisions equal the CPU model's; a fault of 2e-3 of the typical |C| entry is found."""
+    M, N, K = 512, 384, 1024
+    a = (oracle_mod.fill_uniform_matrix(M, K, 910) + np.float32(shift)) * np.float32(scale_a)
+    b = (oracle_mod.fill_uniform_matrix(K, N, 911) + np.float32(shift)) * np.float32(scale_b)
+    c0 = np.zeros((M, N), np.float32)
+    typical = float(np.abs(a[:64].astype(np.float64) @ b.astype(np.float64)).mean())
+    for fault in (None, (3, 100, 50, 2e-3 * typical * 40), (1, 7, 9, -2e-3 * typical * 40)):
+        da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+        status = blas.ft_status_alloc(M, N)
+        blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=-1.0, fault=fault, status=status, ws=_ws(blas, ft_mode, M, N, K))
+        st = blas.ft_status_numpy(status)
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm(M, N, K, a, K, b, N, c_model, N, 1.0, 0.0, blas.FT_TILE_M, blas.FT_TILE_N, -1.0, fault)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (scale_a, shift, fault, f, st[f], st_model[f])
+        if fault is None:
+            assert np.all(st["flag"] == 0)
+        else:
+            assert st["flag"][fault[0]] == 1 and (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3]
+            assert np.count_nonzero(st["flag"]) == 1
+        _assert_values(oracle_mod, M, N, K, a, b, c0, dc.cpu().numpy(), 1.0, 0.0)
