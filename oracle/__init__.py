@@ -97,6 +97,8 @@ def _load():
     lib.oracle_ft_sgemm.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
                                     C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int, C.c_int, C.c_float,
                                     C.c_void_p]
+    lib.oracle_abft_relative_thresholds.restype = None
+    lib.oracle_abft_relative_thresholds.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, C.c_float, dp, dp]
     lib.oracle_sgemv_f64.restype = None
     lib.oracle_sgemv_f64.argtypes = [C.c_int, C.c_int, C.c_int, C.c_float, fp, C.c_int, fp, C.c_float, fp, dp, dp]
     lib.oracle_offline_ft_sgemm.restype = None
@@ -248,3 +250,12 @@ def offline_ft_sgemm(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, panel, fault=
     _load().oracle_offline_ft_sgemm(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, panel, int(fp_), int(fr),
                                     int(fc), float(fd), _d(res))
     return res[:2 * panels]
+
+
+def abft_relative_thresholds(acc: np.ndarray, K: int, factor: float = 1.0):
+    """Per-row and per-column thresholds of the data-scaled mode for one tile of accumulators."""
+    tm, tn = acc.shape
+    acc = np.ascontiguousarray(acc, dtype=np.float32)
+    tr, tc = np.empty(tm, np.float64), np.empty(tn, np.float64)
+    _load().oracle_abft_relative_thresholds(tm, tn, K, _f(acc), tn, factor, _d(tr), _d(tc))
+    return tr, tc

@@ -25,6 +25,9 @@
  *     (AB)e = A(Be)) and to the one known-answer case the reference holds
  *     (+1.0 at tile-local (0,1), threshold 0.1 -> row 0, col 1, magnitude 1;
  *     kernel/ft_sgemm/include/ft_sgemm_huge.cuh:40,145,263,358).  Bit-level
+ *     oracle_abft_relative_thresholds (data-scaled thresholds, an addition
+ *     with no reference counterpart): pinned to closed forms (constant and
+ *     single-entry tiles) and to its scaling laws.  Bit-level
  *     agreement with the reference's CUDA kernels or cuBLAS: parity unpinned
  *     (neither can be built or run without an NVIDIA toolchain, and the
  *     reference's ABFT locate/correct step is unfinished).

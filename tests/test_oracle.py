@@ -294,3 +294,24 @@ def test_offline_ft_model_closed_form(oracle_mod, alpha, beta, panel):
         assert abs(diff[5, 7] + 3.5) < 1e-5
         diff[5, 7] = 0.0
         assert np.abs(diff).max() < 1e-5
+
+
+def test_relative_thresholds_closed_forms_and_scaling(oracle_mod):
+    """Constant tile: every row holds tn copies of |c|, so its threshold is rel * |c| * sqrt(tn) (and sqrt(tm) for
+    columns) with rel = 2.56e-7 * sqrt(K); a single non-zero entry only raises its own row and column; thresholds
+    are linear in the data, in the factor, and grow like sqrt(K)."""
+    tm, tn, K = 48, 20, 400
+    rel = 2.56e-7 * np.sqrt(K)
+    tr, tc = oracle_mod.abft_relative_thresholds(np.full((tm, tn), -3.0, np.float32), K)
+    assert np.allclose(tr, rel * 3.0 * np.sqrt(tn), rtol=1e-6) and np.allclose(tc, rel * 3.0 * np.sqrt(tm), rtol=1e-6)
+    one = np.zeros((tm, tn), np.float32)
+    one[5, 7] = 2.0
+    tr, tc = oracle_mod.abft_relative_thresholds(one, K)
+    assert np.count_nonzero(tr) == 1 and np.count_nonzero(tc) == 1
+    assert np.isclose(tr[5], rel * 2.0 / np.sqrt(tn), rtol=1e-6) and np.isclose(tc[7], rel * 2.0 / np.sqrt(tm), rtol=1e-6)
+    rng = np.random.default_rng(3)
+    acc = rng.standard_normal((tm, tn)).astype(np.float32)
+    tr1, tc1 = oracle_mod.abft_relative_thresholds(acc, K)
+    tr2, tc2 = oracle_mod.abft_relative_thresholds(acc * np.float32(8.0), 4 * K, factor=0.5)
+    assert np.allclose(tr2, tr1 * 8.0 * 2.0 * 0.5, rtol=1e-6) and np.allclose(tc2, tc1 * 8.0, rtol=1e-6)
+    assert np.allclose(tr1, rel * np.abs(acc.astype(np.float64)).sum(axis=1) / np.sqrt(tn), rtol=1e-5)
