@@ -315,3 +315,35 @@ def test_relative_thresholds_closed_forms_and_scaling(oracle_mod):
     tr2, tc2 = oracle_mod.abft_relative_thresholds(acc * np.float32(8.0), 4 * K, factor=0.5)
     assert np.allclose(tr2, tr1 * 8.0 * 2.0 * 0.5, rtol=1e-6) and np.allclose(tc2, tc1 * 8.0, rtol=1e-6)
     assert np.allclose(tr1, rel * np.abs(acc.astype(np.float64)).sum(axis=1) / np.sqrt(tn), rtol=1e-5)
+
+
+def _fixtures():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fixtures.json")) as f:
+        return json.load(f)
+
+
+def test_golden_fixtures_pin_rng_saxpy_and_the_reference_fault_case(oracle_mod):
+    """tests/golden/fixtures.json holds values computed with Python integers / exact fractions
+    (tests/golden/make_fixtures.py), independent of the oracle's C code."""
+    fx = _fixtures()
+    for r in fx["rng"]:
+        assert oracle_mod.uniform(r["seed"], r["idx"]) == r["value"], r
+    differs = 0
+    for c in fx["saxpy"]:
+        x, y = np.array([c["x"]], np.float32), np.array([c["y"]], np.float32)
+        oracle_mod.saxpy(c["a"], x, y)
+        assert float(y[0]) == c["fused"], c
+        differs += c["fused"] != c["unfused"]
+    assert differs >= 3  # the set does tell a fused multiply-add from a*x rounded, then + y
+    k = fx["abft"]
+    tm, tn = k["tile_m"], k["tile_n"]
+    dr, dc = np.zeros(tm), np.zeros(tn)
+    f = k["fault"]
+    dr[f["row"]] -= f["delta"]  # residual = reference - observed, the fault sits in the observed sums
+    dc[f["col"]] -= f["delta"]
+    st, fix = oracle_mod.abft_decide(dr, dc, k["threshold"])
+    for name in ("flag", "row", "col", "n_bad_rows", "n_bad_cols"):
+        assert st[name] == k["expect"][name], name
+    assert fix == k["expect"]["correction"]

@@ -175,3 +175,26 @@ def test_vectors_longer_than_2_pow_31_elements(blas, oracle_mod):
             assert np.float32(g) == ys[0], i
         else:
             assert np.float32(g) == y0, i  # past n: untouched
+
+
+def test_golden_fixtures_on_the_device(blas):
+    """The device generator and SAXPY against tests/golden/fixtures.json (values from Python integers and exact
+    fractions, tests/golden/make_fixtures.py)."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fixtures.json")) as f:
+        fx = json.load(f)
+    for seed in sorted({r["seed"] for r in fx["rng"]}):
+        want = {r["idx"]: r["value"] for r in fx["rng"] if r["seed"] == seed and r["idx"] < (1 << 20)}
+        buf = torch.empty(max(want) + 1, dtype=torch.float32, device="cuda")
+        blas.fill_uniform(buf, seed)
+        got = buf.cpu().numpy()
+        for idx, value in want.items():
+            assert float(got[idx]) == value, (seed, idx)
+    cases = fx["saxpy"]
+    for a in sorted({c["a"] for c in cases}):
+        sel = [c for c in cases if c["a"] == a]
+        x = torch.tensor([c["x"] for c in sel], dtype=torch.float32, device="cuda")
+        y = torch.tensor([c["y"] for c in sel], dtype=torch.float32, device="cuda")
+        blas.saxpy(len(sel), a, x, y)
+        assert y.cpu().numpy().tolist() == [np.float32(c["fused"]) for c in sel]
