@@ -283,3 +283,36 @@ def test_data_scaled_threshold(blas, oracle_mod, ft_mode, scale_a, scale_b, shif
             assert st["flag"][fault[0]] == 1 and (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3]
             assert np.count_nonzero(st["flag"]) == 1
         _assert_values(oracle_mod, M, N, K, a, b, c0, dc.cpu().numpy(), 1.0, 0.0)
+
+
+def test_fault_campaign_with_data_scaled_threshold(blas, oracle_mod):
+    """200 seeded single faults at 2048 x 2048 x 2048 on operands that are neither unit-range nor zero-mean, with the
+    data-scaled threshold (tau = -1): every fault of at least 1e-3 of the typical |C| entry is detected, located
+    and corrected, nothing else is flagged."""
+    M = N = K = 2048
+    dev = "cuda"
+    da, db = torch.empty(M, K, device=dev), torch.empty(K, N, device=dev)
+    blas.fill_uniform_matrix(da, M, K, 30)
+    blas.fill_uniform_matrix(db, K, N, 31)
+    da.mul_(100.0).add_(25.0)
+    db.mul_(0.5).add_(0.125)
+    dc = torch.zeros(M, N, device=dev)
+    status = blas.ft_status_alloc(M, N)
+    ws = blas.workspace(blas.ft_workspace_bytes(M, N, K))
+    blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=-1.0, status=status, ws=ws)
+    clean = blas.ft_status_numpy(status)
+    assert np.count_nonzero(clean["flag"]) == 0
+    c_clean = dc.clone()
+    typical = float(c_clean.abs().mean())
+    ntiles = blas.ft_num_tiles(M, N)
+    rng = np.random.default_rng(77)
+    for launch in range(200):
+        tile = int(rng.integers(ntiles))
+        i, j = int(rng.integers(blas.FT_TILE_M)), int(rng.integers(blas.FT_TILE_N))
+        delta = float(np.float32((1 if rng.integers(2) else -1) * typical * 10.0 ** rng.uniform(-3, 1)))
+        blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=-1.0, fault=(tile, i, j, delta), status=status, ws=ws)
+        st = blas.ft_status_numpy(status)
+        assert st["flag"][tile] == 1 and (st["row"][tile], st["col"][tile]) == (i, j), (launch, tile, i, j, delta, st[tile])
+        assert np.count_nonzero(st["flag"]) == 1, launch
+        diff = (dc - c_clean).abs()
+        assert int(torch.count_nonzero(diff)) <= 1 and float(diff.max()) < 3e-4 * typical, (launch, float(diff.max()))
