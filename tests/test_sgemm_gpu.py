@@ -274,3 +274,26 @@ def test_row_split_gives_the_same_bits_as_one_launch(blas, oracle_mod):
         c_one = _sampled_check(oracle_mod, blas, n, n, n, 1.0, 1.0, nrows=6, seed=950 + n, tile=t1, split_k=1)
         assert torch.equal(c_auto, c_one), n
     assert found >= 1
+
+
+def test_seeded_random_shapes_every_path(blas, oracle_mod):
+    """Seeded random (M, N, K, leading dimensions, alpha, beta) with and without workspace, so that whatever the
+    selector picks for them (tile, split-K, tail split, row split, ragged kernels) is checked on every element."""
+    rng = np.random.default_rng(2025)
+    seen = set()
+    for case in range(48):
+        M, N = int(rng.integers(1, 1400)), int(rng.integers(1, 1400))
+        K = int(rng.choice([1, 7, 16, 100, 257, 1024, 3000, 9000]))
+        if case % 6 == 0:   # shapes with many tiles, where the splits come into play
+            M, N, K = int(rng.integers(2000, 2600)), int(rng.integers(2000, 2600)), int(rng.choice([512, 1040]))
+        lda, ldb, ldc = K + int(rng.integers(0, 9)), N + int(rng.integers(0, 9)), N + int(rng.integers(0, 9))
+        alpha = float(rng.choice([1.0, -0.5, 2.0]))
+        beta = float(rng.choice([0.0, 1.0, -1.5]))
+        use_ws = bool(case % 2)
+        need = blas.sgemm_workspace_bytes(M, N, K)
+        ws = blas.workspace(max(need, 4)) if use_ws else None
+        plan = blas.sgemm_plan(M, N, K, need if use_ws else 0)
+        rows = blas.sgemm_row_split(M, N, K, need if use_ws else 0)[0]
+        seen.add(("rows" if rows else "split" if plan[1] > 1 else "tail" if plan[1] < -1 else "plain"))
+        _check(oracle_mod, blas, M, N, K, alpha, beta, lda=lda, ldb=ldb, ldc=ldc, ws=ws, seed=3000 + case)
+    assert {"plain", "split"} <= seen, seen
