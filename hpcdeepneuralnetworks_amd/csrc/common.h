@@ -22,16 +22,16 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Compute units of the current device (256 on an MI355X); 256 when no device can be queried.
 inline int device_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            return 256;
+    constexpr int kMaxDevices = 64;
+    static int cus[kMaxDevices] = {};  // written once per device with the same value: racing threads agree
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+        cus[dev] = n;
     }
-    return cus;
+    return cus[dev];
 }
 
 // ---- counter-based RNG: splitmix64 finaliser of seed*golden + index ------

@@ -78,19 +78,26 @@ static const FtClass kFtClasses[HPCDNN_FT_NUM_CLASSES] = {
     HPCDNN_FT_CLASS(64, 2, 2, 2, 2),   // 2 wide
 };
 
-// Kernels that use more than the default 64 KiB of LDS must opt in once.
+// Kernels that use more than the default 64 KiB of LDS must opt in once per device.
 static int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {
     if (bytes <= 64 * 1024) return HPCDNN_OK;
+    struct Done {
+        const void* fn;
+        int device;
+    };
     static std::mutex mu;
-    static const void* done[8 * kNumTiles] = {};
+    static Done done[16 * kNumTiles] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
     std::lock_guard<std::mutex> lock(mu);
     const void* key = reinterpret_cast<const void*>(fn);
-    for (const void* d : done)
-        if (d == key) return HPCDNN_OK;
-    hipError_t e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+    for (const Done& d : done)
+        if (d.fn == key && d.device == dev) return HPCDNN_OK;
+    e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
     if (e != hipSuccess) return static_cast<int>(e);
-    for (const void*& d : done)
-        if (!d) { d = key; break; }
+    for (Done& d : done)
+        if (!d.fn) { d = Done{key, dev}; break; }  // a full table only costs a repeated call
     return HPCDNN_OK;
 }
 
