@@ -1,5 +1,6 @@
 // SGEMM / ABFT-SGEMM entry points: argument checks, tile + split-K choice, launch.
 #include "sgemm_kernel.h"
+#include "sgemm_small_kernel.h"
 
 #include <mutex>
 
@@ -13,12 +14,19 @@ struct TileConfig {
     void (*plain)(const GemmArgs);
     void (*edge)(const GemmArgs);
     float eff;  // fitted steady-state fraction of the FP32 MFMA peak of one CU
+    bool wave_split_k;  // small-problem kernel: the waves of a workgroup split K (other summation order, no tail split)
 };
 
 #define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, EFF)                                                          \
     {                                                                                                    \
         BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
             sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC>, EFF \
+    }
+
+#define HPCDNN_SMALL_TILE(TMB, OCC, EFF)                                                                  \
+    {                                                                                                    \
+        32 * TMB, 32, kSmallBK, kSmallThreads, OCC, small_lds_bytes<TMB>(), sgemm_small_kernel<TMB, false, OCC>, \
+            sgemm_small_kernel<TMB, true, OCC>, EFF, true                                                \
     }
 
 // The counterpart of the reference's small/medium/large/tall/wide/huge shape table
@@ -37,6 +45,9 @@ static const TileConfig kTiles[] = {
     HPCDNN_TILE(256, 256, 2, 4, 1, 1.000f),  // 8 giant, eight waves
     HPCDNN_TILE(256, 128, 4, 2, 1, 1.000f),  // 9 huge, eight waves
     HPCDNN_TILE(256, 256, 4, 2, 1, 1.000f),  // 10 giant, eight waves (4 x 2)
+    // 11 small: 32 x 32, K split between the four waves.  Every lane fetches its own operands, so the rate is set by
+    // the vector memory path, about half the matrix peak: for problems with too few 64 x 64 tiles to go round
+    HPCDNN_SMALL_TILE(1, 4, 0.50f),
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
@@ -129,7 +140,7 @@ static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int
     const bool edge = (M % t.bm) || (N % t.bn) || (K % t.bk);
     double eff = t.eff;
     const double resident = t.blocks_per_cu < n ? t.blocks_per_cu : n;
-    if (t.blocks_per_cu >= 4) eff *= 1.0 - kThinPenalty * (t.blocks_per_cu - resident) / t.blocks_per_cu;
+    if (t.blocks_per_cu >= 4 && !t.wave_split_k) eff *= 1.0 - kThinPenalty * (t.blocks_per_cu - resident) / t.blocks_per_cu;
     const double per_tile = 2.0 * t.bm * t.bn * k_slice / (kPeakFlopsPerCu * eff) * (edge ? kEdgePenalty : 1.0);
     const double fixed = kFixedBase + kFixedPer32K * t.bm * t.bn / 32768.0;
     const double exposed = t.blocks_per_cu == 1 ? n : 1.0 + kCoveredFraction * (n - 1.0);
@@ -165,7 +176,7 @@ static double tail_plan_cost(const TileConfig& t, int M, int N, int K, int cus, 
 }
 
 static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, bool allow_tail = true,
-                        double* cost_out = nullptr) {
+                        double* cost_out = nullptr, bool same_bits_only = false) {
     const int cus = device_cus();
     struct Candidate {
         Plan plan;
@@ -176,6 +187,7 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
     double best_cost = 1e300;
     for (int t = 0; t < kNumTiles; ++t) {
         const TileConfig& cfg = kTiles[t];
+        if (same_bits_only && cfg.wave_split_k) continue;
         for (int split = 1; split <= 64; split *= 2) {
             if (split > 1) {
                 if (!allow_split) break;
@@ -186,7 +198,7 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
             cand[n_cand++] = Candidate{Plan{t, split}, c};
             if (c < best_cost) best_cost = c;
         }
-        if (allow_split && allow_tail) {
+        if (allow_split && allow_tail && !cfg.wave_split_k) {
             int ways = 0;
             const double c = tail_plan_cost(cfg, M, N, K, cus, ws_bytes, &ways);
             if (ways >= 2) {
@@ -221,6 +233,7 @@ static RowSplit choose_row_split(int M, int N, int K, int cus) {
     RowSplit best{-1, 0, -1, 1e300};
     for (int t = 0; t < kNumTiles; ++t) {
         const TileConfig& cfg = kTiles[t];
+        if (cfg.wave_split_k) continue;
         const int64_t tiles_n = ceil_div(N, cfg.bn), tiles_m = ceil_div(M, cfg.bm);
         const int64_t rounds = tiles_m * tiles_n / cus;
         for (int64_t k = rounds; k >= 1 && k + 1 >= rounds; --k) {
@@ -229,7 +242,7 @@ static RowSplit choose_row_split(int M, int N, int K, int cus) {
             if (tile_rows < 1 || rows1 >= M) continue;
             const double c1 = plan_cost(cfg, static_cast<int>(rows1), N, K, 1, cus);
             double c2 = 0.0;
-            const Plan rest = choose_plan(M - static_cast<int>(rows1), N, K, false, 0, false, &c2);
+            const Plan rest = choose_plan(M - static_cast<int>(rows1), N, K, false, 0, false, &c2, true);
             const double c = c1 + c2 + kSecondLaunch;
             if (c < best.cost) best = RowSplit{t, static_cast<int>(rows1), rest.tile, c};
         }
@@ -277,6 +290,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
     if (rc != HPCDNN_OK) return rc;
     if (tile >= kNumTiles || split == -1) return HPCDNN_ERR_INVALID_VALUE;
+    if (tile >= 0 && kTiles[tile].wave_split_k && split < -1) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
 
     if (tile < 0 || split == 0) {

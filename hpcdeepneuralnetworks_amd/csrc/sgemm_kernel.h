@@ -810,8 +810,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
     const int64_t total = static_cast<int64_t>(M) * N;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
     for (int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; e < total; e += stride) {
+        // eight slices are fetched before any is added, so their latencies overlap; the additions keep slice order
         float s = ws[e];
-        for (int z = 1; z < splits; ++z) s += ws[static_cast<size_t>(z) * total + e];
+        int z = 1;
+        for (; z + 8 <= splits; z += 8) {
+            float t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = ws[static_cast<size_t>(z + u) * total + e];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += t[u];
+        }
+        for (; z < splits; ++z) s += ws[static_cast<size_t>(z) * total + e];
         const int64_t r = e / N, c = e - r * N;
         float* dst = C + r * ldc + c;
         const float t = alpha * s;
@@ -836,7 +845,15 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, 
         if (row >= M || col >= N) continue;
         const size_t off = static_cast<size_t>(r) * bn + c;
         v4f s = *reinterpret_cast<const v4f*>(src + off);
-        for (int z = 1; z < splits; ++z) s += *reinterpret_cast<const v4f*>(src + z * tile_elems + off);
+        int z = 1;
+        for (; z + 4 <= splits; z += 4) {  // four slices in flight, added in slice order
+            v4f t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t[u] = *reinterpret_cast<const v4f*>(src + (z + u) * tile_elems + off);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s += t[u];
+        }
+        for (; z < splits; ++z) s += *reinterpret_cast<const v4f*>(src + z * tile_elems + off);
         const float sv[4] = {s.x, s.y, s.z, s.w};
         float* dst = C + static_cast<size_t>(row) * ldc + col;
 #pragma unroll

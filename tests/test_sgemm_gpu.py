@@ -210,6 +210,48 @@ def test_tail_split_forced_matches_and_is_deterministic(blas, oracle_mod):
         _check(oracle_mod, blas, M, N, K, 1.0, 0.0, tile=4, split_k=-8, ws=None)
 
 
+def test_small_problem_tile_splits_k_between_its_waves(blas, oracle_mod):
+    """The 32 x 32 tile: four waves share K block-wise and meet in LDS; picked where 64 x 64 tiles cannot fill the CUs."""
+    small = [t for t, (bm, bn, _) in enumerate(blas.tile_table()) if (bm, bn) == (32, 32)]
+    assert len(small) == 1
+    tile = small[0]
+    # fewer K blocks than waves, every kind of K tail inside a lane's 16-value run, ragged M and N, NaN padding
+    for (M, N, K) in [(32, 32, 1), (32, 32, 31), (40, 50, 33), (64, 96, 64), (70, 45, 95), (33, 65, 129), (96, 32, 160),
+                      (1, 1, 17), (128, 128, 1000), (31, 200, 48)]:
+        _check(oracle_mod, blas, M, N, K, 1.0, 0.0, tile=tile, lda=K + 3, ldb=N + 5, ldc=N + 1, seed=300 + K)
+    for alpha, beta in [(1.5, -1.0), (0.0, 2.0), (-0.5, 0.0), (1.0, 1.0)]:
+        _check(oracle_mod, blas, 200, 150, 90, alpha, beta, tile=tile, lda=96, ldb=152, ldc=160)
+    # K slices through the workspace on top of the split between the waves; fixed order, same bits every run
+    M, N, K = 100, 90, 1000
+    ws = blas.workspace(M * N * 4 * 4)
+    for split in (2, 3, 4):
+        c1 = _check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=tile, split_k=split, ws=ws, ldc=N + 6)
+        c2 = _check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=tile, split_k=split, ws=ws, ldc=N + 6)
+        assert np.array_equal(c1[:, :N], c2[:, :N])
+    with pytest.raises(blas.HpcdnnError):  # no tail split for this tile
+        _check(oracle_mod, blas, M, N, K, 1.0, 0.0, tile=tile, split_k=-2, ws=ws)
+    # K = 0 scales C; exact cases: ones (any summation order), identity
+    n = 96
+    c0 = torch.rand(n, n, device="cuda")
+    c = c0.clone()
+    blas.sgemm(n, n, 0, c0[:, :0], c0[:0, :], c, 1.0, 0.5, tile=tile)
+    assert torch.equal(c, c0 * 0.5)
+    a = torch.rand(n, n, device="cuda") * 2 - 1
+    c = torch.empty(n, n, device="cuda")
+    blas.sgemm(n, n, n, a, torch.eye(n, device="cuda"), c, 1.0, 0.0, tile=tile)
+    assert torch.equal(c, a)
+    blas.sgemm(n, n, 4096, torch.ones(n, 4096, device="cuda"), torch.ones(4096, n, device="cuda"), c, 1.0, 0.0, tile=tile)
+    assert torch.all(c == 4096.0)
+    # the selector: small squares and thin deep shapes without a workspace, never the large squares
+    for shape in [(256, 256, 256), (512, 512, 512), (512, 512, 4096)]:
+        assert blas.sgemm_plan(*shape, 0)[0] == tile
+        c1 = _check(oracle_mod, blas, *shape, 1.0, 0.0)
+        c2 = _check(oracle_mod, blas, *shape, 1.0, 0.0)
+        assert np.array_equal(c1, c2)
+    for shape in [(1024, 1024, 1024), (2048, 2048, 2048), (6144, 6144, 6144)]:
+        assert blas.sgemm_plan(*shape, 0)[0] != tile
+
+
 def test_plan_is_a_function_of_the_shape_and_runs(blas, oracle_mod):
     for shape in [(3072, 3072, 3072), (5120, 5120, 1024), (4352, 4352, 4352)]:
         need = blas.sgemm_workspace_bytes(*shape)
