@@ -15,18 +15,26 @@ struct TileConfig {
     void (*edge)(const GemmArgs);
     float eff;  // fitted steady-state fraction of the FP32 MFMA peak of one CU
     bool wave_split_k;  // small-problem kernel: the waves of a workgroup split K (other summation order, no tail split)
+    int nslot;          // K steps a workgroup keeps on their way from memory (0: not modelled)
 };
 
 #define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, EFF)                                                          \
     {                                                                                                    \
         BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
-            sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC>, EFF \
+            sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC>, EFF, false, 2 \
+    }
+
+#define HPCDNN_TILE_DEEP(BM, BN, WGM, WGN, OCC, EFF, NSLOT)                                               \
+    {                                                                                                    \
+        BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
+            sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC, NSLOT>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC, NSLOT>, EFF, \
+            false, NSLOT                                                                                 \
     }
 
 #define HPCDNN_SMALL_TILE(TMB, OCC, EFF)                                                                  \
     {                                                                                                    \
         32 * TMB, 32, kSmallBK, kSmallThreads, OCC, small_lds_bytes<TMB>(), sgemm_small_kernel<TMB, false, OCC>, \
-            sgemm_small_kernel<TMB, true, OCC>, EFF, true                                                \
+            sgemm_small_kernel<TMB, true, OCC>, EFF, true, 0                                             \
     }
 
 // The counterpart of the reference's small/medium/large/tall/wide/huge shape table
@@ -48,6 +56,9 @@ static const TileConfig kTiles[] = {
     // 11 small: 32 x 32, K split between the four waves.  Every lane fetches its own operands, so the rate is set by
     // the vector memory path, about half the matrix peak: for problems with too few 64 x 64 tiles to go round
     HPCDNN_SMALL_TILE(1, 4, 0.50f),
+    // 12 medium with its loads four K steps ahead: a 64-row tile moves 64 bytes per row and K step, and with one
+    // workgroup per CU two steps in flight do not cover the trip to HBM when A is long and read once
+    HPCDNN_TILE_DEEP(64, 64, 2, 2, 4, 0.890f, 4),
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
@@ -130,6 +141,7 @@ constexpr double kFixedBase = 2.133e-6;        // prologue + epilogue of a tile:
 constexpr double kFixedPer32K = 2.31e-6;       // ... plus this per 32768 elements of tile area
 constexpr double kCoveredFraction = 0.209;     // exposed share of the fixed part behind a co-resident workgroup
 constexpr double kThinPenalty = 0.253;         // efficiency lost by a 4-per-CU tile per missing co-resident (x 1/4)
+constexpr double kStreamLatency = 0.73e-6;     // trip to HBM under load, fitted on 16384 x 64 x 4096
 constexpr double kReduceFixed = 2.5e-6;        // second launch of split-K
 constexpr double kReduceBytesPerSec = 8e12;    // partials written once and read once, C written once
 
@@ -145,6 +157,16 @@ static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int
     const double fixed = kFixedBase + kFixedPer32K * t.bm * t.bn / 32768.0;
     const double exposed = t.blocks_per_cu == 1 ? n : 1.0 + kCoveredFraction * (n - 1.0);
     double cost = n * per_tile + exposed * fixed;
+    if (t.nslot > 0) {
+        // An operand read once from HBM cannot arrive faster than the bytes in flight allow: per busy CU, resident
+        // workgroups x staged K steps x one K step of the tile's rows (A) or columns (B), per trip to memory
+        const double busy = tiles < cus ? tiles : cus;
+        const double steps_in_flight = busy * resident * t.nslot;
+        const double stream_a = static_cast<double>(M) * K * kStreamLatency / (steps_in_flight * t.bm * t.bk);
+        const double stream_b = static_cast<double>(N) * K * kStreamLatency / (steps_in_flight * t.bn * t.bk);
+        const double stream = (stream_a > stream_b ? stream_a : stream_b) + fixed;
+        if (stream > cost) cost = stream;
+    }
     if (split > 1) cost += kReduceFixed + (2.0 * split + 1.0) * M * static_cast<double>(N) * 4.0 / kReduceBytesPerSec;
     return cost;
 }
@@ -187,7 +209,7 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
     double best_cost = 1e300;
     for (int t = 0; t < kNumTiles; ++t) {
         const TileConfig& cfg = kTiles[t];
-        if (same_bits_only && cfg.wave_split_k) continue;
+        if (cfg.eff <= 0.f || (same_bits_only && cfg.wave_split_k)) continue;
         for (int split = 1; split <= 64; split *= 2) {
             if (split > 1) {
                 if (!allow_split) break;
@@ -233,7 +255,7 @@ static RowSplit choose_row_split(int M, int N, int K, int cus) {
     RowSplit best{-1, 0, -1, 1e300};
     for (int t = 0; t < kNumTiles; ++t) {
         const TileConfig& cfg = kTiles[t];
-        if (cfg.wave_split_k) continue;
+        if (cfg.eff <= 0.f || cfg.wave_split_k) continue;
         const int64_t tiles_n = ceil_div(N, cfg.bn), tiles_m = ceil_div(M, cfg.bm);
         const int64_t rounds = tiles_m * tiles_n / cus;
         for (int64_t k = rounds; k >= 1 && k + 1 >= rounds; --k) {

@@ -116,9 +116,14 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
 
 // FT: 0 = plain SGEMM; 1 = ABFT, checksum vectors e^T A and B e formed inside the main loop; 2 = ABFT, checksum
 // vectors read from a workspace filled by abft_encode_kernel (fewer VALU instructions in the main loop).
-template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS>
+//
+// NSLOT: staging register sets.  K step t + 1 waits in one of them while steps up to t + NSLOT are on their way from
+// memory.  Two are enough while a K step takes longer than a trip to memory (big tiles) or the operands come from
+// L2; a small tile that streams an operand from HBM with one workgroup per CU needs its loads further ahead.
+template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS, int NSLOT = 2>
 __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
+    static_assert(NSLOT == 2 || (FT == 0 && NSLOT % 2 == 0), "the ABFT loop is written for two staging sets");
     constexpr int kGemmThreads = WGM * WGN * kWave;
     static_assert(WGM * WGN == 4 || WGM * WGN == 8, "four or eight waves per workgroup");
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -189,12 +194,14 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         b_nvalid[s] = p.N - (n0 + nc);  // columns of this group inside the matrix (may be <= 0 or >= 4)
     }
 
-    v4f ra[2][A_SLOTS], rb[2][B_SLOTS];  // two staging slots: K steps t+1 and t+2 are in flight while t is multiplied
+    v4f ra[NSLOT][A_SLOTS], rb[NSLOT][B_SLOTS];  // staging sets: K steps t+1 .. t+NSLOT are in flight while t is multiplied
     int k_loaded = kbeg;                 // absolute k of the K step the next load call fetches
 
     // One staging load (part P of the K step at a_base/b_base) into slot S.  Nothing here touches the loaded
     // value, so the load stays in flight until the slot is consumed a K step later.
-    int k_slot[2] = {kbeg, kbeg};  // absolute k of the K step held by each staging slot
+    int k_slot[NSLOT];  // absolute k of the K step held by each staging slot
+#pragma unroll
+    for (int i = 0; i < NSLOT; ++i) k_slot[i] = kbeg;
     // FT == 2: the K step's slice of the pre-encoded checksum vectors travels with it (same run-ahead, same
     // slots).  The rows of enc_a / enc_b end with two K steps of zeros, so the fetches that run ahead past the
     // end need no bounds: one descriptor per row, a per-thread offset, and a scalar offset that moves on by one
@@ -514,9 +521,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     //                (+ consume the checksum partials of step kt+1)
     // Work past the end of the slice (kt+1, kt+2 >= nkt) moves duplicate data that is never multiplied, which
     // keeps the loop free of branches (and lets the loads stay two steps ahead).
-    auto step = [&](auto sl_next, auto sl_free, auto flush, auto masked) {
-        // steps alternate between (next = slot 1, LDS stage 0) and (next = slot 0, LDS stage 1)
-        constexpr int st = (decltype(sl_next)::value == 1) ? 0 : 1;
+    auto step_in = [&](auto sl_next, auto sl_free, auto stage, auto flush, auto masked) {
+        constexpr int st = decltype(stage)::value;
         constexpr int NMASK = (EDGE && decltype(masked)::value) ? (FT ? NGL : A_SLOTS) : 0;
         constexpr int NS0 = NRD + NMASK + NPROD + 2 * NGL;
         constexpr int NS1 = NRD + NCONS;
@@ -562,6 +568,17 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         });
     };
 
+    // with two staging sets steps alternate between (next = slot 1, LDS stage 0) and (next = slot 0, LDS stage 1)
+    auto step = [&](auto sl_next, auto sl_free, auto flush, auto masked) {
+        step_in(sl_next, sl_free, std::integral_constant<int, (decltype(sl_next)::value == 1) ? 0 : 1>{}, flush, masked);
+    };
+    // step number kt with kt % NSLOT == phase: its successor waits in slot (phase + 1) % NSLOT, slot phase is free
+    auto step_at = [&](auto phase, auto masked) {
+        constexpr int Ph = decltype(phase)::value;
+        step_in(std::integral_constant<int, (Ph + 1) % NSLOT>{}, std::integral_constant<int, Ph % NSLOT>{},
+                std::integral_constant<int, Ph % 2>{}, std::false_type{}, masked);
+    };
+
     if (nkt > 0) {
         // prologue: step 0 -> LDS stage 0, step 1 -> staging slot 1, first-half fragments of step 0 -> buffer 0
         static_for<NGL>([&](auto s) { gload1(S0{}, s); });
@@ -571,25 +588,41 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         static_for<NPROD>([&](auto e) { produce1(S0{}, e, 0); });
         static_for<NGL>([&](auto s) { gload1(S1{}, s); });
         gload_advance();
+        static_for<NSLOT - 2>([&](auto extra) {  // steps 2 .. NSLOT-1 -> their slots
+            static_for<NGL>([&](auto s) { gload1(std::integral_constant<int, decltype(extra)::value + 2>{}, s); });
+            gload_advance();
+        });
         __syncthreads();
         static_for<NCONS>([&](auto e) { consume1(S0{}, e, 0, std::true_type{}); });
         static_for<NRD>([&](auto s) { fread1(S0{}, s, 0, 0); });
         int kt = 0;
-        if constexpr (EDGE && FT == 0) {
-            // plain SGEMM on a ragged tile: only the last K step can be partial, and step kt consumes the staged
-            // data of step kt+1, so every step before kt = nkt-2 runs without the masks
-            for (; kt + 3 < nkt; kt += 2) {
-                step(S1{}, S0{}, std::false_type{}, std::false_type{});
-                step(S0{}, S1{}, std::false_type{}, std::false_type{});
+        if constexpr (NSLOT > 2) {
+            // whole groups of NSLOT steps; on a ragged tile only the slice's last K step can be partial, and it is
+            // step nkt - 2 that moves it to LDS, so the steps before that one run without the masks
+            const int bulk_end = EDGE ? nkt - 2 : nkt;
+            for (; kt + NSLOT <= bulk_end; kt += NSLOT)
+                static_for<NSLOT>([&](auto ph) { step_at(ph, std::false_type{}); });
+            // what is left (fewer than a group, plus the two last steps of a ragged tile), one step at a time
+            static_for<NSLOT + (EDGE ? 1 : -1)>([&](auto i) {
+                if (kt + decltype(i)::value < nkt) step_at(std::integral_constant<int, decltype(i)::value % NSLOT>{}, std::true_type{});
+            });
+        } else {
+            if constexpr (EDGE && FT == 0) {
+                // plain SGEMM on a ragged tile: only the last K step can be partial, and step kt consumes the staged
+                // data of step kt+1, so every step before kt = nkt-2 runs without the masks
+                for (; kt + 3 < nkt; kt += 2) {
+                    step(S1{}, S0{}, std::false_type{}, std::false_type{});
+                    step(S0{}, S1{}, std::false_type{}, std::false_type{});
+                }
             }
+            for (; kt + 1 < nkt; kt += 2) {
+                step(S1{}, S0{}, std::false_type{}, std::true_type{});
+                flush_now = ((kt & 14) == 14) || (kt + 2 >= nkt);
+                step(S0{}, S1{}, std::true_type{}, std::true_type{});
+            }
+            flush_now = true;
+            if (kt < nkt) step(S1{}, S0{}, std::true_type{}, std::true_type{});
         }
-        for (; kt + 1 < nkt; kt += 2) {
-            step(S1{}, S0{}, std::false_type{}, std::true_type{});
-            flush_now = ((kt & 14) == 14) || (kt + 2 >= nkt);
-            step(S0{}, S1{}, std::true_type{}, std::true_type{});
-        }
-        flush_now = true;
-        if (kt < nkt) step(S1{}, S0{}, std::true_type{}, std::true_type{});
         __syncthreads();  // every wave is done with the staging buffers (the verification below reuses them)
     }
 

@@ -252,6 +252,28 @@ def test_small_problem_tile_splits_k_between_its_waves(blas, oracle_mod):
         assert blas.sgemm_plan(*shape, 0)[0] != tile
 
 
+def test_deep_prefetch_tile_every_k_remainder(blas, oracle_mod):
+    """The 64 x 64 tile that keeps four K steps in flight: its loop runs in groups of four steps plus a remainder."""
+    table = blas.tile_table()
+    tiles = [t for t, shape in enumerate(table) if shape[:2] == (64, 64)]
+    assert len(tiles) == 2
+    deep = tiles[1]
+    for steps in range(1, 12):
+        for extra in (0, 5):
+            K = 16 * steps + extra
+            _check(oracle_mod, blas, 128, 64, K, 1.0, 0.0, tile=deep, seed=400 + K)                       # full tiles
+            _check(oracle_mod, blas, 100, 70, K, 1.5, -1.0, tile=deep, lda=K + 3, ldb=75, ldc=72, seed=500 + K)  # ragged
+    # same summation order as the other large tiles: same bits as the two-slot 64 x 64 tile
+    a = _check(oracle_mod, blas, 192, 128, 1000, 1.0, 0.0, tile=tiles[0])
+    b = _check(oracle_mod, blas, 192, 128, 1000, 1.0, 0.0, tile=deep)
+    assert np.array_equal(a, b)
+    ws = blas.workspace(192 * 128 * 4 * 4)
+    _check(oracle_mod, blas, 192, 128, 1000, 1.0, 1.0, tile=deep, split_k=3, ws=ws)
+    # picked for a long operand that is read once with one workgroup per CU
+    assert blas.sgemm_plan(16384, 64, 4096, 0)[0] == deep
+    _sampled_check(oracle_mod, blas, 16384, 64, 4096, 1.0, 0.0, nrows=16)
+
+
 def test_plan_is_a_function_of_the_shape_and_runs(blas, oracle_mod):
     for shape in [(3072, 3072, 3072), (5120, 5120, 1024), (4352, 4352, 4352)]:
         need = blas.sgemm_workspace_bytes(*shape)
