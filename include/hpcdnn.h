@@ -96,8 +96,11 @@ int hpcdnn_sgemm(int M, int N, int K, const float* A, int lda, const float* B, i
  * as hpcdnn_sgemm does; `split_k` >= 1 forces that many K slices (needs a
  * workspace of M*N*split_k floats when > 1), 0 = pick; `split_k` = -s (s >= 2)
  * splits only the tiles left over after the last full round of CUs, s ways
- * (workspace: leftover tiles * s * tile size floats, 16-byte aligned).  Either
- * way the slices are added in a fixed order. */
+ * (workspace: leftover tiles * s * tile size floats, 16-byte aligned; not
+ * available for the 32 x 32 tile).  Either way the slices are added in a fixed
+ * order.  All tiles but the 32 x 32 one add the products of an element in the
+ * same order and give the same bits; in the 32 x 32 tile the four waves of a
+ * workgroup split K between them. */
 int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                     float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split_k, void* stream);
 
