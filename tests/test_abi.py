@@ -134,3 +134,35 @@ def test_plan_query_without_a_gpu(L):
     assert plan(3072, 3072, 3072, 1 << 30)[1] <= -2              # 3072^3: a partial last round, tail split
     assert plan(4096, 4096, 4096, 1 << 30)[1] == 1               # 4096^3: whole rounds, nothing to split
     assert L.hpcdnn_sgemm_plan(-1, 1, 1, 0, None, None) == 1
+
+
+def test_plans_fit_their_workspace_for_random_shapes(L):
+    """Host arithmetic only: whatever workspace is offered, the plan is valid and never needs more than it was given."""
+    import random
+    rnd = random.Random(5)
+    n_tiles = L.hpcdnn_sgemm_num_tiles()
+    dims = [1, 7, 31, 32, 33, 64, 100, 128, 255, 256, 500, 768, 1000, 1024, 1536, 2048, 3001, 4096, 6144, 16384]
+    for _ in range(300):
+        M, N = rnd.choice(dims), rnd.choice(dims)
+        K = rnd.choice(dims + [65536])
+        need = L.hpcdnn_workspace_bytes(0, M, N, K)
+        for ws in (0, need // 3, need, need + 4096):
+            t, s = C.c_int(-1), C.c_int(0)
+            assert L.hpcdnn_sgemm_plan(M, N, K, ws, C.byref(t), C.byref(s)) == 0
+            assert 0 <= t.value < n_tiles and s.value not in (0, -1)
+            bm, bn, bk = C.c_int(), C.c_int(), C.c_int()
+            assert L.hpcdnn_sgemm_tile_info(t.value, C.byref(bm), C.byref(bn), C.byref(bk)) == 0
+            tiles = -(-M // bm.value) * -(-N // bn.value)
+            if s.value > 1:
+                assert M * N * s.value * 4 <= ws and K // s.value >= 8 * bk.value
+            elif s.value < -1:
+                assert 0 < tiles % 256 and (tiles % 256) * (-s.value) * bm.value * bn.value * 4 <= ws
+            else:
+                assert s.value == 1
+            rows, t1, t2 = C.c_int(-1), C.c_int(-2), C.c_int(-2)
+            assert L.hpcdnn_sgemm_row_split(M, N, K, ws, C.byref(rows), C.byref(t1), C.byref(t2)) == 0
+            if rows.value:
+                assert 0 < rows.value < M and 0 <= t1.value < n_tiles and 0 <= t2.value < n_tiles
+                assert L.hpcdnn_sgemm_tile_info(t1.value, C.byref(bm), None, None) == 0 and rows.value % bm.value == 0
+            else:
+                assert (t1.value, t2.value) == (-1, -1)
