@@ -98,6 +98,11 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* base, i
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, static_cast<int>(clipped), 0x00020000);
 }
 
+// Descriptor without an end, for accesses known to stay inside the allocation.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc_unbounded(const float* base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, -1, 0x00020000);
+}
+
 __device__ __forceinline__ v4f buffer_load_v4f(__amdgpu_buffer_rsrc_t rsrc, int byte_offset) {
     typedef unsigned v4u __attribute__((ext_vector_type(4)));
     const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0);

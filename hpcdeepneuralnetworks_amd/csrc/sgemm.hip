@@ -58,7 +58,7 @@ static const TileConfig kTiles[] = {
     HPCDNN_SMALL_TILE(1, 4, 0.50f),
     // 12 medium with its loads four K steps ahead: a 64-row tile moves 64 bytes per row and K step, and with one
     // workgroup per CU two steps in flight do not cover the trip to HBM when A is long and read once
-    HPCDNN_TILE_DEEP(64, 64, 2, 2, 4, 0.890f, 4),
+    HPCDNN_TILE_DEEP(64, 64, 2, 2, 4, 0.905f, 4),
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
@@ -140,7 +140,7 @@ constexpr double kEdgePenalty = 1.03;          // ragged tiles: partly empty til
 constexpr double kFixedBase = 2.133e-6;        // prologue + epilogue of a tile: base ...
 constexpr double kFixedPer32K = 2.31e-6;       // ... plus this per 32768 elements of tile area
 constexpr double kCoveredFraction = 0.209;     // exposed share of the fixed part behind a co-resident workgroup
-constexpr double kThinPenalty = 0.253;         // efficiency lost by a 4-per-CU tile per missing co-resident (x 1/4)
+constexpr double kThinPenalty = 0.18;          // efficiency lost by a 4-per-CU tile per missing co-resident (x 1/4)
 constexpr double kStreamLatency = 0.73e-6;     // trip to HBM under load, fitted on 16384 x 64 x 4096
 constexpr double kReduceFixed = 2.5e-6;        // second launch of split-K
 constexpr double kReduceBytesPerSec = 8e12;    // partials written once and read once, C written once
@@ -153,7 +153,9 @@ static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int
     double eff = t.eff;
     const double resident = t.blocks_per_cu < n ? t.blocks_per_cu : n;
     if (t.blocks_per_cu >= 4 && !t.wave_split_k) eff *= 1.0 - kThinPenalty * (t.blocks_per_cu - resident) / t.blocks_per_cu;
-    const double per_tile = 2.0 * t.bm * t.bn * k_slice / (kPeakFlopsPerCu * eff) * (edge ? kEdgePenalty : 1.0);
+    // (the ragged-tile variant of a deep-staging kernel runs more masked steps at the end of the slice)
+    const double edge_cost = edge ? kEdgePenalty * (t.nslot > 2 ? 1.06 : 1.0) : 1.0;
+    const double per_tile = 2.0 * t.bm * t.bn * k_slice / (kPeakFlopsPerCu * eff) * edge_cost;
     const double fixed = kFixedBase + kFixedPer32K * t.bm * t.bn / 32768.0;
     const double exposed = t.blocks_per_cu == 1 ? n : 1.0 + kCoveredFraction * (n - 1.0);
     double cost = n * per_tile + exposed * fixed;
@@ -232,12 +234,23 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
     // Among plans the model cannot tell apart (within 1 %), take the one that moves the least data: no split
     // before a split, then the larger tile (A and B are re-read once per tile column / tile row).
     Plan best{0, 1};
-    double best_key = -1.0;
+    bool have = false;
+    double best_area = 0.0, best_c = 0.0;
     for (int i = 0; i < n_cand; ++i) {
         if (cand[i].cost > best_cost * 1.01) continue;
         const TileConfig& cfg = kTiles[cand[i].plan.tile];
-        const double key = (cand[i].plan.split == 1 ? 1e12 : 0.0) + static_cast<double>(cfg.bm) * cfg.bn - cand[i].cost;
-        if (key > best_key) { best_key = key; best = cand[i].plan; if (cost_out) *cost_out = cand[i].cost; }
+        const double area = static_cast<double>(cfg.bm) * cfg.bn;
+        const bool unsplit = cand[i].plan.split == 1, best_unsplit = best.split == 1;
+        const bool better = !have || (unsplit != best_unsplit ? unsplit
+                                      : area != best_area     ? area > best_area
+                                                              : cand[i].cost < best_c);
+        if (better) {
+            have = true;
+            best = cand[i].plan;
+            best_area = area;
+            best_c = cand[i].cost;
+            if (cost_out) *cost_out = cand[i].cost;
+        }
     }
     return best;
 }

@@ -139,6 +139,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int NGL = A_SLOTS + B_SLOTS;  // global loads (and LDS writes) per thread per K step
     constexpr int NRD = TM + TN;            // fragment read groups per half K step
     constexpr int NMG = 4 * TM * TN;        // MFMAs per half K step (8 k values)
+    constexpr bool kShortStep = FT == 0 && NMG <= 8;  // one or two 32x32 blocks per wave: little to hide latencies behind
+    constexpr bool kNoBounds = kShortStep && !EDGE;
 
     extern __shared__ __align__(16) float smem[];
     float* const As = smem;
@@ -220,8 +222,13 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     auto gload1 = [&](auto slot, auto part) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P == 0) k_slot[S] = k_loaded;
-        if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc(a_base, a_left), a_voff[P]);
-        else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[P - A_SLOTS]);
+        if constexpr (kNoBounds) {
+            if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc_unbounded(a_base), a_voff[P]);
+            else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc_unbounded(b_base), b_voff[P - A_SLOTS]);
+        } else {
+            if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc(a_base, a_left), a_voff[P]);
+            else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[P - A_SLOTS]);
+        }
         if constexpr (FT == 2 && P == NGL - 1) {
             static_assert(FT != 2 || B_SLOTS <= 2, "a thread stages one or two k rows of B");
             if constexpr (B_SLOTS == 2) {
@@ -272,6 +279,20 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         b_left = more ? b_left - b_step * 4 : 0;
         k_loaded += more ? BK : 0;
         if constexpr (FT == 2) enc_off += BK * 4;
+    };
+    // The same in two parts, so that the short-step schedule can place them apart.  Its full tiles keep no bounds at
+    // all: nothing they fetch lies outside the matrix, and past the end of the slice they fetch its last K step
+    // again instead of zeros.
+    auto gload_advance_a = [&]() {
+        const bool more = k_loaded + BK < kend;
+        a_base += more ? BK : 0;
+        if constexpr (!kNoBounds) a_left = more ? a_left - BK * 4 : 0;
+    };
+    auto gload_advance_b = [&]() {
+        const bool more = k_loaded + BK < kend;
+        b_base += more ? b_step : 0;
+        if constexpr (!kNoBounds) b_left = more ? b_left - b_step * 4 : 0;
+        k_loaded += more ? BK : 0;
     };
     auto lstore1 = [&](auto slot, auto part, int stage) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
@@ -526,6 +547,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         constexpr int NMASK = (EDGE && decltype(masked)::value) ? (FT ? NGL : A_SLOTS) : 0;
         constexpr int NS0 = NRD + NMASK + NPROD + 2 * NGL;
         constexpr int NS1 = NRD + NCONS;
+        // A wave with few MFMAs per half step (one or two 32x32 blocks) has little to hide latencies behind: its
+        // second half reads the next step's fragments right behind the first MFMA (the next step starts with them),
+        // and the scalar arithmetic that moves the descriptors on goes behind the second one instead of joining
+        // the loads and LDS writes of the first half (a wave alone on its SIMD pays for clumps of scalar work).
         static_for<NMG>([&](auto m) {
             constexpr int Mi = decltype(m)::value;
             mfma1(S0{}, m);
@@ -545,7 +570,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     produce1(sl_next, std::integral_constant<int, o - NRD - NMASK>{}, st ^ 1);
                 } else if constexpr (o < NRD + NMASK + NPROD + NGL) {
                     gload1(sl_free, std::integral_constant<int, o - NRD - NMASK - NPROD>{});
-                    if constexpr (o == NRD + NMASK + NPROD + NGL - 1) gload_advance();
+                    if constexpr (o == NRD + NMASK + NPROD + NGL - 1 && !kShortStep) gload_advance();
                 } else {
                     lstore1(sl_next, std::integral_constant<int, o - NRD - NMASK - NPROD - NGL>{}, st ^ 1);
                 }
@@ -557,13 +582,19 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         static_for<NMG>([&](auto m) {
             constexpr int Mi = decltype(m)::value;
             mfma1(S1{}, m);
-            constexpr int k_lo = (Mi * NS1 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS1 + NMG - 1) / NMG;
-            static_for<k_hi - k_lo>([&](auto d) {
-                constexpr int o = k_lo + decltype(d)::value;
-                // fragment reads first (the next step's first MFMAs wait for them), then the checksum pieces
-                if constexpr (o < NRD) fread1(S0{}, std::integral_constant<int, o>{}, st ^ 1, 0);
-                else consume1(sl_next, std::integral_constant<int, o - NRD>{}, st ^ 1, flush);
-            });
+            if constexpr (kShortStep) {
+                if constexpr (Mi == 0) static_for<NRD>([&](auto o) { fread1(S0{}, o, st ^ 1, 0); });
+                if constexpr (Mi == 1) gload_advance_a();
+                if constexpr (Mi == 2) gload_advance_b();
+            } else {
+                constexpr int k_lo = (Mi * NS1 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS1 + NMG - 1) / NMG;
+                static_for<k_hi - k_lo>([&](auto d) {
+                    constexpr int o = k_lo + decltype(d)::value;
+                    // fragment reads first (the next step's first MFMAs wait for them), then the checksum pieces
+                    if constexpr (o < NRD) fread1(S0{}, std::integral_constant<int, o>{}, st ^ 1, 0);
+                    else consume1(sl_next, std::integral_constant<int, o - NRD>{}, st ^ 1, flush);
+                });
+            }
             __builtin_amdgcn_sched_barrier(0);
         });
     };
