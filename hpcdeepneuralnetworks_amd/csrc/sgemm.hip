@@ -57,7 +57,8 @@ static const TileConfig kTiles[] = {
     // the vector memory path, about half the matrix peak: for problems with too few 64 x 64 tiles to go round
     HPCDNN_SMALL_TILE(1, 4, 0.50f),
     // 12 medium with its loads four K steps ahead: a 64-row tile moves 64 bytes per row and K step, and with one
-    // workgroup per CU two steps in flight do not cover the trip to HBM when A is long and read once
+    // workgroup per CU two steps in flight do not cover the trip to HBM when A is long and read once.  Staged data
+    // is so old when it is needed that the LDS writes lead the step and are done long before the barrier.
     HPCDNN_TILE_DEEP(64, 64, 2, 2, 4, 0.905f, 4),
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
@@ -134,13 +135,14 @@ struct Plan {
 // workgroups share them), plus the part of each tile's prologue and epilogue that nothing overlaps: all of it when
 // one workgroup owns the CU, a fraction of it (after the first) when co-resident workgroups cover for each other.
 // The epilogue grows with the tile's area (C is written at the CU's share of HBM bandwidth).  A four-per-CU tile
-// running with fewer co-residents loses efficiency: one wave per SIMD cannot hide its own barriers.
+// with two staging sets running with fewer co-residents loses efficiency: one wave per SIMD cannot hide its own
+// waits (the deep-staging variant writes LDS early enough not to have them).
 constexpr double kPeakFlopsPerCu = 157.3e12 / 256.0;
 constexpr double kEdgePenalty = 1.03;          // ragged tiles: partly empty tiles are paid in full by tile counting; this is the rest
 constexpr double kFixedBase = 2.133e-6;        // prologue + epilogue of a tile: base ...
 constexpr double kFixedPer32K = 2.31e-6;       // ... plus this per 32768 elements of tile area
 constexpr double kCoveredFraction = 0.209;     // exposed share of the fixed part behind a co-resident workgroup
-constexpr double kThinPenalty = 0.18;          // efficiency lost by a 4-per-CU tile per missing co-resident (x 1/4)
+constexpr double kThinPenalty = 0.12;          // efficiency lost by a small tile when all co-residents are missing
 constexpr double kStreamLatency = 0.73e-6;     // trip to HBM under load, fitted on 16384 x 64 x 4096
 constexpr double kReduceFixed = 2.5e-6;        // second launch of split-K
 constexpr double kReduceBytesPerSec = 8e12;    // partials written once and read once, C written once
@@ -152,7 +154,8 @@ static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int
     const bool edge = (M % t.bm) || (N % t.bn) || (K % t.bk);
     double eff = t.eff;
     const double resident = t.blocks_per_cu < n ? t.blocks_per_cu : n;
-    if (t.blocks_per_cu >= 4 && !t.wave_split_k) eff *= 1.0 - kThinPenalty * (t.blocks_per_cu - resident) / t.blocks_per_cu;
+    // tiles whose waves own one or two 32x32 blocks (two staging sets): alone on a SIMD a wave cannot hide its waits
+    if (t.bm * t.bn <= 128 * 64 && t.nslot == 2) eff *= 1.0 - kThinPenalty * (t.blocks_per_cu - resident) / t.blocks_per_cu;
     // (the ragged-tile variant of a deep-staging kernel runs more masked steps at the end of the slice)
     const double edge_cost = edge ? kEdgePenalty * (t.nslot > 2 ? 1.06 : 1.0) : 1.0;
     const double per_tile = 2.0 * t.bm * t.bn * k_slice / (kPeakFlopsPerCu * eff) * edge_cost;

@@ -141,6 +141,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int NMG = 4 * TM * TN;        // MFMAs per half K step (8 k values)
     constexpr bool kShortStep = FT == 0 && NMG <= 8;  // one or two 32x32 blocks per wave: little to hide latencies behind
     constexpr bool kNoBounds = kShortStep && !EDGE;
+    constexpr bool kEarlyStore = kShortStep && NSLOT > 2;
 
     extern __shared__ __align__(16) float smem[];
     float* const As = smem;
@@ -562,7 +563,14 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 // order: fragment reads (needed soonest); ragged-tile masks and checksum pieces of step kt+1 (its
                 // staged data arrived a step ago; the cross-lane chain must be finished well before the barrier);
                 // global loads of step kt+2; LDS writes of step kt+1
-                if constexpr (o < NRD) {
+                if constexpr (kEarlyStore) {
+                    // deep staging: the data of step kt+1 arrived steps ago, so its LDS writes go first and are
+                    // complete long before the barrier; the loads of the step furthest ahead follow
+                    if constexpr (o < NRD) fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
+                    else if constexpr (o < NRD + NMASK) gmask1(sl_next, std::integral_constant<int, o - NRD>{});
+                    else if constexpr (o < NRD + NMASK + NGL) lstore1(sl_next, std::integral_constant<int, o - NRD - NMASK>{}, st ^ 1);
+                    else gload1(sl_free, std::integral_constant<int, o - NRD - NMASK - NGL>{});
+                } else if constexpr (o < NRD) {
                     fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
                 } else if constexpr (o < NRD + NMASK) {
                     gmask1(sl_next, std::integral_constant<int, o - NRD>{});
