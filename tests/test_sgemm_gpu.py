@@ -361,3 +361,43 @@ def test_seeded_random_shapes_every_path(blas, oracle_mod):
         seen.add(("rows" if rows else "split" if plan[1] > 1 else "tail" if plan[1] < -1 else "plain"))
         _check(oracle_mod, blas, M, N, K, alpha, beta, lda=lda, ldb=ldb, ldc=ldc, ws=ws, seed=3000 + case)
     assert {"plain", "split"} <= seen, seen
+
+
+def test_host_threads_on_their_own_streams(blas, oracle_mod):
+    """Four host threads, each on its own stream with its own shapes and workspace: the library keeps no state that
+    they could trample (the plan memo is per thread), so every result has the bits of the serial run."""
+    import threading
+    shapes = [(512, 512, 512), (1024, 1024, 1024), (700, 900, 300), (128, 128, 8192), (2048, 2048, 512), (1536, 1536, 1536)]
+    ops = {}
+    for i, (M, N, K) in enumerate(shapes):
+        a = torch.empty(M, K, device="cuda"); b = torch.empty(K, N, device="cuda")
+        blas.fill_uniform_matrix(a, M, K, 900 + i); blas.fill_uniform_matrix(b, K, N, 950 + i)
+        ws = blas.workspace(max(blas.sgemm_workspace_bytes(M, N, K), 16))
+        ref = torch.empty(M, N, device="cuda")
+        blas.sgemm(M, N, K, a, b, ref, 1.0, 0.0, ws=ws)
+        ops[(M, N, K)] = (a, b, ref)
+    torch.cuda.synchronize()
+    errors = []
+
+    def work(tid):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for rep in range(6):
+                    M, N, K = shapes[(tid + rep) % len(shapes)]
+                    a, b, ref = ops[(M, N, K)]
+                    ws = blas.workspace(max(blas.sgemm_workspace_bytes(M, N, K), 16))   # own scratch: slices would race
+                    c = torch.empty(M, N, device="cuda")
+                    blas.sgemm(M, N, K, a, b, c, 1.0, 0.0, ws=ws)
+                    stream.synchronize()
+                    if not torch.equal(c, ref):
+                        errors.append((tid, rep, M, N, K))
+        except Exception as e:  # surfaced below: an assert in a thread would be lost
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
