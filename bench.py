@@ -37,7 +37,7 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline SGEMM line only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--ft-launches", type=int, default=1000, help="launches of the ABFT fault campaign")
-    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "ft_sgemm", "saxpy", "sdot", "copy", "sgemv_n", "sgemv_t"],
+    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "sgemm_1024", "ft_sgemm", "saxpy", "sdot", "copy", "sgemv_n", "sgemv_t"],
                     help="run one kernel only for --steps launches (for profiling with rocprofv3) and print a short line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -80,7 +80,13 @@ def main() -> int:
 
     if args.kernel not in ("all", "sgemm"):
         # single-kernel mode for the profiler: same shapes as the full run
-        if args.kernel == "ft_sgemm":
+        if args.kernel == "sgemm_1024":
+            # the reference's CPU-checkable configuration: M=N=K=1024, alpha=1, beta=0
+            m = 1024
+            a, b, c = operands(m, m, m, 10)
+            fn = lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0)
+            work, unit = 2.0 * m ** 3, "GFLOP/s"
+        elif args.kernel == "ft_sgemm":
             m = 4096
             a, b, c = operands(m, m, m, 20)
             status = blas.ft_status_alloc(m, m)
