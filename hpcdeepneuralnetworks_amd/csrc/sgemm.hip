@@ -335,7 +335,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         // The decision is a function of the shape and of what the workspace allows; callers tend to repeat shapes,
         // so each thread remembers its last one instead of re-evaluating the cost model on every call.
         struct Decision {
-            int M, N, K;
+            int M, N, K, cus;
             size_t ws_bytes;
             bool ws_aligned, valid;
             Plan plan;
@@ -345,15 +345,17 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         // the tail split moves 16-byte groups through the workspace
         const bool ws_aligned = (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
         const size_t usable = ws ? ws_bytes : 0;
-        if (!(memo.valid && memo.M == M && memo.N == N && memo.K == K && memo.ws_bytes == usable && memo.ws_aligned == ws_aligned)) {
+        const int cus = device_cus();  // of the current device: the plan depends on it
+        if (!(memo.valid && memo.M == M && memo.N == N && memo.K == K && memo.cus == cus && memo.ws_bytes == usable &&
+              memo.ws_aligned == ws_aligned)) {
             double cost = 0.0;
             memo.plan = choose_plan(M, N, K, ws != nullptr, usable, ws_aligned, &cost);
             memo.rows = RowSplit{-1, 0, -1, 1e300};
             if (K > 0) {
-                const RowSplit rs = choose_row_split(M, N, K, device_cus());
+                const RowSplit rs = choose_row_split(M, N, K, cus);
                 if (rs.tile1 >= 0 && rs.cost < 0.97 * cost) memo.rows = rs;
             }
-            memo.M = M; memo.N = N; memo.K = K;
+            memo.M = M; memo.N = N; memo.K = K; memo.cus = cus;
             memo.ws_bytes = usable;
             memo.ws_aligned = ws_aligned;
             memo.valid = true;
