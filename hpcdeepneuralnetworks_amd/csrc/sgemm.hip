@@ -60,6 +60,7 @@ static const TileConfig kTiles[] = {
     // workgroup per CU two steps in flight do not cover the trip to HBM when A is long and read once.  Staged data
     // is so old when it is needed that the LDS writes lead the step and are done long before the barrier.
     HPCDNN_TILE_DEEP(64, 64, 2, 2, 4, 0.905f, 4),
+    HPCDNN_TILE(192, 192, 2, 2, 1, 0.943f),  // 13 3072-friendly: 16 x 16 tiles = one full round of 256 CUs
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
