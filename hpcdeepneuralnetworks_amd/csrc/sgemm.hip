@@ -539,10 +539,11 @@ extern "C" int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, 
     cfg.bn = fc.bn;
     cfg.bk = kGemmBK;
     GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
-    // tau > 0: absolute; tau == 0: the absolute default for unit-range data; tau < 0: scaled to the data, a line's
-    // threshold being -tau * 4.3 FP32 rounding units * sqrt(K) * sum |acc| / sqrt(elements of the line)
+    // tau > 0: absolute; tau == 0: the absolute default for unit-range data; tau < 0: scaled to the data, the
+    // threshold of a line of n elements being -tau * 4.3 FP32 rounding units * sqrt(max(K, 64)) * sqrt(n) * the larger
+    // of the line's and the tile's mean |accumulator|
     a.tau = (tau > 0.f) ? tau : (tau == 0.f ? hpcdnn_ft_default_tau(K) : 0.f);
-    a.tau_rel = (tau < 0.f) ? -tau * 2.56e-7f * sqrtf(static_cast<float>(K > 1 ? K : 1)) : 0.f;
+    a.tau_rel = (tau < 0.f) ? -tau * 2.56e-7f * sqrtf(static_cast<float>(K > 64 ? K : 64)) : 0.f;
     a.status = status;
     if (inject) {
         if (inject->tile < 0 || inject->tile >= a.tiles_m * a.tiles_n || inject->row < 0 || inject->row >= fc.bm ||

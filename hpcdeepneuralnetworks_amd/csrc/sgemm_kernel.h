@@ -676,8 +676,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         float* const s_crabs = s_ccabs + WGM * BN;                      // [WGN][BM] row sums of |accumulators|
         float* const s_dr = s_crabs + WGN * BM;                         // [BM] row residuals, then [BN] column residuals
         int* const s_meta = reinterpret_cast<int*>(s_dr + BM + BN);     // nbr, nbc, bad row, bad col, max clean (float bits)
+        float* const s_tsum = reinterpret_cast<float*>(s_meta + 8);     // [waves] partial sums of |acc| over the tile
         static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads>() >=
-                          sizeof(double) * (CCP * BN + CRP * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + BM + BN) + 32,
+                          sizeof(double) * (CCP * BN + CRP * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + BM + BN) + 32 +
+                              sizeof(float) * (kGemmThreads / kWave),
                       "verification scratch fits in the staging buffers");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
 
@@ -756,11 +758,29 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         __syncthreads();
 
         // residual = reference - observed per line; |d| > tau marks the line (ft_sgemm_huge.cuh:200-271).  Relative
-        // mode: tau of a line = tau_rel * sum |acc| / sqrt(n), n = elements of the line inside the matrix (rounding
-        // noise of a sum of n accumulators grows like sqrt(n) times their magnitude).
+        // mode: tau of a line of n elements inside the matrix = tau_rel * sqrt(n) * max(mean |acc| of the line, mean
+        // |acc| of the tile): the rounding noise of a sum of n accumulators grows like sqrt(n) times their magnitude,
+        // and the tile mean stands in for a short or cancelling line whose own accumulators say little about the
+        // size of its terms.  The tile sum is formed in a fixed order (per wave, then wave by wave).
         const int rows_in = (p.M - m0 < BM) ? p.M - m0 : BM, cols_in = (p.N - n0 < BN) ? p.N - n0 : BN;
         const float row_scale = p.tau_rel / __builtin_sqrtf(static_cast<float>(cols_in));
         const float col_scale = p.tau_rel / __builtin_sqrtf(static_cast<float>(rows_in));
+        float row_floor = 0.f, col_floor = 0.f;
+        if (relative) {
+            float part = 0.f;
+            for (int r = tid; r < BM; r += kGemmThreads)
+#pragma unroll
+                for (int w = 0; w < WGN; ++w) part += s_crabs[w * BM + r];
+            part = wave_sum_lane63(part);
+            if (lane == kWave - 1) s_tsum[wave] = part;
+            __syncthreads();
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < kGemmThreads / kWave; ++w) total += s_tsum[w];
+            const float mean = total / (static_cast<float>(rows_in) * static_cast<float>(cols_in));
+            row_floor = p.tau_rel * __builtin_sqrtf(static_cast<float>(cols_in)) * mean;
+            col_floor = p.tau_rel * __builtin_sqrtf(static_cast<float>(rows_in)) * mean;
+        }
         for (int line = tid; line < BM + BN; line += kGemmThreads) {
             const bool is_row = line < BM;
             const int idx = is_row ? line : line - BM;
@@ -781,7 +801,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
                 for (int w = 0; w < WGM; ++w) mag += s_ccabs[w * BN + idx];
             }
-            const double tau = relative ? static_cast<double>(mag * (is_row ? row_scale : col_scale)) : static_cast<double>(p.tau);
+            const float own = mag * (is_row ? row_scale : col_scale), floor = is_row ? row_floor : col_floor;
+            const double tau = relative ? static_cast<double>(own > floor ? own : floor) : static_cast<double>(p.tau);
             const double d = ref - obs;
             if (fabs(d) > tau) {
                 atomicAdd(&s_meta[is_row ? 0 : 1], 1);

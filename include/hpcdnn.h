@@ -126,10 +126,11 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * per tile is located (faulty row x faulty column) and corrected before
  * alpha/beta are applied.  `tau` > 0 is an absolute residual threshold, 0
  * selects the default for inputs of magnitude <= 1 (hpcdnn_ft_default_tau),
- * and `tau` < 0 scales the threshold to the data: a line is flagged when its
- * residual exceeds -tau * 2.56e-7 * sqrt(K) * (sum of |accumulators| over the
- * line) / sqrt(elements of the line), -1 being calibrated to twice the
- * largest fault-free residual of uniform operands; `inject` is a HOST
+ * and `tau` < 0 scales the threshold to the data: a line of n elements is
+ * flagged when its residual exceeds -tau * 2.56e-7 * sqrt(max(K, 64)) *
+ * sqrt(n) * m, m being the larger of the mean |accumulator| of the line and
+ * of the whole tile, -1 being calibrated to twice the largest fault-free
+ * residual of uniform operands; `inject` is a HOST
  * pointer to one fault or NULL; `status` is DEVICE memory for
  * hpcdnn_ft_num_tiles(M,N) records or NULL.
  * `ws`/`ws_bytes`: optional DEVICE scratch of
@@ -160,7 +161,7 @@ int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, const float
 int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
 int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N);
 int hpcdnn_ft_pick_class(int M, int N, int K);
-/* Threshold hpcdnn_ft_sgemm uses when tau <= 0: 1.1e-6 * max(K, 64), twice the
+/* Threshold hpcdnn_ft_sgemm uses when tau == 0: 1.1e-6 * max(K, 64), twice the
  * largest fault-free residual measured for operands uniform in [-1, 1] (the
  * rounding noise of the FP32 accumulators grows linearly with K).  Scale it by
  * max|A| * max|B| for other data. */

@@ -297,14 +297,18 @@ float oracle_abft_decide(int tm, int tn, const double* dr, const double* dc, flo
     return fix;
 }
 
-/* Data-scaled thresholds (no reference counterpart; the reference's thresholds are constants): a line's threshold
- * is rel * sum |acc| over the line / sqrt(elements in the line), with rel = factor * 2.56e-7 * sqrt(K) (4.3 units of
- * FP32 rounding per sqrt(K)): the rounding noise of a sum of n accumulators grows like sqrt(n) times their
- * magnitude, and that of one accumulator like sqrt(K) times the rounding unit. */
+/* Data-scaled thresholds (no reference counterpart; the reference's thresholds are constants): a line of n
+ * accumulators gets rel * sqrt(n) * max(mean |acc| over the line, mean |acc| over the tile), with
+ * rel = factor * 2.56e-7 * sqrt(max(K, 64)) (4.3 units of FP32 rounding per sqrt(K)): the rounding noise of a sum of n
+ * accumulators grows like sqrt(n) times their magnitude, and that of one accumulator like sqrt(K) times the rounding
+ * unit.  The tile mean keeps a short or cancelling line (whose own |acc| says little about the size of its terms)
+ * from getting a threshold below its noise; the floor on K covers the rounding of the sums themselves, which does
+ * not shrink with K. */
 void oracle_abft_relative_thresholds(int tm, int tn, int K, const float* acc, int ldacc, float factor,
                                      double* tau_r, double* tau_c) {
-    float rel = factor * 2.56e-7f * sqrtf((float)K);
+    float rel = factor * 2.56e-7f * sqrtf((float)(K > 64 ? K : 64));
     float rs = rel / sqrtf((float)tn), cs = rel / sqrtf((float)tm);
+    double total = 0.0;
     for (int n = 0; n < tn; ++n) tau_c[n] = 0.0;
     for (int m = 0; m < tm; ++m) {
         double s = 0.0;
@@ -313,9 +317,19 @@ void oracle_abft_relative_thresholds(int tm, int tn, int K, const float* acc, in
             s += v;
             tau_c[n] += v;
         }
-        tau_r[m] = (double)((float)s * rs);
+        tau_r[m] = s;
+        total += s;
     }
-    for (int n = 0; n < tn; ++n) tau_c[n] = (double)((float)tau_c[n] * cs);
+    float mean = (float)total / ((float)tm * (float)tn);
+    float row_floor = rel * sqrtf((float)tn) * mean, col_floor = rel * sqrtf((float)tm) * mean;
+    for (int m = 0; m < tm; ++m) {
+        float t = (float)tau_r[m] * rs;
+        tau_r[m] = (double)(t > row_floor ? t : row_floor);
+    }
+    for (int n = 0; n < tn; ++n) {
+        float t = (float)tau_c[n] * cs;
+        tau_c[n] = (double)(t > col_floor ? t : col_floor);
+    }
 }
 
 /* Whole-matrix model: C = alpha*acc + beta*C with acc = A*B accumulated in

@@ -297,9 +297,10 @@ def test_offline_ft_model_closed_form(oracle_mod, alpha, beta, panel):
 
 
 def test_relative_thresholds_closed_forms_and_scaling(oracle_mod):
-    """Constant tile: every row holds tn copies of |c|, so its threshold is rel * |c| * sqrt(tn) (and sqrt(tm) for
-    columns) with rel = 2.56e-7 * sqrt(K); a single non-zero entry only raises its own row and column; thresholds
-    are linear in the data, in the factor, and grow like sqrt(K)."""
+    """Constant tile: line mean = tile mean = |c|, so a row's threshold is rel * |c| * sqrt(tn) (sqrt(tm) for columns)
+    with rel = 2.56e-7 * sqrt(max(K, 64)); a single non-zero entry raises its own row and column above the floor the
+    tile mean gives every line; thresholds are linear in the data and in the factor, grow like sqrt(K) from K = 64 up
+    and stay put below."""
     tm, tn, K = 48, 20, 400
     rel = 2.56e-7 * np.sqrt(K)
     tr, tc = oracle_mod.abft_relative_thresholds(np.full((tm, tn), -3.0, np.float32), K)
@@ -307,14 +308,30 @@ def test_relative_thresholds_closed_forms_and_scaling(oracle_mod):
     one = np.zeros((tm, tn), np.float32)
     one[5, 7] = 2.0
     tr, tc = oracle_mod.abft_relative_thresholds(one, K)
-    assert np.count_nonzero(tr) == 1 and np.count_nonzero(tc) == 1
+    tile_mean = 2.0 / (tm * tn)
     assert np.isclose(tr[5], rel * 2.0 / np.sqrt(tn), rtol=1e-6) and np.isclose(tc[7], rel * 2.0 / np.sqrt(tm), rtol=1e-6)
+    others_r, others_c = np.delete(tr, 5), np.delete(tc, 7)
+    assert np.allclose(others_r, rel * np.sqrt(tn) * tile_mean, rtol=1e-6) and np.allclose(others_c, rel * np.sqrt(tm) * tile_mean, rtol=1e-6)
+    assert tr[5] > 10 * others_r[0] and tc[7] > 10 * others_c[0]
     rng = np.random.default_rng(3)
     acc = rng.standard_normal((tm, tn)).astype(np.float32)
     tr1, tc1 = oracle_mod.abft_relative_thresholds(acc, K)
     tr2, tc2 = oracle_mod.abft_relative_thresholds(acc * np.float32(8.0), 4 * K, factor=0.5)
     assert np.allclose(tr2, tr1 * 8.0 * 2.0 * 0.5, rtol=1e-6) and np.allclose(tc2, tc1 * 8.0, rtol=1e-6)
-    assert np.allclose(tr1, rel * np.abs(acc.astype(np.float64)).sum(axis=1) / np.sqrt(tn), rtol=1e-5)
+    a64 = np.abs(acc.astype(np.float64))
+    want = rel * np.sqrt(tn) * np.maximum(a64.mean(axis=1), a64.mean())
+    assert np.allclose(tr1, want, rtol=1e-5)
+    assert np.any(a64.mean(axis=1) < a64.mean()) and np.any(a64.mean(axis=1) > a64.mean())  # both branches are exercised
+    # below K = 64 the rounding of the sums themselves dominates: the threshold stops shrinking
+    t1, _ = oracle_mod.abft_relative_thresholds(acc, 1)
+    t64, _ = oracle_mod.abft_relative_thresholds(acc, 64)
+    t256, _ = oracle_mod.abft_relative_thresholds(acc, 256)
+    assert np.array_equal(t1, t64) and np.allclose(t256, 2.0 * t64, rtol=1e-6)
+    # a one-element line that cancels to nearly nothing still gets the tile's scale
+    thin = np.full((tm, 1), 1.0, np.float32)
+    thin[3, 0] = 1e-6
+    tr, _ = oracle_mod.abft_relative_thresholds(thin, K)
+    assert np.isclose(tr[3], rel * (47.0 + 1e-6) / 48.0, rtol=1e-5) and np.isclose(tr[0], rel * 1.0, rtol=1e-6)
 
 
 def _fixtures():
