@@ -316,3 +316,36 @@ def test_fault_campaign_with_data_scaled_threshold(blas, oracle_mod):
         assert np.count_nonzero(st["flag"]) == 1, launch
         diff = (dc - c_clean).abs()
         assert int(torch.count_nonzero(diff)) <= 1 and float(diff.max()) < 3e-4 * typical, (launch, float(diff.max()))
+
+
+@pytest.mark.parametrize("M,N,K,tile_class", [(512, 129, 256, 1), (600, 1, 250, 0), (512, 384, 1, 0), (200, 129, 15, 2),
+                                              (129, 127, 1, 1), (64, 129, 7, 1), (257, 300, 16, 2), (1, 512, 7, 2)])
+def test_data_scaled_threshold_on_thin_edge_tiles_and_short_k(blas, oracle_mod, ft_mode, M, N, K, tile_class):
+    """One-column edge tiles and K below 64 (found by a randomized sweep against the CPU model): a line's own
+    |accumulators| can cancel to far less than its terms, and the rounding of the sums does not shrink with K; the
+    tile-wide mean and the floor on K keep fault-free lines below the threshold, and a fault is still located."""
+    bm, bn = blas.ft_tile(tile_class)
+    ntn = -(-N // bn)
+    for trial, with_fault in enumerate([False, False, True]):
+        a = oracle_mod.fill_uniform_matrix(M, K, 1600 + trial, ld=K + 1)
+        b = oracle_mod.fill_uniform_matrix(K, N, 1700 + trial, ld=N + 3)
+        c0 = oracle_mod.fill_uniform_matrix(M, N, 1800 + trial, ld=N)
+        fault = None
+        if with_fault:
+            tile = blas.ft_num_tiles(M, N, tile_class) - 1          # the last tile: clipped in both directions
+            tm, tn = M - (tile // ntn) * bm, N - (tile % ntn) * bn
+            fault = (tile, tm - 1, tn - 1, -3.25)
+        da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+        status = blas.ft_status_alloc(M, N, tile_class=tile_class)
+        blas.ft_sgemm(M, N, K, da, db, dc, 1.0, -0.75, tau=-1.0, fault=fault, status=status, ws=_ws(blas, ft_mode, M, N, K),
+                      tile_class=tile_class)
+        st = blas.ft_status_numpy(status)
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm(M, N, K, a, K + 1, b, N + 3, c_model, N, 1.0, -0.75, bm, bn, -1.0, fault)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (fault, f, st[f], st_model[f])
+        if fault is None:
+            assert np.all(st["flag"] == 0)
+        else:
+            assert st["flag"][fault[0]] == 1 and (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3]
+            assert np.sum(st["flag"] != 0) == 1
