@@ -401,3 +401,27 @@ def test_host_threads_on_their_own_streams(blas, oracle_mod):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+def test_maximum_leading_dimensions(blas):
+    """lda and ldb at the documented limits (32-bit byte offsets inside one tile), for every kernel family; one more
+    is refused."""
+    lda, ldb = (1 << 21) - 64, (1 << 25) - 1024
+    M, N, K = 300, 100, 40
+    abuf = torch.empty(M * lda, device="cuda")
+    bbuf = torch.empty(K * ldb + 8, device="cuda")
+    a, b = abuf.view(M, lda)[:, :K], bbuf[:K * ldb].view(K, ldb)[:, :N]
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    a.copy_(torch.rand(M, K, device="cuda", generator=gen) * 2 - 1)
+    b.copy_(torch.rand(K, N, device="cuda", generator=gen) * 2 - 1)
+    ref = a.double() @ b.double()
+    den = a.abs().double() @ b.abs().double()
+    small = [t for t, shape in enumerate(blas.tile_table()) if shape[:2] == (32, 32)][0]
+    for tile in (-1, 0, 4, 8, small, len(blas.tile_table()) - 1):
+        c = torch.zeros(M, N, device="cuda")
+        blas.sgemm(M, N, K, a, b, c, 1.0, 0.0, tile=tile, split_k=0 if tile < 0 else 1)
+        assert float(((c.double() - ref).abs() / den).max()) <= TOL, tile
+    with pytest.raises(blas.HpcdnnError):
+        blas.sgemm(M, N, K, a, bbuf[:(K - 1) * (ldb + 1) + N].as_strided((K, N), (ldb + 1, 1)), torch.zeros(M, N, device="cuda"), 1.0, 0.0)
+    with pytest.raises(blas.HpcdnnError):
+        blas.sgemm(8, N, K, abuf[:7 * (lda + 1) + K].as_strided((8, K), (lda + 1, 1)), b, torch.zeros(8, N, device="cuda"), 1.0, 0.0)
