@@ -349,3 +349,46 @@ def test_data_scaled_threshold_on_thin_edge_tiles_and_short_k(blas, oracle_mod, 
         else:
             assert st["flag"][fault[0]] == 1 and (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3]
             assert np.sum(st["flag"] != 0) == 1
+
+
+def test_seeded_random_cases_equal_the_model(blas, oracle_mod):
+    """Random shapes, leading dimensions, alpha/beta, tile classes, both encode modes, absolute and data-scaled
+    thresholds, with and without a fault: decisions equal the CPU model's, the fault is located, C is right."""
+    import random
+    rnd = random.Random(11)
+    dims = [1, 5, 31, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 300, 384, 400, 512, 600]
+    kd = [1, 7, 15, 16, 17, 33, 64, 100, 128, 250, 256, 400, 512, 1000]
+    for case in range(80):
+        M, N, K = rnd.choice(dims), rnd.choice(dims), rnd.choice(kd)
+        lda, ldb, ldc = K + rnd.choice([0, 0, 1, 4]), N + rnd.choice([0, 0, 3, 4]), N + rnd.choice([0, 0, 8])
+        alpha, beta = rnd.choice([1.0, 1.0, -1.5, 0.5]), rnd.choice([0.0, 1.0, -0.75])
+        cls, mode = rnd.choice([0, 1, 2]), rnd.choice(["fused", "workspace"])
+        tau = -1.0 if rnd.random() < 0.4 else blas.ft_default_tau(K)
+        bm, bn = blas.ft_tile(cls)
+        ntm, ntn = -(-M // bm), -(-N // bn)
+        fault = None
+        if rnd.random() < 0.7:
+            tile = rnd.randrange(ntm * ntn)
+            tm, tn = min(bm, M - (tile // ntn) * bm), min(bn, N - (tile % ntn) * bn)
+            fault = (tile, rnd.randrange(tm), rnd.randrange(tn), float(np.float32(rnd.choice([-1, 1]) * 10.0 ** rnd.uniform(-1.3, 1.5))))
+        what = (case, M, N, K, lda, ldb, ldc, alpha, beta, cls, mode, tau, fault)
+        a = oracle_mod.fill_uniform_matrix(M, K, 5000 + case, ld=lda)
+        b = oracle_mod.fill_uniform_matrix(K, N, 6000 + case, ld=ldb)
+        c0 = oracle_mod.fill_uniform_matrix(M, N, 7000 + case, ld=ldc)
+        da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+        status = blas.ft_status_alloc(M, N, tile_class=cls)
+        blas.ft_sgemm(M, N, K, da, db, dc, alpha, beta, tau=tau, fault=fault, status=status, ws=_ws(blas, mode, M, N, K),
+                      tile_class=cls)
+        st = blas.ft_status_numpy(status)
+        c = dc.cpu().numpy()
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm(M, N, K, a, lda, b, ldb, c_model, ldc, alpha, beta, bm, bn, tau, fault)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (what, f, st[f], st_model[f])
+        assert np.all(np.isnan(c[:, N:])), what
+        caught = fault is not None and st_model["flag"][fault[0]] == 1
+        if caught:
+            assert (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3], what
+        if (fault is None or caught) and K >= 16:   # a sub-threshold fault stays in C; K < 16: |A||B| is too small a yardstick for the corrected element
+            ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, lda, b, ldb, c0, ldc, alpha, beta)
+            assert oracle_mod.gemm_max_err(N, c, ldc, ref, den) <= TOL, what
