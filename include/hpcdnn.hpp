@@ -9,6 +9,7 @@
 #pragma once
 
 #include <chrono>
+#include <cmath>
 
 #include "hpcdnn.h"
 
@@ -34,6 +35,23 @@ inline int sdot(int N, const float* x, const float* y, float* out, void* ws, siz
 }
 inline void cpu_gemm(float alpha, float beta, const float* mat1, const float* mat2, int n, float* mat3) {
     hpcdnn_cpu_gemm(alpha, beta, mat1, mat2, n, mat3);
+}
+
+// The reference's acceptance checks on host arrays (utils/utils.cu:60-91): square n x n matrices agree when every
+// element differs by at most 1e-2; vectors agree when every element is within 5e-3 relative.  (The reference
+// divides by the signed first argument, so its vector check never fails on negative values; the magnitude is used
+// here.)  Silent: the reference also prints the first offending element.
+inline bool verify_matrix(const float* mat1, const float* mat2, int n) {
+    for (long i = 0; i < static_cast<long>(n) * n; ++i)
+        if (!(std::fabs(static_cast<double>(mat1[i]) - static_cast<double>(mat2[i])) <= 1e-2)) return false;
+    return true;
+}
+inline bool verify_vector(const float* vec1, const float* vec2, int n) {
+    for (int i = 0; i < n; ++i) {
+        const double diff = std::fabs(static_cast<double>(vec1[i]) - static_cast<double>(vec2[i]));
+        if (!(diff <= 5e-3 * std::fabs(static_cast<double>(vec1[i])))) return false;
+    }
+    return true;
 }
 
 // utils/utils.cuh:53 and :56-77

@@ -166,3 +166,52 @@ def test_plans_fit_their_workspace_for_random_shapes(L):
                 assert L.hpcdnn_sgemm_tile_info(t1.value, C.byref(bm), None, None) == 0 and rows.value % bm.value == 0
             else:
                 assert (t1.value, t2.value) == (-1, -1)
+
+
+def test_cpp_header_helpers_compile_and_behave(tmp_path):
+    """include/hpcdnn.hpp: the reference's host helpers (verify_matrix, verify_vector, cpu_gemm, CEIL_DIV, the timer;
+    utils/utils.cu:60-103, utils.cuh:53-77) compile with a plain C++ compiler against the library and do what the
+    reference's do."""
+    import os
+    import shutil
+    import subprocess
+    if shutil.which("g++") is None:
+        pytest.skip("no host C++ compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    libdir = os.path.join(root, "hpcdeepneuralnetworks_amd", "lib")
+    src = tmp_path / "t.cpp"
+    src.write_text(r"""
+#include <cstdio>
+#include <vector>
+#include "hpcdnn.hpp"
+int main() {
+    const int n = 8;
+    std::vector<float> a(n * n), b(n * n, 0.f), c(n * n, 1.f), c2;
+    for (int i = 0; i < n * n; ++i) a[i] = 0.25f * (i % 7) - 0.5f;
+    for (int i = 0; i < n; ++i) b[i * n + i] = 1.f;                    // identity
+    hpcdnn::cpu_gemm(2.f, 3.f, a.data(), b.data(), n, c.data());       // c = 2 a + 3
+    for (int i = 0; i < n * n; ++i) if (c[i] != 2.f * a[i] + 3.f) return 1;
+    c2 = c;
+    if (!hpcdnn::verify_matrix(c.data(), c2.data(), n)) return 2;
+    c2[5] += 0.009f;
+    if (!hpcdnn::verify_matrix(c.data(), c2.data(), n)) return 3;       // within the absolute 1e-2
+    c2[5] += 0.002f;
+    if (hpcdnn::verify_matrix(c.data(), c2.data(), n)) return 4;        // beyond it
+    std::vector<float> v = {1.f, -2.f, 100.f}, w = {1.004f, -2.009f, 100.4f};
+    if (!hpcdnn::verify_vector(v.data(), w.data(), 3)) return 5;         // all within 5e-3 relative
+    w[1] = -2.02f;
+    if (hpcdnn::verify_vector(v.data(), w.data(), 3)) return 6;          // 1 % off on a negative element
+    if (hpcdnn::ceil_div(10, 4) != 3 || hpcdnn::ceil_div(8, 4) != 2) return 7;
+    hpcdnn::timer t;
+    if (t.elapsed() < 0.0 || t.elapsed_msec(true) < 0.0) return 8;
+    std::printf("%s\n", hpcdnn_version());
+    return 0;
+}
+""")
+    exe = tmp_path / "t"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-I", os.path.join(root, "include"), str(src), "-o", str(exe),
+                    "-L", libdir, "-lhpcdnn", "-L/opt/rocm/lib", "-lamdhip64", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib"],
+                   check=True, capture_output=True, timeout=120)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, (out.returncode, out.stderr)
+    assert out.stdout.startswith("hpcdnn")
