@@ -291,6 +291,21 @@ def main() -> int:
         }
         del a, b, c
 
+        # ---- ABFT overhead across the square sweep (workspace variant, the tile class the library suggests)
+        sweep = {}
+        for m in (2048, 3072, 5120, 6144):
+            a, b, c = operands(m, m, m, 26)
+            cls = blas.ft_pick_class(m, m, m)
+            status_s = blas.ft_status_alloc(m, m, tile_class=cls)
+            ft_ws_s = blas.workspace(blas.ft_workspace_bytes(m, m, m))
+            ms_plain = median_timed(lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0), 10, 5, batches=3)
+            ms_ft = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, status=status_s, ws=ft_ws_s, tile_class=cls), 10, 5, batches=3)
+            sweep[str(m)] = {"tile_class": cls, "sgemm_gflops": round(2.0 * m ** 3 / ms_plain / 1e6, 1),
+                             "ft_sgemm_gflops": round(2.0 * m ** 3 / ms_ft / 1e6, 1),
+                             "overhead_pct_vs_sgemm": round((ms_ft - ms_plain) / ms_plain * 100.0, 2)}
+            del a, b, c
+        extras["abft_square_sweep"] = sweep
+
         # ---- SAXPY / SDOT at n = 2^28 (12 and 8 algorithmic bytes per element)
         nv = 1 << 28
         x = torch.empty(nv, device=dev)
