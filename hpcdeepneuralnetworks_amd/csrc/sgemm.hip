@@ -496,17 +496,49 @@ extern "C" int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N) {
 
 extern "C" int hpcdnn_ft_num_tiles(int M, int N) { return hpcdnn_ft_num_tiles_ex(0, M, N); }
 
-// The class with the shortest predicted run: rounds of tiles over the CUs times the tile height (all classes are
-// 128 columns wide), with the measured efficiency of the smaller tiles relative to the 256-row one.
+// ABFT with a workspace splits the tiles of a partial last round of CUs along K, like plain SGEMM's tail split: every
+// slice is a workgroup that verifies (and corrects) its own partial product - the checksums are linear in K - and
+// writes it raw; tail_reduce_kernel adds the slices, ft_tail_status_kernel merges their records.  With fewer tiles
+// than half the CUs every tile is split.  Returns the number of ways (1: no split) and the tiles it applies to.
+struct FtTail {
+    int ways, tiles;
+};
+static FtTail ft_tail_plan(const FtClass& fc, int M, int N, int K) {
+    const int cus = device_cus();
+    const int64_t tiles = ceil_div(M, fc.bm) * ceil_div(N, fc.bn);
+    const int64_t r = tiles % cus;
+    if (r == 0 || 2 * r > cus) return FtTail{1, 0};
+    int64_t s = cus / r;
+    const int64_t most = K / (16 * kGemmBK);  // at least 16 K steps per slice: each slice pays a verification
+    if (s > most) s = most;
+    if (s > 8) s = 8;
+    if (s < 2) return FtTail{1, 0};
+    return FtTail{static_cast<int>(s), static_cast<int>(r)};
+}
+static size_t ft_enc_bytes(const FtClass& fc, int M, int N, int K) {
+    const size_t b = static_cast<size_t>(ceil_div(M, fc.bm) + ceil_div(N, fc.bn)) * ft_enc_ld(K) * sizeof(float);
+    return (b + 15) & ~static_cast<size_t>(15);
+}
+static size_t ft_tail_bytes(const FtClass& fc, const FtTail& t) {
+    return t.ways < 2 ? 0
+                      : static_cast<size_t>(t.tiles) * t.ways * (static_cast<size_t>(fc.bm) * fc.bn * sizeof(float) + sizeof(hpcdnn_ft_status));
+}
+
+// The class with the shortest predicted run (workspace variant): rounds of tiles over the CUs times the tile height
+// (all classes are 128 columns wide), a partial last round counting for what its K split leaves of it plus the
+// second pass over those tiles, with the measured efficiency of the smaller tiles relative to the 256-row one.
 extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
-    (void)K;
     static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 0.97, 0.90};
     const int cus = device_cus();
     int best = 0;
     double best_cost = 1e300;
     for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
         const int64_t tiles = hpcdnn_ft_num_tiles_ex(c, M, N);
-        const double cost = static_cast<double>(ceil_div(tiles > 0 ? tiles : 1, cus)) * kFtClasses[c].bm / rel_eff[c];
+        const FtTail tail = ft_tail_plan(kFtClasses[c], M, N, K);
+        double rounds = static_cast<double>(ceil_div(tiles > 0 ? tiles : 1, cus));
+        if (tail.ways >= 2)
+            rounds = static_cast<double>(tiles / cus) + static_cast<double>(ceil_div(static_cast<int64_t>(tail.tiles) * tail.ways, cus)) / tail.ways + 0.06;
+        const double cost = rounds * kFtClasses[c].bm / rel_eff[c];
         if (cost < best_cost) { best_cost = cost; best = c; }
     }
     return best;
@@ -523,7 +555,7 @@ extern "C" float hpcdnn_ft_default_tau(int K) {
 static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     const FtClass& fc = kFtClasses[tile_class];
-    return static_cast<size_t>(ceil_div(M, fc.bm) + ceil_div(N, fc.bn)) * ft_enc_ld(K) * sizeof(float);
+    return ft_enc_bytes(fc, M, N, K) + ft_tail_bytes(fc, ft_tail_plan(fc, M, N, K));
 }
 
 extern "C" int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
@@ -560,8 +592,11 @@ extern "C" int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, 
     // With a workspace the checksum vectors of A and B are formed once per tile row / tile column by a small
     // bandwidth-bound kernel and the main loop only reads them; without one every workgroup forms them itself.
     if (ws && K > 0) {
-        if (ws_bytes < ft_class_workspace_bytes(tile_class, M, N, K) || (reinterpret_cast<uintptr_t>(ws) & 15u))
-            return HPCDNN_ERR_WORKSPACE;
+        const size_t enc_bytes = ft_enc_bytes(fc, M, N, K);
+        if (ws_bytes < enc_bytes || (reinterpret_cast<uintptr_t>(ws) & 15u)) return HPCDNN_ERR_WORKSPACE;
+        // the K split of a partial last round is taken when the workspace has room for it
+        FtTail tail = ft_tail_plan(fc, M, N, K);
+        if (ws_bytes < enc_bytes + ft_tail_bytes(fc, tail)) tail = FtTail{1, 0};
         a.enc_ld = ft_enc_ld(K);
         float* enc_a = static_cast<float*>(ws);
         float* enc_b = enc_a + static_cast<size_t>(a.tiles_m) * a.enc_ld;
@@ -575,7 +610,29 @@ extern "C" int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, 
         void (*fn)(const GemmArgs) = edge ? fc.pre_edge : fc.pre_plain;
         rc = enable_lds(fn, fc.lds_pre);
         if (rc != HPCDNN_OK) return rc;
+        const int tiles = a.tiles_m * a.tiles_n;
+        a.full_tiles = tiles;
+        a.tail_split = 1;
+        if (tail.ways >= 2) {
+            a.tail_k_chunk = static_cast<int>(ceil_div(ceil_div(K, tail.ways), kGemmBK)) * kGemmBK;
+            tail.ways = static_cast<int>(ceil_div(K, a.tail_k_chunk));  // drop empty slices
+        }
+        if (tail.ways >= 2) {
+            a.full_tiles = tiles - tail.tiles;
+            a.tail_split = tail.ways;
+            a.tail_partial = reinterpret_cast<float*>(static_cast<char*>(ws) + enc_bytes);
+            a.tail_status = reinterpret_cast<hpcdnn_ft_status*>(a.tail_partial + static_cast<size_t>(tail.tiles) * tail.ways * fc.bm * fc.bn);
+            grid = dim3(a.full_tiles + tail.tiles * tail.ways, 1, 1);
+        }
         hipLaunchKernelGGL(fn, grid, dim3(fc.threads_pre), fc.lds_pre, s, a);
+        rc = launch_status();
+        if (rc != HPCDNN_OK || a.tail_split < 2) return rc;
+        tail_reduce_kernel<<<dim3(tail.tiles, fc.bm / 32), 256, 0, s>>>(M, N, fc.bm, fc.bn, a.tiles_m, a.tiles_n, a.full_tiles,
+                                                                       a.tail_split, a.tail_partial, C, ldc, alpha, beta);
+        rc = launch_status();
+        if (rc != HPCDNN_OK || !status) return rc;
+        ft_tail_status_kernel<<<static_cast<int>(ceil_div(tail.tiles, 64)), 64, 0, s>>>(tail.tiles, a.tail_split, a.tiles_m, a.tiles_n,
+                                                                                      a.full_tiles, a.tail_status, status);
         return launch_status();
     }
     void (*fn)(const GemmArgs) = edge ? fc.fused_edge : fc.fused_plain;

@@ -58,6 +58,7 @@ struct GemmArgs {
     // ways along K (tail_k_chunk per slice) and write raw accumulators to tail_partial[tile - full_tiles][slice][BM*BN]
     int full_tiles, tail_split, tail_k_chunk;
     float* tail_partial;
+    hpcdnn_ft_status* tail_status;  // ABFT with a tail split: one record per slice, [tile - full_tiles][slice]
     // ABFT
     float tau;      // absolute residual threshold; 0 = relative mode
     float tau_rel;  // relative mode: threshold of a line = tau_rel * sum |accumulators of the line| / sqrt(elements in it)
@@ -155,8 +156,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     int tile_m, tile_n;
     int tile_id = blockIdx.x, k_slice = blockIdx.z, k_chunk = p.k_chunk;
     float* tail_out = nullptr;
-    if (FT == 0 && p.tail_split > 1 && tile_id >= p.full_tiles) {
+    int tail_slot = 0;  // index of this slice among all tail slices
+    if (FT != 1 && p.tail_split > 1 && tile_id >= p.full_tiles) {
         const int r = tile_id - p.full_tiles;
+        tail_slot = r;
         tile_id = p.full_tiles + r / p.tail_split;
         k_slice = r % p.tail_split;
         k_chunk = p.tail_k_chunk;
@@ -700,7 +703,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 
         // Soft-error injection: one accumulator, after the K loop, before the checks
         // (run-time form of `t[2].x += error_inject`, ft_sgemm_huge.cuh:40,145).
-        if (tile_linear == p.fault_tile) add_at(p.fault_row, p.fault_col, p.fault_delta);
+        // (a tile split along K verifies every slice on its own - the checksums are linear in K; the test fault goes
+        // into its first slice)
+        if (tile_linear == p.fault_tile && k_slice == 0) add_at(p.fault_row, p.fault_col, p.fault_delta);
 
         if (tid == 0) { s_meta[0] = 0; s_meta[1] = 0; s_meta[2] = -1; s_meta[3] = -1; s_meta[4] = 0; }
 
@@ -834,7 +839,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             st.row_residual = (flag == 1) ? s_dr[bad_r] : 0.f;
             st.col_residual = (flag == 1) ? s_dr[BM + bad_c] : 0.f;
             st.max_clean_residual = __int_as_float(s_meta[4]);
-            p.status[tile_linear] = st;
+            if (tail_out) p.tail_status[tail_slot] = st;
+            else p.status[tile_linear] = st;
         }
     }
 
@@ -842,7 +848,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int row_base = m0 + wm * WM + lh * 4;  // + i*32 + 8*(v/4) + v%4
     const int col_base = n0 + wn * WN + lr;      // + j*32
 
-    if (FT == 0 && tail_out) {
+    if (FT != 1 && tail_out) {
         // whole tile, no bounds: rows and columns past the matrix hold zeros (their operands read as zeros)
         float* out = tail_out + (wm * WM + lh * 4) * BN + wn * WN + lr;
 #pragma unroll
@@ -956,6 +962,37 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, 
                 dst[e] = (beta == 0.f) ? t : __builtin_fmaf(beta, dst[e], t);
             }
     }
+}
+
+// ABFT with a tail split: the records of a tile's K slices become the tile's record.  Bad-line counts add up; a
+// slice that could not locate its fault makes the tile uncorrectable (2); otherwise the tile is corrected (1) if any
+// slice corrected an element, and reports the first such slice's location and residuals (more than one corrected
+// slice shows in the counts).
+__global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int splits, int tiles_m, int tiles_n,
+                                                            int full_tiles, const hpcdnn_ft_status* __restrict__ slices,
+                                                            hpcdnn_ft_status* __restrict__ status) {
+    const int t = blockIdx.x * 64 + threadIdx.x;
+    if (t >= tail_tiles) return;
+    int tile_m, tile_n;
+    tile_of_block(full_tiles + t, tiles_m, tiles_n, tile_m, tile_n);
+    hpcdnn_ft_status out;
+    out.flag = 0; out.row = -1; out.col = -1; out.n_bad_rows = 0; out.n_bad_cols = 0;
+    out.row_residual = 0.f; out.col_residual = 0.f; out.max_clean_residual = 0.f;
+    bool located = false;
+    for (int z = 0; z < splits; ++z) {
+        const hpcdnn_ft_status s = slices[t * splits + z];
+        out.n_bad_rows += s.n_bad_rows;
+        out.n_bad_cols += s.n_bad_cols;
+        out.max_clean_residual = s.max_clean_residual > out.max_clean_residual ? s.max_clean_residual : out.max_clean_residual;
+        if (s.flag == 2) out.flag = 2;
+        if (s.flag == 1 && !located) {
+            located = true;
+            out.row = s.row; out.col = s.col; out.row_residual = s.row_residual; out.col_residual = s.col_residual;
+        }
+    }
+    if (out.flag == 2) { out.row = -1; out.col = -1; out.row_residual = 0.f; out.col_residual = 0.f; }
+    else if (located) out.flag = 1;
+    status[tile_m * tiles_n + tile_n] = out;
 }
 
 // ---- ABFT pre-encode: the checksum vectors of the operands, one per tile row / tile column, in one launch of

@@ -139,6 +139,13 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * once per tile row / tile column by two small kernels ahead of the GEMM
  * (faster); with ws == NULL each workgroup forms them in its main loop, as the
  * reference does.  Detection, location and correction are the same in both.
+ * The size the query returns also has room for the K slices of a partial last
+ * round of tiles: those tiles are then split along K, every slice verifying
+ * and correcting its own partial product (the checksums are linear in K), and
+ * a second pass adds the slices in order and merges their records into the
+ * tile's (bad-line counts add up; the location is that of the first slice that
+ * corrected something).  A workspace that only holds the checksum vectors
+ * (the size without that room) runs without the split.
  * Replaces ft_sgemm_huge <<<dim3(M/128,N/128),256>>>(M,N,K,A,B,C,alpha,beta)
  * (kernel/ft_sgemm/sgemm.cu:159-165, kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21). */
 int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,

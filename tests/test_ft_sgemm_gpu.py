@@ -23,7 +23,8 @@ def _ws(blas, mode, M, N, K):
     if mode == "fused":
         return None
     nbytes = blas.ft_workspace_bytes(M, N, K)
-    assert nbytes == 4 * (-(-M // 64) + -(-N // 128)) * ((-(-K // 16) + 2) * 16)  # covers the class with the most tile rows
+    # the checksum vectors of the class with the most tile rows, plus room for the K slices of a partial last round
+    assert nbytes >= 4 * (-(-M // 64) + -(-N // 128)) * ((-(-K // 16) + 2) * 16)
     # poisoned: the library must not rely on the workspace's previous contents
     return torch.full((max(nbytes // 4, 4),), float("nan"), dtype=torch.float32, device="cuda")
 
@@ -238,7 +239,8 @@ def test_pick_class_and_bad_class(blas):
     assert blas.ft_pick_class(4096, 4096, 4096) == 0      # 512 tiles of 256x128: every CU has one
     assert blas.ft_pick_class(2048, 2048, 1024) == 1      # 128 tiles of 256x128, 256 of 128x128
     assert blas.ft_pick_class(512, 512, 512) == 2
-    assert blas.ft_pick_class(3072, 3072, 3072) == 2      # 288 tiles of 256x128 would leave a nearly empty second round
+    assert blas.ft_pick_class(3072, 3072, 3072) == 0      # 288 tiles of 256x128: one round, the 32 left over split 8 ways along K
+    assert blas.ft_pick_class(3072, 3072, 128) == 2       # too short a K to split: 64x128 tiles fill the rounds best
     t = torch.zeros(64, 64, device="cuda")
     with pytest.raises(blas.HpcdnnError):
         blas.ft_sgemm(64, 64, 64, t, t, t.clone(), 1.0, 0.0, tile_class=3)
@@ -392,3 +394,56 @@ def test_seeded_random_cases_equal_the_model(blas, oracle_mod):
         if (fault is None or caught) and K >= 16:   # a sub-threshold fault stays in C; K < 16: |A||B| is too small a yardstick for the corrected element
             ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, lda, b, ldb, c0, ldc, alpha, beta)
             assert oracle_mod.gemm_max_err(N, c, ldc, ref, den) <= TOL, what
+
+
+def test_partial_last_round_is_split_along_k(blas, oracle_mod):
+    """With room in the workspace the tiles of a partial last round of CUs are split along K; every slice verifies its
+    own partial product, a second pass adds the slices and merges their records.  Decisions and C must not depend on
+    whether the split happened."""
+    M, N, K = 700, 300, 2048                      # 3 x 3 tiles of 256x128 on 256 CUs: all nine are split (8 ways)
+    enc_only = 4 * (-(-M // 256) + -(-N // 128)) * ((-(-K // 16) + 2) * 16)
+    enc_only = (enc_only + 15) // 16 * 16
+    need = blas.ft_workspace_bytes(M, N, K)
+    assert need > enc_only + 9 * 2 * 256 * 128 * 4  # the query includes the slices
+    tau = blas.ft_default_tau(K)
+    a = oracle_mod.fill_uniform_matrix(M, K, 2100, ld=K + 4)
+    b = oracle_mod.fill_uniform_matrix(K, N, 2101, ld=N + 4)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, 2102, ld=N + 8)
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    for fault in [None, (8, 700 - 512 - 1, 300 - 256 - 1, -0.75), (4, 17, 90, 12.5)]:
+        for t in (tau, -1.0):
+            results = []
+            for nbytes in (need, enc_only, need):   # split, not split, split again
+                ws = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+                dc = torch.from_numpy(c0).cuda()
+                status = blas.ft_status_alloc(M, N)
+                blas.ft_sgemm(M, N, K, da, db, dc, 1.5, -1.0, tau=t, fault=fault, status=status, ws=ws)
+                results.append((dc.cpu().numpy(), blas.ft_status_numpy(status)))
+            c_model = c0.copy()
+            st_model = oracle_mod.ft_sgemm(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, 256, 128, t, fault)
+            for c, st in results:
+                for f in DECISION_FIELDS:
+                    assert np.array_equal(st[f], st_model[f]), (fault, t, f, st[f], st_model[f])
+                _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.5, -1.0)
+                if fault is not None:
+                    assert abs(st["row_residual"][fault[0]] + fault[3]) < 2e-3
+            assert np.array_equal(results[0][0][:, :N], results[2][0][:, :N])      # fixed order: same bits on every run
+            assert not np.array_equal(results[0][0][:, :N], results[1][0][:, :N])  # the split did change the summation order
+    # no status array: the slices keep no records either
+    dc = torch.from_numpy(c0).cuda()
+    blas.ft_sgemm(M, N, K, da, db, dc, 1.5, -1.0, tau=tau, ws=torch.empty(need // 4, dtype=torch.float32, device="cuda"))
+    _assert_values(oracle_mod, M, N, K, a, b, c0, dc.cpu().numpy(), 1.5, -1.0)
+    # a real partial round: 288 tiles of 256x128 at 3072^2, 32 of them split; sampled rows + every record clean
+    n = 3072
+    a3 = torch.empty(n, n, device="cuda"); b3 = torch.empty(n, n, device="cuda"); c3 = torch.zeros(n, n, device="cuda")
+    blas.fill_uniform_matrix(a3, n, n, 2200); blas.fill_uniform_matrix(b3, n, n, 2201)
+    status = blas.ft_status_alloc(n, n)
+    ws = blas.workspace(blas.ft_workspace_bytes(n, n, n))
+    fault = (287, 255, 127, 0.5)   # the last tile, one of the split ones
+    blas.ft_sgemm(n, n, n, a3, b3, c3, 1.0, 0.0, fault=fault, status=status, ws=ws)
+    st = blas.ft_status_numpy(status)
+    assert st["flag"].sum() == 1 and st["flag"][287] == 1 and (st["row"][287], st["col"][287]) == (255, 127)
+    rows = torch.tensor([0, 1500, 2816, 3071], device="cuda")
+    ref = a3[rows].double() @ b3.double()
+    den = a3[rows].abs().double() @ b3.abs().double()
+    assert float(((c3[rows].double() - ref).abs() / den).max()) <= TOL
