@@ -528,7 +528,9 @@ static size_t ft_tail_bytes(const FtClass& fc, const FtTail& t) {
 // (all classes are 128 columns wide), a partial last round counting for what its K split leaves of it plus the
 // second pass over those tiles, with the measured efficiency of the smaller tiles relative to the 256-row one.
 extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
-    static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 0.97, 0.90};
+    // measured on squares 1024 ... 6144: the 128-row class keeps up with the 256-row one (two of its workgroups share a CU
+    // and cover each other's verification), the 64-row class runs 4-5 % behind
+    static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 1.0, 0.955};
     const int cus = device_cus();
     int best = 0;
     double best_cost = 1e300;
