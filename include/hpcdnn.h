@@ -157,8 +157,9 @@ int hpcdnn_ft_num_tiles(int M, int N);
  * verification, status records and `inject` coordinates are per tile of that
  * class, so `status` holds hpcdnn_ft_num_tiles_ex(tile_class, M, N) records.
  * Smaller tiles keep more CUs busy on smaller problems; hpcdnn_ft_pick_class
- * returns the class with the shortest predicted run (rounds of tiles over the
- * CUs times the tile height).  The workspace
+ * returns the class with the shortest predicted run for a call that passes the
+ * workspace (rounds of tiles over the CUs times the tile height, a partial
+ * last round counting for what its K split leaves of it).  The workspace
  * size of HPCDNN_OP_FT_SGEMM covers every class.  Counterpart of the reference's
  * abft_kernel_{huge,large,wide} series (kernel/ft_sgemm/sgemm.cu:187-188,
  * kernel/ft_sgemm/code_gen/main.py:8-16). */
