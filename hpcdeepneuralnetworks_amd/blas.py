@@ -251,3 +251,19 @@ def cpu_gemm(alpha: float, beta: float, mat1: np.ndarray, mat2: np.ndarray, n: i
         if not (isinstance(a, np.ndarray) and a.dtype == np.float32 and a.flags.c_contiguous and a.size >= n * n):
             raise HpcdnnError("cpu_gemm takes C-contiguous float32 numpy arrays of n*n elements")
     _lib.lib().hpcdnn_cpu_gemm(alpha, beta, mat1.ctypes.data, mat2.ctypes.data, n, mat3.ctypes.data)
+
+
+def verify_matrix(mat1: np.ndarray, mat2: np.ndarray, n: int) -> bool:
+    """The reference's matrix acceptance check (utils/utils.cu:74-91): every element of the two n x n host arrays
+    within 1e-2 absolute."""
+    a = np.asarray(mat1, dtype=np.float64).reshape(-1)[: n * n]
+    b = np.asarray(mat2, dtype=np.float64).reshape(-1)[: n * n]
+    return bool(np.all(np.abs(a - b) <= 1e-2))
+
+
+def verify_vector(vec1: np.ndarray, vec2: np.ndarray, n: int) -> bool:
+    """The reference's vector acceptance check (utils/utils.cu:60-72): every element within 5e-3 relative to the
+    first argument (its magnitude; the reference divides by the signed value)."""
+    a = np.asarray(vec1, dtype=np.float64).reshape(-1)[:n]
+    b = np.asarray(vec2, dtype=np.float64).reshape(-1)[:n]
+    return bool(np.all(np.abs(a - b) <= 5e-3 * np.abs(a)))

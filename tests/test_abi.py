@@ -215,3 +215,17 @@ int main() {
     out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
     assert out.returncode == 0, (out.returncode, out.stderr)
     assert out.stdout.startswith("hpcdnn")
+
+
+def test_python_host_helpers_mirror_the_reference_checks():
+    from hpcdeepneuralnetworks_amd import blas
+    a = np.arange(16, dtype=np.float32).reshape(4, 4)
+    b = a.copy()
+    assert blas.verify_matrix(a, b, 4)
+    b[1, 2] += 0.009
+    assert blas.verify_matrix(a, b, 4)
+    b[1, 2] += 0.002
+    assert not blas.verify_matrix(a, b, 4)
+    v = np.array([1.0, -2.0, 100.0], np.float32)
+    assert blas.verify_vector(v, v * np.float32(1.004), 3)
+    assert not blas.verify_vector(v, np.array([1.0, -2.02, 100.0], np.float32), 3)
