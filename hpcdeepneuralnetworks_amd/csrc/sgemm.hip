@@ -235,6 +235,18 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
             }
         }
     }
+    // A split has to promise more than the model's error on it (measured: predicted gains below 2-3 % turned out
+    // as losses of about 1 %): if some unsplit plan is within 2.5 % of the best, only unsplit plans compete.
+    double best_unsplit = 1e300;
+    for (int i = 0; i < n_cand; ++i)
+        if (cand[i].plan.split == 1 && cand[i].cost < best_unsplit) best_unsplit = cand[i].cost;
+    if (best_unsplit <= best_cost * 1.025) {
+        best_cost = best_unsplit;
+        int kept = 0;
+        for (int i = 0; i < n_cand; ++i)
+            if (cand[i].plan.split == 1) cand[kept++] = cand[i];
+        n_cand = kept;
+    }
     // Among plans the model cannot tell apart (within 1 %), take the one that moves the least data: no split
     // before a split, then the larger tile (A and B are re-read once per tile column / tile row).
     Plan best{0, 1};
