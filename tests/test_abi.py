@@ -115,7 +115,8 @@ def test_plan_query_without_a_gpu(L):
         return t.value, s.value
 
     n_tiles = L.hpcdnn_sgemm_num_tiles()
-    for shape in [(1024, 1024, 1024), (4096, 4096, 4096), (6144, 6144, 6144), (3072, 3072, 3072), (128, 128, 65536), (16384, 64, 4096)]:
+    for shape in [(1024, 1024, 1024), (4096, 4096, 4096), (6144, 6144, 6144), (3072, 3072, 3072), (2560, 2560, 2560), (128, 128, 65536),
+                  (16384, 64, 4096)]:
         t, s = plan(*shape, 0)
         assert 0 <= t < n_tiles and s == 1                      # no workspace: nothing is split
         need = L.hpcdnn_workspace_bytes(0, *shape)
@@ -131,7 +132,8 @@ def test_plan_query_without_a_gpu(L):
             tiles = -(-shape[0] // bm.value) * -(-shape[1] // bn.value)
             assert 0 < tiles % 256 <= 128 and need == (tiles % 256) * (-s) * bm.value * bn.value * 4
     assert plan(128, 128, 65536, 1 << 30)[1] >= 16               # deep K: split-K
-    assert plan(3072, 3072, 3072, 1 << 30)[1] <= -2              # 3072^3: a partial last round, tail split
+    assert plan(2560, 2560, 2560, 1 << 30)[1] <= -2              # 2560^3: a partial last round whatever the tile, tail split
+    assert plan(3072, 3072, 3072, 1 << 30)[1] == 1               # 3072^3: 16 x 16 tiles of 192 x 192 fill one round
     assert plan(4096, 4096, 4096, 1 << 30)[1] == 1               # 4096^3: whole rounds, nothing to split
     assert L.hpcdnn_sgemm_plan(-1, 1, 1, 0, None, None) == 1
 
