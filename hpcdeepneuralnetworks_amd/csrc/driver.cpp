@@ -148,8 +148,14 @@ int run_ft_sgemm(int start, int end, int gap, int first, int last) {
     LIB_OK(hpcdnn_fill_uniform(a, static_cast<int64_t>(nn), 1, nullptr));
     LIB_OK(hpcdnn_fill_uniform(b, static_cast<int64_t>(nn), 2, nullptr));
     const float alpha = 1.0f, beta = -1.5f;
-    const size_t ft_ws_bytes = hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM, max_n, max_n, K);
-    const size_t off_ws_bytes = hpcdnn_workspace_bytes(HPCDNN_OP_OFFLINE_FT_SGEMM, max_n, max_n, K);
+    // neither size grows monotonically with n (K-split room, SGEMV chunking): take the largest need over the sweep
+    size_t ft_ws_bytes = 0, off_ws_bytes = 0;
+    for (int n = start; n <= end; n += gap) {
+        const size_t f = hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM, n, n, K);
+        const size_t o = hpcdnn_workspace_bytes(HPCDNN_OP_OFFLINE_FT_SGEMM, n, n, K);
+        if (f > ft_ws_bytes) ft_ws_bytes = f;
+        if (o > off_ws_bytes) off_ws_bytes = o;
+    }
     void *ft_ws = nullptr, *off_ws = nullptr;
     HIP_OK(hipMalloc(&ft_ws, ft_ws_bytes ? ft_ws_bytes : 16));
     HIP_OK(hipMalloc(&off_ws, off_ws_bytes ? off_ws_bytes : 16));

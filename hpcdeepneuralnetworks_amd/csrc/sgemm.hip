@@ -373,7 +373,9 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
             memo.ws_aligned = ws_aligned;
             memo.valid = true;
         }
-        const Plan plan = memo.plan;
+        Plan plan = memo.plan;
+        // a forced tail split needs a tile that has one (not the 32 x 32 tile, whose waves split K among themselves)
+        if (tile < 0 && split < -1) plan = choose_plan(M, N, K, false, 0, false, nullptr, true);
         const RowSplit rs = memo.rows;  // copied: the nested calls below do not touch the memo, but keep it simple
         if (tile < 0 && split == 0 && rs.tile1 >= 0) {
             rc = run_sgemm(rs.rows1, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, rs.tile1, 1, stream);
@@ -389,6 +391,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         }
     }
     const TileConfig& cfg = kTiles[tile];
+    if (cfg.wave_split_k && split < -1) return HPCDNN_ERR_INVALID_VALUE;  // whichever way the tile was chosen
     GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
     const int tiles = a.tiles_m * a.tiles_n;
     a.full_tiles = tiles;

@@ -37,6 +37,7 @@ __global__ __launch_bounds__(kSmallThreads, MIN_BLOCKS) void sgemm_small_kernel(
     const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int li = lane & 31, lh = lane >> 5;
 
+    if (static_cast<int>(blockIdx.x) >= p.tiles_m * p.tiles_n) return;  // this kernel has no tail split: one workgroup per tile
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;

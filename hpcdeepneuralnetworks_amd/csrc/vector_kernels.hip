@@ -3,8 +3,8 @@
 // Layout: contiguous FP32 vectors.  Algorithmic traffic: SAXPY 12 B/element
 // (two loads, one store), SDOT 8 B/element (two loads).  Launch shapes follow
 // what the HBM3E stacks of this part sustain: for the read+write stream of
-// SAXPY many small workgroups, one 16-byte lane per thread (a grid-stride loop
-// that runs once unless n exceeds the grid cap), reach ~6.7 TB/s where
+// SAXPY many one-wave workgroups, 8 bytes per lane (a grid-stride loop
+// that runs once unless n exceeds the grid cap), reach ~7.1 TB/s where
 // long-running grid-stride blocks stay near 4.6 TB/s; for the read-only stream
 // of SDOT one workgroup per CU walks one contiguous slice of both vectors with
 // four 16-byte loads per vector in flight (~7.2 TB/s against ~6.0 TB/s
@@ -18,31 +18,47 @@ constexpr int kVecThreads = 256;
 
 // ------------------------------------------------------------------ SAXPY --
 // Stands in for saxpy / saxpy3 / _saxpy (kernel/saxpy/saxpy.cu:15-48).  The
-// reference's f128 kernels need n % 4 == 0; here the n % 4 tail is done by the
-// first lanes of block 0 and misaligned vectors take the dword kernel.
-// One wave per workgroup: measured 6.67 TB/s against 6.46 with two waves and less with more (n = 2^28).
+// reference's f128 kernels need n % 4 == 0 and 16-byte alignment; here any n
+// and any pair of pointers with the same alignment modulo 8 take the vector
+// kernel (a leading and a trailing single element are done by two lanes of
+// block 0), and the rest takes the dword kernel.
+//
+// One wave per workgroup and 8 bytes per lane: a wave moves 512 contiguous
+// bytes of x and of y.  The memory system sustains more the smaller and the
+// shorter-lived the waves are (n = 2^28, 12 B/element: 16 bytes per lane in
+// 256-thread workgroups 6.4 TB/s, in 64-thread workgroups 6.65, 8 bytes per
+// lane in 64-thread workgroups 7.1): the requests then reach the DRAM
+// channels in address order at the pace the dispatcher launches waves, which
+// at 512 bytes per wave is just below what the channels can take (4 bytes per
+// lane is bound by the wave launch rate at 3.6 TB/s).  Loads carry the
+// non-temporal hint, stores write through (sc0 sc1 nt): measured 1-3 % over
+// non-temporal stores alone, and less dependent on where x and y lie.
 constexpr int kSaxpyThreads = 64;
-constexpr int kSaxpyMaxBlocks = 1 << 22;
+constexpr int64_t kSaxpySegment = int64_t{1} << 29;  // elements per launch: byte offsets stay below 2^31
+constexpr int kAuxNt = 2;            // cache-policy bits of the raw buffer instructions on gfx950: sc0 = 1, nt = 2, sc1 = 16
+constexpr int kAuxWriteThroughNt = 19;
 
-__global__ __launch_bounds__(kSaxpyThreads) void saxpy_vec4_kernel(int64_t n, float alpha, const float* __restrict__ x,
-                                                                   float* __restrict__ y) {
-    const int64_t n4 = n >> 2;
-    const v4f* __restrict__ x4 = reinterpret_cast<const v4f*>(x);
-    v4f* __restrict__ y4 = reinterpret_cast<v4f*>(y);
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kSaxpyThreads;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kSaxpyThreads + threadIdx.x; i < n4; i += stride) {
-        const v4f xv = __builtin_nontemporal_load(&x4[i]);
-        const v4f yv = __builtin_nontemporal_load(&y4[i]);
-        v4f r;
-        r.x = __builtin_fmaf(alpha, xv.x, yv.x);
-        r.y = __builtin_fmaf(alpha, xv.y, yv.y);
-        r.z = __builtin_fmaf(alpha, xv.z, yv.z);
-        r.w = __builtin_fmaf(alpha, xv.w, yv.w);
-        __builtin_nontemporal_store(r, &y4[i]);
-    }
-    if (blockIdx.x == 0) {
-        const int64_t t = (n4 << 2) + threadIdx.x;
-        if (t < n) y[t] = __builtin_fmaf(alpha, x[t], y[t]);
+// One launch covers `nbytes` (a multiple of 8, at most 4 * kSaxpySegment) of x and y from 8-byte aligned xb, yb.
+// The whole byte offset of a lane goes into the vector offset of one descriptor over the segment: rebasing the
+// descriptor per wave, or moving the wave's part into the scalar offset, measured 3 % slower.  Lanes past the end
+// load zeros and their stores are dropped by the descriptor's range check.
+// extra bit 0: also do the single element in front of the segment (xb[-1]); bit 1: the one behind it.
+__global__ __launch_bounds__(kSaxpyThreads) void saxpy_vec2_kernel(unsigned nbytes, float alpha, const float* __restrict__ xb,
+                                                                   float* __restrict__ yb, int extra) {
+    typedef float v2f __attribute__((ext_vector_type(2)));
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(xb), 0, nbytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(yb, 0, nbytes, 0x00020000);
+    const unsigned off = blockIdx.x * (kSaxpyThreads * 8) + threadIdx.x * 8;
+    const v2f xv = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(rx, off, 0, kAuxNt));
+    const v2f yv = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(ry, off, 0, kAuxNt));
+    v2f r;
+    r.x = __builtin_fmaf(alpha, xv.x, yv.x);
+    r.y = __builtin_fmaf(alpha, xv.y, yv.y);
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, r), ry, off, 0, kAuxWriteThroughNt);
+    if (blockIdx.x == 0 && extra != 0 && threadIdx.x < 2) {
+        const int64_t t = threadIdx.x == 0 ? -1 : static_cast<int64_t>(nbytes >> 2);
+        if (extra & (1 << threadIdx.x)) yb[t] = __builtin_fmaf(alpha, xb[t], yb[t]);
     }
 }
 
@@ -204,12 +220,27 @@ extern "C" int hpcdnn_saxpy(int64_t n, float alpha, const float* x, float* y, vo
     if (n < 0 || (n > 0 && (!x || !y))) return HPCDNN_ERR_INVALID_VALUE;
     if (n == 0) return HPCDNN_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3u) return HPCDNN_ERR_INVALID_VALUE;
+    // the vector kernel pairs elements on 8-byte boundaries: x and y must agree modulo 8
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(y)) & 7u) == 0;
     if (aligned) {
-        int64_t grid = ceil_div((n >> 2) + 1, kSaxpyThreads);
-        if (grid > kSaxpyMaxBlocks) grid = kSaxpyMaxBlocks;
-        saxpy_vec4_kernel<<<static_cast<int>(grid), kSaxpyThreads, 0, s>>>(n, alpha, x, y);
+        // a leading element when both pointers are 4 bytes off an 8-byte boundary, pairs, a trailing element
+        const int head = static_cast<int>((reinterpret_cast<uintptr_t>(x) >> 2) & 1);
+        const int64_t pairs = (n - head) >> 1;
+        const bool tail = head + 2 * pairs < n;
+        const float* xb = x + head;
+        float* yb = y + head;
+        int64_t done = 0;
+        do {
+            const int64_t left = 2 * pairs - done;
+            const int64_t count = left < kSaxpySegment ? left : kSaxpySegment;
+            const bool last = done + count == 2 * pairs;
+            const int extra = ((done == 0 && head) ? 1 : 0) | ((last && tail) ? 2 : 0);
+            const unsigned nbytes = static_cast<unsigned>(count * 4);
+            const int64_t grid = count > 0 ? ceil_div(count * 4, kSaxpyThreads * 8) : 1;
+            saxpy_vec2_kernel<<<static_cast<int>(grid), kSaxpyThreads, 0, s>>>(nbytes, alpha, xb + done, yb + done, extra);
+            done += count;
+        } while (done < 2 * pairs);
     } else {
         const int grid = stream_grid(n, 16);
         saxpy_dword_kernel<<<grid, kVecThreads, 0, s>>>(n, alpha, x, y);
@@ -222,6 +253,7 @@ extern "C" int hpcdnn_sdot(int64_t n, const float* x, const float* y, float* out
     if (n < 0 || !out || (n > 0 && (!x || !y))) return HPCDNN_ERR_INVALID_VALUE;
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3u) return HPCDNN_ERR_INVALID_VALUE;
     if (!ws || ws_bytes < hpcdnn_workspace_bytes(HPCDNN_OP_SDOT, 0, 0, 0)) return HPCDNN_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(ws) & 7u) return HPCDNN_ERR_INVALID_VALUE;  // the block partials are doubles
     hipStream_t s = static_cast<hipStream_t>(stream);
     unsigned int* ticket = static_cast<unsigned int*>(ws);
     double* partials = reinterpret_cast<double*>(static_cast<char*>(ws) + kSdotPartialOffset);

@@ -80,7 +80,10 @@ const char* hpcdnn_version(void);
 const char* hpcdnn_error_string(int code);
 
 /* C = alpha*A*B + beta*C, A is MxK, B is KxN, C is MxN, any M,N,K >= 0 and any
- * lda >= K, ldb >= N, ldc >= N.  C is not read when beta == 0.
+ * lda >= K, ldb >= N, ldc >= N with lda <= 2^21 - 64 and ldb <= 2^25 - 1024 (byte
+ * offsets inside one tile are 32-bit; larger values return
+ * HPCDNN_ERR_INVALID_VALUE).  A, B and C are 4-byte aligned.  C is not read
+ * when beta == 0.
  * Replaces sgemm_1..sgemm_14 <<<dim3(ceil(N/bt),ceil(N/bt)),256>>>(N,A,B,C,alpha,beta)
  * (kernel/sgemm/sgemm.cu:70-141, kernel/sgemm/include/kernel_13.cuh:14) and
  * sgemm_{small,medium,large,tall,wide,huge} <<<dim3(ceil(M/ms),ceil(N/ns)),T>>>

@@ -93,6 +93,8 @@ def _load():
     lib.oracle_abft_residuals.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, dp, dp]
     lib.oracle_abft_decide.restype = C.c_float
     lib.oracle_abft_decide.argtypes = [C.c_int, C.c_int, dp, dp, C.c_float, C.POINTER(FtStatus)]
+    lib.oracle_abft_decide_lines.restype = C.c_float
+    lib.oracle_abft_decide_lines.argtypes = [C.c_int, C.c_int, dp, dp, dp, dp, C.POINTER(FtStatus)]
     lib.oracle_ft_sgemm.restype = None
     lib.oracle_ft_sgemm.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
                                     C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int, C.c_int, C.c_float,
@@ -219,6 +221,15 @@ def abft_decide(dr: np.ndarray, dc: np.ndarray, tau: float):
     dr = np.ascontiguousarray(dr, dtype=np.float64)
     dc = np.ascontiguousarray(dc, dtype=np.float64)
     fix = _load().oracle_abft_decide(len(dr), len(dc), _d(dr), _d(dc), tau, C.byref(st))
+    return {k: getattr(st, k) for k, _ in FtStatus._fields_}, float(fix)
+
+
+def abft_decide_lines(dr: np.ndarray, dc: np.ndarray, tau_r: np.ndarray, tau_c: np.ndarray):
+    """Like abft_decide with one threshold per row (tau_r) and per column (tau_c)."""
+    st = FtStatus()
+    dr, dc, tau_r, tau_c = (np.ascontiguousarray(v, dtype=np.float64) for v in (dr, dc, tau_r, tau_c))
+    assert len(tau_r) == len(dr) and len(tau_c) == len(dc)
+    fix = _load().oracle_abft_decide_lines(len(dr), len(dc), _d(dr), _d(dc), _d(tau_r), _d(tau_c), C.byref(st))
     return {k: getattr(st, k) for k, _ in FtStatus._fields_}, float(fix)
 
 

@@ -49,6 +49,12 @@ def test_status_and_fault_struct_sizes():
     assert C.sizeof(_lib.Fault) == 16 and FT_STATUS_DTYPE.itemsize == 32
 
 
+def _tile(L, t):
+    bm, bn, bk = C.c_int(), C.c_int(), C.c_int()
+    assert L.hpcdnn_sgemm_tile_info(t, C.byref(bm), C.byref(bn), C.byref(bk)) == 0
+    return bm.value, bn.value, bk.value
+
+
 def test_bad_arguments_are_rejected_without_a_gpu(L):
     INVALID, WORKSPACE = 1, 2
     dummy = C.c_void_p(0x1000)
@@ -59,6 +65,7 @@ def test_bad_arguments_are_rejected_without_a_gpu(L):
     assert L.hpcdnn_sdot(4, dummy, dummy, None, dummy, 1 << 20, None) == INVALID
     assert L.hpcdnn_sdot(4, dummy, dummy, dummy, None, 0, None) == WORKSPACE
     assert L.hpcdnn_sdot(4, dummy, dummy, dummy, dummy, 8, None) == WORKSPACE
+    assert L.hpcdnn_sdot(4, dummy, dummy, dummy, C.c_void_p(0x1004), 1 << 20, None) == INVALID  # the block partials are doubles
     # GEMM: negative dims, leading dimensions smaller than the row length, null operands
     assert L.hpcdnn_sgemm(-1, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
     assert L.hpcdnn_sgemm(4, 4, 4, dummy, 3, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
@@ -68,6 +75,13 @@ def test_bad_arguments_are_rejected_without_a_gpu(L):
     assert L.hpcdnn_sgemm(0, 4, 4, None, 4, None, 4, None, 4, 1.0, 0.0, None, 0, None) == 0  # empty: nothing to do
     assert L.hpcdnn_sgemm_ex(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, 99, 1, None) == INVALID
     assert L.hpcdnn_sgemm_ex(4, 4, 64, dummy, 64, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, 0, 2, None) == WORKSPACE
+    # the 32 x 32 tile has no tail split (its waves split K among themselves)
+    small = [t for t in range(L.hpcdnn_sgemm_num_tiles()) if _tile(L, t)[:2] == (32, 32)]
+    assert len(small) == 1
+    assert L.hpcdnn_sgemm_ex(256, 1056, 256, dummy, 256, dummy, 1056, dummy, 1056, 1.0, 0.0, dummy, 1 << 30, small[0], -2, None) == INVALID
+    # leading dimensions beyond the 32-bit tile offsets
+    assert L.hpcdnn_sgemm(4, 4, 4, dummy, (1 << 21) - 63, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
+    assert L.hpcdnn_sgemm(4, 4, 4, dummy, 4, dummy, (1 << 25) - 1023, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
     from hpcdeepneuralnetworks_amd._lib import Fault
 
     bad = Fault(5, 0, 0, 1.0)  # only one tile exists

@@ -231,6 +231,147 @@ def test_abft_decide_cases(oracle_mod):
     assert st["flag"] == 2 and st["n_bad_rows"] == 2
 
 
+def test_tile_acc_matches_numpy_on_a_padded_rectangular_tile(oracle_mod):
+    """The accumulator model of the fault campaigns: float accumulators, one fused multiply-add per k, k ascending."""
+    tm, tn, K, lda, ldb = 7, 5, 96, 101, 9
+    a = oracle_mod.fill_uniform_matrix(tm, K, 41, ld=lda)   # NaN padding: a wrong stride or an over-read shows
+    b = oracle_mod.fill_uniform_matrix(K, tn, 42, ld=ldb)
+    acc = oracle_mod.tile_acc(a, lda, b, ldb, tm, tn, K)
+    ref = a[:, :K].astype(np.float64) @ b[:, :tn].astype(np.float64)
+    assert acc.shape == (tm, tn) and acc.dtype == np.float32
+    assert np.max(np.abs(acc - ref)) < 4e-6          # float rounding of a 96-term sum of products below 1
+    # a sub-block of a larger matrix: pointer + leading dimension select it
+    big_a = oracle_mod.fill_uniform_matrix(16, K, 43)
+    big_b = oracle_mod.fill_uniform_matrix(K, 24, 44)
+    sub = oracle_mod.tile_acc(big_a[8:], K, big_b[:, 16:], 24, 8, 8, K)
+    want = big_a[8:].astype(np.float64) @ big_b[:, 16:].astype(np.float64)
+    assert np.max(np.abs(sub - want)) < 4e-6
+
+
+def test_tile_acc_is_not_transposed_and_keeps_float_fma_order(oracle_mod):
+    # rectangular hand case: a transposed operand or swapped tm/tn cannot give this
+    a = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.float32)                    # 2 x 3
+    b = np.array([[1, 0, 2, 0], [0, 1, 0, 2], [1, 1, 1, 1]], dtype=np.float32)  # 3 x 4
+    acc = oracle_mod.tile_acc(a, 3, b, 4, 2, 4, 3)
+    assert acc.tolist() == [[4.0, 5.0, 5.0, 7.0], [10.0, 11.0, 14.0, 16.0]]
+    # float accumulator, k ascending: 2^24 + 1 + 1 stays 2^24 (a double accumulator, or k descending, gives 2^24 + 2)
+    a = np.array([[16777216.0, 1.0, 1.0]], dtype=np.float32)
+    b = np.ones((3, 1), dtype=np.float32)
+    assert oracle_mod.tile_acc(a, 3, b, 1, 1, 1, 3)[0, 0] == np.float32(16777216.0)
+    a = np.array([[1.0, 1.0, 16777216.0]], dtype=np.float32)
+    assert oracle_mod.tile_acc(a, 3, b, 1, 1, 1, 3)[0, 0] == np.float32(16777218.0)
+    # fused: (1 + 2^-12)^2 - 1 keeps the 2^-24 term that a rounded product loses
+    h = np.float32(1.0 + 2.0**-12)
+    a = np.array([[-1.0, h]], dtype=np.float32)
+    b = np.array([[1.0], [h]], dtype=np.float32)
+    assert float(oracle_mod.tile_acc(a, 2, b, 1, 1, 1, 2)[0, 0]) == 2.0**-11 + 2.0**-24
+
+
+def test_decide_lines_uses_each_lines_own_threshold(oracle_mod):
+    tm, tn = 5, 4
+    dr, dc = np.zeros(tm), np.zeros(tn)
+    tau_r = np.array([1.0, 0.1, 1.0, 0.01, 1.0])
+    tau_c = np.array([0.5, 0.05, 0.5, 0.5])
+    # 0.2 is above row 1's threshold but below its neighbours'; the same residual in row 2 is clean
+    dr[1] = -0.2
+    st, fix = oracle_mod.abft_decide_lines(dr, dc, tau_r, tau_c)
+    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"]) == (2, 1, 0) and fix == 0.0
+    dr[:] = 0.0
+    dr[2] = -0.2
+    st, fix = oracle_mod.abft_decide_lines(dr, dc, tau_r, tau_c)
+    assert st["flag"] == 0 and st["max_clean_residual"] == pytest.approx(0.2)
+    # row 1 and column 1 flagged by their own thresholds, the equally large residuals of row 0 / column 0 are clean
+    dr[:] = [0.2, -0.2, 0.0, 0.0, 0.0]
+    dc[:] = [0.2, -0.21, 0.0, 0.0]
+    st, fix = oracle_mod.abft_decide_lines(dr, dc, tau_r, tau_c)
+    assert (st["flag"], st["row"], st["col"], st["n_bad_rows"], st["n_bad_cols"]) == (1, 1, 1, 1, 1)
+    assert fix == pytest.approx(-0.2) and st["col_residual"] == pytest.approx(-0.21)
+    assert st["max_clean_residual"] == pytest.approx(0.2)
+    # rows and columns are not mixed up: tau_c applied to rows would flag row 0 (0.2 > 0.05 is column 1's threshold)
+    st, _ = oracle_mod.abft_decide_lines(dr, dc, tau_r, np.array([0.5, 0.5, 0.5, 0.5]))
+    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"]) == (2, 1, 0)
+    # the uniform form is the special case
+    st_u, fix_u = oracle_mod.abft_decide(dr, dc, 0.1)
+    st_l, fix_l = oracle_mod.abft_decide_lines(dr, dc, np.full(tm, np.float32(0.1), np.float64), np.full(tn, np.float32(0.1), np.float64))
+    assert st_u == st_l and fix_u == fix_l
+
+
+def _numpy_relative_decision(acc, cr_ref, cc_ref, K):
+    """The data-scaled decision of one tile composed in numpy: thresholds rel * sqrt(n) * max(line mean |acc|, tile
+    mean |acc|) with rel = 2.56e-7 * sqrt(max(K, 64)), residual = reference - line sum, strict comparison."""
+    tm, tn = acc.shape
+    a64 = np.abs(acc.astype(np.float64))
+    rel = 2.56e-7 * np.sqrt(max(K, 64))
+    tau_r = rel * np.sqrt(tn) * np.maximum(a64.mean(axis=1), a64.mean())
+    tau_c = rel * np.sqrt(tm) * np.maximum(a64.mean(axis=0), a64.mean())
+    dr = cr_ref - acc.astype(np.float64).sum(axis=1)
+    dc = cc_ref - acc.astype(np.float64).sum(axis=0)
+    bad_r, bad_c = np.flatnonzero(np.abs(dr) > tau_r), np.flatnonzero(np.abs(dc) > tau_c)
+    if len(bad_r) == 0 and len(bad_c) == 0:
+        flag = 0
+    elif len(bad_r) == 1 and len(bad_c) == 1:
+        flag = 1
+    else:
+        flag = 2
+    return flag, bad_r, bad_c, tau_r, tau_c, dr, dc
+
+
+@pytest.mark.parametrize("fault_tile", [None, 0, 1, 4, 5])
+@pytest.mark.parametrize("level", ["below both", "between", "above both"])
+def test_ft_sgemm_model_with_data_scaled_threshold_against_numpy_composition(oracle_mod, fault_tile, level):
+    """oracle_ft_sgemm with tau = -1 on a ragged 3 x 2 tile problem, against the same pipeline composed in numpy
+    (float64 accumulators are exact here: small-integer operands, so the fault-free residuals are exactly zero and
+    the decision depends only on how the thresholds are composed: clipped tile extents, line mean against tile
+    mean, rows against columns).  The fault is sized relative to the two thresholds of its row and column."""
+    M, N, K, tm, tn = 20, 12, 70, 8, 8   # tiles: rows 8, 8, 4; columns 8, 4
+    rng = np.random.default_rng(17)
+    a = rng.integers(-8, 9, (M, K)).astype(np.float32)
+    b = rng.integers(-8, 9, (K, N)).astype(np.float32)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.abs(exact).max() < 2**20   # every partial sum is an exact float
+    ntn = 2
+    fault = None
+    if fault_tile is not None:
+        bm, bn = fault_tile // ntn, fault_tile % ntn
+        h, w = min(tm, M - bm * tm), min(tn, N - bn * tn)
+        blk = exact[bm * tm:bm * tm + h, bn * tn:bn * tn + w].astype(np.float32)
+        # thresholds barely move with the fault (it is far below the accumulators): size it from the fault-free ones
+        _, _, _, tau_r, tau_c, _, _ = _numpy_relative_decision(blk, blk.astype(np.float64).sum(axis=1), blk.astype(np.float64).sum(axis=0), K)
+        # the row with the largest and the column with the smallest threshold: they differ, so a fault can sit between
+        i, j = int(np.argmax(tau_r)), int(np.argmin(tau_c))
+        lo, hi = sorted((tau_r[i], tau_c[j]))
+        assert hi > 1.15 * lo, "row and column thresholds must differ for the in-between case to exist"
+        delta = {"below both": 0.85 * lo, "between": 0.5 * (lo + hi), "above both": 1.15 * hi}[level]
+        fault = (fault_tile, i, j, float(np.float32(-delta)))
+    elif level != "below both":
+        pytest.skip("no fault: one case is enough")
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, -1.0, fault)
+    for t in range(6):
+        bm, bn = t // ntn, t % ntn
+        h, w = min(tm, M - bm * tm), min(tn, N - bn * tn)
+        blk64 = exact[bm * tm:bm * tm + h, bn * tn:bn * tn + w]
+        acc = blk64.astype(np.float32)
+        if fault is not None and t == fault[0]:
+            acc[fault[1], fault[2]] += np.float32(fault[3])
+        flag, bad_r, bad_c, tau_r, tau_c, dr, dc = _numpy_relative_decision(acc, blk64.sum(axis=1), blk64.sum(axis=0), K)
+        # the sized fault keeps a clear distance from both thresholds, so float rounding of the thresholds cannot flip it
+        for d, tau in ((dr, tau_r), (dc, tau_c)):
+            assert np.all(np.abs(np.abs(d) - tau) > 0.05 * tau)
+        assert st["flag"][t] == flag, (t, level)
+        assert (st["n_bad_rows"][t], st["n_bad_cols"][t]) == (len(bad_r), len(bad_c)), (t, level)
+        if flag == 1:
+            assert (st["row"][t], st["col"][t]) == (bad_r[0], bad_c[0])
+            assert st["row_residual"][t] == np.float32(dr[bad_r[0]])
+        else:
+            assert (st["row"][t], st["col"][t]) == (-1, -1)
+    if fault is not None:
+        want = {"below both": 0, "between": 2, "above both": 1}[level]
+        assert st["flag"][fault[0]] == want and np.count_nonzero(st["flag"]) == (want != 0)
+        if want == 1:   # corrected: C is the exact product again
+            assert np.array_equal(c, exact.astype(np.float32))
+
+
 @pytest.mark.parametrize("fault", [None, (1, 3, 2, 0.5), (2, 7, 0, -20.0)])
 def test_ft_sgemm_model_detects_and_corrects(oracle_mod, fault):
     M, N, K, tm, tn = 20, 12, 64, 8, 8   # 3 x 2 tiles, ragged in both directions

@@ -208,6 +208,11 @@ def test_tail_split_forced_matches_and_is_deterministic(blas, oracle_mod):
     _check(oracle_mod, blas, 1024, 1024, 256, 1.0, 0.0, tile=4, split_k=-4, ws=ws)
     with pytest.raises(blas.HpcdnnError):
         _check(oracle_mod, blas, M, N, K, 1.0, 0.0, tile=4, split_k=-8, ws=None)
+    # tail split forced, tile left to the library: a shape whose unforced plan is the 32 x 32 tile (which has no tail
+    # split) must get a tile that has one
+    big = blas.workspace(64 << 20)
+    assert blas.tile_table()[blas.sgemm_plan(256, 1056, 256, ws_bytes=64 << 20)[0]][:2] == (32, 32)
+    _check(oracle_mod, blas, 256, 1056, 256, 1.0, 1.0, split_k=-2, ws=big)
 
 
 def test_small_problem_tile_splits_k_between_its_waves(blas, oracle_mod):

@@ -53,7 +53,7 @@ def test_saxpy_alpha_values(blas, oracle_mod, alpha):
     assert np.array_equal(dy.cpu().numpy(), y)
 
 
-@pytest.mark.parametrize("ox,oy", [(1, 0), (0, 3), (1, 1), (2, 3)])
+@pytest.mark.parametrize("ox,oy", [(1, 0), (0, 3), (1, 1), (2, 3), (1, 3), (3, 5), (2, 4), (0, 2)])
 def test_saxpy_misaligned_base_pointers(blas, oracle_mod, ox, oy):
     n = 5003
     x = oracle_mod.fill_uniform(n + 8, seed=25)
