@@ -36,6 +36,7 @@ EXPORTS = (
     "hpcdnn_ft_sgemm",
     "hpcdnn_ft_num_tiles",
     "hpcdnn_ft_sgemm_ex",
+    "hpcdnn_ft_sgemm_static",
     "hpcdnn_ft_tile_info",
     "hpcdnn_ft_num_tiles_ex",
     "hpcdnn_ft_pick_class",
@@ -99,6 +100,8 @@ def lib():
     L.hpcdnn_sgemm_row_split.argtypes = [i, i, i, sz, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.hpcdnn_ft_sgemm.restype = i
     L.hpcdnn_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, vp]
+    L.hpcdnn_ft_sgemm_static.restype = i
+    L.hpcdnn_ft_sgemm_static.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp]
     L.hpcdnn_ft_sgemm_ex.restype = i
     L.hpcdnn_ft_sgemm_ex.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, i, vp]
     L.hpcdnn_ft_tile_info.restype = i

@@ -136,6 +136,30 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
           "hpcdnn_ft_sgemm")
 
 
+FT_STATIC_SCRATCH_BYTES = 4 << 20
+
+
+def ft_sgemm_static(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
+                    tau: float = 0.0, fault=None, status: torch.Tensor | None = None) -> None:
+    """``ft_sgemm`` with the library's own fixed scratch array instead of a workspace: allocates nothing; refuses
+    problems whose checksum vectors exceed ``FT_STATIC_SCRATCH_BYTES``; calls on one device must not overlap."""
+    pa, lda = _matrix(A, M, K, "A")
+    pb, ldb = _matrix(B, K, N, "B")
+    pc, ldc = _matrix(Cm, M, N, "C")
+    L = _lib.lib()
+    sp = None
+    if status is not None:
+        need = 8 * L.hpcdnn_ft_num_tiles(M, N)
+        if not (status.is_cuda and status.dtype == torch.int32 and status.numel() >= need and status.is_contiguous()):
+            raise HpcdnnError(f"status must be a contiguous int32 GPU tensor with >= {need} elements")
+        sp = status.data_ptr()
+    f = None
+    if fault is not None:
+        f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
+    check(L.hpcdnn_ft_sgemm_static(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, f, sp, _stream()),
+          "hpcdnn_ft_sgemm_static")
+
+
 def ft_workspace_bytes(M: int, N: int, K: int) -> int:
     return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_FT_SGEMM, M, N, K))
 

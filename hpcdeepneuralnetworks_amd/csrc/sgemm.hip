@@ -665,6 +665,48 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
     return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws, ws_bytes, 0, stream);
 }
 
+// ---- ABFT SGEMM for callers that can neither allocate nor pass a workspace: the checksum vectors (and, when they
+// fit, the K slices of a partial last round) live in a fixed device array of this library.  Every device the
+// library runs on holds its own copy of the array at its own address, looked up once per device.
+static __device__ __align__(256) unsigned char scratch[HPCDNN_FT_STATIC_SCRATCH_BYTES];
+
+static int static_scratch_address(void** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* address[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return HPCDNN_ERR_INVALID_VALUE;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!address[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // the address on the current device
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!p) return HPCDNN_ERR_WORKSPACE;
+        address[dev] = p;
+    }
+    *out = address[dev];
+    return HPCDNN_OK;
+}
+
+extern "C" int hpcdnn_ft_sgemm_static(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                                      int ldc, float alpha, float beta, float tau, const hpcdnn_fault* inject,
+                                      hpcdnn_ft_status* status, void* stream) {
+    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
+    if (rc != HPCDNN_OK) return rc;
+    if (M == 0 || N == 0) return HPCDNN_OK;
+    // the checksum vectors of the 256 x 128 class must fit; beyond that the call is refused, never silently slower
+    if (K > 0 && ft_enc_bytes(kFtClasses[0], M, N, K) > HPCDNN_FT_STATIC_SCRATCH_BYTES) return HPCDNN_ERR_WORKSPACE;
+    void* ws = nullptr;
+    rc = static_scratch_address(&ws);
+    if (rc != HPCDNN_OK) return rc;
+    // Nothing in the array has to start at zero: the pre-pass rewrites every word of the checksum vectors the GEMM
+    // reads (their zero padding included), and the K slices and their records are written before they are read.
+    return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws,
+                              HPCDNN_FT_STATIC_SCRATCH_BYTES, 0, stream);
+}
+
 namespace hpcdnn {
 // enough for any tile class (the lowest class has the most tile rows)
 size_t ft_workspace_bytes(int M, int N, int K) {

@@ -178,6 +178,27 @@ int hpcdnn_ft_pick_class(int M, int N, int K);
  * max|A| * max|B| for other data. */
 float hpcdnn_ft_default_tau(int K);
 
+/* hpcdnn_ft_sgemm for callers that cannot allocate device memory or carry a
+ * workspace around (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): same arguments and results as
+ * hpcdnn_ft_sgemm called with a workspace, but the scratch (checksum vectors of
+ * A and B, K slices of a partial last round when they fit as well) is a fixed
+ * array of HPCDNN_FT_STATIC_SCRATCH_BYTES inside the library, one copy per
+ * device.  The call allocates and frees nothing.  Problems whose checksum
+ * vectors need more than the array,
+ *   (ceil(M/256) + ceil(N/128)) * (ceil(K/16) + 2) * 64 bytes > HPCDNN_FT_STATIC_SCRATCH_BYTES,
+ * are refused with HPCDNN_ERR_WORKSPACE (e.g. 8192^3 needs 3.0 MiB and fits,
+ * 12288^3 does not).  All calls on one device share the array: calls that may
+ * overlap in time on one device (different streams, different host threads)
+ * race on it and must be serialised by the caller; the array needs no
+ * initialisation and keeps nothing between calls.
+ * No counterpart in the reference, whose driver allocates everything up front
+ * (kernel/ft_sgemm/sgemm.cu:60-83). */
+#define HPCDNN_FT_STATIC_SCRATCH_BYTES (4u << 20)
+int hpcdnn_ft_sgemm_static(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                           float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
+                           void* stream);
+
 /* Row-major SGEMV, A is M x N with leading dimension lda >= N:
  *   trans = 0:  y[M] = alpha * A   * x[N] + beta * y
  *   trans = 1:  y[N] = alpha * A^T * x[M] + beta * y
