@@ -238,6 +238,23 @@ def main() -> int:
             "no_workspace_overhead_pct_vs_sgemm": round((ms_ft_fused - ms_plain) / ms_plain * 100.0, 2),
             "tau": tau,
         }
+        # checksum granularity and verification cadence (the reference's block- / warp- / thread-level study and its
+        # verification every 256 k): time over plain SGEMM at the same size, the reference's own figures beside it
+        status_w = blas.ft_status_alloc(m, m, granularity=blas.FT_GRAN_WAVE)
+        ms_wave = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status_w, ws=ft_ws,
+                                                     granularity=blas.FT_GRAN_WAVE), st, wu)
+        ms_cad = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ft_ws, check_interval=256), st, wu)
+        ms_cad_fused = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, check_interval=256), st, wu)
+        pct = lambda t: round((t - ms_plain) / ms_plain * 100.0, 2)
+        extras["abft_granularity_4096"] = {
+            "tile_256x128_overhead_pct": pct(ms_ft), "wave_tile_128x32_overhead_pct": pct(ms_wave),
+            "tile_verify_every_256k_overhead_pct": pct(ms_cad), "tile_verify_every_256k_no_workspace_overhead_pct": pct(ms_cad_fused),
+            "wave_tile_gflops": round(2.0 * m ** 3 / ms_wave / 1e6, 1),
+            "reference_T4_block_warp_thread_overhead_pct": [13.49, 27.52, 45.13],    # 4761.49 / {4195.57, 3733.88, 3280.92} - 1
+            "reference_A100_block_warp_thread_overhead_pct": [11.27, 13.20, 68.07],  # 17885.44 / {16073.50, 15800.36, 10641.73} - 1
+            "note": "time over plain SGEMM at 4096^3; reference: fig/ABFT_GEMM/T4/fig12_step_wise_abft_plot.py:30-31, "
+                    "A100/fig17_step_wise_abft_plot.py:28-29 against sgemm_huge (performance.py:22 / :21), other hardware",
+        }
         ntiles = blas.ft_num_tiles(m, m)
         blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ft_ws)
         clean = blas.ft_status_numpy(status)

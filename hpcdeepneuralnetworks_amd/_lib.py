@@ -37,6 +37,9 @@ EXPORTS = (
     "hpcdnn_ft_num_tiles",
     "hpcdnn_ft_sgemm_ex",
     "hpcdnn_ft_sgemm_static",
+    "hpcdnn_ft_sgemm_opt",
+    "hpcdnn_ft_check_tile_info",
+    "hpcdnn_ft_num_check_tiles",
     "hpcdnn_ft_tile_info",
     "hpcdnn_ft_num_tiles_ex",
     "hpcdnn_ft_pick_class",
@@ -55,6 +58,20 @@ EXPORTS = (
 
 class Fault(C.Structure):
     _fields_ = [("tile", C.c_int32), ("row", C.c_int32), ("col", C.c_int32), ("delta", C.c_float)]
+
+
+FT_GRAN_TILE = 0
+FT_GRAN_WAVE = 1
+FT_MAX_FAULTS = 4
+
+
+class FaultAt(C.Structure):
+    _fields_ = [("tile", C.c_int32), ("row", C.c_int32), ("col", C.c_int32), ("delta", C.c_float), ("check", C.c_int32)]
+
+
+class FtOptions(C.Structure):
+    _fields_ = [("tile_class", C.c_int32), ("granularity", C.c_int32), ("check_interval", C.c_int32),
+                ("n_faults", C.c_int32), ("faults", FaultAt * FT_MAX_FAULTS)]
 
 
 class HpcdnnError(RuntimeError):
@@ -102,6 +119,12 @@ def lib():
     L.hpcdnn_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, vp]
     L.hpcdnn_ft_sgemm_static.restype = i
     L.hpcdnn_ft_sgemm_static.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp]
+    L.hpcdnn_ft_sgemm_opt.restype = i
+    L.hpcdnn_ft_sgemm_opt.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(FtOptions), vp, vp, sz, vp]
+    L.hpcdnn_ft_check_tile_info.restype = i
+    L.hpcdnn_ft_check_tile_info.argtypes = [i, i, C.POINTER(i), C.POINTER(i)]
+    L.hpcdnn_ft_num_check_tiles.restype = i
+    L.hpcdnn_ft_num_check_tiles.argtypes = [i, i, i, i]
     L.hpcdnn_ft_sgemm_ex.restype = i
     L.hpcdnn_ft_sgemm_ex.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, i, vp]
     L.hpcdnn_ft_tile_info.restype = i

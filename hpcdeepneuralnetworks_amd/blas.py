@@ -110,13 +110,17 @@ def sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Te
 
 def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
              tau: float = 0.0, fault=None, status: torch.Tensor | None = None, ws: torch.Tensor | None = None,
-             tile_class: int = 0) -> None:
-    """ABFT GEMM; ``fault`` = (tile, row, col, delta) or None; ``status`` = int32 tensor of 8*ft_num_tiles words;
+             tile_class: int = 0, granularity: int = 0, check_interval: int = 0, faults=None) -> None:
+    """ABFT GEMM; ``fault`` = (tile, row, col, delta) or None; ``status`` = int32 tensor of 8*ft_num_check_tiles words;
     ``ws`` = optional scratch tensor of ``ft_workspace_bytes(M, N, K)`` bytes (checksum vectors are then formed
     by a pre-pass instead of inside the main loop); ``tile_class`` selects the ABFT tile (0 = 256x128, 1 = 128x128,
-    2 = 64x128: tiles, status records and fault coordinates are per tile of that class).
+    2 = 64x128).  ``granularity`` FT_GRAN_TILE keeps one checksum pair, verification and status record per tile of the
+    class, FT_GRAN_WAVE one per wave tile (``ft_check_tile``); ``check_interval`` > 0 also verifies every that many
+    values of k inside the K loop, with re-synchronised references; ``faults`` = up to four
+    (tile, row, col, delta[, check]) in check-tile units, ``check`` = the verification each precedes.
 
-    Counterpart of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)`` (kernel/ft_sgemm/sgemm.cu:159-165).
+    Counterpart of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)`` (kernel/ft_sgemm/sgemm.cu:159-165), of its
+    warp- and thread-level variants and of its verification every 256 k (ft_sgemm_huge.cuh:143).
     """
     pa, lda = _matrix(A, M, K, "A")
     pb, ldb = _matrix(B, K, N, "B")
@@ -124,18 +128,30 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
     L = _lib.lib()
     sp = None
     if status is not None:
-        need = 8 * L.hpcdnn_ft_num_tiles_ex(tile_class, M, N)
+        need = 8 * L.hpcdnn_ft_num_check_tiles(tile_class, granularity, M, N)
         if not (status.is_cuda and status.dtype == torch.int32 and status.numel() >= need and status.is_contiguous()):
             raise HpcdnnError(f"status must be a contiguous int32 GPU tensor with >= {need} elements")
         sp = status.data_ptr()
-    f = None
-    if fault is not None:
-        f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
     wp, wb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
-    check(L.hpcdnn_ft_sgemm_ex(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, f, sp, wp, wb, tile_class, _stream()),
-          "hpcdnn_ft_sgemm")
+    if granularity == 0 and check_interval == 0 and not faults:
+        f = None
+        if fault is not None:
+            f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
+        check(L.hpcdnn_ft_sgemm_ex(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, f, sp, wp, wb, tile_class, _stream()),
+              "hpcdnn_ft_sgemm")
+        return
+    every = list(faults or []) + ([fault] if fault is not None else [])
+    if len(every) > _lib.FT_MAX_FAULTS:
+        raise HpcdnnError(f"at most {_lib.FT_MAX_FAULTS} faults per call")
+    opt = _lib.FtOptions()
+    opt.tile_class, opt.granularity, opt.check_interval, opt.n_faults = tile_class, granularity, check_interval, len(every)
+    for i, fl in enumerate(every):
+        opt.faults[i] = _lib.FaultAt(int(fl[0]), int(fl[1]), int(fl[2]), float(fl[3]), int(fl[4]) if len(fl) > 4 else 0)
+    check(L.hpcdnn_ft_sgemm_opt(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, C.byref(opt), sp, wp, wb, _stream()),
+          "hpcdnn_ft_sgemm_opt")
 
 
+FT_GRAN_TILE, FT_GRAN_WAVE = _lib.FT_GRAN_TILE, _lib.FT_GRAN_WAVE
 FT_STATIC_SCRATCH_BYTES = 4 << 20
 
 
@@ -225,8 +241,19 @@ def ft_default_tau(K: int) -> float:
     return float(_lib.lib().hpcdnn_ft_default_tau(K))
 
 
-def ft_status_alloc(M: int, N: int, device=None, tile_class: int = 0) -> torch.Tensor:
-    return torch.zeros(8 * ft_num_tiles(M, N, tile_class), dtype=torch.int32, device=device or "cuda")
+def ft_check_tile(tile_class: int = 0, granularity: int = 0):
+    """(rows, columns) of the unit that has its own checksum pair, verification and status record."""
+    cm, cn = C.c_int(), C.c_int()
+    check(_lib.lib().hpcdnn_ft_check_tile_info(tile_class, granularity, C.byref(cm), C.byref(cn)), "hpcdnn_ft_check_tile_info")
+    return cm.value, cn.value
+
+
+def ft_num_check_tiles(M: int, N: int, tile_class: int = 0, granularity: int = 0) -> int:
+    return int(_lib.lib().hpcdnn_ft_num_check_tiles(tile_class, granularity, M, N))
+
+
+def ft_status_alloc(M: int, N: int, device=None, tile_class: int = 0, granularity: int = 0) -> torch.Tensor:
+    return torch.zeros(8 * ft_num_check_tiles(M, N, tile_class, granularity), dtype=torch.int32, device=device or "cuda")
 
 
 def ft_status_numpy(status: torch.Tensor) -> np.ndarray:

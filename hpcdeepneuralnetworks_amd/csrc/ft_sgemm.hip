@@ -1,0 +1,357 @@
+// ABFT-SGEMM entry points: tile classes, checksum granularity, verification cadence, workspace layout, launch.
+#include "gemm_host.h"
+
+namespace hpcdnn {
+
+// row length of the pre-encoded checksum vectors: K rounded up to the K step, plus two K steps of zeros for the
+// fetches that run ahead of the main loop
+static int ft_enc_ld(int K) { return (static_cast<int>(ceil_div(K, kGemmBK)) + 2) * kGemmBK; }
+size_t ft_workspace_bytes(int M, int N, int K);
+
+// ABFT tile classes (the counterpart of the reference's abft_kernel_{huge,large,wide,...} family,
+// kernel/ft_sgemm/sgemm.cu:187-188): class 0 is the 256 x 128 tile of HPCDNN_FT_TILE_M/N; the smaller classes keep
+// more CUs busy on smaller problems.  The encode is laid out for 128-column tiles, so the classes differ in height.
+//
+// Without a workspace (FT = 1) four waves: on this part every VALU instruction takes its issue cycles away from the
+// FP32 matrix pipe of the same SIMD, whichever wave it comes from, so more waves do not hide the checksum arithmetic;
+// fewer, fatter threads need the fewest VALU instructions per K step.  With the operands' checksum vectors read from
+// a workspace (FT = 2) no cross-lane reductions are left in the loop, the thread count no longer changes the VALU
+// work per SIMD, and eight waves (two per SIMD) hide each other's barriers and LDS latency: measured 2 % faster.
+//
+// Wave-tile granularity (the counterpart of ft_sgemm_huge_warp.cuh / ft_sgemm_huge_thread.cuh) runs the FT = 2 kernel
+// with one checksum pair per wave tile: the tile a wave of the workspace kernel owns, (bm / wgm) x (bn / wgn).
+struct FtKernel {
+    void (*plain)(const GemmArgs);
+    void (*edge)(const GemmArgs);
+    int threads;
+    size_t lds;
+};
+typedef void (*EncodeFn)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int);
+struct FtClass {
+    int bm, bn;
+    int wgm, wgn;        // wave layout of the workspace kernels
+    FtKernel fused;      // checksum vectors formed in the main loop, one pair per workgroup tile
+    FtKernel pre;        // checksum vectors from the workspace, one pair per workgroup tile
+    FtKernel wave;       // checksum vectors from the workspace, one pair per wave tile
+    FtKernel fused_cad;  // the first two with a verification every check_interval k (class 0 only)
+    FtKernel pre_cad;
+    EncodeFn encode, encode_wave;
+};
+
+#define HPCDNN_FT_KERNEL(BM, WM_, WN_, FT, GRAN, CAD)                                                      \
+    FtKernel {                                                                                             \
+        sgemm_kernel<BM, 128, WM_, WN_, false, FT, 1, 2, GRAN, CAD>,                                       \
+            sgemm_kernel<BM, 128, WM_, WN_, true, FT, 1, 2, GRAN, CAD>, WM_ * WN_ * kWave,                 \
+            gemm_lds_bytes<BM, 128, FT, WM_ * WN_ * kWave, WM_, WN_, GRAN>()                               \
+    }
+#define HPCDNN_FT_NO_KERNEL \
+    FtKernel { nullptr, nullptr, 0, 0 }
+
+static const FtClass kFtClasses[HPCDNN_FT_NUM_CLASSES] = {
+    // 0 huge
+    {256, 128, 2, 4, HPCDNN_FT_KERNEL(256, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(256, 2, 4, 2, 0, false),
+     HPCDNN_FT_KERNEL(256, 2, 4, 2, 1, false), HPCDNN_FT_KERNEL(256, 2, 2, 1, 0, true),
+     HPCDNN_FT_KERNEL(256, 2, 4, 2, 0, true), abft_encode_kernel<256, 128>, abft_encode_kernel<128, 32>},
+    // 1 large
+    {128, 128, 2, 2, HPCDNN_FT_KERNEL(128, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(128, 2, 2, 2, 0, false),
+     HPCDNN_FT_KERNEL(128, 2, 2, 2, 1, false), HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<128, 128>,
+     abft_encode_kernel<64, 64>},
+    // 2 wide
+    {64, 128, 2, 2, HPCDNN_FT_KERNEL(64, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(64, 2, 2, 2, 0, false),
+     HPCDNN_FT_KERNEL(64, 2, 2, 2, 1, false), HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<64, 128>,
+     abft_encode_kernel<32, 64>},
+};
+
+// check tile of a class at a granularity: the unit that has a checksum pair, a verification and a status record
+static void check_tile(const FtClass& fc, int granularity, int* cm, int* cn) {
+    *cm = granularity == HPCDNN_FT_GRAN_WAVE ? fc.bm / fc.wgm : fc.bm;
+    *cn = granularity == HPCDNN_FT_GRAN_WAVE ? fc.bn / fc.wgn : fc.bn;
+}
+
+// ABFT with a workspace splits the tiles of a partial last round of CUs along K, like plain SGEMM's tail split: every
+// slice is a workgroup that verifies (and corrects) its own partial product - the checksums are linear in K - and
+// writes it raw; tail_reduce_kernel adds the slices, ft_tail_status_kernel merges their records.  With fewer tiles
+// than half the CUs every tile is split.  Returns the number of ways (1: no split) and the tiles it applies to.
+struct FtTail {
+    int ways, tiles;
+};
+static FtTail ft_tail_plan(const FtClass& fc, int M, int N, int K) {
+    const int cus = device_cus();
+    const int64_t tiles = ceil_div(M, fc.bm) * ceil_div(N, fc.bn);
+    const int64_t r = tiles % cus;
+    if (r == 0 || 2 * r > cus) return FtTail{1, 0};
+    int64_t s = cus / r;
+    const int64_t most = K / (16 * kGemmBK);  // at least 16 K steps per slice: each slice pays a verification
+    if (s > most) s = most;
+    if (s > 8) s = 8;
+    if (s < 2) return FtTail{1, 0};
+    return FtTail{static_cast<int>(s), static_cast<int>(r)};
+}
+// checksum vectors: one row per row group and per column group of the granularity
+static size_t ft_enc_bytes(const FtClass& fc, int granularity, int M, int N, int K) {
+    const int gm = granularity == HPCDNN_FT_GRAN_WAVE ? fc.wgm : 1, gn = granularity == HPCDNN_FT_GRAN_WAVE ? fc.wgn : 1;
+    const size_t b = static_cast<size_t>(ceil_div(M, fc.bm) * gm + ceil_div(N, fc.bn) * gn) * ft_enc_ld(K) * sizeof(float);
+    return (b + 15) & ~static_cast<size_t>(15);
+}
+static size_t ft_tail_bytes(const FtClass& fc, const FtTail& t) {
+    return t.ways < 2 ? 0
+                      : static_cast<size_t>(t.tiles) * t.ways * (static_cast<size_t>(fc.bm) * fc.bn * sizeof(float) + sizeof(hpcdnn_ft_status));
+}
+
+static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const FtClass& fc = kFtClasses[tile_class];
+    const size_t tile_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_TILE, M, N, K) + ft_tail_bytes(fc, ft_tail_plan(fc, M, N, K));
+    const size_t wave_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_WAVE, M, N, K);
+    return tile_mode > wave_mode ? tile_mode : wave_mode;
+}
+
+static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                        float alpha, float beta, float tau, const hpcdnn_ft_options& opt, hpcdnn_ft_status* status, void* ws,
+                        size_t ws_bytes, hipStream_t s) {
+    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
+    if (rc != HPCDNN_OK) return rc;
+    if (opt.tile_class < 0 || opt.tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
+    if (opt.granularity != HPCDNN_FT_GRAN_TILE && opt.granularity != HPCDNN_FT_GRAN_WAVE) return HPCDNN_ERR_INVALID_VALUE;
+    if (opt.check_interval < 0 || opt.check_interval % kGemmBK != 0) return HPCDNN_ERR_INVALID_VALUE;
+    if (opt.n_faults < 0 || opt.n_faults > HPCDNN_FT_MAX_FAULTS) return HPCDNN_ERR_INVALID_VALUE;
+    const FtClass& fc = kFtClasses[opt.tile_class];
+    const bool wave = opt.granularity == HPCDNN_FT_GRAN_WAVE;
+    // an interval that covers all of K is a single verification after the loop
+    const bool cadence = opt.check_interval > 0 && opt.check_interval < K;
+    if (cadence && (wave || !fc.pre_cad.plain)) return HPCDNN_ERR_INVALID_VALUE;
+    if (M == 0 || N == 0) return HPCDNN_OK;
+    if (wave && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
+
+    GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, fc.bm, fc.bn);
+    // tau > 0: absolute; tau == 0: the absolute default for unit-range data; tau < 0: scaled to the data, the
+    // threshold of a line of n elements being -tau * 4.3 FP32 rounding units * sqrt(max(K, 64)) * sqrt(n) * the larger
+    // of the line's and the check tile's mean |accumulator|
+    a.tau = (tau > 0.f) ? tau : (tau == 0.f ? hpcdnn_ft_default_tau(K) : 0.f);
+    a.tau_rel = (tau < 0.f) ? -tau * 2.56e-7f * sqrtf(static_cast<float>(K > 64 ? K : 64)) : 0.f;
+    a.status = status;
+    a.check_interval = cadence ? opt.check_interval : 0;
+    int cm = 0, cn = 0;
+    check_tile(fc, opt.granularity, &cm, &cn);
+    const int gm = fc.bm / cm, gn = fc.bn / cn;
+    a.status_rows = static_cast<int>(ceil_div(M, cm));
+    a.status_ld = static_cast<int>(ceil_div(N, cn));
+    // faults come in check-tile units; the kernel takes them per workgroup tile
+    a.n_faults = opt.n_faults;
+    for (int f = 0; f < opt.n_faults; ++f) {
+        const hpcdnn_ft_fault_at& in = opt.faults[f];
+        if (in.tile < 0 || in.tile >= a.status_rows * a.status_ld || in.row < 0 || in.row >= cm || in.col < 0 ||
+            in.col >= cn || in.check < 0)
+            return HPCDNN_ERR_INVALID_VALUE;
+        const int srow = in.tile / a.status_ld, scol = in.tile % a.status_ld;
+        a.faults[f].tile = (srow / gm) * a.tiles_n + scol / gn;
+        a.faults[f].row = (srow % gm) * cm + in.row;
+        a.faults[f].col = (scol % gn) * cn + in.col;
+        a.faults[f].delta = in.delta;
+        a.faults[f].check = in.check;
+    }
+    const bool edge = needs_edge(a, fc.bm, fc.bn, kGemmBK);
+    dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
+    // With a workspace the checksum vectors of A and B are formed once per row group / column group by a small
+    // bandwidth-bound kernel and the main loop only reads them; without one every workgroup forms them itself.
+    if (ws && K > 0) {
+        const size_t enc_bytes = ft_enc_bytes(fc, opt.granularity, M, N, K);
+        if (ws_bytes < enc_bytes || (reinterpret_cast<uintptr_t>(ws) & 15u)) return HPCDNN_ERR_WORKSPACE;
+        // the K split of a partial last round is taken when the workspace has room for it (one checksum pair per
+        // workgroup tile and one verification only: a slice keeps one record)
+        FtTail tail = (wave || cadence) ? FtTail{1, 0} : ft_tail_plan(fc, M, N, K);
+        if (ws_bytes < enc_bytes + ft_tail_bytes(fc, tail)) tail = FtTail{1, 0};
+        a.enc_ld = ft_enc_ld(K);
+        const int row_groups = a.tiles_m * gm, col_groups = a.tiles_n * gn;
+        float* enc_a = static_cast<float*>(ws);
+        float* enc_b = enc_a + static_cast<size_t>(row_groups) * a.enc_ld;
+        (void)col_groups;
+        a.enc_a = enc_a;
+        a.enc_b = enc_b;
+        const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
+        hipLaunchKernelGGL(wave ? fc.encode_wave : fc.encode, dim3(k_blocks * (row_groups + a.tiles_n)), dim3(1024), 0, s, M, N, K,
+                           A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups);
+        rc = launch_status();
+        if (rc != HPCDNN_OK) return rc;
+        const FtKernel& k = wave ? fc.wave : (cadence ? fc.pre_cad : fc.pre);
+        void (*fn)(const GemmArgs) = edge ? k.edge : k.plain;
+        rc = enable_lds(fn, k.lds);
+        if (rc != HPCDNN_OK) return rc;
+        const int tiles = a.tiles_m * a.tiles_n;
+        if (tail.ways >= 2) {
+            a.tail_k_chunk = static_cast<int>(ceil_div(ceil_div(K, tail.ways), kGemmBK)) * kGemmBK;
+            tail.ways = static_cast<int>(ceil_div(K, a.tail_k_chunk));  // drop empty slices
+        }
+        if (tail.ways >= 2) {
+            a.full_tiles = tiles - tail.tiles;
+            a.tail_split = tail.ways;
+            a.tail_partial = reinterpret_cast<float*>(static_cast<char*>(ws) + enc_bytes);
+            a.tail_status = reinterpret_cast<hpcdnn_ft_status*>(a.tail_partial + static_cast<size_t>(tail.tiles) * tail.ways * fc.bm * fc.bn);
+            grid = dim3(a.full_tiles + tail.tiles * tail.ways, 1, 1);
+        }
+        hipLaunchKernelGGL(fn, grid, dim3(k.threads), k.lds, s, a);
+        rc = launch_status();
+        if (rc != HPCDNN_OK || a.tail_split < 2) return rc;
+        tail_reduce_kernel<><<<dim3(tail.tiles, fc.bm / 32), 256, 0, s>>>(M, N, fc.bm, fc.bn, a.tiles_m, a.tiles_n, a.full_tiles,
+                                                                         a.tail_split, a.tail_partial, C, ldc, alpha, beta);
+        rc = launch_status();
+        if (rc != HPCDNN_OK || !status) return rc;
+        ft_tail_status_kernel<><<<static_cast<int>(ceil_div(tail.tiles, 64)), 64, 0, s>>>(tail.tiles, a.tail_split, a.tiles_m, a.tiles_n,
+                                                                                        a.full_tiles, a.tail_status, status);
+        return launch_status();
+    }
+    const FtKernel& k = cadence ? fc.fused_cad : fc.fused;
+    void (*fn)(const GemmArgs) = edge ? k.edge : k.plain;
+    rc = enable_lds(fn, k.lds);
+    if (rc != HPCDNN_OK) return rc;
+    hipLaunchKernelGGL(fn, grid, dim3(k.threads), k.lds, s, a);
+    return launch_status();
+}
+
+}  // namespace hpcdnn
+
+using namespace hpcdnn;
+
+extern "C" int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn) {
+    if (tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
+    if (bm) *bm = kFtClasses[tile_class].bm;
+    if (bn) *bn = kFtClasses[tile_class].bn;
+    return HPCDNN_OK;
+}
+
+extern "C" int hpcdnn_ft_check_tile_info(int tile_class, int granularity, int* cm, int* cn) {
+    if (tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
+    if (granularity != HPCDNN_FT_GRAN_TILE && granularity != HPCDNN_FT_GRAN_WAVE) return HPCDNN_ERR_INVALID_VALUE;
+    int m = 0, n = 0;
+    check_tile(kFtClasses[tile_class], granularity, &m, &n);
+    if (cm) *cm = m;
+    if (cn) *cn = n;
+    return HPCDNN_OK;
+}
+
+extern "C" int hpcdnn_ft_num_check_tiles(int tile_class, int granularity, int M, int N) {
+    int cm = 0, cn = 0;
+    if (M < 0 || N < 0 || hpcdnn_ft_check_tile_info(tile_class, granularity, &cm, &cn) != HPCDNN_OK) return 0;
+    return static_cast<int>(ceil_div(M, cm) * ceil_div(N, cn));
+}
+
+extern "C" int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N) {
+    return hpcdnn_ft_num_check_tiles(tile_class, HPCDNN_FT_GRAN_TILE, M, N);
+}
+
+extern "C" int hpcdnn_ft_num_tiles(int M, int N) { return hpcdnn_ft_num_tiles_ex(0, M, N); }
+
+// The class with the shortest predicted run (workspace variant): rounds of tiles over the CUs times the tile height
+// (all classes are 128 columns wide), a partial last round counting for what its K split leaves of it plus the
+// second pass over those tiles, with the measured efficiency of the smaller tiles relative to the 256-row one.
+extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
+    // measured on squares 1024 ... 6144: the 128-row class keeps up with the 256-row one (two of its workgroups share a CU
+    // and cover each other's verification), the 64-row class runs 4-5 % behind
+    static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 1.0, 0.955};
+    const int cus = device_cus();
+    int best = 0;
+    double best_cost = 1e300;
+    for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
+        const int64_t tiles = hpcdnn_ft_num_tiles_ex(c, M, N);
+        const FtTail tail = ft_tail_plan(kFtClasses[c], M, N, K);
+        double rounds = static_cast<double>(ceil_div(tiles > 0 ? tiles : 1, cus));
+        if (tail.ways >= 2)
+            rounds = static_cast<double>(tiles / cus) + static_cast<double>(ceil_div(static_cast<int64_t>(tail.tiles) * tail.ways, cus)) / tail.ways + 0.06;
+        const double cost = rounds * kFtClasses[c].bm / rel_eff[c];
+        if (cost < best_cost) { best_cost = cost; best = c; }
+    }
+    return best;
+}
+
+// Fault-free residuals are the FP32 rounding of the accumulators added over a tile line; for operands uniform in
+// [-1, 1] their maximum over a whole matrix grows linearly with K (measured 4.0e-7 ... 4.9e-7 per unit of K from
+// K = 256 to 65536).  The default leaves a factor of two to that and stays below the 1e-2 faults at K = 4096.
+extern "C" float hpcdnn_ft_default_tau(int K) {
+    const int k = K > 64 ? K : 64;
+    return 1.1e-6f * static_cast<float>(k);
+}
+
+extern "C" int hpcdnn_ft_sgemm_opt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                                   float alpha, float beta, float tau, const hpcdnn_ft_options* opt, hpcdnn_ft_status* status,
+                                   void* ws, size_t ws_bytes, void* stream) {
+    hpcdnn_ft_options none{};
+    return run_ft_sgemm(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, opt ? *opt : none, status, ws, ws_bytes,
+                        static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                                  float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
+                                  void* ws, size_t ws_bytes, int tile_class, void* stream) {
+    hpcdnn_ft_options opt{};
+    opt.tile_class = tile_class;
+    if (inject) {
+        opt.n_faults = 1;
+        opt.faults[0].tile = inject->tile;
+        opt.faults[0].row = inject->row;
+        opt.faults[0].col = inject->col;
+        opt.faults[0].delta = inject->delta;
+        opt.faults[0].check = 0;
+    }
+    return run_ft_sgemm(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, opt, status, ws, ws_bytes,
+                        static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                               float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
+                               void* ws, size_t ws_bytes, void* stream) {
+    return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws, ws_bytes, 0, stream);
+}
+
+// ---- ABFT SGEMM for callers that can neither allocate nor pass a workspace: the checksum vectors (and, when they
+// fit, the K slices of a partial last round) live in a fixed device array of this library.  Every device the
+// library runs on holds its own copy of the array at its own address, looked up once per device.
+static __device__ __align__(256) unsigned char scratch[HPCDNN_FT_STATIC_SCRATCH_BYTES];
+
+static int static_scratch_address(void** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* address[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return HPCDNN_ERR_INVALID_VALUE;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!address[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // the address on the current device
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!p) return HPCDNN_ERR_WORKSPACE;
+        address[dev] = p;
+    }
+    *out = address[dev];
+    return HPCDNN_OK;
+}
+
+extern "C" int hpcdnn_ft_sgemm_static(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                                      int ldc, float alpha, float beta, float tau, const hpcdnn_fault* inject,
+                                      hpcdnn_ft_status* status, void* stream) {
+    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
+    if (rc != HPCDNN_OK) return rc;
+    if (M == 0 || N == 0) return HPCDNN_OK;
+    // the checksum vectors of the 256 x 128 class must fit; beyond that the call is refused, never silently slower
+    if (K > 0 && ft_enc_bytes(kFtClasses[0], HPCDNN_FT_GRAN_TILE, M, N, K) > HPCDNN_FT_STATIC_SCRATCH_BYTES) return HPCDNN_ERR_WORKSPACE;
+    void* ws = nullptr;
+    rc = static_scratch_address(&ws);
+    if (rc != HPCDNN_OK) return rc;
+    // Nothing in the array has to start at zero: the pre-pass rewrites every word of the checksum vectors the GEMM
+    // reads (their zero padding included), and the K slices and their records are written before they are read.
+    return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws,
+                              HPCDNN_FT_STATIC_SCRATCH_BYTES, 0, stream);
+}
+
+namespace hpcdnn {
+// enough for any tile class at either granularity (the lowest class has the most tile rows)
+size_t ft_workspace_bytes(int M, int N, int K) {
+    size_t most = 0;
+    for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
+        const size_t b = ft_class_workspace_bytes(c, M, N, K);
+        if (b > most) most = b;
+    }
+    return most;
+}
+}  // namespace hpcdnn

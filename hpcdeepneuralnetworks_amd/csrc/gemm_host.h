@@ -1,0 +1,70 @@
+// Host-side helpers shared by the SGEMM and ABFT-SGEMM entry points.
+#pragma once
+
+#include <mutex>
+
+#include "sgemm_kernel.h"
+
+namespace hpcdnn {
+
+constexpr int kMaxLda = (1 << 21) - 64;    // 256 * lda * 4 < 2^31
+constexpr int kMaxLdb = (1 << 25) - 1024;  // 16 * ldb * 4 + row < 2^31
+
+inline int check_gemm_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+    if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
+    if (lda < (K > 1 ? K : 1) || ldb < (N > 1 ? N : 1) || ldc < (N > 1 ? N : 1)) return HPCDNN_ERR_INVALID_VALUE;
+    if (M > 0 && N > 0 && !C) return HPCDNN_ERR_INVALID_VALUE;
+    if (M > 0 && N > 0 && K > 0 && (!A || !B)) return HPCDNN_ERR_INVALID_VALUE;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) & 3u)
+        return HPCDNN_ERR_INVALID_VALUE;
+    // byte offsets inside one tile are 32-bit: 256 rows of A, 16 rows of B
+    if (lda > kMaxLda || ldb > kMaxLdb) return HPCDNN_ERR_INVALID_VALUE;
+    return HPCDNN_OK;
+}
+
+inline GemmArgs make_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                          float alpha, float beta, int bm, int bn) {
+    GemmArgs a{};
+    a.M = M; a.N = N; a.K = K;
+    a.A = A; a.lda = lda; a.B = B; a.ldb = ldb; a.C = C; a.ldc = ldc;
+    a.alpha = alpha; a.beta = beta;
+    a.tiles_m = static_cast<int>(ceil_div(M, bm));
+    a.tiles_n = static_cast<int>(ceil_div(N, bn));
+    a.k_chunk = static_cast<int>(ceil_div(K > 0 ? K : 1, kGemmBK)) * kGemmBK;
+    a.partial = nullptr;
+    a.n_faults = 0;
+    a.full_tiles = a.tiles_m * a.tiles_n;
+    a.tail_split = 1;
+    return a;
+}
+
+// The ragged-tile kernel masks the K tail and the columns past N; full tiles with K a multiple of the K step
+// (per slice, which k_chunk guarantees for all but the last) skip that work.
+inline bool needs_edge(const GemmArgs& a, int bm, int bn, int bk) {
+    return !(a.M % bm == 0 && a.N % bn == 0 && a.K % bk == 0);
+}
+
+// Kernels that use more than the default 64 KiB of LDS must opt in once per device.
+inline int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {
+    if (bytes <= 64 * 1024) return HPCDNN_OK;
+    struct Done {
+        const void* fn;
+        int device;
+    };
+    static std::mutex mu;
+    static Done done[512] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    std::lock_guard<std::mutex> lock(mu);
+    const void* key = reinterpret_cast<const void*>(fn);
+    for (const Done& d : done)
+        if (d.fn == key && d.device == dev) return HPCDNN_OK;
+    e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+    if (e != hipSuccess) return static_cast<int>(e);
+    for (Done& d : done)
+        if (!d.fn) { d = Done{key, dev}; break; }  // a full table only costs a repeated call
+    return HPCDNN_OK;
+}
+
+}  // namespace hpcdnn

@@ -1,8 +1,6 @@
 // SGEMM / ABFT-SGEMM entry points: argument checks, tile + split-K choice, launch.
-#include "sgemm_kernel.h"
+#include "gemm_host.h"
 #include "sgemm_small_kernel.h"
-
-#include <mutex>
 
 namespace hpcdnn {
 
@@ -63,67 +61,6 @@ static const TileConfig kTiles[] = {
     HPCDNN_TILE(192, 192, 2, 2, 1, 0.943f),  // 13 3072-friendly: 16 x 16 tiles = one full round of 256 CUs
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
-
-// row length of the pre-encoded checksum vectors: K rounded up to the K step, plus two K steps of zeros for the
-// fetches that run ahead of the main loop
-static int ft_enc_ld(int K) { return (static_cast<int>(ceil_div(K, kGemmBK)) + 2) * kGemmBK; }
-size_t ft_workspace_bytes(int M, int N, int K);
-// ABFT tile classes (the counterpart of the reference's abft_kernel_{huge,large,wide,...} family,
-// kernel/ft_sgemm/sgemm.cu:187-188): class 0 is the 256 x 128 tile of HPCDNN_FT_TILE_M/N; the smaller classes keep
-// more CUs busy on smaller problems.  The encode is laid out for 128-column tiles, so the classes differ in height.
-//
-// Without a workspace (FT = 1) four waves: on this part every VALU instruction takes its issue cycles away from the
-// FP32 matrix pipe of the same SIMD, whichever wave it comes from, so more waves do not hide the checksum arithmetic;
-// fewer, fatter threads need the fewest VALU instructions per K step.  With the operands' checksum vectors read from
-// a workspace (FT = 2) no cross-lane reductions are left in the loop, the thread count no longer changes the VALU
-// work per SIMD, and eight waves (two per SIMD) hide each other's barriers and LDS latency: measured 2 % faster.
-struct FtClass {
-    int bm, bn;
-    int threads_fused, threads_pre;
-    size_t lds_fused, lds_pre;
-    void (*fused_plain)(const GemmArgs);
-    void (*fused_edge)(const GemmArgs);
-    void (*pre_plain)(const GemmArgs);
-    void (*pre_edge)(const GemmArgs);
-    void (*encode)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int);
-};
-
-#define HPCDNN_FT_CLASS(BM, FM, FN, PM, PN)                                                                      \
-    {                                                                                                            \
-        BM, 128, FM * FN * kWave, PM * PN * kWave, gemm_lds_bytes<BM, 128, 1, FM * FN * kWave>(),                \
-            gemm_lds_bytes<BM, 128, 2, PM * PN * kWave>(), sgemm_kernel<BM, 128, FM, FN, false, 1, 1>,           \
-            sgemm_kernel<BM, 128, FM, FN, true, 1, 1>, sgemm_kernel<BM, 128, PM, PN, false, 2, 1>,               \
-            sgemm_kernel<BM, 128, PM, PN, true, 2, 1>, abft_encode_kernel<BM, 128>                               \
-    }
-
-static const FtClass kFtClasses[HPCDNN_FT_NUM_CLASSES] = {
-    HPCDNN_FT_CLASS(256, 2, 2, 2, 4),  // 0 huge
-    HPCDNN_FT_CLASS(128, 2, 2, 2, 2),  // 1 large
-    HPCDNN_FT_CLASS(64, 2, 2, 2, 2),   // 2 wide
-};
-
-// Kernels that use more than the default 64 KiB of LDS must opt in once per device.
-static int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {
-    if (bytes <= 64 * 1024) return HPCDNN_OK;
-    struct Done {
-        const void* fn;
-        int device;
-    };
-    static std::mutex mu;
-    static Done done[16 * kNumTiles] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return static_cast<int>(e);
-    std::lock_guard<std::mutex> lock(mu);
-    const void* key = reinterpret_cast<const void*>(fn);
-    for (const Done& d : done)
-        if (d.fn == key && d.device == dev) return HPCDNN_OK;
-    e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
-    if (e != hipSuccess) return static_cast<int>(e);
-    for (Done& d : done)
-        if (!d.fn) { d = Done{key, dev}; break; }  // a full table only costs a repeated call
-    return HPCDNN_OK;
-}
 
 struct Plan {
     int tile;
@@ -301,41 +238,6 @@ static RowSplit choose_row_split(int M, int N, int K, int cus) {
     return best;
 }
 
-constexpr int kMaxLda = (1 << 21) - 64;   // 256 * lda * 4 < 2^31
-constexpr int kMaxLdb = (1 << 25) - 1024;  // 16 * ldb * 4 + row < 2^31
-
-static int check_gemm_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
-    if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
-    if (lda < (K > 1 ? K : 1) || ldb < (N > 1 ? N : 1) || ldc < (N > 1 ? N : 1)) return HPCDNN_ERR_INVALID_VALUE;
-    if (M > 0 && N > 0 && !C) return HPCDNN_ERR_INVALID_VALUE;
-    if (M > 0 && N > 0 && K > 0 && (!A || !B)) return HPCDNN_ERR_INVALID_VALUE;
-    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) & 3u)
-        return HPCDNN_ERR_INVALID_VALUE;
-    // byte offsets inside one tile are 32-bit: 256 rows of A, 16 rows of B
-    if (lda > kMaxLda || ldb > kMaxLdb) return HPCDNN_ERR_INVALID_VALUE;
-    return HPCDNN_OK;
-}
-
-static GemmArgs make_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
-                          float alpha, float beta, const TileConfig& cfg) {
-    GemmArgs a{};
-    a.M = M; a.N = N; a.K = K;
-    a.A = A; a.lda = lda; a.B = B; a.ldb = ldb; a.C = C; a.ldc = ldc;
-    a.alpha = alpha; a.beta = beta;
-    a.tiles_m = static_cast<int>(ceil_div(M, cfg.bm));
-    a.tiles_n = static_cast<int>(ceil_div(N, cfg.bn));
-    a.k_chunk = static_cast<int>(ceil_div(K > 0 ? K : 1, cfg.bk)) * cfg.bk;
-    a.partial = nullptr;
-    a.fault_tile = -1;
-    return a;
-}
-
-// The ragged-tile kernel masks the K tail and the columns past N; full tiles with K a multiple of the K step
-// (per slice, which k_chunk guarantees for all but the last) skip that work.
-static bool needs_edge(const GemmArgs& a, const TileConfig& cfg) {
-    return !(a.M % cfg.bm == 0 && a.N % cfg.bn == 0 && a.K % cfg.bk == 0);
-}
-
 static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                      float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split, hipStream_t stream) {
     int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
@@ -392,7 +294,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     }
     const TileConfig& cfg = kTiles[tile];
     if (cfg.wave_split_k && split < -1) return HPCDNN_ERR_INVALID_VALUE;  // whichever way the tile was chosen
-    GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
+    GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg.bm, cfg.bn);
     const int tiles = a.tiles_m * a.tiles_n;
     a.full_tiles = tiles;
     a.tail_split = 1;
@@ -423,7 +325,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         split = static_cast<int>(ceil_div(K, a.k_chunk));  // drop empty slices
         if (split > 1) a.partial = static_cast<float*>(ws);
     }
-    const bool edge = needs_edge(a, cfg);
+    const bool edge = needs_edge(a, cfg.bm, cfg.bn, cfg.bk);
     void (*fn)(const GemmArgs) = edge ? cfg.edge : cfg.plain;
     rc = enable_lds(fn, cfg.lds_bytes);
     if (rc != HPCDNN_OK) return rc;
@@ -433,7 +335,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     rc = launch_status();
     if (rc != HPCDNN_OK) return rc;
     if (tail_tiles > 0) {
-        tail_reduce_kernel<<<dim3(tail_tiles, cfg.bm / 32), 256, 0, stream>>>(M, N, cfg.bm, cfg.bn, a.tiles_m, a.tiles_n,
+        tail_reduce_kernel<><<<dim3(tail_tiles, cfg.bm / 32), 256, 0, stream>>>(M, N, cfg.bm, cfg.bn, a.tiles_m, a.tiles_n,
                                                                              a.full_tiles, a.tail_split, a.tail_partial, C,
                                                                              ldc, alpha, beta);
         return launch_status();
@@ -444,7 +346,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     int rgrid = static_cast<int>(ceil_div(total, 256));
     const int cap = device_cus() * 8;
     if (rgrid > cap) rgrid = cap;
-    splitk_reduce_kernel<<<rgrid, 256, 0, stream>>>(M, N, split, static_cast<const float*>(ws), C, ldc, alpha, beta);
+    splitk_reduce_kernel<><<<rgrid, 256, 0, stream>>>(M, N, split, static_cast<const float*>(ws), C, ldc, alpha, beta);
     return launch_status();
 }
 
@@ -497,226 +399,7 @@ extern "C" int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int*
     return HPCDNN_OK;
 }
 
-extern "C" int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn) {
-    if (tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
-    if (bm) *bm = kFtClasses[tile_class].bm;
-    if (bn) *bn = kFtClasses[tile_class].bn;
-    return HPCDNN_OK;
-}
-
-extern "C" int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N) {
-    if (M < 0 || N < 0 || tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return 0;
-    return static_cast<int>(ceil_div(M, kFtClasses[tile_class].bm) * ceil_div(N, kFtClasses[tile_class].bn));
-}
-
-extern "C" int hpcdnn_ft_num_tiles(int M, int N) { return hpcdnn_ft_num_tiles_ex(0, M, N); }
-
-// ABFT with a workspace splits the tiles of a partial last round of CUs along K, like plain SGEMM's tail split: every
-// slice is a workgroup that verifies (and corrects) its own partial product - the checksums are linear in K - and
-// writes it raw; tail_reduce_kernel adds the slices, ft_tail_status_kernel merges their records.  With fewer tiles
-// than half the CUs every tile is split.  Returns the number of ways (1: no split) and the tiles it applies to.
-struct FtTail {
-    int ways, tiles;
-};
-static FtTail ft_tail_plan(const FtClass& fc, int M, int N, int K) {
-    const int cus = device_cus();
-    const int64_t tiles = ceil_div(M, fc.bm) * ceil_div(N, fc.bn);
-    const int64_t r = tiles % cus;
-    if (r == 0 || 2 * r > cus) return FtTail{1, 0};
-    int64_t s = cus / r;
-    const int64_t most = K / (16 * kGemmBK);  // at least 16 K steps per slice: each slice pays a verification
-    if (s > most) s = most;
-    if (s > 8) s = 8;
-    if (s < 2) return FtTail{1, 0};
-    return FtTail{static_cast<int>(s), static_cast<int>(r)};
-}
-static size_t ft_enc_bytes(const FtClass& fc, int M, int N, int K) {
-    const size_t b = static_cast<size_t>(ceil_div(M, fc.bm) + ceil_div(N, fc.bn)) * ft_enc_ld(K) * sizeof(float);
-    return (b + 15) & ~static_cast<size_t>(15);
-}
-static size_t ft_tail_bytes(const FtClass& fc, const FtTail& t) {
-    return t.ways < 2 ? 0
-                      : static_cast<size_t>(t.tiles) * t.ways * (static_cast<size_t>(fc.bm) * fc.bn * sizeof(float) + sizeof(hpcdnn_ft_status));
-}
-
-// The class with the shortest predicted run (workspace variant): rounds of tiles over the CUs times the tile height
-// (all classes are 128 columns wide), a partial last round counting for what its K split leaves of it plus the
-// second pass over those tiles, with the measured efficiency of the smaller tiles relative to the 256-row one.
-extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
-    // measured on squares 1024 ... 6144: the 128-row class keeps up with the 256-row one (two of its workgroups share a CU
-    // and cover each other's verification), the 64-row class runs 4-5 % behind
-    static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 1.0, 0.955};
-    const int cus = device_cus();
-    int best = 0;
-    double best_cost = 1e300;
-    for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
-        const int64_t tiles = hpcdnn_ft_num_tiles_ex(c, M, N);
-        const FtTail tail = ft_tail_plan(kFtClasses[c], M, N, K);
-        double rounds = static_cast<double>(ceil_div(tiles > 0 ? tiles : 1, cus));
-        if (tail.ways >= 2)
-            rounds = static_cast<double>(tiles / cus) + static_cast<double>(ceil_div(static_cast<int64_t>(tail.tiles) * tail.ways, cus)) / tail.ways + 0.06;
-        const double cost = rounds * kFtClasses[c].bm / rel_eff[c];
-        if (cost < best_cost) { best_cost = cost; best = c; }
-    }
-    return best;
-}
-
-// Fault-free residuals are the FP32 rounding of the accumulators added over a tile line; for operands uniform in
-// [-1, 1] their maximum over a whole matrix grows linearly with K (measured 4.0e-7 ... 4.9e-7 per unit of K from
-// K = 256 to 65536).  The default leaves a factor of two to that and stays below the 1e-2 faults at K = 4096.
-extern "C" float hpcdnn_ft_default_tau(int K) {
-    const int k = K > 64 ? K : 64;
-    return 1.1e-6f * static_cast<float>(k);
-}
-
-static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
-    const FtClass& fc = kFtClasses[tile_class];
-    return ft_enc_bytes(fc, M, N, K) + ft_tail_bytes(fc, ft_tail_plan(fc, M, N, K));
-}
-
-extern "C" int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
-                                  float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
-                                  void* ws, size_t ws_bytes, int tile_class, void* stream) {
-    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
-    if (rc != HPCDNN_OK) return rc;
-    if (tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
-    if (M == 0 || N == 0) return HPCDNN_OK;
-    const FtClass& fc = kFtClasses[tile_class];
-    TileConfig cfg{};
-    cfg.bm = fc.bm;
-    cfg.bn = fc.bn;
-    cfg.bk = kGemmBK;
-    GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, cfg);
-    // tau > 0: absolute; tau == 0: the absolute default for unit-range data; tau < 0: scaled to the data, the
-    // threshold of a line of n elements being -tau * 4.3 FP32 rounding units * sqrt(max(K, 64)) * sqrt(n) * the larger
-    // of the line's and the tile's mean |accumulator|
-    a.tau = (tau > 0.f) ? tau : (tau == 0.f ? hpcdnn_ft_default_tau(K) : 0.f);
-    a.tau_rel = (tau < 0.f) ? -tau * 2.56e-7f * sqrtf(static_cast<float>(K > 64 ? K : 64)) : 0.f;
-    a.status = status;
-    if (inject) {
-        if (inject->tile < 0 || inject->tile >= a.tiles_m * a.tiles_n || inject->row < 0 || inject->row >= fc.bm ||
-            inject->col < 0 || inject->col >= fc.bn)
-            return HPCDNN_ERR_INVALID_VALUE;
-        a.fault_tile = inject->tile;
-        a.fault_row = inject->row;
-        a.fault_col = inject->col;
-        a.fault_delta = inject->delta;
-    }
-    const bool edge = needs_edge(a, cfg);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
-    // With a workspace the checksum vectors of A and B are formed once per tile row / tile column by a small
-    // bandwidth-bound kernel and the main loop only reads them; without one every workgroup forms them itself.
-    if (ws && K > 0) {
-        const size_t enc_bytes = ft_enc_bytes(fc, M, N, K);
-        if (ws_bytes < enc_bytes || (reinterpret_cast<uintptr_t>(ws) & 15u)) return HPCDNN_ERR_WORKSPACE;
-        // the K split of a partial last round is taken when the workspace has room for it
-        FtTail tail = ft_tail_plan(fc, M, N, K);
-        if (ws_bytes < enc_bytes + ft_tail_bytes(fc, tail)) tail = FtTail{1, 0};
-        a.enc_ld = ft_enc_ld(K);
-        float* enc_a = static_cast<float*>(ws);
-        float* enc_b = enc_a + static_cast<size_t>(a.tiles_m) * a.enc_ld;
-        a.enc_a = enc_a;
-        a.enc_b = enc_b;
-        const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
-        hipLaunchKernelGGL(fc.encode, dim3(k_blocks * (a.tiles_m + a.tiles_n)), dim3(1024), 0, s, M, N, K, A, lda, B, ldb,
-                           enc_a, enc_b, a.enc_ld, k_blocks, a.tiles_m);
-        rc = launch_status();
-        if (rc != HPCDNN_OK) return rc;
-        void (*fn)(const GemmArgs) = edge ? fc.pre_edge : fc.pre_plain;
-        rc = enable_lds(fn, fc.lds_pre);
-        if (rc != HPCDNN_OK) return rc;
-        const int tiles = a.tiles_m * a.tiles_n;
-        a.full_tiles = tiles;
-        a.tail_split = 1;
-        if (tail.ways >= 2) {
-            a.tail_k_chunk = static_cast<int>(ceil_div(ceil_div(K, tail.ways), kGemmBK)) * kGemmBK;
-            tail.ways = static_cast<int>(ceil_div(K, a.tail_k_chunk));  // drop empty slices
-        }
-        if (tail.ways >= 2) {
-            a.full_tiles = tiles - tail.tiles;
-            a.tail_split = tail.ways;
-            a.tail_partial = reinterpret_cast<float*>(static_cast<char*>(ws) + enc_bytes);
-            a.tail_status = reinterpret_cast<hpcdnn_ft_status*>(a.tail_partial + static_cast<size_t>(tail.tiles) * tail.ways * fc.bm * fc.bn);
-            grid = dim3(a.full_tiles + tail.tiles * tail.ways, 1, 1);
-        }
-        hipLaunchKernelGGL(fn, grid, dim3(fc.threads_pre), fc.lds_pre, s, a);
-        rc = launch_status();
-        if (rc != HPCDNN_OK || a.tail_split < 2) return rc;
-        tail_reduce_kernel<<<dim3(tail.tiles, fc.bm / 32), 256, 0, s>>>(M, N, fc.bm, fc.bn, a.tiles_m, a.tiles_n, a.full_tiles,
-                                                                       a.tail_split, a.tail_partial, C, ldc, alpha, beta);
-        rc = launch_status();
-        if (rc != HPCDNN_OK || !status) return rc;
-        ft_tail_status_kernel<<<static_cast<int>(ceil_div(tail.tiles, 64)), 64, 0, s>>>(tail.tiles, a.tail_split, a.tiles_m, a.tiles_n,
-                                                                                      a.full_tiles, a.tail_status, status);
-        return launch_status();
-    }
-    void (*fn)(const GemmArgs) = edge ? fc.fused_edge : fc.fused_plain;
-    rc = enable_lds(fn, fc.lds_fused);
-    if (rc != HPCDNN_OK) return rc;
-    hipLaunchKernelGGL(fn, grid, dim3(fc.threads_fused), fc.lds_fused, s, a);
-    return launch_status();
-}
-
-extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
-                               float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
-                               void* ws, size_t ws_bytes, void* stream) {
-    return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws, ws_bytes, 0, stream);
-}
-
-// ---- ABFT SGEMM for callers that can neither allocate nor pass a workspace: the checksum vectors (and, when they
-// fit, the K slices of a partial last round) live in a fixed device array of this library.  Every device the
-// library runs on holds its own copy of the array at its own address, looked up once per device.
-static __device__ __align__(256) unsigned char scratch[HPCDNN_FT_STATIC_SCRATCH_BYTES];
-
-static int static_scratch_address(void** out) {
-    constexpr int kMaxDevices = 64;
-    static std::mutex mu;
-    static void* address[kMaxDevices] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return static_cast<int>(e);
-    if (dev < 0 || dev >= kMaxDevices) return HPCDNN_ERR_INVALID_VALUE;
-    std::lock_guard<std::mutex> lock(mu);
-    if (!address[dev]) {
-        void* p = nullptr;
-        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // the address on the current device
-        if (e != hipSuccess) return static_cast<int>(e);
-        if (!p) return HPCDNN_ERR_WORKSPACE;
-        address[dev] = p;
-    }
-    *out = address[dev];
-    return HPCDNN_OK;
-}
-
-extern "C" int hpcdnn_ft_sgemm_static(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
-                                      int ldc, float alpha, float beta, float tau, const hpcdnn_fault* inject,
-                                      hpcdnn_ft_status* status, void* stream) {
-    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
-    if (rc != HPCDNN_OK) return rc;
-    if (M == 0 || N == 0) return HPCDNN_OK;
-    // the checksum vectors of the 256 x 128 class must fit; beyond that the call is refused, never silently slower
-    if (K > 0 && ft_enc_bytes(kFtClasses[0], M, N, K) > HPCDNN_FT_STATIC_SCRATCH_BYTES) return HPCDNN_ERR_WORKSPACE;
-    void* ws = nullptr;
-    rc = static_scratch_address(&ws);
-    if (rc != HPCDNN_OK) return rc;
-    // Nothing in the array has to start at zero: the pre-pass rewrites every word of the checksum vectors the GEMM
-    // reads (their zero padding included), and the K slices and their records are written before they are read.
-    return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws,
-                              HPCDNN_FT_STATIC_SCRATCH_BYTES, 0, stream);
-}
-
 namespace hpcdnn {
-// enough for any tile class (the lowest class has the most tile rows)
-size_t ft_workspace_bytes(int M, int N, int K) {
-    size_t most = 0;
-    for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
-        const size_t b = ft_class_workspace_bytes(c, M, N, K);
-        if (b > most) most = b;
-    }
-    return most;
-}
 size_t sgemm_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     const Plan plan = choose_plan(M, N, K, true, static_cast<size_t>(-1));

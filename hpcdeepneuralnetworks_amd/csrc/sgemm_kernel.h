@@ -33,7 +33,9 @@
 // keep the compiler from regrouping them.
 //
 // With FT != 0 the kernel is the online-ABFT variant: see "ABFT encode" in the
-// main loop and "ABFT verification" after it.
+// main loop and "ABFT verification" after it.  GRAN = 1 keeps one checksum pair
+// per wave tile instead of one per workgroup tile; CADENCE verifies every
+// check_interval values of k inside the K loop as well as after it.
 #pragma once
 
 #include <type_traits>
@@ -41,6 +43,8 @@
 #include "common.h"
 
 namespace hpcdnn {
+
+constexpr int kMaxFaults = HPCDNN_FT_MAX_FAULTS;
 
 struct GemmArgs {
     int M, N, K;
@@ -62,11 +66,17 @@ struct GemmArgs {
     // ABFT
     float tau;      // absolute residual threshold; 0 = relative mode
     float tau_rel;  // relative mode: threshold of a line = tau_rel * sum |accumulators of the line| / sqrt(elements in it)
-    int fault_tile, fault_row, fault_col;
-    float fault_delta;
+    int n_faults;   // test faults: delta is added to accumulator (row, col) of workgroup tile `tile` before verification `check`
+    struct {
+        int tile, row, col;
+        float delta;
+        int check;
+    } faults[kMaxFaults];
+    int check_interval;          // CADENCE kernels: values of k between two verifications, a multiple of the K step
+    int status_rows, status_ld;  // records are laid out as a status_rows x status_ld grid of check tiles
     hpcdnn_ft_status* status;
-    const float* enc_a;  // FT == 2: [tiles_m][enc_ld] column sums of A over each tile's rows
-    const float* enc_b;  // FT == 2: [tiles_n][enc_ld] row sums of B over each tile's columns
+    const float* enc_a;  // FT == 2: [row groups][enc_ld] column sums of A over the rows of each check tile
+    const float* enc_b;  // FT == 2: [column groups][enc_ld] row sums of B over the columns of each check tile
     int enc_ld;          // row length: K rounded up to the K step, plus two K steps of zeros
 };
 
@@ -74,13 +84,26 @@ constexpr int kGemmBK = 16;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tiles share A and B panels
 
-template <int BM, int BN, int FT = 0, int THREADS = 256>
+// LDS the ABFT verification needs (it reuses the staging buffers once the K loop has drained): FP64 partials of the
+// reference checksums, observed line sums and their absolute counterparts per wave row / wave column, one residual
+// per line, one record per check tile, per-wave sums of |acc| per check tile.  GM x GN check tiles per workgroup tile.
+template <int BM, int BN, int WGM, int WGN, int GM, int GN>
+constexpr size_t ft_verify_lds_bytes() {
+    constexpr size_t threads = static_cast<size_t>(WGM) * WGN * 64;
+    constexpr size_t ccp = 2 * threads / 64, crp = kGemmBK / 4, lines = static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
+    return sizeof(double) * (GM * ccp * BN + GN * crp * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + lines) +
+           32 * GM * GN + sizeof(float) * GM * GN * (threads / 64);
+}
+
+template <int BM, int BN, int FT = 0, int THREADS = 256, int WGM = 2, int WGN = 2, int GRAN = 0>
 constexpr size_t gemm_lds_bytes() {
     // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x one column
     // sum per wave, 16 row sums) and a dump area for the branch-free predicated writes of the lanes that
     // publish nothing (one word per thread plus the reach of the strided writes)
-    return sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8)) +
+    constexpr size_t staging = sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8)) +
            (FT == 1 ? sizeof(float) * (2 * (kGemmBK * (THREADS / 64) + kGemmBK) + THREADS + 2 * kGemmBK * (THREADS / 64)) : 0);
+    constexpr size_t verify = FT ? ft_verify_lds_bytes<BM, BN, WGM, WGN, GRAN ? WGM : 1, GRAN ? WGN : 1>() : 0;
+    return staging > verify ? staging : verify;
 }
 
 template <int N, class F>
@@ -121,10 +144,21 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
 // NSLOT: staging register sets.  K step t + 1 waits in one of them while steps up to t + NSLOT are on their way from
 // memory.  Two are enough while a K step takes longer than a trip to memory (big tiles) or the operands come from
 // L2; a small tile that streams an operand from HBM with one workgroup per CU needs its loads further ahead.
-template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS, int NSLOT = 2>
+//
+// GRAN (ABFT only): 0 = one checksum pair, one verification and one status record per workgroup tile; 1 = per wave
+// tile (BM / WGM) x (BN / WGN): every wave tile is verified, located and corrected on its own, so one fault per wave
+// tile is correctable.  Needs the pre-encoded checksum vectors (FT == 2), one per wave row / wave column.
+// CADENCE (ABFT only): the K loop runs in intervals of p.check_interval; after each interval the pipeline drains,
+// the accumulators are verified against the references of the k range done so far, and the references are
+// re-synchronised, as the reference kernel does every 256 k (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:143,263-271).
+template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS, int NSLOT = 2, int GRAN = 0, bool CADENCE = false>
 __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
     static_assert(NSLOT == 2 || (FT == 0 && NSLOT % 2 == 0), "the ABFT loop is written for two staging sets");
+    static_assert(FT != 0 || (GRAN == 0 && !CADENCE), "granularity and cadence belong to the ABFT kernels");
+    static_assert(GRAN == 0 || FT == 2, "wave-tile checksums come from the pre-encoded vectors");
+    constexpr int GM = GRAN ? WGM : 1, GN = GRAN ? WGN : 1;  // check tiles per workgroup tile
+    constexpr int CM = BM / GM, CN = BN / GN;                // check tile
     constexpr int kGemmThreads = WGM * WGN * kWave;
     static_assert(WGM * WGN == 4 || WGM * WGN == 8, "four or eight waves per workgroup");
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -167,9 +201,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     }
     tile_of_block(tile_id, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int kbeg = k_slice * k_chunk;
-    const int kend = (p.K - kbeg < k_chunk) ? p.K : kbeg + k_chunk;
-    const int nkt = (kend - kbeg + BK - 1) / BK;
+    // the K range of one pass of the pipeline: the slice, or one verification interval of it
+    int kbeg = k_slice * k_chunk;
+    int kend = (p.K - kbeg < k_chunk) ? p.K : kbeg + k_chunk;
+    int nkt = (kend - kbeg + BK - 1) / BK;
 
     // ---- global -> register staging: which 16-byte groups of the A and B tiles this thread moves.
     // Descriptors start at the tile's first element of the current K step and end with the matrix, so that
@@ -212,17 +247,20 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // slots).  The rows of enc_a / enc_b end with two K steps of zeros, so the fetches that run ahead past the
     // end need no bounds: one descriptor per row, a per-thread offset, and a scalar offset that moves on by one
     // K step per fetch.
+    // (with wave-tile checksums the tile's GM / GN rows of the vectors follow each other: one descriptor over all
+    // of them, the row chosen by the scalar offset)
     const __amdgpu_buffer_rsrc_t enc_a_rsrc =
-        make_rsrc(FT == 2 ? p.enc_a + static_cast<int64_t>(tile_m) * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * 4);
+        make_rsrc(FT == 2 ? p.enc_a + static_cast<int64_t>(tile_m) * GM * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * GM * 4);
     const __amdgpu_buffer_rsrc_t enc_b_rsrc =
-        make_rsrc(FT == 2 ? p.enc_b + static_cast<int64_t>(tile_n) * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * 4);
+        make_rsrc(FT == 2 ? p.enc_b + static_cast<int64_t>(tile_n) * GN * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * GN * 4);
+    const int enc_row_bytes = p.enc_ld * 4;
     // a_c of the k rows of B this thread stages: k = tid/32 (and k + 8 with four waves), which the pre-encode kernel
     // stores side by side (order 0, 8, 1, 9, ... inside each K step)
     const int enc_a_voff = B_SLOTS == 2 ? (tid >> 5) * 8 : ((((tid >> 5) & 7) * 2 + (tid >> 8)) * 4);
     const int enc_b_voff = (tid & 3) * 16;  // b_r of the four k values of A this thread stages
     int enc_off = kbeg * 4;
-    float g_ac[2][B_SLOTS];
-    v4f g_br[2];
+    float g_ac[2][GM][B_SLOTS];
+    v4f g_br[2][GN];
     auto gload1 = [&](auto slot, auto part) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P == 0) k_slot[S] = k_loaded;
@@ -235,15 +273,21 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         }
         if constexpr (FT == 2 && P == NGL - 1) {
             static_assert(FT != 2 || B_SLOTS <= 2, "a thread stages one or two k rows of B");
-            if constexpr (B_SLOTS == 2) {
-                typedef float v2f __attribute__((ext_vector_type(2)));
-                const v2f t = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(enc_a_rsrc, enc_a_voff, enc_off, 0));
-                g_ac[S][0] = t[0];
-                g_ac[S][B_SLOTS - 1] = t[1];
-            } else {
-                g_ac[S][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(enc_a_rsrc, enc_a_voff, enc_off, 0));
+#pragma unroll
+            for (int gm = 0; gm < GM; ++gm) {
+                const int soff = enc_off + gm * enc_row_bytes;
+                if constexpr (B_SLOTS == 2) {
+                    typedef float v2f __attribute__((ext_vector_type(2)));
+                    const v2f t = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(enc_a_rsrc, enc_a_voff, soff, 0));
+                    g_ac[S][gm][0] = t[0];
+                    g_ac[S][gm][B_SLOTS - 1] = t[1];
+                } else {
+                    g_ac[S][gm][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(enc_a_rsrc, enc_a_voff, soff, 0));
+                }
             }
-            g_br[S] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_b_rsrc, enc_b_voff, enc_off, 0));
+#pragma unroll
+            for (int gn = 0; gn < GN; ++gn)
+                g_br[S][gn] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_b_rsrc, enc_b_voff, enc_off + gn * enc_row_bytes, 0));
         }
     };
     // Ragged tiles only, applied when the slot is consumed: columns k >= kend of A hold padding, the next K
@@ -306,6 +350,18 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             *reinterpret_cast<v4f*>(Bs + stage * B_STAGE + b_lds[P - A_SLOTS]) = rb[S][P - A_SLOTS];
     };
 
+    // CADENCE: point the staging state at the start of the next verification interval [kbeg, kend)
+    auto k_range_reset = [&]() {
+        a_base = p.A + static_cast<int64_t>(m0) * p.lda + kbeg;
+        b_base = p.B + static_cast<int64_t>(kbeg) * p.ldb + n0;
+        a_left = (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - kbeg)) * 4;
+        b_left = (static_cast<int64_t>(p.K - 1 - kbeg) * p.ldb + (p.N - n0)) * 4;
+        k_loaded = kbeg;
+#pragma unroll
+        for (int i = 0; i < NSLOT; ++i) k_slot[i] = kbeg;
+        enc_off = kbeg * 4;
+    };
+
     // ---- LDS -> fragment registers -> MFMA
     v16f acc[TM][TN];
 #pragma unroll
@@ -365,27 +421,40 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     float* const pub_a = (lane < 4) ? s_apart + (4 * (tid & 3)) * kParts + wave : s_dump;
     float* const pub_b = (lr < B_SLOTS) ? s_br + (tid >> 5) + kHalfWaves * lr : s_dump;
     const int x32_addr = (lane ^ 32) * 4;  // ds_bpermute address of the partner lane in the other half wave
-    double cc_ref[4], cr_ref[A_SLOTS];
-    float cc_lo[B_SLOTS][4], cr_lo[A_SLOTS][4];  // FP32 partials of the running sums, one per staged element
+    // With wave-tile checksums a thread keeps one column sum per wave row gm (its columns lie in one wave column)
+    // and one row sum per wave column gn (its rows lie in one wave row).
+    double cc_ref[GM][4], cr_ref[GN][A_SLOTS];
+    float cc_lo[GM][B_SLOTS][4], cr_lo[GN][A_SLOTS][4];  // FP32 partials of the running sums, one per staged element
 #pragma unroll
-    for (int e = 0; e < 4; ++e) cc_ref[e] = 0.0;
+    for (int gm = 0; gm < GM; ++gm)
 #pragma unroll
-    for (int sl = 0; sl < A_SLOTS; ++sl) cr_ref[sl] = 0.0;
+        for (int e = 0; e < 4; ++e) cc_ref[gm][e] = 0.0;
 #pragma unroll
-    for (int sl = 0; sl < B_SLOTS; ++sl)
+    for (int gn = 0; gn < GN; ++gn)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) cc_lo[sl][e] = 0.f;
+        for (int sl = 0; sl < A_SLOTS; ++sl) cr_ref[gn][sl] = 0.0;
 #pragma unroll
-    for (int sl = 0; sl < A_SLOTS; ++sl)
+    for (int gm = 0; gm < GM; ++gm)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) cr_lo[sl][e] = 0.f;
+        for (int sl = 0; sl < B_SLOTS; ++sl)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cc_lo[gm][sl][e] = 0.f;
+#pragma unroll
+    for (int gn = 0; gn < GN; ++gn)
+#pragma unroll
+        for (int sl = 0; sl < A_SLOTS; ++sl)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cr_lo[gn][sl][e] = 0.f;
     float e_pa[4], e_sw[4];
-    v4f e_t[kPartV4 * B_SLOTS], e_brv;
-    float e_pb0, e_pb1, e_pk, e_swb, e_ac[B_SLOTS];
+    v4f e_t[kPartV4 * B_SLOTS], e_brv[GN];
+    float e_pb0, e_pb1, e_pk, e_swb, e_ac[GM][B_SLOTS];
     const int e_hw = tid >> 5;           // half wave = first k row this thread stages of B
     const int e_class = tid & 3;         // k group (4 k values) this thread stages of A
     constexpr int NPROD = (FT == 1) ? 11 : 0;  // pieces before the barrier
-    constexpr int NCONS = FT ? 6 : 0;          // pieces after the barrier
+    // pieces after the barrier: fetch, combine (FT == 1), column checksums (one piece per wave row), row checksums
+    // (one piece per wave column; two halves of the staged rows with one checksum pair per tile), flush
+    constexpr int NCR = GRAN ? GN : 2;
+    constexpr int NCONS = FT ? 2 + GM + NCR + 1 : 0;
     constexpr int kDppRor4 = 0x124, kDppRor8 = 0x128;  // rotate right inside each row of 16 lanes
 
     auto produce1 = [&](auto slot, auto piece, int par) {
@@ -464,8 +533,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         if constexpr (FT == 2 && E <= 1) {
             if constexpr (E == 0) {
 #pragma unroll
-                for (int sl = 0; sl < B_SLOTS; ++sl) e_ac[sl] = g_ac[S][sl];
-                e_brv = g_br[S];
+                for (int gm = 0; gm < GM; ++gm)
+#pragma unroll
+                    for (int sl = 0; sl < B_SLOTS; ++sl) e_ac[gm][sl] = g_ac[S][gm][sl];
+#pragma unroll
+                for (int gn = 0; gn < GN; ++gn) e_brv[gn] = g_br[S][gn];
             }
         } else if constexpr (E == 0) {
 #pragma unroll
@@ -474,62 +546,69 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
                 for (int v = 0; v < kPartV4; ++v) e_t[kPartV4 * sl + v] = *reinterpret_cast<const v4f*>(row + 4 * v);
             }
-            e_brv = *reinterpret_cast<const v4f*>(br + 4 * e_class);
+            e_brv[0] = *reinterpret_cast<const v4f*>(br + 4 * e_class);
         } else if constexpr (E == 1) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
                 v4f u = e_t[kPartV4 * sl];
 #pragma unroll
                 for (int v = 1; v < kPartV4; ++v) u += e_t[kPartV4 * sl + v];
-                e_ac[sl] = (u.x + u.y) + (u.z + u.w);
-                HPCDNN_PIN(e_ac[sl]);
+                e_ac[0][sl] = (u.x + u.y) + (u.z + u.w);
+                HPCDNN_PIN(e_ac[0][sl]);
             }
-        } else if constexpr (E == 2) {
+        } else if constexpr (E < 2 + GM) {
             // independent accumulators: a wave alone on its SIMD cannot hide the latency of dependent VALU
             // instructions behind other waves
+            constexpr int gm = E - 2;
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {
-                cc_lo[sl][0] = __builtin_fmaf(e_ac[sl], rb[S][sl].x, cc_lo[sl][0]);
-                cc_lo[sl][1] = __builtin_fmaf(e_ac[sl], rb[S][sl].y, cc_lo[sl][1]);
-                cc_lo[sl][2] = __builtin_fmaf(e_ac[sl], rb[S][sl].z, cc_lo[sl][2]);
-                cc_lo[sl][3] = __builtin_fmaf(e_ac[sl], rb[S][sl].w, cc_lo[sl][3]);
+                cc_lo[gm][sl][0] = __builtin_fmaf(e_ac[gm][sl], rb[S][sl].x, cc_lo[gm][sl][0]);
+                cc_lo[gm][sl][1] = __builtin_fmaf(e_ac[gm][sl], rb[S][sl].y, cc_lo[gm][sl][1]);
+                cc_lo[gm][sl][2] = __builtin_fmaf(e_ac[gm][sl], rb[S][sl].z, cc_lo[gm][sl][2]);
+                cc_lo[gm][sl][3] = __builtin_fmaf(e_ac[gm][sl], rb[S][sl].w, cc_lo[gm][sl][3]);
             }
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) HPCDNN_PIN(cc_lo[sl][e]);
-        } else if constexpr (E == 3 || E == 4) {
-            constexpr int lo = (E == 3) ? 0 : A_SLOTS / 2, hi = (E == 3) ? A_SLOTS / 2 : A_SLOTS;
+                for (int e = 0; e < 4; ++e) HPCDNN_PIN(cc_lo[gm][sl][e]);
+        } else if constexpr (E < 2 + GM + NCR) {
+            constexpr int piece = E - 2 - GM;
+            constexpr int gn = GRAN ? piece : 0;
+            constexpr int lo = GRAN ? 0 : (piece == 0 ? 0 : A_SLOTS / 2), hi = GRAN ? A_SLOTS : (piece == 0 ? A_SLOTS / 2 : A_SLOTS);
 #pragma unroll
             for (int sl = lo; sl < hi; ++sl) {
-                cr_lo[sl][0] = __builtin_fmaf(ra[S][sl].x, e_brv.x, cr_lo[sl][0]);
-                cr_lo[sl][1] = __builtin_fmaf(ra[S][sl].y, e_brv.y, cr_lo[sl][1]);
-                cr_lo[sl][2] = __builtin_fmaf(ra[S][sl].z, e_brv.z, cr_lo[sl][2]);
-                cr_lo[sl][3] = __builtin_fmaf(ra[S][sl].w, e_brv.w, cr_lo[sl][3]);
+                cr_lo[gn][sl][0] = __builtin_fmaf(ra[S][sl].x, e_brv[gn].x, cr_lo[gn][sl][0]);
+                cr_lo[gn][sl][1] = __builtin_fmaf(ra[S][sl].y, e_brv[gn].y, cr_lo[gn][sl][1]);
+                cr_lo[gn][sl][2] = __builtin_fmaf(ra[S][sl].z, e_brv[gn].z, cr_lo[gn][sl][2]);
+                cr_lo[gn][sl][3] = __builtin_fmaf(ra[S][sl].w, e_brv[gn].w, cr_lo[gn][sl][3]);
             }
 #pragma unroll
             for (int sl = lo; sl < hi; ++sl)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) HPCDNN_PIN(cr_lo[sl][e]);
+                for (int e = 0; e < 4; ++e) HPCDNN_PIN(cr_lo[gn][sl][e]);
         } else if constexpr (kFlush) {
             // every 16th K step (and after the last one): FP32 partials -> FP64 running sums.  FP64 VALU
             // instructions are twice as expensive as FP32 ones, so this is kept rare.
             if (flush_now) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float t = cc_lo[0][e];
+                for (int gm = 0; gm < GM; ++gm)
 #pragma unroll
-                    for (int sl = 1; sl < B_SLOTS; ++sl) t += cc_lo[sl][e];
-                    cc_ref[e] += static_cast<double>(t);
+                    for (int e = 0; e < 4; ++e) {
+                        float t = cc_lo[gm][0][e];
 #pragma unroll
-                    for (int sl = 0; sl < B_SLOTS; ++sl) cc_lo[sl][e] = 0.f;
-                }
+                        for (int sl = 1; sl < B_SLOTS; ++sl) t += cc_lo[gm][sl][e];
+                        cc_ref[gm][e] += static_cast<double>(t);
 #pragma unroll
-                for (int sl = 0; sl < A_SLOTS; ++sl) {
-                    cr_ref[sl] += static_cast<double>((cr_lo[sl][0] + cr_lo[sl][1]) + (cr_lo[sl][2] + cr_lo[sl][3]));
+                        for (int sl = 0; sl < B_SLOTS; ++sl) cc_lo[gm][sl][e] = 0.f;
+                    }
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) cr_lo[sl][e] = 0.f;
-                }
+                for (int gn = 0; gn < GN; ++gn)
+#pragma unroll
+                    for (int sl = 0; sl < A_SLOTS; ++sl) {
+                        cr_ref[gn][sl] += static_cast<double>((cr_lo[gn][sl][0] + cr_lo[gn][sl][1]) + (cr_lo[gn][sl][2] + cr_lo[gn][sl][3]));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) cr_lo[gn][sl][e] = 0.f;
+                    }
             }
         }
     };
@@ -621,6 +700,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 std::integral_constant<int, Ph % 2>{}, std::false_type{}, masked);
     };
 
+    // One pass of the software pipeline over [kbeg, kend).
+    auto run_k_range = [&]() {
     if (nkt > 0) {
         // prologue: step 0 -> LDS stage 0, step 1 -> staging slot 1, first-half fragments of step 0 -> buffer 0
         static_for<NGL>([&](auto s) { gload1(S0{}, s); });
@@ -667,23 +748,37 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         }
         __syncthreads();  // every wave is done with the staging buffers (the verification below reuses them)
     }
+    };
 
-    // ---- ABFT verification: inject (testing aid), observe, compare, locate, correct
-    if constexpr (FT) {
-        constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;             // partials per column / per row checksum
-        double* const s_ccref = reinterpret_cast<double*>(smem);        // [CCP][BN] reference column checksum partials
-        double* const s_crref = s_ccref + CCP * BN;                     // [CRP][BM] reference row checksum partials
-        float* const s_ccobs = reinterpret_cast<float*>(s_crref + CRP * BM);  // [WGM][BN] observed column sums
+    if constexpr (FT == 0) {
+        run_k_range();
+    } else {
+    // ---- ABFT verification: inject (testing aid), observe, compare, locate, correct, re-synchronise
+    constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;   // partials per column / per row checksum
+    constexpr int NCT = GM * GN;                          // check tiles per workgroup tile
+    constexpr int kRowLines = GN * BM;                    // row lines (gn, m) come first, column lines (gm, n) after them
+    constexpr int kLines = kRowLines + GM * BN;
+    constexpr int LPT = (kLines + kGemmThreads - 1) / kGemmThreads;  // lines per thread
+    static_assert(NCT <= kGemmThreads, "one thread per check tile keeps its record");
+    double line_off[LPT];          // CADENCE: what re-synchronisation has taken out of each of this thread's lines
+#pragma unroll
+    for (int it = 0; it < LPT; ++it) line_off[it] = 0.0;
+    hpcdnn_ft_status rec;          // thread ct < NCT: the record of check tile ct, merged over the verifications
+    rec.flag = 0; rec.row = -1; rec.col = -1; rec.n_bad_rows = 0; rec.n_bad_cols = 0;
+    rec.row_residual = 0.f; rec.col_residual = 0.f; rec.max_clean_residual = 0.f;
+
+    auto verify = [&](int check, bool last) {
+        double* const s_ccref = reinterpret_cast<double*>(smem);        // [GM][CCP][BN] reference column checksum partials
+        double* const s_crref = s_ccref + GM * CCP * BN;                // [GN][CRP][BM] reference row checksum partials
+        float* const s_ccobs = reinterpret_cast<float*>(s_crref + GN * CRP * BM);  // [WGM][BN] observed column sums
         float* const s_crobs = s_ccobs + WGM * BN;                      // [WGN][BM] observed row sums
         float* const s_ccabs = s_crobs + WGN * BM;                      // [WGM][BN] column sums of |accumulators|
         float* const s_crabs = s_ccabs + WGM * BN;                      // [WGN][BM] row sums of |accumulators|
-        float* const s_dr = s_crabs + WGN * BM;                         // [BM] row residuals, then [BN] column residuals
-        int* const s_meta = reinterpret_cast<int*>(s_dr + BM + BN);     // nbr, nbc, bad row, bad col, max clean (float bits)
-        float* const s_tsum = reinterpret_cast<float*>(s_meta + 8);     // [waves] partial sums of |acc| over the tile
-        static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads>() >=
-                          sizeof(double) * (CCP * BN + CRP * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + BM + BN) + 32 +
-                              sizeof(float) * (kGemmThreads / kWave),
-                      "verification scratch fits in the staging buffers");
+        float* const s_dr = s_crabs + WGN * BM;                         // [kLines] residuals
+        int* const s_meta = reinterpret_cast<int*>(s_dr + kLines);      // [NCT][8] nbr, nbc, bad row, bad col, max clean (float bits)
+        float* const s_tsum = reinterpret_cast<float*>(s_meta + 8 * NCT);  // [NCT][waves] partial sums of |acc| over a check tile
+        static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads, WGM, WGN, GRAN>() >= ft_verify_lds_bytes<BM, BN, WGM, WGN, GM, GN>(),
+                      "verification scratch fits in the kernel's LDS");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
 
         // acc element (r, c) of the tile lives in wave (r/WM, c/WN), block (i, j), lane (c%32, (r%32/4)%2), register v
@@ -701,20 +796,31 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             }
         };
 
-        // Soft-error injection: one accumulator, after the K loop, before the checks
-        // (run-time form of `t[2].x += error_inject`, ft_sgemm_huge.cuh:40,145).
-        // (a tile split along K verifies every slice on its own - the checksums are linear in K; the test fault goes
+        // Soft-error injection: one accumulator per fault, after the K loop (or interval), before the checks
+        // (run-time form of `t[2].x += error_inject`, ft_sgemm_huge.cuh:40,145).  A fault aimed at a row or column
+        // of an edge tile that lies outside the matrix is ignored.  A kernel that verifies once injects every fault
+        // before that verification.
+        // (a tile split along K verifies every slice on its own - the checksums are linear in K; the test faults go
         // into its first slice)
-        if (tile_linear == p.fault_tile && k_slice == 0) add_at(p.fault_row, p.fault_col, p.fault_delta);
+#pragma unroll 1
+        for (int f = 0; f < p.n_faults; ++f)
+            if (tile_linear == p.faults[f].tile && k_slice == 0 && (!CADENCE || p.faults[f].check == check) &&
+                m0 + p.faults[f].row < p.M && n0 + p.faults[f].col < p.N)
+                add_at(p.faults[f].row, p.faults[f].col, p.faults[f].delta);
 
-        if (tid == 0) { s_meta[0] = 0; s_meta[1] = 0; s_meta[2] = -1; s_meta[3] = -1; s_meta[4] = 0; }
+        if (tid < NCT) { s_meta[8 * tid] = 0; s_meta[8 * tid + 1] = 0; s_meta[8 * tid + 2] = -1; s_meta[8 * tid + 3] = -1; s_meta[8 * tid + 4] = 0; }
 
         // reference checksums: every thread publishes its partial sums (columns nc..nc+3 over its k rows, its
         // rows over its k group); the residual step below adds the partials in a fixed order
 #pragma unroll
-        for (int e = 0; e < 4; ++e) s_ccref[e_hw * BN + (tid & 31) * 4 + e] = cc_ref[e];
+        for (int gm = 0; gm < GM; ++gm)
 #pragma unroll
-        for (int sl = 0; sl < A_SLOTS; ++sl) s_crref[e_class * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = cr_ref[sl];
+            for (int e = 0; e < 4; ++e) s_ccref[(gm * CCP + e_hw) * BN + (tid & 31) * 4 + e] = cc_ref[gm][e];
+#pragma unroll
+        for (int gn = 0; gn < GN; ++gn)
+#pragma unroll
+            for (int sl = 0; sl < A_SLOTS; ++sl)
+                s_crref[(gn * CRP + e_class) * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = cr_ref[gn][sl];
         // observed column sums of the accumulators (ft_sgemm_huge.cuh:147-154): lane = column.  In relative mode the
         // sums of absolute values go with them: they scale the threshold to the data.
         const bool relative = p.tau <= 0.f;
@@ -764,85 +870,155 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 
         // residual = reference - observed per line; |d| > tau marks the line (ft_sgemm_huge.cuh:200-271).  Relative
         // mode: tau of a line of n elements inside the matrix = tau_rel * sqrt(n) * max(mean |acc| of the line, mean
-        // |acc| of the tile): the rounding noise of a sum of n accumulators grows like sqrt(n) times their magnitude,
-        // and the tile mean stands in for a short or cancelling line whose own accumulators say little about the
-        // size of its terms.  The tile sum is formed in a fixed order (per wave, then wave by wave).
-        const int rows_in = (p.M - m0 < BM) ? p.M - m0 : BM, cols_in = (p.N - n0 < BN) ? p.N - n0 : BN;
-        const float row_scale = p.tau_rel / __builtin_sqrtf(static_cast<float>(cols_in));
-        const float col_scale = p.tau_rel / __builtin_sqrtf(static_cast<float>(rows_in));
-        float row_floor = 0.f, col_floor = 0.f;
+        // |acc| of the check tile): the rounding noise of a sum of n accumulators grows like sqrt(n) times their
+        // magnitude, and the tile mean stands in for a short or cancelling line whose own accumulators say little about
+        // the size of its terms.  The tile sum is formed in a fixed order (per wave, then wave by wave).
+        constexpr int WPGM = WGM / GM, WPGN = WGN / GN;  // wave rows / wave columns per check tile
         if (relative) {
-            float part = 0.f;
-            for (int r = tid; r < BM; r += kGemmThreads)
 #pragma unroll
-                for (int w = 0; w < WGN; ++w) part += s_crabs[w * BM + r];
-            part = wave_sum_lane63(part);
-            if (lane == kWave - 1) s_tsum[wave] = part;
+            for (int ct = 0; ct < NCT; ++ct) {
+                const int gm = ct / GN, gn = ct % GN;
+                float part = 0.f;
+                for (int r = tid; r < CM; r += kGemmThreads)
+#pragma unroll
+                    for (int w = 0; w < WPGN; ++w) part += s_crabs[(gn * WPGN + w) * BM + gm * CM + r];
+                part = wave_sum_lane63(part);
+                if (lane == kWave - 1) s_tsum[ct * (kGemmThreads / kWave) + wave] = part;
+            }
             __syncthreads();
-            float total = 0.f;
-#pragma unroll
-            for (int w = 0; w < kGemmThreads / kWave; ++w) total += s_tsum[w];
-            const float mean = total / (static_cast<float>(rows_in) * static_cast<float>(cols_in));
-            row_floor = p.tau_rel * __builtin_sqrtf(static_cast<float>(cols_in)) * mean;
-            col_floor = p.tau_rel * __builtin_sqrtf(static_cast<float>(rows_in)) * mean;
         }
-        for (int line = tid; line < BM + BN; line += kGemmThreads) {
-            const bool is_row = line < BM;
-            const int idx = is_row ? line : line - BM;
-            double ref = 0.0, obs = 0.0;
-            float mag = 0.f;
-            if (is_row) {
+        double d_line[LPT];
 #pragma unroll
-                for (int w = 0; w < CRP; ++w) ref += s_crref[w * BM + idx];
+        for (int it = 0; it < LPT; ++it) {
+            const int line = tid + it * kGemmThreads;
+            d_line[it] = 0.0;
+            if (line < kLines) {
+                const bool is_row = line < kRowLines;
+                // row line (gn, idx): row idx of the tile against wave column gn; column line (gm, idx) likewise
+                const int grp = is_row ? line / BM : (line - kRowLines) / BN;
+                const int idx = is_row ? line - grp * BM : (line - kRowLines) - grp * BN;
+                const int gm = is_row ? idx / CM : grp, gn = is_row ? grp : idx / CN;
+                const int ct = gm * GN + gn;
+                int rows_in = p.M - (m0 + gm * CM), cols_in = p.N - (n0 + gn * CN);
+                rows_in = rows_in < CM ? rows_in : CM;
+                cols_in = cols_in < CN ? cols_in : CN;
+                double ref = 0.0, obs = 0.0;
+                float mag = 0.f;
+                if (is_row) {
 #pragma unroll
-                for (int w = 0; w < WGN; ++w) obs += static_cast<double>(s_crobs[w * BM + idx]);
+                    for (int w = 0; w < CRP; ++w) ref += s_crref[(grp * CRP + w) * BM + idx];
 #pragma unroll
-                for (int w = 0; w < WGN; ++w) mag += s_crabs[w * BM + idx];
-            } else {
+                    for (int w = 0; w < WPGN; ++w) obs += static_cast<double>(s_crobs[(grp * WPGN + w) * BM + idx]);
 #pragma unroll
-                for (int w = 0; w < CCP; ++w) ref += s_ccref[w * BN + idx];
+                    for (int w = 0; w < WPGN; ++w) mag += s_crabs[(grp * WPGN + w) * BM + idx];
+                } else {
 #pragma unroll
-                for (int w = 0; w < WGM; ++w) obs += static_cast<double>(s_ccobs[w * BN + idx]);
+                    for (int w = 0; w < CCP; ++w) ref += s_ccref[(grp * CCP + w) * BN + idx];
 #pragma unroll
-                for (int w = 0; w < WGM; ++w) mag += s_ccabs[w * BN + idx];
+                    for (int w = 0; w < WPGM; ++w) obs += static_cast<double>(s_ccobs[(grp * WPGM + w) * BN + idx]);
+#pragma unroll
+                    for (int w = 0; w < WPGM; ++w) mag += s_ccabs[(grp * WPGM + w) * BN + idx];
+                }
+                const double d = (CADENCE ? ref - line_off[it] : ref) - obs;
+                d_line[it] = d;
+                if (rows_in > 0 && cols_in > 0) {  // check tiles of an edge tile that lie outside the matrix have no lines
+                    double tau = static_cast<double>(p.tau);
+                    if (relative) {
+                        float total = 0.f;
+#pragma unroll
+                        for (int w = 0; w < kGemmThreads / kWave; ++w) total += s_tsum[ct * (kGemmThreads / kWave) + w];
+                        const float mean = total / (static_cast<float>(rows_in) * static_cast<float>(cols_in));
+                        const float n_line = static_cast<float>(is_row ? cols_in : rows_in);
+                        const float own = mag * (p.tau_rel / __builtin_sqrtf(n_line));
+                        const float floor = p.tau_rel * __builtin_sqrtf(n_line) * mean;
+                        tau = static_cast<double>(own > floor ? own : floor);
+                    }
+                    if (fabs(d) > tau) {
+                        atomicAdd(&s_meta[8 * ct + (is_row ? 0 : 1)], 1);
+                        atomicMax(&s_meta[8 * ct + (is_row ? 2 : 3)], idx);
+                    } else {
+                        atomicMax(&s_meta[8 * ct + 4], __float_as_int(static_cast<float>(fabs(d))));
+                    }
+                }
+                s_dr[line] = static_cast<float>(d);
             }
-            const float own = mag * (is_row ? row_scale : col_scale), floor = is_row ? row_floor : col_floor;
-            const double tau = relative ? static_cast<double>(own > floor ? own : floor) : static_cast<double>(p.tau);
-            const double d = ref - obs;
-            if (fabs(d) > tau) {
-                atomicAdd(&s_meta[is_row ? 0 : 1], 1);
-                atomicMax(&s_meta[is_row ? 2 : 3], idx);
-            } else {
-                atomicMax(&s_meta[4], __float_as_int(static_cast<float>(fabs(d))));
-            }
-            s_dr[line] = static_cast<float>(d);  // column residuals follow the row residuals
         }
         __syncthreads();
 
-        // locate: one faulty row x one faulty column (ft_sgemm_huge.cuh:273-296); correct with the signed
-        // row residual (the reference's round(|residual|), :358, only fits its +1.0 test fault)
-        const int nbr = s_meta[0], nbc = s_meta[1], bad_r = s_meta[2], bad_c = s_meta[3];
-        int flag = 0;
-        if (nbr == 1 && nbc == 1) {
-            flag = 1;
-            add_at(bad_r, bad_c, s_dr[bad_r]);
-        } else if (nbr != 0 || nbc != 0) {
-            flag = 2;
+        // locate: one faulty row x one faulty column of a check tile (ft_sgemm_huge.cuh:273-296); correct with the
+        // signed row residual (the reference's round(|residual|), :358, only fits its +1.0 test fault)
+#pragma unroll 1
+        for (int ct = 0; ct < NCT; ++ct) {
+            const int gn = ct % GN;
+            if (s_meta[8 * ct] == 1 && s_meta[8 * ct + 1] == 1) {
+                const int bad_r = s_meta[8 * ct + 2], bad_c = s_meta[8 * ct + 3];
+                add_at(bad_r, bad_c, s_dr[gn * BM + bad_r]);
+            }
         }
-        if (tid == 0 && p.status) {
-            hpcdnn_ft_status st;
-            st.flag = flag;
-            st.row = (flag == 1) ? bad_r : -1;
-            st.col = (flag == 1) ? bad_c : -1;
-            st.n_bad_rows = nbr;
-            st.n_bad_cols = nbc;
-            st.row_residual = (flag == 1) ? s_dr[bad_r] : 0.f;
-            st.col_residual = (flag == 1) ? s_dr[BM + bad_c] : 0.f;
-            st.max_clean_residual = __int_as_float(s_meta[4]);
-            if (tail_out) p.tail_status[tail_slot] = st;
-            else p.status[tile_linear] = st;
+        if constexpr (CADENCE) {
+            // re-synchronise (ft_sgemm_huge.cuh:268-271): every line starts the next interval with what is left of
+            // its residual after the correction taken out of its reference
+#pragma unroll
+            for (int it = 0; it < LPT; ++it) {
+                const int line = tid + it * kGemmThreads;
+                if (line < kLines) {
+                    const bool is_row = line < kRowLines;
+                    const int grp = is_row ? line / BM : (line - kRowLines) / BN;
+                    const int idx = is_row ? line - grp * BM : (line - kRowLines) - grp * BN;
+                    const int gm = is_row ? idx / CM : grp, gn = is_row ? grp : idx / CN;
+                    const int ct = gm * GN + gn;
+                    double fixed = 0.0;
+                    if (s_meta[8 * ct] == 1 && s_meta[8 * ct + 1] == 1 && idx == s_meta[8 * ct + (is_row ? 2 : 3)])
+                        fixed = static_cast<double>(s_dr[gn * BM + s_meta[8 * ct + 2]]);
+                    line_off[it] += d_line[it] - fixed;
+                }
+            }
         }
+        if (tid < NCT) {
+            const int ct = tid, gm = ct / GN, gn = ct % GN;
+            const int nbr = s_meta[8 * ct], nbc = s_meta[8 * ct + 1], bad_r = s_meta[8 * ct + 2], bad_c = s_meta[8 * ct + 3];
+            const int flag = (nbr == 1 && nbc == 1) ? 1 : ((nbr != 0 || nbc != 0) ? 2 : 0);
+            rec.n_bad_rows += nbr;
+            rec.n_bad_cols += nbc;
+            const float clean = __int_as_float(s_meta[8 * ct + 4]);
+            rec.max_clean_residual = clean > rec.max_clean_residual ? clean : rec.max_clean_residual;
+            if (flag == 2) {
+                rec.flag = 2;
+            } else if (flag == 1 && rec.flag == 0) {
+                rec.flag = 1;
+                rec.row = bad_r - gm * CM;
+                rec.col = bad_c - gn * CN;
+                rec.row_residual = s_dr[gn * BM + bad_r];
+                rec.col_residual = s_dr[kRowLines + gm * BN + bad_c];
+            }
+            if (last && p.status) {
+                hpcdnn_ft_status st = rec;
+                if (st.flag == 2) { st.row = -1; st.col = -1; st.row_residual = 0.f; st.col_residual = 0.f; }
+                const int srow = tile_m * GM + gm, scol = tile_n * GN + gn;
+                if (tail_out) p.tail_status[tail_slot] = st;
+                else if (srow < p.status_rows && scol < p.status_ld) p.status[srow * p.status_ld + scol] = st;
+            }
+        }
+        if constexpr (CADENCE) __syncthreads();  // the next interval's prologue writes the staging buffers again
+    };
+
+    if constexpr (CADENCE) {
+        const int slice_end = kend;
+        for (int check = 0;; ++check) {
+            kend = (slice_end - kbeg > p.check_interval) ? kbeg + p.check_interval : slice_end;
+            nkt = (kend - kbeg + BK - 1) / BK;
+            const bool last = kend >= slice_end;
+            if (check > 0) k_range_reset();
+            run_k_range();
+            verify(check, last);
+            if (last) break;
+            kbeg = kend;
+        }
+    } else {
+        run_k_range();
+        verify(0, true);
     }
+    }  // FT != 0
 
     // ---- epilogue
     const int row_base = m0 + wm * WM + lh * 4;  // + i*32 + 8*(v/4) + v%4
@@ -904,6 +1080,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 }
 
 // Fixed-order second phase of split-K: C = alpha * (ws[0] + ws[1] + ...) + beta*C.
+template <int kUnused = 0>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int splits, const float* __restrict__ ws,
                                                             float* __restrict__ C, int ldc, float alpha, float beta) {
     const int64_t total = static_cast<int64_t>(M) * N;
@@ -929,6 +1106,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
 
 // Fixed-order second phase of the tail split: for the tiles after the first full_tiles, C = alpha * (slice 0 +
 // slice 1 + ...) + beta*C.  grid = (tail tiles, bm / 32): one block adds 32 rows of one tile, 4 columns per thread.
+template <int kUnused = 0>
 __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, int bn, int tiles_m, int tiles_n,
                                                           int full_tiles, int splits, const float* __restrict__ partial,
                                                           float* __restrict__ C, int ldc, float alpha, float beta) {
@@ -968,6 +1146,7 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, 
 // slice that could not locate its fault makes the tile uncorrectable (2); otherwise the tile is corrected (1) if any
 // slice corrected an element, and reports the first such slice's location and residuals (more than one corrected
 // slice shows in the counts).
+template <int kUnused = 0>
 __global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int splits, int tiles_m, int tiles_n,
                                                             int full_tiles, const hpcdnn_ft_status* __restrict__ slices,
                                                             hpcdnn_ft_status* __restrict__ status) {
@@ -995,34 +1174,41 @@ __global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int 
     status[tile_m * tiles_n + tile_n] = out;
 }
 
-// ---- ABFT pre-encode: the checksum vectors of the operands, one per tile row / tile column, in one launch of
-// 1024-thread blocks that each cover 256 values of k: the first k_blocks * tiles_m blocks encode A, the rest B.
+// ---- ABFT pre-encode: the checksum vectors of the operands, one per row group (RM rows) / column group (CN
+// columns), in one launch of 1024-thread blocks that each cover 256 values of k: the first k_blocks * row_groups
+// blocks encode A, the rest B (one block per 128 columns, i.e. 128 / CN column groups).  A group is a workgroup tile's
+// rows or columns, or a wave tile's with wave-tile checksums.
 //
-// enc_a[tm][k'] = sum over the rows m of tile row tm (m < M) of A[m][k]; zero for K <= k < enc_ld; k' is k with
+// enc_a[g][k'] = sum over the rows m of row group g (m < M) of A[m][k]; zero for K <= k < enc_ld; k' is k with
 // the order inside each group of 16 changed to 0, 8, 1, 9, ...  Lane q of a wave owns 4 consecutive k, wave w (16
-// of them) owns 16 of the tile's 256 rows; the 16 partials are added in wave order, so the result does not depend
+// of them) owns RM / 16 of the group's rows; the 16 partials are added in wave order, so the result does not depend
 // on timing.
 //
-// enc_b[tn][k] = sum over the columns n of tile column tn (n < N) of B[k][n]; zero for K <= k < enc_ld.  A half
-// wave reads one k row of the tile (32 lanes x 4 columns) and owns 8 of the block's 256 rows.
-template <int BM, int BN>
+// enc_b[g][k] = sum over the columns n of column group g (n < N) of B[k][n]; zero for K <= k < enc_ld.  A half
+// wave reads 128 columns of one k row (32 lanes x 4 columns) and owns 8 of the block's 256 rows; CN / 4 neighbouring
+// lanes share a column group.
+template <int RM, int CN>
 __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
                                                            const float* __restrict__ B, int ldb,
                                                            float* __restrict__ enc_a, float* __restrict__ enc_b,
-                                                           int enc_ld, int k_blocks, int tiles_m) {
-    static_assert(BN == 128, "a half wave covers the tile's columns with one 16-byte load per lane");
-    constexpr int kWaves = 16, kRows = BM / kWaves;
+                                                           int enc_ld, int k_blocks, int row_groups) {
+    static_assert(CN == 128 || CN == 64 || CN == 32, "column groups are 8, 16 or 32 lanes of a half wave");
+    static_assert(RM % 16 == 0, "the rows of a group split evenly over 16 waves");
+    constexpr int kWaves = 16, kRows = RM / kWaves;
     constexpr int kHalves = 2 * kWaves, kRowsPerHalf = 256 / kHalves;
+    constexpr int kGroupLanes = CN / 4, kGroupsPer128 = 128 / CN;
+    static_assert(kRowsPerHalf <= kGroupLanes, "every k row of a half wave has a lane of each group to write it");
     __shared__ v4f part[kWaves][kWave];
-    const int a_blocks = k_blocks * tiles_m;
+    const int a_blocks = k_blocks * row_groups;
     if (static_cast<int>(blockIdx.x) < a_blocks) {
         const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-        const int tile_m = blockIdx.x / k_blocks, m0 = tile_m * BM;
+        const int group = blockIdx.x / k_blocks, m0 = group * RM;
         const int k = ((blockIdx.x % k_blocks) * kWave + lane) * 4;
         const float* base = A + static_cast<int64_t>(m0) * lda;
-        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base, (static_cast<int64_t>(M - 1 - m0) * lda + K) * 4);
+        // a group past the last row (the lower wave tiles of an edge tile) reads nothing and is all zeros
+        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base, m0 < M ? (static_cast<int64_t>(M - 1 - m0) * lda + K) * 4 : 0);
         v4f s = {0.f, 0.f, 0.f, 0.f};
-        if (k < K) {
+        if (k < K && m0 < M) {
             v4f v[kRows];
 #pragma unroll
             for (int r = 0; r < kRows; ++r) v[r] = buffer_load_v4f(rsrc, ((wave * kRows + r) * lda + k) * 4);
@@ -1041,7 +1227,7 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
             for (int w = 1; w < kWaves; ++w) t += part[w][lane];
             // within each K step of 16, k and k + 8 sit side by side: the GEMM thread that stages rows k and
             // k + 8 of the B tile fetches both with one 8-byte load
-            float* dst = enc_a + static_cast<int64_t>(tile_m) * enc_ld + (k & ~15);
+            float* dst = enc_a + static_cast<int64_t>(group) * enc_ld + (k & ~15);
             const int q = k & 15, pos = (q & 7) * 2 + (q >> 3);
             dst[pos] = t.x;
             dst[pos + 2] = t.y;
@@ -1051,7 +1237,7 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
     } else {
         const int bid = blockIdx.x - a_blocks;
         const int lr = threadIdx.x & 31, half = threadIdx.x >> 5;
-        const int tile_n = bid / k_blocks, n0 = tile_n * BN;
+        const int tile_n = bid / k_blocks, n0 = tile_n * 128;
         const int kb = (bid % k_blocks) * 256;
         float s[kRowsPerHalf];
         v4f v[kRowsPerHalf];
@@ -1065,15 +1251,24 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
 #pragma unroll
         for (int i = 0; i < kRowsPerHalf; ++i) {
             const int k = kb + half + kHalves * i;
-            const float t = (v[i].x + v[i].y) + (v[i].z + v[i].w);
-            s[i] = half32_allsum(k < K ? t : 0.f);
+            float t = (v[i].x + v[i].y) + (v[i].z + v[i].w);
+            t = k < K ? t : 0.f;
+            // sum over the lanes of the column group; every lane of the group gets it
+            t += dpp_mov<kDppXor1>(t);
+            t += dpp_mov<kDppXor2>(t);
+            t += dpp_mov<kDppHalfMirror>(t);
+            if constexpr (kGroupLanes >= 16) t += dpp_mov<kDppMirror>(t);
+            if constexpr (kGroupLanes >= 32) t += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, t), 0x401F));
+            s[i] = t;
         }
-        if (lr < kRowsPerHalf) {
+        // lane l of a group writes the group's sum of k row l of this half wave
+        const int in_group = lr % kGroupLanes, group = tile_n * kGroupsPer128 + lr / kGroupLanes;
+        if (in_group < kRowsPerHalf) {
             float out = s[0];
 #pragma unroll
-            for (int i = 1; i < kRowsPerHalf; ++i) out = (lr == i) ? s[i] : out;
-            const int k = kb + half + kHalves * lr;
-            if (k < enc_ld) enc_b[static_cast<int64_t>(tile_n) * enc_ld + k] = out;
+            for (int i = 1; i < kRowsPerHalf; ++i) out = (in_group == i) ? s[i] : out;
+            const int k = kb + half + kHalves * in_group;
+            if (k < enc_ld) enc_b[static_cast<int64_t>(group) * enc_ld + k] = out;
         }
     }
 }

@@ -149,6 +149,14 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * tile's (bad-line counts add up; the location is that of the first slice that
  * corrected something).  A workspace that only holds the checksum vectors
  * (the size without that room) runs without the split.
+ * Accuracy of a corrected element: the correction is the FP32-rounded row
+ * residual, so with a fault of size delta the element ends up within
+ *   |fault-free row residual| + 16 * 2^-24 * |delta|
+ * of its fault-free accumulator (before alpha/beta): the first term is the
+ * rounding noise the threshold is calibrated against (below tau / 2 for the
+ * default), the second the rounding of the FP32 line sums that contain the
+ * fault.  It does not scale with (|A||B|)_ij: for K of a few tens and a large
+ * delta it can exceed the 1e-5 componentwise criterion of the plain product.
  * Replaces ft_sgemm_huge <<<dim3(M/128,N/128),256>>>(M,N,K,A,B,C,alpha,beta)
  * (kernel/ft_sgemm/sgemm.cu:159-165, kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21). */
 int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
@@ -170,6 +178,65 @@ int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, const float
                        float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
                        void* ws, size_t ws_bytes, int tile_class, void* stream);
 int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
+
+/* Checksum granularity and verification cadence (the reference's block- /
+ * warp- / thread-level kernels and its in-loop verification:
+ * kernel/ft_sgemm/include/ft_sgemm_huge.cuh:143,263-271 verifies every 256 k
+ * and re-synchronises; ft_sgemm_huge_warp.cuh:111-207 keeps one checksum pair
+ * per warp tile, ft_sgemm_huge_thread.cuh:106-177 one per thread tile).
+ *
+ * granularity HPCDNN_FT_GRAN_TILE: one checksum pair, one verification and one
+ * status record per workgroup tile of the class (what hpcdnn_ft_sgemm_ex does).
+ * HPCDNN_FT_GRAN_WAVE: one per wave tile, the part of the workgroup tile one
+ * 64-lane wave accumulates on the matrix cores (class 0: 128x32, class 1:
+ * 64x64, class 2: 32x64; hpcdnn_ft_check_tile_info): every wave tile is
+ * verified, located and corrected on its own, so one fault per wave tile is
+ * correctable where tile granularity reports two faults in one 256x128 tile
+ * as uncorrectable.  Needs the workspace (HPCDNN_ERR_WORKSPACE without one).
+ * The wave tile is the finest granularity on this hardware: a matrix-core
+ * instruction spreads its 32x32 result over all 64 lanes, so there is no
+ * per-thread tile to keep checksums for.
+ *
+ * check_interval 0: one verification, after the K loop.  > 0 (a multiple of
+ * 16; the reference uses 256): also every check_interval values of k inside
+ * the K loop, against reference checksums of the k range done so far; after
+ * each verification the references are re-synchronised with the (corrected)
+ * accumulators, so every verification sees what happened since the one
+ * before, and one fault per check tile *per interval* is correctable.  The
+ * record of a check tile merges its verifications: bad-line counts add up,
+ * flag 2 if any verification could not locate its fault, else 1 if any
+ * corrected an element; row, col and the residuals are those of the first
+ * correction.  Tile granularity, class 0 only.
+ *
+ * Check tiles are numbered row-major over the matrix,
+ * t = (i / cm) * ceil(N / cn) + (j / cn); `status` holds
+ * hpcdnn_ft_num_check_tiles() records, and the tile / row / col of a fault
+ * are in check-tile units.  `check` of a fault is the verification (0 = first)
+ * before which it is added; a run that verifies once adds every fault before
+ * that verification.  Faults aimed outside the matrix are ignored. */
+#define HPCDNN_FT_GRAN_TILE 0
+#define HPCDNN_FT_GRAN_WAVE 1
+#define HPCDNN_FT_MAX_FAULTS 4
+typedef struct hpcdnn_ft_fault_at {
+    int32_t tile;
+    int32_t row, col;
+    float delta;
+    int32_t check;
+} hpcdnn_ft_fault_at;
+typedef struct hpcdnn_ft_options {
+    int32_t tile_class;      /* as for hpcdnn_ft_sgemm_ex */
+    int32_t granularity;     /* HPCDNN_FT_GRAN_* */
+    int32_t check_interval;  /* 0, or a positive multiple of 16 */
+    int32_t n_faults;        /* 0 .. HPCDNN_FT_MAX_FAULTS */
+    hpcdnn_ft_fault_at faults[HPCDNN_FT_MAX_FAULTS];
+} hpcdnn_ft_options;
+/* hpcdnn_ft_sgemm_ex with the options above (`opt` is a HOST pointer, NULL =
+ * class 0, tile granularity, one verification, no faults). */
+int hpcdnn_ft_sgemm_opt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                        float alpha, float beta, float tau, const hpcdnn_ft_options* opt, hpcdnn_ft_status* status,
+                        void* ws, size_t ws_bytes, void* stream);
+int hpcdnn_ft_check_tile_info(int tile_class, int granularity, int* cm, int* cn);
+int hpcdnn_ft_num_check_tiles(int tile_class, int granularity, int M, int N);
 int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N);
 int hpcdnn_ft_pick_class(int M, int N, int K);
 /* Threshold hpcdnn_ft_sgemm uses when tau == 0: 1.1e-6 * max(K, 64), twice the

@@ -99,6 +99,9 @@ def _load():
     lib.oracle_ft_sgemm.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
                                     C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int, C.c_int, C.c_float,
                                     C.c_void_p]
+    lib.oracle_ft_sgemm_checked.restype = None
+    lib.oracle_ft_sgemm_checked.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
+                                            C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     lib.oracle_abft_relative_thresholds.restype = None
     lib.oracle_abft_relative_thresholds.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, C.c_float, dp, dp]
     lib.oracle_sgemv_f64.restype = None
@@ -240,6 +243,23 @@ def ft_sgemm(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, tile_m, tile_n, tau, 
     ft, fi, fj, fd = (-1, 0, 0, 0.0) if fault is None else fault
     _load().oracle_ft_sgemm(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, tile_m, tile_n, tau,
                             int(ft), int(fi), int(fj), float(fd), status.ctypes.data_as(C.c_void_p))
+    return status
+
+
+FAULT_AT_DTYPE = np.dtype([("tile", "<i4"), ("row", "<i4"), ("col", "<i4"), ("delta", "<f4"), ("check", "<i4")])
+
+
+def ft_sgemm_checked(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, tile_m, tile_n, tau, check_interval=0, faults=()):
+    """In-place ABFT GEMM model with a verification every ``check_interval`` values of k (0: once, at the end) and
+    re-synchronised references; ``faults`` = iterable of (tile, i, j, delta, check).  Returns the per-tile status array."""
+    ntiles = ((M + tile_m - 1) // tile_m) * ((N + tile_n - 1) // tile_n)
+    status = np.zeros(ntiles, dtype=FT_STATUS_DTYPE)
+    fa = np.zeros(max(len(faults), 1), dtype=FAULT_AT_DTYPE)
+    for i, f in enumerate(faults):
+        fa[i] = (int(f[0]), int(f[1]), int(f[2]), float(f[3]), int(f[4]) if len(f) > 4 else 0)
+    _load().oracle_ft_sgemm_checked(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, tile_m, tile_n, tau,
+                                    int(check_interval), len(faults), fa.ctypes.data_as(C.c_void_p),
+                                    status.ctypes.data_as(C.c_void_p))
     return status
 
 

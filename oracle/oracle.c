@@ -383,6 +383,107 @@ void oracle_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     }
 }
 
+/* One soft error with the verification it precedes: delta is added to accumulator (row, col) of tile `tile` right
+ * before verification number `check` of that tile (0 = the first).  A model run that verifies only once, after the
+ * whole K loop, injects every fault before that one verification. */
+typedef struct {
+    int32_t tile, row, col;
+    float delta;
+    int32_t check;
+} oracle_fault_at;
+
+/* The whole-matrix model with the reference's verification cadence: the accumulators of a tile are verified every
+ * check_interval values of k inside the K loop (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:143, `if (k % 256 == 0)`)
+ * and once more after the last k, against reference checksums that cover the k range done so far; after every
+ * verification the references are re-synchronised with the accumulators (`C_c -= C_c_`, ft_sgemm_huge.cuh:263-271):
+ * what is left of each line's residual after the correction is absorbed, so the next verification sees only what
+ * happened since this one.  (The reference leaves a line that exceeded the threshold unsynchronised and has no
+ * working locate/correct step; here every line is re-synchronised, a located element is corrected first, and a
+ * verification that could not locate its fault marks the tile uncorrectable for good.)
+ * check_interval <= 0: one verification after the K loop (then this is oracle_ft_sgemm with several faults).
+ * The tile's record merges its verifications: bad-line counts add up, flag 2 if any verification was
+ * uncorrectable, else 1 if any corrected an element; row, col and the residuals are those of the first correction;
+ * max_clean_residual is the largest over all verifications. */
+void oracle_ft_sgemm_checked(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                             int ldc, float alpha, float beta, int tile_m, int tile_n, float tau,
+                             int check_interval, int n_faults, const oracle_fault_at* faults,
+                             oracle_ft_status* status) {
+    int ntm = (M + tile_m - 1) / tile_m, ntn = (N + tile_n - 1) / tile_n;
+    int ci = (check_interval > 0 && check_interval < K) ? check_interval : (K > 0 ? K : 1);
+    int checks = (K > 0) ? (K + ci - 1) / ci : 1;
+    #pragma omp parallel for schedule(dynamic, 1)
+    for (int t = 0; t < ntm * ntn; ++t) {
+        int bm = t / ntn, bn = t % ntn;
+        int m0 = bm * tile_m, n0 = bn * tile_n;
+        int tm = (M - m0 < tile_m) ? M - m0 : tile_m;
+        int tn = (N - n0 < tile_n) ? N - n0 : tile_n;
+        float* acc = (float*)calloc((size_t)tm * tn, sizeof(float));
+        double* buf = (double*)calloc((size_t)(tm + tn) * 5, sizeof(double));
+        double *cr_ref = buf, *cc_ref = buf + tm;              /* cumulative references */
+        double *off_r = buf + (tm + tn), *off_c = off_r + tm;  /* what re-synchronisation has absorbed so far */
+        double *dr = buf + 2 * (tm + tn), *dc = dr + tm;
+        double *part_r = buf + 3 * (tm + tn), *part_c = part_r + tm;
+        double *thr = buf + 4 * (tm + tn);
+        oracle_ft_status rec;
+        memset(&rec, 0, sizeof rec);
+        rec.row = rec.col = -1;
+        for (int c = 0; c < checks; ++c) {
+            int k0 = c * ci, k1 = (k0 + ci < K) ? k0 + ci : K;
+            for (int m = 0; m < tm; ++m)
+                for (int k = k0; k < k1; ++k) {
+                    float a = A[(size_t)(m0 + m) * lda + k];
+                    const float* brow = B + (size_t)k * ldb + n0;
+                    float* arow = acc + (size_t)m * tn;
+                    for (int n = 0; n < tn; ++n) arow[n] = fmaf(a, brow[n], arow[n]);
+                }
+            if (k1 > k0) {
+                oracle_abft_reference_checksums(tm, tn, k1 - k0, A + (size_t)m0 * lda + k0, lda,
+                                                B + (size_t)k0 * ldb + n0, ldb, part_r, part_c);
+                for (int m = 0; m < tm; ++m) cr_ref[m] += part_r[m];
+                for (int n = 0; n < tn; ++n) cc_ref[n] += part_c[n];
+            }
+            for (int f = 0; f < n_faults; ++f)
+                if (faults[f].tile == t && (checks == 1 || faults[f].check == c) && faults[f].row < tm && faults[f].col < tn)
+                    acc[(size_t)faults[f].row * tn + faults[f].col] += faults[f].delta;
+            /* residual against the re-synchronised references */
+            for (int m = 0; m < tm; ++m) part_r[m] = cr_ref[m] - off_r[m];
+            for (int n = 0; n < tn; ++n) part_c[n] = cc_ref[n] - off_c[n];
+            oracle_abft_observe(tm, tn, acc, tn, part_r, part_c, dr, dc);
+            oracle_ft_status cur;
+            float fix;
+            if (tau < 0.0f) {
+                oracle_abft_relative_thresholds(tm, tn, K, acc, tn, -tau, thr, thr + tm);
+                fix = oracle_abft_decide_lines(tm, tn, dr, dc, thr, thr + tm, &cur);
+            } else {
+                fix = oracle_abft_decide(tm, tn, dr, dc, tau, &cur);
+            }
+            if (cur.flag == 1) acc[(size_t)cur.row * tn + cur.col] += fix;
+            /* re-synchronise every line with what it shows after the correction */
+            for (int m = 0; m < tm; ++m) off_r[m] += dr[m] - ((cur.flag == 1 && m == cur.row) ? (double)fix : 0.0);
+            for (int n = 0; n < tn; ++n) off_c[n] += dc[n] - ((cur.flag == 1 && n == cur.col) ? (double)fix : 0.0);
+            /* merge */
+            rec.n_bad_rows += cur.n_bad_rows;
+            rec.n_bad_cols += cur.n_bad_cols;
+            if (cur.max_clean_residual > rec.max_clean_residual) rec.max_clean_residual = cur.max_clean_residual;
+            if (cur.flag == 2) rec.flag = 2;
+            else if (cur.flag == 1 && rec.flag == 0) {
+                rec.flag = 1; rec.row = cur.row; rec.col = cur.col;
+                rec.row_residual = cur.row_residual; rec.col_residual = cur.col_residual;
+            }
+        }
+        if (rec.flag == 2) { rec.row = rec.col = -1; rec.row_residual = rec.col_residual = 0.0f; }
+        status[t] = rec;
+        for (int m = 0; m < tm; ++m)
+            for (int n = 0; n < tn; ++n) {
+                float* c = &C[(size_t)(m0 + m) * ldc + n0 + n];
+                float v = alpha * acc[(size_t)m * tn + n];
+                *c = (beta == 0.0f) ? v : fmaf(beta, *c, v);
+            }
+        free(acc);
+        free(buf);
+    }
+}
+
 /* ----------------------------------------------- SGEMV / offline ABFT -- */
 
 /* Row-major SGEMV in FP64 on an M x N matrix: trans = 0: out[m] = alpha *

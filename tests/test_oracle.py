@@ -394,6 +394,117 @@ def test_ft_sgemm_model_detects_and_corrects(oracle_mod, fault):
         assert st["row_residual"][fault[0]] == pytest.approx(-fault[3], abs=1e-4)
 
 
+def test_checked_model_with_one_verification_is_the_plain_model(oracle_mod):
+    M, N, K, tm, tn = 20, 12, 64, 8, 8
+    rng = np.random.default_rng(6)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    c0 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    for tau in (1e-3, -1.0):
+        for fault in (None, (1, 3, 2, 0.5), (5, 3, 1, -20.0)):
+            c1, c2 = c0.copy(), c0.copy()
+            st1 = oracle_mod.ft_sgemm(M, N, K, a, K, b, N, c1, N, 1.5, -0.5, tm, tn, tau, fault)
+            st2 = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c2, N, 1.5, -0.5, tm, tn, tau, 0, [] if fault is None else [fault + (7,)])
+            assert np.array_equal(c1, c2) and np.array_equal(st1, st2)
+            # an interval of K or more is a single verification too
+            c3 = c0.copy()
+            st3 = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c3, N, 1.5, -0.5, tm, tn, tau, K, [] if fault is None else [fault + (0,)])
+            assert np.array_equal(c1, c3) and np.array_equal(st1, st3)
+
+
+def _exact_problem(M, N, K, seed):
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-8, 9, (M, K)).astype(np.float32)
+    b = rng.integers(-8, 9, (K, N)).astype(np.float32)
+    return a, b, a.astype(np.float64) @ b.astype(np.float64)
+
+
+def test_checked_model_corrects_one_fault_per_verification(oracle_mod):
+    """Small-integer operands: accumulators and checksums are exact, so every expectation below is exact.  Two faults
+    in one tile cannot be located by a single verification (two bad rows, two bad columns), but can when they fall
+    into different K intervals; the record adds the bad-line counts and keeps the first location."""
+    M, N, K, tm, tn = 16, 24, 96, 16, 8   # 1 x 3 tiles, three intervals of 32
+    a, b, exact = _exact_problem(M, N, K, 21)
+    faults = [(1, 3, 5, 64.0, 0), (1, 9, 2, -32.0, 2)]
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, 32, faults)
+    assert np.array_equal(c, exact.astype(np.float32))             # both removed
+    assert st["flag"].tolist() == [0, 1, 0]
+    assert (st["row"][1], st["col"][1], st["n_bad_rows"][1], st["n_bad_cols"][1]) == (3, 5, 2, 2)
+    assert (st["row_residual"][1], st["col_residual"][1]) == (-64.0, -64.0)
+    assert st["max_clean_residual"].tolist() == [0.0, 0.0, 0.0]
+    # the same two faults seen by one verification: detected, not correctable, left in C
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, 0, faults)
+    assert st["flag"].tolist() == [0, 2, 0] and (st["n_bad_rows"][1], st["n_bad_cols"][1]) == (2, 2)
+    assert (st["row"][1], st["col"][1]) == (-1, -1)
+    want = exact.copy()
+    want[3, 8 + 5] += 64.0
+    want[9, 8 + 2] -= 32.0
+    assert np.array_equal(c, want.astype(np.float32))
+    # both in the same interval: that verification fails, the tile stays uncorrectable, later ones find nothing new
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, 32,
+                                     [(1, 3, 5, 64.0, 1), (1, 9, 2, -32.0, 1)])
+    assert st["flag"][1] == 2 and (st["n_bad_rows"][1], st["n_bad_cols"][1]) == (2, 2)
+    assert np.array_equal(c, want.astype(np.float32))
+    # an uncorrectable verification followed by a locatable fault: the later fault is still corrected in C
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, 32,
+                                     [(1, 3, 5, 64.0, 0), (1, 9, 2, -32.0, 0), (1, 0, 0, 16.0, 2)])
+    assert st["flag"][1] == 2 and (st["n_bad_rows"][1], st["n_bad_cols"][1]) == (3, 3)
+    assert np.array_equal(c, want.astype(np.float32))
+
+
+def test_checked_model_resynchronises_after_every_verification(oracle_mod):
+    """Two faults of 0.75 tau in one row, in different intervals: each verification sees one of them and absorbs it,
+    so nothing is ever flagged (and both stay in C); a single verification at the end sees 1.5 tau in that row and in
+    two columns.  The residual a verification reports is what happened since the one before."""
+    M, N, K, tm, tn = 8, 8, 64, 8, 8
+    a, b, exact = _exact_problem(M, N, K, 22)
+    tau = 1.0
+    faults = [(0, 2, 1, 0.75, 0), (0, 2, 6, 0.75, 1)]
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, tau, 32, faults)
+    assert st["flag"][0] == 0 and st["max_clean_residual"][0] == 0.75
+    want = exact.copy()
+    want[2, 1] += 0.75
+    want[2, 6] += 0.75
+    assert np.array_equal(c, want.astype(np.float32))
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, tau, 0, faults)
+    assert (st["flag"][0], st["n_bad_rows"][0], st["n_bad_cols"][0]) == (2, 1, 0) and st["max_clean_residual"][0] == 0.75
+    # the interval boundaries are k = 32, 64: a fault before verification 1 is seen by verification 1, not 0
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, tau, 32, [(0, 4, 4, 8.0, 1)])
+    assert (st["flag"][0], st["row"][0], st["col"][0], st["row_residual"][0]) == (1, 4, 4, -8.0)
+    assert np.array_equal(c, exact.astype(np.float32))
+    # a ragged last interval (K = 70: verifications after k = 32, 64, 70) and a fault before the last one
+    a, b, exact = _exact_problem(M, N, 70, 23)
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, 70, a, 70, b, N, c, N, 1.0, 0.0, tm, tn, tau, 32, [(0, 7, 0, -4.0, 2)])
+    assert (st["flag"][0], st["row"][0], st["col"][0]) == (1, 7, 0) and np.array_equal(c, exact.astype(np.float32))
+    # a verification index past the last one never happens: the fault is not injected
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, 70, a, 70, b, N, c, N, 1.0, 0.0, tm, tn, tau, 32, [(0, 7, 0, -4.0, 3)])
+    assert st["flag"][0] == 0 and np.array_equal(c, exact.astype(np.float32))
+
+
+def test_checked_model_references_cover_the_k_range_done_so_far(oracle_mod):
+    """Float operands: the residuals of every verification are rounding noise, far below a fault; an intermediate
+    verification that compared the accumulators of k < 32 with references over all of K (or the other way round)
+    would flag every line."""
+    M, N, K, tm, tn = 24, 16, 200, 8, 16
+    rng = np.random.default_rng(24)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 1e-3, 32, [(2, 1, 9, 0.05, 4)])
+    assert st["flag"].tolist() == [0, 0, 1] and (st["row"][2], st["col"][2]) == (1, 9)
+    assert st["max_clean_residual"].max() < 5e-5
+    assert np.max(np.abs(c - a.astype(np.float64) @ b.astype(np.float64))) < 5e-5
+
+
 @pytest.mark.parametrize("trans", [False, True])
 def test_sgemv_f64_matches_numpy_and_is_not_transposed(oracle_mod, trans):
     M, N, lda = 13, 29, 37
