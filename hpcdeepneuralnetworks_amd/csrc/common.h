@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "hpcdnn.h"
 
 namespace hpcdnn {
@@ -76,6 +78,54 @@ __device__ __forceinline__ float half32_allsum(float v) {
     // swap with lane ^ 16: bit-mask swizzle, and=0x1f or=0 xor=0x10
     v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
     return v;
+}
+
+// Value of lane (l ^ X) for X = 1, 2 (DPP quad permutes) or 4, 8, 16 (bit-mask swizzles).
+template <int X>
+__device__ __forceinline__ float lane_xor(float v) {
+    static_assert(X == 1 || X == 2 || X == 4 || X == 8 || X == 16, "partner inside a 32-lane half");
+    if constexpr (X == 1) return dpp_mov<kDppXor1>(v);
+    else if constexpr (X == 2) return dpp_mov<kDppXor2>(v);
+    else return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x1F | (X << 10)));
+}
+
+// Transposing sum over each 32-lane half of the wave.  On entry every lane holds N values (N = 16 or 32); on return
+// v[0] of lane l holds the sum over the lanes of its half of value l % N.  Each stage halves the values a lane keeps
+// and doubles the lanes summed into them (lane bit b decides which of a pair stays and which travels), so the whole
+// costs N - 1 additions per lane instead of 5 N for N separate all-reduces.  The order of the additions is fixed.
+template <int N>
+__device__ __forceinline__ void half32_transpose_sum(float (&v)[N], int lane) {
+    static_assert(N == 16 || N == 32, "16 or 32 values per lane");
+    auto stage = [&](auto bit, auto count) {
+        constexpr int B = decltype(bit)::value, C = decltype(count)::value;
+        const bool up = (lane >> B) & 1;
+        float send[C / 2];
+#pragma unroll
+        for (int i = 0; i < C / 2; ++i) {
+            send[i] = up ? v[2 * i] : v[2 * i + 1];
+            v[i] = up ? v[2 * i + 1] : v[2 * i];
+        }
+#pragma unroll
+        for (int i = 0; i < C / 2; ++i) send[i] = lane_xor<(1 << B)>(send[i]);
+#pragma unroll
+        for (int i = 0; i < C / 2; ++i) v[i] += send[i];
+    };
+    using std::integral_constant;
+    stage(integral_constant<int, 0>{}, integral_constant<int, N>{});
+    stage(integral_constant<int, 1>{}, integral_constant<int, N / 2>{});
+    stage(integral_constant<int, 2>{}, integral_constant<int, N / 4>{});
+    stage(integral_constant<int, 3>{}, integral_constant<int, N / 8>{});
+    if constexpr (N == 32) stage(integral_constant<int, 4>{}, integral_constant<int, 2>{});
+    else v[0] += lane_xor<16>(v[0]);
+}
+
+// Maximum over each 32-lane half of the wave; every lane of the half gets it.
+__device__ __forceinline__ float half32_allmax(float v) {
+    v = __builtin_fmaxf(v, dpp_mov<kDppXor1>(v));
+    v = __builtin_fmaxf(v, dpp_mov<kDppXor2>(v));
+    v = __builtin_fmaxf(v, dpp_mov<kDppHalfMirror>(v));
+    v = __builtin_fmaxf(v, dpp_mov<kDppMirror>(v));
+    return __builtin_fmaxf(v, lane_xor<16>(v));
 }
 
 // Sum over the whole wave; the total is valid in lane 63 only.

@@ -159,6 +159,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     static_assert(GRAN == 0 || FT == 2, "wave-tile checksums come from the pre-encoded vectors");
     constexpr int GM = GRAN ? WGM : 1, GN = GRAN ? WGN : 1;  // check tiles per workgroup tile
     constexpr int CM = BM / GM, CN = BN / GN;                // check tile
+    static_assert(CM % 32 == 0 && CN % 32 == 0, "check tiles are made of 32x32 blocks");
     constexpr int kGemmThreads = WGM * WGN * kWave;
     static_assert(WGM * WGN == 4 || WGM * WGN == 8, "four or eight waves per workgroup");
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -847,25 +848,44 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 s_ccabs[wm * BN + wn * WN + j * 32 + lr] = sa;
             }
         }
-        // observed row sums (ft_sgemm_huge.cuh:156-171): register = row, summed over the 32 column lanes
+        // observed row sums (ft_sgemm_huge.cuh:156-171): register = row, summed over the 32 column lanes.  The
+        // TM * 16 sums of a lane are reduced together, 32 (or 16) at a time: afterwards lane lr of each half holds
+        // the sum of row number lr of the group, and every lane stores one
+        constexpr int RG = TM >= 2 ? 32 : 16;      // rows reduced together
+        constexpr int NRG = TM * 16 / RG;          // groups per wave tile
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int g = 0; g < NRG; ++g) {
+            float rs[RG], ra_[RG];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                float s = acc[i][0][v], sa = 0.f;
+            for (int e = 0; e < RG; ++e) {
+                const int i = (g * RG + e) / 16, v = (g * RG + e) % 16;
+                float s = acc[i][0][v];
 #pragma unroll
                 for (int j = 1; j < TN; ++j) s += acc[i][j][v];
-                s = half32_allsum(s);
-                if (relative) {
+                rs[e] = s;
+            }
+            half32_transpose_sum<RG>(rs, lane);
+            if (relative) {
+#pragma unroll
+                for (int e = 0; e < RG; ++e) {
+                    const int i = (g * RG + e) / 16, v = (g * RG + e) % 16;
+                    float sa = 0.f;
 #pragma unroll
                     for (int j = 0; j < TN; ++j) sa += __builtin_fabsf(acc[i][j][v]);
-                    sa = half32_allsum(sa);
+                    ra_[e] = sa;
                 }
-                if (lr == 0) {
-                    s_crobs[wn * BM + wm * WM + i * 32 + 8 * (v / 4) + 4 * lh + (v % 4)] = s;
-                    s_crabs[wn * BM + wm * WM + i * 32 + 8 * (v / 4) + 4 * lh + (v % 4)] = sa;
-                }
+                half32_transpose_sum<RG>(ra_, lane);
+            } else {
+                ra_[0] = 0.f;
             }
+            // this lane's row: number e = lr % RG of the group -> block i, register v
+            const int e = g * RG + (lr & (RG - 1)), v = e & 15;
+            const int row = wm * WM + (e >> 4) * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (RG == 32 || lr < RG) {
+                s_crobs[wn * BM + row] = rs[0];
+                s_crabs[wn * BM + row] = ra_[0];
+            }
+        }
         __syncthreads();
 
         // residual = reference - observed per line; |d| > tau marks the line (ft_sgemm_huge.cuh:200-271).  Relative
@@ -892,6 +912,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         for (int it = 0; it < LPT; ++it) {
             const int line = tid + it * kGemmThreads;
             d_line[it] = 0.0;
+            float clean = 0.f;
+            int line_ct = -1;  // check tile of this line, if it has one inside the matrix
             if (line < kLines) {
                 const bool is_row = line < kRowLines;
                 // row line (gn, idx): row idx of the tile against wave column gn; column line (gm, idx) likewise
@@ -937,11 +959,16 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                         atomicAdd(&s_meta[8 * ct + (is_row ? 0 : 1)], 1);
                         atomicMax(&s_meta[8 * ct + (is_row ? 2 : 3)], idx);
                     } else {
-                        atomicMax(&s_meta[8 * ct + 4], __float_as_int(static_cast<float>(fabs(d))));
+                        clean = static_cast<float>(fabs(d));
                     }
+                    line_ct = ct;
                 }
                 s_dr[line] = static_cast<float>(d);
             }
+            // largest residual among the clean lines: the 32 lines of a half wave belong to one check tile (check
+            // tiles are multiples of 32 rows and columns), so one lane per half records their maximum
+            const float half_max = half32_allmax(clean);
+            if (lr == 0 && line_ct >= 0) atomicMax(&s_meta[8 * line_ct + 4], __float_as_int(half_max));
         }
         __syncthreads();
 
