@@ -159,4 +159,11 @@ __device__ __forceinline__ v4f buffer_load_v4f(__amdgpu_buffer_rsrc_t rsrc, int 
     return __builtin_bit_cast(v4f, v);
 }
 
+// The same with the non-temporal hint, for data that is read once (aux bit 1 of the raw buffer instructions).
+__device__ __forceinline__ v4f buffer_load_v4f_nt(__amdgpu_buffer_rsrc_t rsrc, int byte_offset) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 2);
+    return __builtin_bit_cast(v4f, v);
+}
+
 }  // namespace hpcdnn

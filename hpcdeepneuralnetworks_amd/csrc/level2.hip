@@ -8,7 +8,7 @@ namespace hpcdnn {
 constexpr int kGemvThreads = 256;
 constexpr int kGemvWaves = kGemvThreads / kWave;
 constexpr int kGemvColsPerBlock = 4 * kWave;  // one 16-byte load per lane
-constexpr int kGemvMaxChunks = 64;
+constexpr int kGemvMaxChunks = 128;
 
 // y[m] = alpha * sum_n A[m][n] x[n] + beta * y[m].  One wave per group of kGemvRows rows: the rows are read in 1 KiB
 // pieces (one 16-byte load per lane), 8 / kGemvRows pieces of each row in flight, against the same two pieces of x, so x is
@@ -56,6 +56,65 @@ __global__ __launch_bounds__(kGemvThreads) void sgemv_n_kernel(int M, int N, flo
             const float s = wave_sum_lane63((acc[r].x + acc[r].y) + (acc[r].z + acc[r].w));
             if (lane == kWave - 1 && m + r < M) y[m + r] = (beta == 0.f) ? alpha * s : __builtin_fmaf(beta, y[m + r], alpha * s);
         }
+    }
+}
+
+// The same product for matrices with rows of 2048 ... 16384 elements: x is copied to LDS once per workgroup (zeros
+// behind its end), every wave walks one row at a time in pieces of 16 KiB (sixteen 16-byte loads per lane in flight)
+// and multiplies them with x from LDS, so the only traffic to memory is the stream of A.  Workgroup b owns the
+// contiguous rows [b * rows_per_block, ...), wave w every fourth of them.  Measured 6.97 TB/s at 16384^2 against
+// 6.4 for the kernel above, whose x comes from L2 with every piece.
+constexpr int kGemvLdsMaxN = 16384;
+constexpr int kGemvLdsLoads = 16;
+constexpr int kGemvLdsStep = kGemvLdsLoads * kGemvColsPerBlock;  // 4096 columns per wave and pass
+
+__global__ __launch_bounds__(kGemvThreads) void sgemv_n_lds_kernel(int M, int N, int rows_per_block, float alpha,
+                                                                   const float* __restrict__ A, int lda,
+                                                                   const float* __restrict__ x, float beta,
+                                                                   float* __restrict__ y) {
+    extern __shared__ __align__(16) float xs[];  // N rounded up to a multiple of kGemvLdsStep
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int padded = (N + kGemvLdsStep - 1) / kGemvLdsStep * kGemvLdsStep;
+    // 16-byte groups through a descriptor over x (zeros behind its end), eight in flight per thread
+    {
+        const __amdgpu_buffer_rsrc_t xr = make_rsrc(x, static_cast<int64_t>(N) * 4);
+        constexpr int kBatch = 8;
+        for (int i = threadIdx.x * 4; i < padded; i += kBatch * kGemvThreads * 4) {
+            v4f t[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) t[u] = buffer_load_v4f(xr, (i + u * kGemvThreads * 4) * 4);
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u)
+                if (i + u * kGemvThreads * 4 < padded) *reinterpret_cast<v4f*>(xs + i + u * kGemvThreads * 4) = t[u];
+        }
+    }
+    __syncthreads();
+    const int first = blockIdx.x * rows_per_block;
+    const int last = (M - first < rows_per_block) ? M : first + rows_per_block;
+    for (int m = first + wave; m < last; m += kGemvWaves) {
+        const __amdgpu_buffer_rsrc_t ar = make_rsrc(A + static_cast<int64_t>(m) * lda, static_cast<int64_t>(N) * 4);
+        float acc[kGemvLdsLoads];
+#pragma unroll
+        for (int u = 0; u < kGemvLdsLoads; ++u) acc[u] = 0.f;
+        for (int n0 = 0; n0 < N; n0 += kGemvLdsStep) {
+            v4f a[kGemvLdsLoads];
+#pragma unroll
+            for (int u = 0; u < kGemvLdsLoads; ++u) a[u] = buffer_load_v4f_nt(ar, (n0 + u * kGemvColsPerBlock + lane * 4) * 4);
+#pragma unroll
+            for (int u = 0; u < kGemvLdsLoads; ++u) {
+                const v4f xv = *reinterpret_cast<const v4f*>(xs + n0 + u * kGemvColsPerBlock + lane * 4);
+                acc[u] = __builtin_fmaf(a[u].x, xv.x, acc[u]);
+                acc[u] = __builtin_fmaf(a[u].y, xv.y, acc[u]);
+                acc[u] = __builtin_fmaf(a[u].z, xv.z, acc[u]);
+                acc[u] = __builtin_fmaf(a[u].w, xv.w, acc[u]);
+            }
+        }
+        float s = acc[0];
+#pragma unroll
+        for (int u = 1; u < kGemvLdsLoads; ++u) s += acc[u];
+        s = wave_sum_lane63(s);
+        if (lane == kWave - 1) y[m] = (beta == 0.f) ? alpha * s : __builtin_fmaf(beta, y[m], alpha * s);
     }
 }
 
@@ -113,13 +172,81 @@ __global__ __launch_bounds__(kGemvThreads) void sgemv_t_kernel(int M, int N, int
     }
 }
 
+// The transposed product for wide matrices: every *wave* owns a strip of 2048 columns and a chunk of rows, keeps
+// the strip's 2048 partial sums in registers (8 x 4 per lane) and walks its rows two at a time (sixteen 16-byte
+// loads in flight, each row 8 KiB of contiguous memory); no LDS, no barrier.  Partial sums go to
+// partial[chunk][n] and sgemv_t_finish_kernel adds the chunks in order; with a single chunk the wave finishes y.
+// Measured 6.7 TB/s at 16384^2 with 128 chunks (finish included) against 6.1 for the kernel above.
+constexpr int kGemvStripLoads = 8;
+constexpr int kGemvStripCols = kGemvStripLoads * kGemvColsPerBlock;  // 2048
+
+__global__ __launch_bounds__(kGemvThreads) void sgemv_t_strip_kernel(int M, int N, int rows_per_chunk, int strips, int waves,
+                                                                     float alpha, const float* __restrict__ A, int lda,
+                                                                     const float* __restrict__ x, float beta,
+                                                                     float* __restrict__ y, float* __restrict__ partial) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int gw = __builtin_amdgcn_readfirstlane(blockIdx.x * kGemvWaves + threadIdx.x / kWave);
+    if (gw >= waves) return;
+    const int strip = gw % strips, chunk = gw / strips;
+    const int c0 = strip * kGemvStripCols;
+    const int first = chunk * rows_per_chunk;
+    const int last = (M - first < rows_per_chunk) ? M : first + rows_per_chunk;
+    const int64_t row_bytes = static_cast<int64_t>(N - c0) * 4;
+    v4f acc[kGemvStripLoads];
+#pragma unroll
+    for (int u = 0; u < kGemvStripLoads; ++u) acc[u] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int m = first; m < last; m += 2) {
+        v4f a[2][kGemvStripLoads];
+        float xm[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const bool valid = m + q < last;
+            const int mc = valid ? m + q : first;
+            const __amdgpu_buffer_rsrc_t ar = make_rsrc(A + static_cast<int64_t>(mc) * lda + c0, valid ? row_bytes : 0);
+            xm[q] = valid ? x[mc] : 0.f;
+#pragma unroll
+            for (int u = 0; u < kGemvStripLoads; ++u) a[q][u] = buffer_load_v4f_nt(ar, (u * kGemvColsPerBlock + lane * 4) * 4);
+        }
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int u = 0; u < kGemvStripLoads; ++u) {
+                acc[u].x = __builtin_fmaf(a[q][u].x, xm[q], acc[u].x);
+                acc[u].y = __builtin_fmaf(a[q][u].y, xm[q], acc[u].y);
+                acc[u].z = __builtin_fmaf(a[q][u].z, xm[q], acc[u].z);
+                acc[u].w = __builtin_fmaf(a[q][u].w, xm[q], acc[u].w);
+            }
+    }
+#pragma unroll
+    for (int u = 0; u < kGemvStripLoads; ++u) {
+        const float tv[4] = {acc[u].x, acc[u].y, acc[u].z, acc[u].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = c0 + u * kGemvColsPerBlock + lane * 4 + e;
+            if (n < N) {
+                if (partial)
+                    partial[static_cast<int64_t>(chunk) * N + n] = tv[e];
+                else
+                    y[n] = (beta == 0.f) ? alpha * tv[e] : __builtin_fmaf(beta, y[n], alpha * tv[e]);
+            }
+        }
+    }
+}
+
 __global__ __launch_bounds__(kGemvThreads) void sgemv_t_finish_kernel(int N, int chunks, float alpha,
                                                                       const float* __restrict__ partial, float beta,
                                                                       float* __restrict__ y) {
     const int n = blockIdx.x * kGemvThreads + threadIdx.x;
     if (n >= N) return;
-    float s = partial[n];
-    for (int c = 1; c < chunks; ++c) s += partial[static_cast<int64_t>(c) * N + n];
+    // chunk partials of column n, added in chunk order; eight loads in flight
+    float s = 0.f;
+    for (int c = 0; c < chunks; c += 8) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = (c + u < chunks) ? partial[static_cast<int64_t>(c + u) * N + n] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += t[u];
+    }
     y[n] = (beta == 0.f) ? alpha * s : __builtin_fmaf(beta, y[n], alpha * s);
 }
 
@@ -130,10 +257,16 @@ __global__ __launch_bounds__(kGemvThreads) void fill_const_kernel(float* __restr
 
 __global__ void add_to_element_kernel(float* __restrict__ p, float delta) { *p += delta; }
 
-// Row chunks of the transposed product: enough blocks to fill the device, at least 32 rows each.
+// Row chunks of the transposed product: enough workgroups (narrow matrices, 256-column blocks) or waves (wide ones,
+// 2048-column strips) to fill the device, at least 32 rows each.  A function of the shape only.
+static bool gemv_t_wide(int N) { return N >= kGemvStripCols; }
+
 static int gemv_t_chunks(int M, int N) {
-    const int64_t col_blocks = ceil_div(N, kGemvColsPerBlock);
-    int64_t want = ceil_div(2 * 256, col_blocks);  // about two blocks per CU of an MI355X; a function of the shape only
+    int64_t want;
+    if (gemv_t_wide(N))
+        want = ceil_div(4 * 256, ceil_div(N, kGemvStripCols));  // about four waves per CU of an MI355X
+    else
+        want = ceil_div(2 * 256, ceil_div(N, kGemvColsPerBlock));  // about two blocks per CU
     const int64_t most = ceil_div(M, 32);
     if (want > most) want = most;
     if (want > kGemvMaxChunks) want = kGemvMaxChunks;
@@ -155,6 +288,14 @@ static int run_sgemv(int trans, int M, int N, float alpha, const float* A, int l
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 3u)
         return HPCDNN_ERR_INVALID_VALUE;
     if (!trans) {
+        if (N >= 2048 && N <= kGemvLdsMaxN && M >= kGemvWaves) {
+            // x in LDS, one contiguous range of rows per workgroup, one workgroup per CU when there are enough rows
+            int rows_per_block = static_cast<int>(ceil_div(ceil_div(M, device_cus()), kGemvWaves)) * kGemvWaves;
+            const int grid = static_cast<int>(ceil_div(M, rows_per_block));
+            const size_t lds = static_cast<size_t>(ceil_div(N, kGemvLdsStep)) * kGemvLdsStep * sizeof(float);
+            sgemv_n_lds_kernel<<<grid, kGemvThreads, lds, s>>>(M, N, rows_per_block, alpha, A, lda, x, beta, y);
+            return launch_status();
+        }
         const bool grouped = N >= 4096 && M >= 8192;  // long rows and enough of them: share x between four rows
         int64_t grid = ceil_div(M, (grouped ? 4 : 1) * kGemvWaves);
         const int64_t cap = static_cast<int64_t>(device_cus()) * 16;
@@ -170,48 +311,319 @@ static int run_sgemv(int trans, int M, int N, float alpha, const float* A, int l
     if (M == 0) chunks = 1;
     const int rows_per_chunk = M > 0 ? static_cast<int>(ceil_div(M, chunks)) : 1;
     chunks = M > 0 ? static_cast<int>(ceil_div(M, rows_per_chunk)) : 1;
-    const dim3 grid(static_cast<unsigned>(ceil_div(N, kGemvColsPerBlock)), chunks);
     float* partial = chunks > 1 ? static_cast<float*>(ws) : nullptr;
-    sgemv_t_kernel<8><<<grid, kGemvThreads, 0, s>>>(M, N, rows_per_chunk, alpha, A, lda, x, beta, y, partial);
+    if (gemv_t_wide(N)) {
+        const int strips = static_cast<int>(ceil_div(N, kGemvStripCols)), waves = strips * chunks;
+        sgemv_t_strip_kernel<<<static_cast<int>(ceil_div(waves, kGemvWaves)), kGemvThreads, 0, s>>>(M, N, rows_per_chunk, strips, waves,
+                                                                                                   alpha, A, lda, x, beta, y, partial);
+    } else {
+        const dim3 grid(static_cast<unsigned>(ceil_div(N, kGemvColsPerBlock)), chunks);
+        sgemv_t_kernel<8><<<grid, kGemvThreads, 0, s>>>(M, N, rows_per_chunk, alpha, A, lda, x, beta, y, partial);
+    }
     if (chunks > 1)
         sgemv_t_finish_kernel<<<static_cast<int>(ceil_div(N, kGemvThreads)), kGemvThreads, 0, s>>>(N, chunks, alpha, partial,
                                                                                                   beta, y);
     return launch_status();
 }
 
-// ---- offline ABFT: workspace carving (all sizes in floats, each region 64-float aligned)
+// ---- offline ABFT (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:3-31), three launches per K panel behind the GEMM:
+//   sums   one pass over C for its row *and* column sums (partial per 1024-column / 64-row block), the column sums
+//          of the A panel and the row sums of the B panel, all in one grid;
+//   carry  the checksums carried through the operands, added to the running references, and next to them the
+//          residual vectors (sums of C minus references) reduced to one partial per block;
+//   the residual sums of panel p are finished by one extra block of the sums launch of panel p + 1 (a last small
+//   launch after the loop finishes the last panel's).
+// Every sum is formed in a fixed order: lanes, then waves, then blocks by index.
+constexpr int kSumRows = 64;            // rows of one block of the sums pass: 16 per wave
+constexpr int kSumPieceCols = 4 * kWave;  // one 16-byte load per lane
+constexpr int kSumPieces = 2;           // 1 KiB pieces of a row per block: 512 columns
+constexpr int kSumCols = kSumPieces * kSumPieceCols;
+constexpr int kCarryCols = 256;         // columns per block of the carried column checksum
+
+// rows [r0, r0 + 64) x columns [c0, c0 + PIECES * 256) of a row-major matrix: rowsum[r] = sum over the block's
+// columns of row r (lane partials combined by DPP), colsum[c] = sum over the block's rows of column c (in-lane over
+// the rows of a wave, then the four waves in order).  Wave w takes rows r0 + w, r0 + w + 4, ..., four of them in
+// flight.  Rows >= rows and columns >= cols read as zeros through the descriptors and are not written.
+template <int PIECES, bool WANT_ROW, bool WANT_COL>
+__device__ __forceinline__ void sums_block(const float* __restrict__ mat, int ld, int rows, int cols, int r0, int c0,
+                                           float* __restrict__ rowsum, float* __restrict__ colsum,
+                                           v4f (*part)[kSumPieces][kWave]) {
+    constexpr int kUnroll = 8;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int64_t row_bytes = static_cast<int64_t>(cols - c0) * 4;
+    v4f acc[PIECES];
+#pragma unroll
+    for (int pc = 0; pc < PIECES; ++pc) acc[pc] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < kSumRows / kGemvWaves; i += kUnroll) {
+        v4f a[kUnroll][PIECES];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int r = r0 + wave + kGemvWaves * (i + u);
+            const bool valid = r < rows;
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(mat + static_cast<int64_t>(valid ? r : r0) * ld + c0, valid ? row_bytes : 0);
+#pragma unroll
+            for (int pc = 0; pc < PIECES; ++pc) a[u][pc] = buffer_load_v4f(rs, (pc * kSumPieceCols + lane * 4) * 4);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if constexpr (WANT_COL) {
+#pragma unroll
+                for (int pc = 0; pc < PIECES; ++pc) acc[pc] += a[u][pc];
+            }
+            if constexpr (WANT_ROW) {
+                float s = (a[u][0].x + a[u][0].y) + (a[u][0].z + a[u][0].w);
+#pragma unroll
+                for (int pc = 1; pc < PIECES; ++pc) s += (a[u][pc].x + a[u][pc].y) + (a[u][pc].z + a[u][pc].w);
+                s = wave_sum_lane63(s);
+                const int r = r0 + wave + kGemvWaves * (i + u);
+                if (lane == kWave - 1 && r < rows) rowsum[r] = s;
+            }
+        }
+    }
+    if constexpr (WANT_COL) {
+#pragma unroll
+        for (int pc = 0; pc < PIECES; ++pc) part[wave][pc][lane] = acc[pc];
+        __syncthreads();
+        const int pc = threadIdx.x / kWave, l = lane;  // 256 threads = 4 pieces x 64 lanes
+        if (pc < PIECES) {
+            v4f t = part[0][pc][l];
+#pragma unroll
+            for (int w = 1; w < kGemvWaves; ++w) t += part[w][pc][l];
+            const float tv[4] = {t.x, t.y, t.z, t.w};
+            const int c = c0 + pc * kSumPieceCols + l * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (c + e < cols) colsum[c + e] = tv[e];
+        }
+    }
+}
+
+// base[0] + base[stride] + ... (count terms, added in index order): sixteen loads are in flight before the first
+// addition waits, instead of one trip to memory per term
+__device__ __forceinline__ float strided_sum(const float* __restrict__ base, size_t stride, int count) {
+    constexpr int kBatch = 16;
+    float s = 0.f;
+    int i = 0;
+    for (; i + kBatch <= count; i += kBatch) {
+        float t[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) t[u] = base[static_cast<size_t>(i + u) * stride];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) s += t[u];
+    }
+    float t[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) t[u] = (i + u < count) ? base[static_cast<size_t>(i + u) * stride] : 0.f;
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) s += t[u];
+    return s;
+}
+
+struct OfflineArgs {
+    int M, N, kp;  // kp: columns of the A panel = rows of the B panel (<= HPCDNN_OFFLINE_FT_PANEL_K)
+    const float* C;
+    int ldc;
+    const float* Ap;
+    int lda;
+    const float* Bp;
+    int ldb;
+    float alpha;
+    float* rowpart;  // [col blocks of C][M]   row sums of C per 1024-column block
+    float* colpart;  // [row blocks of C][N]   column sums of C per 64-row block
+    float* apart;    // [row blocks][panel]    column sums of the A panel per 64-row block
+    float* bpart;    // [col blocks][panel]    row sums of the B panel per 1024-column block
+    float* ref_row;  // [M] running reference row checksum
+    float* ref_col;  // [N] running reference column checksum
+    double* row_slots;  // [row blocks]        sum of (row sums of C - reference) per carry block
+    double* col_slots;  // [N / 256]           the same for the column sums
+    float* res_out;     // where the residual sums of the panel before this one go (sums launch), or nullptr
+    int c_blocks, a_blocks, b_blocks;  // roles of the sums launch, in this order; one more block when res_out is set
+    int row_blocks, col_blocks;        // 64-row blocks of C, 1024-column blocks of C
+    int carry_col_blocks;              // 256-column blocks of the carry launch (after its row_blocks row blocks)
+};
+
+// residual sums of a panel: the block partials added in block order
+__device__ __forceinline__ void finish_residuals(const OfflineArgs& p) {
+    if (threadIdx.x != 0) return;
+    double sc = 0.0, sr = 0.0;
+    for (int b = 0; b < p.carry_col_blocks; ++b) sc += p.col_slots[b];
+    for (int b = 0; b < p.row_blocks; ++b) sr += p.row_slots[b];
+    p.res_out[0] = static_cast<float>(sc);
+    p.res_out[1] = static_cast<float>(sr);
+}
+
+__global__ __launch_bounds__(kGemvThreads) void offline_sums_kernel(const OfflineArgs p) {
+    __shared__ v4f part[kGemvWaves][kSumPieces][kWave];
+    int b = blockIdx.x;
+    if (b < p.c_blocks) {
+        const int rb = b / p.col_blocks, cb = b % p.col_blocks;
+        sums_block<kSumPieces, true, true>(p.C, p.ldc, p.M, p.N, rb * kSumRows, cb * kSumCols, p.rowpart + static_cast<size_t>(cb) * p.M,
+                                           p.colpart + static_cast<size_t>(rb) * p.N, part);
+        return;
+    }
+    b -= p.c_blocks;
+    if (b < p.a_blocks) {  // column sums of the A panel (M x kp): one 256-column piece
+        sums_block<1, false, true>(p.Ap, p.lda, p.M, p.kp, b * kSumRows, 0, nullptr, p.apart + static_cast<size_t>(b) * HPCDNN_OFFLINE_FT_PANEL_K, part);
+        return;
+    }
+    b -= p.a_blocks;
+    if (b < p.b_blocks) {  // row sums of the B panel (kp x N)
+        const int rb = b / p.col_blocks, cb = b % p.col_blocks;
+        sums_block<kSumPieces, true, false>(p.Bp, p.ldb, p.kp, p.N, rb * kSumRows, cb * kSumCols,
+                                            p.bpart + static_cast<size_t>(cb) * HPCDNN_OFFLINE_FT_PANEL_K, nullptr, part);
+        return;
+    }
+    finish_residuals(p);
+}
+
+// sum of a double over the block, valid in thread 0 (wave partials added in wave order)
+__device__ __forceinline__ double block_sum_f64(double v, double* lds) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = v;
+    __syncthreads();
+    double s = 0.0;
+    if (threadIdx.x == 0)
+        for (int w = 0; w < kGemvWaves; ++w) s += lds[w];
+    return s;
+}
+
+// Blocks 0 .. row_blocks-1: ref_row[m] += alpha * sum_k A_p[m][k] * b_row[k] for 64 rows (b_row = the B panel's row
+// sums, its column-block partials added in order), then the row residuals c_row[m] - ref_row[m] of those rows, summed.
+// The other blocks: ref_col[n] += alpha * sum_k a_col[k] * B_p[k][n] for 256 columns (a_col likewise from its
+// row-block partials), and the column residuals.  (baseline_ft_sgemm.cuh:20-30)
+__global__ __launch_bounds__(kGemvThreads) void offline_carry_kernel(const OfflineArgs p) {
+    constexpr int pk = HPCDNN_OFFLINE_FT_PANEL_K;
+    static_assert(pk == kGemvThreads && pk == kSumPieceCols, "one thread per k of a panel, one piece per panel row of A");
+    __shared__ float vec[pk];
+    __shared__ v4f part[kGemvWaves][kWave];
+    __shared__ float colsum[kCarryCols];  // carried sums of the block's columns (or of its 64 rows)
+    __shared__ double red[kGemvWaves];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    if (static_cast<int>(blockIdx.x) < p.row_blocks) {
+        vec[tid] = tid < p.kp ? strided_sum(p.bpart + tid, pk, p.col_blocks) : 0.f;
+        __syncthreads();
+        const v4f bv = *reinterpret_cast<const v4f*>(vec + lane * 4);
+        const int r0 = blockIdx.x * kSumRows;
+        constexpr int kUnroll = 8;
+        for (int i = 0; i < kSumRows / kGemvWaves; i += kUnroll) {
+            v4f a[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int r = r0 + wave + kGemvWaves * (i + u);
+                const bool valid = r < p.M;
+                a[u] = buffer_load_v4f(make_rsrc(p.Ap + static_cast<int64_t>(valid ? r : r0) * p.lda, valid ? static_cast<int64_t>(p.kp) * 4 : 0), lane * 16);
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                float s = __builtin_fmaf(a[u].x, bv.x, 0.f);
+                s = __builtin_fmaf(a[u].y, bv.y, s);
+                s = __builtin_fmaf(a[u].z, bv.z, s);
+                s = __builtin_fmaf(a[u].w, bv.w, s);
+                s = wave_sum_lane63(s);
+                if (lane == kWave - 1) colsum[wave + kGemvWaves * (i + u)] = s;  // row number inside the block
+            }
+        }
+        __syncthreads();
+        // one thread per row: reference, sum of C's row from its column-block partials, residual
+        double d = 0.0;
+        const int r = r0 + tid;
+        if (tid < kSumRows && r < p.M) {
+            const float ref = __builtin_fmaf(p.alpha, colsum[tid], p.ref_row[r]);
+            p.ref_row[r] = ref;
+            const float c = strided_sum(p.rowpart + r, p.M, p.col_blocks);
+            d = static_cast<double>(c - ref);
+        }
+        const double s = block_sum_f64(d, red);
+        if (tid == 0) p.row_slots[blockIdx.x] = s;
+        return;
+    }
+    const int cbk = blockIdx.x - p.row_blocks, c0 = cbk * kCarryCols;
+    vec[tid] = tid < p.kp ? strided_sum(p.apart + tid, pk, p.row_blocks) : 0.f;
+    __syncthreads();
+    const int64_t row_bytes = static_cast<int64_t>(p.N - c0) * 4;
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    constexpr int kUnroll = 8;
+    for (int k = wave; k < p.kp; k += kUnroll * kGemvWaves) {
+        v4f bq[kUnroll];
+        float av[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int kk = k + u * kGemvWaves;
+            const bool valid = kk < p.kp;
+            bq[u] = buffer_load_v4f(make_rsrc(p.Bp + static_cast<int64_t>(valid ? kk : 0) * p.ldb + c0, valid ? row_bytes : 0), lane * 16);
+            av[u] = valid ? vec[kk] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            acc.x = __builtin_fmaf(bq[u].x, av[u], acc.x);
+            acc.y = __builtin_fmaf(bq[u].y, av[u], acc.y);
+            acc.z = __builtin_fmaf(bq[u].z, av[u], acc.z);
+            acc.w = __builtin_fmaf(bq[u].w, av[u], acc.w);
+        }
+    }
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+        v4f t = part[0][lane];
+#pragma unroll
+        for (int w = 1; w < kGemvWaves; ++w) t += part[w][lane];
+        *reinterpret_cast<v4f*>(colsum + lane * 4) = t;
+    }
+    __syncthreads();
+    const int n = c0 + tid;
+    double d = 0.0;
+    if (n < p.N) {
+        const float ref = __builtin_fmaf(p.alpha, colsum[tid], p.ref_col[n]);
+        p.ref_col[n] = ref;
+        const float c = strided_sum(p.colpart + n, p.N, p.row_blocks);
+        d = static_cast<double>(c - ref);
+    }
+    const double s = block_sum_f64(d, red);
+    if (tid == 0) p.col_slots[cbk] = s;
+}
+
+// running references before the first panel: beta times the sums of the C that is there, or zeros
+__global__ __launch_bounds__(kGemvThreads) void offline_init_kernel(const OfflineArgs p, float beta) {
+    const int i = blockIdx.x * kGemvThreads + threadIdx.x;
+    if (i < p.M) {
+        p.ref_row[i] = beta != 0.f ? beta * strided_sum(p.rowpart + i, p.M, p.col_blocks) : 0.f;
+    }
+    if (i < p.N) {
+        p.ref_col[i] = beta != 0.f ? beta * strided_sum(p.colpart + i, p.N, p.row_blocks) : 0.f;
+    }
+}
+
+__global__ void offline_finish_kernel(const OfflineArgs p) { finish_residuals(p); }
+
+// ---- workspace carving (sizes in floats, each region 64-float aligned)
 struct OfflineWs {
-    size_t ones, c_row, c_col, ref_row, ref_col, a_col, b_row, gemv, sdot, total;
+    size_t rowpart, colpart, apart, bpart, ref_row, ref_col, slots, total;
 };
 
 static size_t align64(size_t v) { return (v + 63) & ~static_cast<size_t>(63); }
 
-size_t sdot_workspace_bytes();
-
-static OfflineWs offline_layout(int M, int N, int panel_k) {
+static OfflineWs offline_layout(int M, int N) {
+    constexpr size_t pk = HPCDNN_OFFLINE_FT_PANEL_K;
+    const size_t rb = static_cast<size_t>(ceil_div(M, kSumRows)), cb = static_cast<size_t>(ceil_div(N, kSumCols));
     OfflineWs w{};
-    const size_t mx = static_cast<size_t>(M > N ? M : N);
     size_t off = 0;
-    w.ones = off; off += align64(mx > static_cast<size_t>(panel_k) ? mx : panel_k);
-    w.c_row = off; off += align64(M);
-    w.c_col = off; off += align64(N);
+    w.rowpart = off; off += align64(cb * M);
+    w.colpart = off; off += align64(rb * N);
+    w.apart = off; off += align64(rb * pk);
+    w.bpart = off; off += align64(cb * pk);
     w.ref_row = off; off += align64(M);
     w.ref_col = off; off += align64(N);
-    w.a_col = off; off += align64(panel_k);
-    w.b_row = off; off += align64(panel_k);
-    size_t g = sgemv_workspace_bytes(M, N);
-    const size_t g2 = sgemv_workspace_bytes(M, panel_k), g3 = sgemv_workspace_bytes(panel_k, N);
-    if (g2 > g) g = g2;
-    if (g3 > g) g = g3;
-    w.gemv = off; off += align64(g / sizeof(float));
-    w.sdot = off; off += align64(sdot_workspace_bytes() / sizeof(float));
+    w.slots = off; off += align64(2 * (rb + static_cast<size_t>(ceil_div(N, kCarryCols))));  // doubles
     w.total = off;
     return w;
 }
 
 size_t offline_ft_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return offline_layout(M, N, HPCDNN_OFFLINE_FT_PANEL_K).total * sizeof(float);
+    return offline_layout(M, N).total * sizeof(float);
 }
 
 }  // namespace hpcdnn
@@ -234,7 +646,7 @@ extern "C" int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int 
     if (inject && (inject->tile < 0 || inject->tile >= panels || inject->row < 0 || inject->row >= M || inject->col < 0 ||
                    inject->col >= N))
         return HPCDNN_ERR_INVALID_VALUE;
-    const OfflineWs w = offline_layout(M, N, pk);
+    const OfflineWs w = offline_layout(M, N);
     if (K > 0 && (!ws || ws_bytes < w.total * sizeof(float) || (reinterpret_cast<uintptr_t>(ws) & 15u)))
         return HPCDNN_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -242,52 +654,52 @@ extern "C" int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int 
         return hpcdnn_sgemm(M, N, 0, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, stream);
 
     float* base = static_cast<float*>(ws);
-    float *ones = base + w.ones, *c_row = base + w.c_row, *c_col = base + w.c_col, *ref_row = base + w.ref_row,
-          *ref_col = base + w.ref_col, *a_col = base + w.a_col, *b_row = base + w.b_row;
-    void* gws = base + w.gemv;
-    const size_t gws_bytes = (w.sdot - w.gemv) * sizeof(float);
-    void* dws = base + w.sdot;
-    const size_t dws_bytes = (w.total - w.sdot) * sizeof(float);
-    const int64_t n_ones = static_cast<int64_t>(w.c_row - w.ones);
-    fill_const_kernel<<<static_cast<int>(ceil_div(n_ones, kGemvThreads)), kGemvThreads, 0, s>>>(ones, n_ones, 1.0f);
-    int rc = hpcdnn_workspace_init(dws, dws_bytes, stream);
-    if (rc != HPCDNN_OK) return rc;
-#define HPCDNN_TRY(call)              \
-    do {                              \
-        rc = (call);                  \
-        if (rc != HPCDNN_OK) return rc; \
-    } while (0)
+    OfflineArgs a{};
+    a.M = M; a.N = N;
+    a.C = C; a.ldc = ldc; a.lda = lda; a.ldb = ldb;
+    a.alpha = alpha;
+    a.rowpart = base + w.rowpart; a.colpart = base + w.colpart; a.apart = base + w.apart; a.bpart = base + w.bpart;
+    a.ref_row = base + w.ref_row; a.ref_col = base + w.ref_col;
+    a.row_blocks = static_cast<int>(ceil_div(M, kSumRows));
+    a.col_blocks = static_cast<int>(ceil_div(N, kSumCols));
+    a.carry_col_blocks = static_cast<int>(ceil_div(N, kCarryCols));
+    a.row_slots = reinterpret_cast<double*>(base + w.slots);
+    a.col_slots = a.row_slots + a.row_blocks;
+    a.c_blocks = a.row_blocks * a.col_blocks;
+    int rc = HPCDNN_OK;
     // running reference checksums start from what C already holds (nothing when beta == 0: C is not read then)
     if (beta != 0.f) {
-        HPCDNN_TRY(run_sgemv(0, M, N, beta, C, ldc, ones, 0.f, ref_row, nullptr, 0, s));
-        HPCDNN_TRY(run_sgemv(1, M, N, beta, C, ldc, ones, 0.f, ref_col, gws, gws_bytes, s));
-    } else {
-        fill_const_kernel<<<static_cast<int>(ceil_div(M, kGemvThreads)), kGemvThreads, 0, s>>>(ref_row, M, 0.f);
-        fill_const_kernel<<<static_cast<int>(ceil_div(N, kGemvThreads)), kGemvThreads, 0, s>>>(ref_col, N, 0.f);
+        OfflineArgs first = a;
+        first.a_blocks = first.b_blocks = 0;
+        offline_sums_kernel<<<first.c_blocks, kGemvThreads, 0, s>>>(first);
     }
+    const int most = M > N ? M : N;
+    offline_init_kernel<<<static_cast<int>(ceil_div(most, kGemvThreads)), kGemvThreads, 0, s>>>(a, beta);
+    rc = launch_status();
+    if (rc != HPCDNN_OK) return rc;
     for (int p = 0; p < panels; ++p) {
         const int k0 = p * pk, kp = (K - k0 < pk) ? K - k0 : pk;
-        const float* Ap = A + k0;
-        const float* Bp = B + static_cast<int64_t>(k0) * ldb;
+        a.kp = kp;
+        a.Ap = A + k0;
+        a.Bp = B + static_cast<int64_t>(k0) * ldb;
         // the panel's product (baseline_ft_sgemm.cuh:5)
-        HPCDNN_TRY(hpcdnn_sgemm(M, N, kp, Ap, lda, Bp, ldb, C, ldc, alpha, p == 0 ? beta : 1.f, nullptr, 0, stream));
+        rc = hpcdnn_sgemm(M, N, kp, a.Ap, lda, a.Bp, ldb, C, ldc, alpha, p == 0 ? beta : 1.f, nullptr, 0, stream);
+        if (rc != HPCDNN_OK) return rc;
         if (inject && inject->tile == p)
             add_to_element_kernel<<<1, 1, 0, s>>>(C + static_cast<int64_t>(inject->row) * ldc + inject->col, inject->delta);
-        // row and column sums of C (:8,:11)
-        HPCDNN_TRY(run_sgemv(0, M, N, 1.f, C, ldc, ones, 0.f, c_row, nullptr, 0, s));
-        HPCDNN_TRY(run_sgemv(1, M, N, 1.f, C, ldc, ones, 0.f, c_col, gws, gws_bytes, s));
-        // column sums of the A panel, row sums of the B panel (:14,:17)
-        HPCDNN_TRY(run_sgemv(1, M, kp, 1.f, Ap, lda, ones, 0.f, a_col, gws, gws_bytes, s));
-        HPCDNN_TRY(run_sgemv(0, kp, N, 1.f, Bp, ldb, ones, 0.f, b_row, nullptr, 0, s));
-        // checksums carried through the operands, added to the running references (:20,:23)
-        HPCDNN_TRY(run_sgemv(1, kp, N, alpha, Bp, ldb, a_col, 1.f, ref_col, gws, gws_bytes, s));
-        HPCDNN_TRY(run_sgemv(0, M, kp, alpha, Ap, lda, b_row, 1.f, ref_row, nullptr, 0, s));
-        // residual vectors and their sums (:26-30)
-        HPCDNN_TRY(hpcdnn_saxpy(N, -1.f, ref_col, c_col, stream));
-        HPCDNN_TRY(hpcdnn_sdot(N, c_col, ones, residuals + 2 * p, dws, dws_bytes, stream));
-        HPCDNN_TRY(hpcdnn_saxpy(M, -1.f, ref_row, c_row, stream));
-        HPCDNN_TRY(hpcdnn_sdot(M, c_row, ones, residuals + 2 * p + 1, dws, dws_bytes, stream));
+        // row and column sums of C, column sums of the A panel, row sums of the B panel (:8-17); one more block
+        // finishes the residual sums of the panel before
+        a.a_blocks = a.row_blocks;
+        a.b_blocks = static_cast<int>(ceil_div(kp, kSumRows)) * a.col_blocks;
+        a.res_out = p > 0 ? residuals + 2 * (p - 1) : nullptr;
+        offline_sums_kernel<<<a.c_blocks + a.a_blocks + a.b_blocks + (p > 0 ? 1 : 0), kGemvThreads, 0, s>>>(a);
+        // checksums carried through the operands into the running references, residual vectors and their block sums
+        // (:20-30)
+        offline_carry_kernel<<<a.row_blocks + a.carry_col_blocks, kGemvThreads, 0, s>>>(a);
+        rc = launch_status();
+        if (rc != HPCDNN_OK) return rc;
     }
-#undef HPCDNN_TRY
+    a.res_out = residuals + 2 * (panels - 1);
+    offline_finish_kernel<<<1, kWave, 0, s>>>(a);
     return launch_status();
 }
