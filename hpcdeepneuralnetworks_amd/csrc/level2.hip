@@ -343,7 +343,9 @@ constexpr int kCarryCols = 256;         // columns per block of the carried colu
 // rows [r0, r0 + 64) x columns [c0, c0 + PIECES * 256) of a row-major matrix: rowsum[r] = sum over the block's
 // columns of row r (lane partials combined by DPP), colsum[c] = sum over the block's rows of column c (in-lane over
 // the rows of a wave, then the four waves in order).  Wave w takes rows r0 + w, r0 + w + 4, ..., four of them in
-// flight.  Rows >= rows and columns >= cols read as zeros through the descriptors and are not written.
+// flight.  Rows >= rows and columns >= cols read as zeros through the descriptors and are not written.  Plain
+// loads on purpose: C stays in the memory-side cache for the next panel's GEMM, which reads it again (with the
+// non-temporal hint that GEMM ran 4 % slower).
 template <int PIECES, bool WANT_ROW, bool WANT_COL>
 __device__ __forceinline__ void sums_block(const float* __restrict__ mat, int ld, int rows, int cols, int r0, int c0,
                                            float* __restrict__ rowsum, float* __restrict__ colsum,
