@@ -21,7 +21,7 @@ OP_OFFLINE_FT_SGEMM = 4
 OFFLINE_FT_PANEL_K = 256
 FT_TILE_M = 256
 FT_TILE_N = 128
-FT_NUM_CLASSES = 3
+FT_NUM_CLASSES = 5
 
 # every symbol include/hpcdnn.h declares
 EXPORTS = (

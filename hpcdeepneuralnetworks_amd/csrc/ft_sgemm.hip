@@ -26,7 +26,7 @@ struct FtKernel {
     int threads;
     size_t lds;
 };
-typedef void (*EncodeFn)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int);
+typedef void (*EncodeFn)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int, int);
 struct FtClass {
     int bm, bn;
     int wgm, wgn;        // wave layout of the workspace kernels
@@ -38,12 +38,13 @@ struct FtClass {
     EncodeFn encode, encode_wave;
 };
 
-#define HPCDNN_FT_KERNEL(BM, WM_, WN_, FT, GRAN, CAD)                                                      \
+#define HPCDNN_FT_KERNEL_N(BM, BN, WM_, WN_, FT, GRAN, CAD)                                                \
     FtKernel {                                                                                             \
-        sgemm_kernel<BM, 128, WM_, WN_, false, FT, 1, 2, GRAN, CAD>,                                       \
-            sgemm_kernel<BM, 128, WM_, WN_, true, FT, 1, 2, GRAN, CAD>, WM_ * WN_ * kWave,                 \
-            gemm_lds_bytes<BM, 128, FT, WM_ * WN_ * kWave, WM_, WN_, GRAN>()                               \
+        sgemm_kernel<BM, BN, WM_, WN_, false, FT, 1, 2, GRAN, CAD>,                                        \
+            sgemm_kernel<BM, BN, WM_, WN_, true, FT, 1, 2, GRAN, CAD>, WM_ * WN_ * kWave,                  \
+            gemm_lds_bytes<BM, BN, FT, WM_ * WN_ * kWave, WM_, WN_, GRAN>()                                \
     }
+#define HPCDNN_FT_KERNEL(BM, WM_, WN_, FT, GRAN, CAD) HPCDNN_FT_KERNEL_N(BM, 128, WM_, WN_, FT, GRAN, CAD)
 #define HPCDNN_FT_NO_KERNEL \
     FtKernel { nullptr, nullptr, 0, 0 }
 
@@ -60,6 +61,12 @@ static const FtClass kFtClasses[HPCDNN_FT_NUM_CLASSES] = {
     {64, 128, 2, 2, HPCDNN_FT_KERNEL(64, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(64, 2, 2, 2, 0, false),
      HPCDNN_FT_KERNEL(64, 2, 2, 2, 1, false), HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<64, 128>,
      abft_encode_kernel<32, 64>},
+    // 3 tall, 4 medium: 64 columns wide, for products with few columns (the reference's tall 128 x 32 and medium
+    // 32 x 32 shapes, kernel/ft_sgemm/code_gen/main.py:8-16, at the size of four waves of 32 x 32 matrix-core blocks)
+    {128, 64, 2, 2, HPCDNN_FT_KERNEL_N(128, 64, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL_N(128, 64, 2, 2, 2, 0, false),
+     HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<128, 64>, nullptr},
+    {64, 64, 2, 2, HPCDNN_FT_KERNEL_N(64, 64, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL_N(64, 64, 2, 2, 2, 0, false),
+     HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<64, 64>, nullptr},
 };
 
 // check tile of a class at a granularity: the unit that has a checksum pair, a verification and a status record
@@ -102,7 +109,7 @@ static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     const FtClass& fc = kFtClasses[tile_class];
     const size_t tile_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_TILE, M, N, K) + ft_tail_bytes(fc, ft_tail_plan(fc, M, N, K));
-    const size_t wave_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_WAVE, M, N, K);
+    const size_t wave_mode = fc.wave.plain ? ft_enc_bytes(fc, HPCDNN_FT_GRAN_WAVE, M, N, K) : 0;
     return tile_mode > wave_mode ? tile_mode : wave_mode;
 }
 
@@ -117,6 +124,7 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     if (opt.n_faults < 0 || opt.n_faults > HPCDNN_FT_MAX_FAULTS) return HPCDNN_ERR_INVALID_VALUE;
     const FtClass& fc = kFtClasses[opt.tile_class];
     const bool wave = opt.granularity == HPCDNN_FT_GRAN_WAVE;
+    if (wave && !fc.wave.plain) return HPCDNN_ERR_INVALID_VALUE;  // the 64-column classes check per workgroup tile only
     // an interval that covers all of K is a single verification after the loop
     const bool cadence = opt.check_interval > 0 && opt.check_interval < K;
     if (cadence && (wave || !fc.pre_cad.plain)) return HPCDNN_ERR_INVALID_VALUE;
@@ -165,12 +173,12 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         const int row_groups = a.tiles_m * gm, col_groups = a.tiles_n * gn;
         float* enc_a = static_cast<float*>(ws);
         float* enc_b = enc_a + static_cast<size_t>(row_groups) * a.enc_ld;
-        (void)col_groups;
         a.enc_a = enc_a;
         a.enc_b = enc_b;
         const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
-        hipLaunchKernelGGL(wave ? fc.encode_wave : fc.encode, dim3(k_blocks * (row_groups + a.tiles_n)), dim3(1024), 0, s, M, N, K,
-                           A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups);
+        const int b_blocks = static_cast<int>(ceil_div(N, 128));  // the pre-pass walks B in blocks of 128 columns
+        hipLaunchKernelGGL(wave ? fc.encode_wave : fc.encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(1024), 0, s, M, N, K,
+                           A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;
         const FtKernel& k = wave ? fc.wave : (cadence ? fc.pre_cad : fc.pre);
@@ -222,6 +230,7 @@ extern "C" int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn) {
 extern "C" int hpcdnn_ft_check_tile_info(int tile_class, int granularity, int* cm, int* cn) {
     if (tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
     if (granularity != HPCDNN_FT_GRAN_TILE && granularity != HPCDNN_FT_GRAN_WAVE) return HPCDNN_ERR_INVALID_VALUE;
+    if (granularity == HPCDNN_FT_GRAN_WAVE && !kFtClasses[tile_class].wave.plain) return HPCDNN_ERR_INVALID_VALUE;
     int m = 0, n = 0;
     check_tile(kFtClasses[tile_class], granularity, &m, &n);
     if (cm) *cm = m;
@@ -241,13 +250,14 @@ extern "C" int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N) {
 
 extern "C" int hpcdnn_ft_num_tiles(int M, int N) { return hpcdnn_ft_num_tiles_ex(0, M, N); }
 
-// The class with the shortest predicted run (workspace variant): rounds of tiles over the CUs times the tile height
-// (all classes are 128 columns wide), a partial last round counting for what its K split leaves of it plus the
-// second pass over those tiles, with the measured efficiency of the smaller tiles relative to the 256-row one.
+// The class with the shortest predicted run (workspace variant): rounds of tiles over the CUs times the tile area, a
+// partial last round counting for what its K split leaves of it plus the second pass over those tiles, with the
+// measured efficiency of the smaller tiles relative to the 256-row one.
 extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
     // measured on squares 1024 ... 6144: the 128-row class keeps up with the 256-row one (two of its workgroups share a CU
-    // and cover each other's verification), the 64-row class runs 4-5 % behind
-    static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 1.0, 0.955};
+    // and cover each other's verification), the 64-row class runs 4-5 % behind; the 64-column classes move twice the
+    // operand bytes per flop and only pay where the 128-column ones would multiply empty columns
+    static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 1.0, 0.955, 0.92, 0.88};
     const int cus = device_cus();
     int best = 0;
     double best_cost = 1e300;
@@ -257,7 +267,7 @@ extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
         double rounds = static_cast<double>(ceil_div(tiles > 0 ? tiles : 1, cus));
         if (tail.ways >= 2)
             rounds = static_cast<double>(tiles / cus) + static_cast<double>(ceil_div(static_cast<int64_t>(tail.tiles) * tail.ways, cus)) / tail.ways + 0.06;
-        const double cost = rounds * kFtClasses[c].bm / rel_eff[c];
+        const double cost = rounds * kFtClasses[c].bm * kFtClasses[c].bn / rel_eff[c];
         if (cost < best_cost) { best_cost = cost; best = c; }
     }
     return best;

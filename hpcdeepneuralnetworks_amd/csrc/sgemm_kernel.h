@@ -90,7 +90,7 @@ constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tile
 template <int BM, int BN, int WGM, int WGN, int GM, int GN>
 constexpr size_t ft_verify_lds_bytes() {
     constexpr size_t threads = static_cast<size_t>(WGM) * WGN * 64;
-    constexpr size_t ccp = 2 * threads / 64, crp = kGemmBK / 4, lines = static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
+    constexpr size_t ccp = threads / (BN / 4), crp = kGemmBK / 4, lines = static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
     return sizeof(double) * (GM * ccp * BN + GN * crp * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + lines) +
            32 * GM * GN + sizeof(float) * GM * GN * (threads / 64);
 }
@@ -255,9 +255,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const __amdgpu_buffer_rsrc_t enc_b_rsrc =
         make_rsrc(FT == 2 ? p.enc_b + static_cast<int64_t>(tile_n) * GN * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * GN * 4);
     const int enc_row_bytes = p.enc_ld * 4;
-    // a_c of the k rows of B this thread stages: k = tid/32 (and k + 8 with four waves), which the pre-encode kernel
-    // stores side by side (order 0, 8, 1, 9, ... inside each K step)
-    const int enc_a_voff = B_SLOTS == 2 ? (tid >> 5) * 8 : ((((tid >> 5) & 7) * 2 + (tid >> 8)) * 4);
+    // a_c of the k rows of B this thread stages: k = tid / (BN / 4) (and k + 8 when it stages two), which the
+    // pre-encode kernel stores side by side (order 0, 8, 1, 9, ... inside each K step)
+    const int enc_a_voff = B_SLOTS == 2 ? (tid / B_V4_PER_ROW) * 8 : ((((tid / B_V4_PER_ROW) & 7) * 2 + (tid / B_V4_PER_ROW) / 8) * 4);
     const int enc_b_voff = (tid & 3) * 16;  // b_r of the four k values of A this thread stages
     int enc_off = kbeg * 4;
     float g_ac[2][GM][B_SLOTS];
@@ -410,17 +410,18 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     //     of their own over a long K.
     // Per thread the running sums cover columns nc..nc+3 over the k rows it stages (8 threads share a column)
     // and rows row(s) over the k group it stages (4 threads share a row); the verification step adds them up.
-    constexpr int kHalfWaves = 2 * kGemmThreads / kWave;  // 8 or 16
+    constexpr int kHalfWaves = kGemmThreads / B_V4_PER_ROW;  // threads that share a column of the B tile = k rows staged per slot
     constexpr int kParts = kGemmThreads / kWave;          // column-sum partials per k: one per wave
     constexpr int kPartV4 = kParts / 4;                   // 16-byte groups of them
-    static_assert(!FT || (A_V4_PER_ROW == 4 && B_V4_PER_ROW == 32), "ABFT encode is laid out for a 128-column tile");
+    static_assert(!FT || (A_V4_PER_ROW == 4 && (B_V4_PER_ROW == 32 || B_V4_PER_ROW == 16)), "ABFT encode is laid out for 128- and 64-column tiles");
+    static_assert(!FT || kHalfWaves * B_SLOTS == BK, "the threads of a column group stage the 16 k rows between them");
     float* const s_apart = smem + 2 * (A_STAGE + B_STAGE);          // [2][16 k][waves]
     float* const s_br = s_apart + 2 * BK * kParts;                  // [2][16 k]
     float* const s_dump = s_br + 2 * BK + tid;                      // where the lanes that publish nothing write
     // destinations of this lane's publishes (parity 0); strides and the parity distance are the same for the
     // publishing lanes and the dump, so every write is base + immediate offset
     float* const pub_a = (lane < 4) ? s_apart + (4 * (tid & 3)) * kParts + wave : s_dump;
-    float* const pub_b = (lr < B_SLOTS) ? s_br + (tid >> 5) + kHalfWaves * lr : s_dump;
+    float* const pub_b = (tid % B_V4_PER_ROW < B_SLOTS) ? s_br + tid / B_V4_PER_ROW + kHalfWaves * (tid % B_V4_PER_ROW) : s_dump;
     const int x32_addr = (lane ^ 32) * 4;  // ds_bpermute address of the partner lane in the other half wave
     // With wave-tile checksums a thread keeps one column sum per wave row gm (its columns lie in one wave column)
     // and one row sum per wave column gn (its rows lie in one wave row).
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     float e_pa[4], e_sw[4];
     v4f e_t[kPartV4 * B_SLOTS], e_brv[GN];
     float e_pb0, e_pb1, e_pk, e_swb, e_ac[GM][B_SLOTS];
-    const int e_hw = tid >> 5;           // half wave = first k row this thread stages of B
+    const int e_hw = tid / B_V4_PER_ROW;  // first k row this thread stages of B (a half wave per row of a 128-column tile)
     const int e_class = tid & 3;         // k group (4 k values) this thread stages of A
     constexpr int NPROD = (FT == 1) ? 11 : 0;  // pieces before the barrier
     // pieces after the barrier: fetch, combine (FT == 1), column checksums (one piece per wave row), row checksums
@@ -504,14 +505,15 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             e_pk += dpp_mov<kDppRor8>(e_pk);
             HPCDNN_PIN(e_pk);
         } else if constexpr (E == 7) {
-            e_swb = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pk), 0x401F));
+            // a k row of a 64-column tile lies in one row of 16 lanes and is complete here
+            if constexpr (B_V4_PER_ROW == 32) e_swb = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pk), 0x401F));
         } else if constexpr (E == 8) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 e_pa[e] += e_sw[e];
                 e_sw[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(x32_addr, __builtin_bit_cast(int, e_pa[e])));
             }
-            e_pk += e_swb;
+            if constexpr (B_V4_PER_ROW == 32) e_pk += e_swb;
             HPCDNN_PIN(e_pk);
         } else if constexpr (E == 9) {
 #pragma unroll
@@ -816,7 +818,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
         for (int gm = 0; gm < GM; ++gm)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) s_ccref[(gm * CCP + e_hw) * BN + (tid & 31) * 4 + e] = cc_ref[gm][e];
+            for (int e = 0; e < 4; ++e) s_ccref[(gm * CCP + e_hw) * BN + (tid % B_V4_PER_ROW) * 4 + e] = cc_ref[gm][e];
 #pragma unroll
         for (int gn = 0; gn < GN; ++gn)
 #pragma unroll
@@ -1203,7 +1205,7 @@ __global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int 
 
 // ---- ABFT pre-encode: the checksum vectors of the operands, one per row group (RM rows) / column group (CN
 // columns), in one launch of 1024-thread blocks that each cover 256 values of k: the first k_blocks * row_groups
-// blocks encode A, the rest B (one block per 128 columns, i.e. 128 / CN column groups).  A group is a workgroup tile's
+// blocks encode A, the rest B (one block per 128 columns of B, i.e. 128 / CN column groups).  A group is a workgroup tile's
 // rows or columns, or a wave tile's with wave-tile checksums.
 //
 // enc_a[g][k'] = sum over the rows m of row group g (m < M) of A[m][k]; zero for K <= k < enc_ld; k' is k with
@@ -1218,7 +1220,7 @@ template <int RM, int CN>
 __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
                                                            const float* __restrict__ B, int ldb,
                                                            float* __restrict__ enc_a, float* __restrict__ enc_b,
-                                                           int enc_ld, int k_blocks, int row_groups) {
+                                                           int enc_ld, int k_blocks, int row_groups, int col_groups) {
     static_assert(CN == 128 || CN == 64 || CN == 32, "column groups are 8, 16 or 32 lanes of a half wave");
     static_assert(RM % 16 == 0, "the rows of a group split evenly over 16 waves");
     constexpr int kWaves = 16, kRows = RM / kWaves;
@@ -1295,7 +1297,8 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
 #pragma unroll
             for (int i = 1; i < kRowsPerHalf; ++i) out = (in_group == i) ? s[i] : out;
             const int k = kb + half + kHalves * in_group;
-            if (k < enc_ld) enc_b[static_cast<int64_t>(group) * enc_ld + k] = out;
+            // (the last block of 128 columns may reach past the last column group)
+            if (k < enc_ld && group < col_groups) enc_b[static_cast<int64_t>(group) * enc_ld + k] = out;
         }
     }
 }

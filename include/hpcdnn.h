@@ -39,8 +39,9 @@ extern "C" {
  * tile = (i / 256) * ceil(N / 128) + (j / 128). */
 #define HPCDNN_FT_TILE_M 256
 #define HPCDNN_FT_TILE_N 128
-/* ABFT tile classes: 0 = 256x128 (above), 1 = 128x128, 2 = 64x128. */
-#define HPCDNN_FT_NUM_CLASSES 3
+/* ABFT tile classes: 0 = 256x128 (above), 1 = 128x128, 2 = 64x128, and for
+ * products with few columns 3 = 128x64, 4 = 64x64. */
+#define HPCDNN_FT_NUM_CLASSES 5
 
 /* Operation selectors for hpcdnn_workspace_bytes(). */
 #define HPCDNN_OP_SGEMM 0
@@ -172,8 +173,9 @@ int hpcdnn_ft_num_tiles(int M, int N);
  * workspace (rounds of tiles over the CUs times the tile height, a partial
  * last round counting for what its K split leaves of it).  The workspace
  * size of HPCDNN_OP_FT_SGEMM covers every class.  Counterpart of the reference's
- * abft_kernel_{huge,large,wide} series (kernel/ft_sgemm/sgemm.cu:187-188,
- * kernel/ft_sgemm/code_gen/main.py:8-16). */
+ * abft_kernel_{huge,large,wide,tall,medium} series (kernel/ft_sgemm/sgemm.cu:187-188,
+ * kernel/ft_sgemm/code_gen/main.py:8-16; its tall 128x32 and medium 32x32 shapes
+ * become 128x64 and 64x64 here: four waves of 32x32 matrix-core blocks). */
 int hpcdnn_ft_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                        float alpha, float beta, float tau, const hpcdnn_fault* inject, hpcdnn_ft_status* status,
                        void* ws, size_t ws_bytes, int tile_class, void* stream);
@@ -189,7 +191,8 @@ int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
  * status record per workgroup tile of the class (what hpcdnn_ft_sgemm_ex does).
  * HPCDNN_FT_GRAN_WAVE: one per wave tile, the part of the workgroup tile one
  * 64-lane wave accumulates on the matrix cores (class 0: 128x32, class 1:
- * 64x64, class 2: 32x64; hpcdnn_ft_check_tile_info): every wave tile is
+ * 64x64, class 2: 32x64; classes 3 and 4 have tile granularity only;
+ * hpcdnn_ft_check_tile_info): every wave tile is
  * verified, located and corrected on its own, so one fault per wave tile is
  * correctable where tile granularity reports two faults in one 256x128 tile
  * as uncorrectable.  Needs the workspace (HPCDNN_ERR_WORKSPACE without one).

@@ -203,11 +203,11 @@ def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod, ft_mode):
           f"fault-free max residual {clean['max_clean_residual'].max():.3e}, tau {tau:.1e}")
 
 
-@pytest.mark.parametrize("tile_class", [1, 2])
+@pytest.mark.parametrize("tile_class", [1, 2, 3, 4])
 def test_smaller_tile_classes_match_the_model(blas, oracle_mod, ft_mode, tile_class):
     """The 128x128 and 64x128 ABFT tiles: tiles, status records and fault coordinates are per tile of the class."""
     bm, bn = blas.ft_tile(tile_class)
-    assert (bm, bn) == {1: (128, 128), 2: (64, 128)}[tile_class]
+    assert (bm, bn) == {1: (128, 128), 2: (64, 128), 3: (128, 64), 4: (64, 64)}[tile_class]
     M, N, K = 333, 300, 520  # ragged in every dimension
     tau = blas.ft_default_tau(K)
     ntm, ntn = -(-M // bm), -(-N // bn)
@@ -241,12 +241,13 @@ def test_smaller_tile_classes_match_the_model(blas, oracle_mod, ft_mode, tile_cl
 def test_pick_class_and_bad_class(blas):
     assert blas.ft_pick_class(4096, 4096, 4096) == 0      # 512 tiles of 256x128: every CU has one
     assert blas.ft_pick_class(2048, 2048, 1024) == 1      # 128 tiles of 256x128, 256 of 128x128
-    assert blas.ft_pick_class(512, 512, 512) == 2
+    assert blas.ft_pick_class(512, 512, 512) == 4         # 64 tiles of 64x64 against 32 of 64x128
     assert blas.ft_pick_class(3072, 3072, 3072) in (0, 1)  # either class ends its partial round with a K split
-    assert blas.ft_pick_class(3072, 3072, 128) == 2       # too short a K to split: 64x128 tiles fill the rounds best
+    assert blas.ft_pick_class(3072, 3072, 128) in (2, 4)  # too short a K to split: small tiles fill the rounds best
+    assert blas.ft_pick_class(16384, 64, 4096) == 3       # 64 columns: the 128-column classes would multiply empty ones
     t = torch.zeros(64, 64, device="cuda")
     with pytest.raises(blas.HpcdnnError):
-        blas.ft_sgemm(64, 64, 64, t, t, t.clone(), 1.0, 0.0, tile_class=3)
+        blas.ft_sgemm(64, 64, 64, t, t, t.clone(), 1.0, 0.0, tile_class=5)
 
 
 def test_k_zero_scales_c_and_flags_nothing(blas, ft_mode):
