@@ -117,7 +117,7 @@ int run_sgemm(int start, int end, int gap) {
 struct Series {
     int number;        // the reference's kernel_number (kernel/ft_sgemm/sgemm.cu:186)
     const char* name;  // the reference's series name (:187-188) where a counterpart exists
-    int kind;          // 0 plain SGEMM, 1 offline ABFT, 2 ABFT without workspace, 3 ABFT with workspace
+    int kind;          // 0 plain SGEMM, 1 offline ABFT, 2 ABFT without workspace, 3 ABFT with workspace, 4 wave-tile ABFT
     int tile;          // plain SGEMM: row of the tile table, -1 = chosen by the library; ABFT: tile class
 };
 
@@ -131,9 +131,14 @@ const Series kSeries[] = {
     {5, "kernel_sgemm_wide", 0, 3},    // 64 x 128
     {6, "kernel_sgemm_huge", 0, 8},    // 256 x 256
     {10, "abft_baseline", 1, -1},
-    {13, "abft_kernel_large", 2, 1},  // 128 x 128
-    {15, "abft_kernel_wide", 2, 2},   // 64 x 128
-    {16, "abft_kernel_huge", 2, 0},   // 256 x 128
+    {12, "abft_kernel_medium", 2, 4},  // 64 x 64
+    {13, "abft_kernel_large", 2, 1},   // 128 x 128
+    {14, "abft_kernel_tall", 2, 3},    // 128 x 64
+    {15, "abft_kernel_wide", 2, 2},    // 64 x 128
+    {16, "abft_kernel_huge", 2, 0},    // 256 x 128
+    // one checksum pair per wave tile (128 x 32 of the 256 x 128 tile): the matrix-core counterpart of the warp-level
+    // kernel; the thread-level one (series 17) has none, a matrix-core result being spread over all lanes of a wave
+    {18, "warp_abft_kernel", 4, 0},
     // no reference counterpart: checksum vectors from the pre-pass
     {19, "abft_kernel_huge_workspace", 3, 0},
     {20, "abft_kernel_large_workspace", 3, 1},
@@ -214,6 +219,15 @@ int run_ft_sgemm(int start, int end, int gap, int first, int last) {
                         LIB_OK(hpcdnn_ft_sgemm_ex(n, n, K, a, K, b, n, c, n, alpha, beta, 0.f, nullptr, nullptr, nullptr, 0, sr.tile, nullptr));
                     });
                     break;
+                case 4: {
+                    hpcdnn_ft_options opt{};
+                    opt.tile_class = sr.tile;
+                    opt.granularity = HPCDNN_FT_GRAN_WAVE;
+                    perf = timed_gflops(flop, kNumTests, [&] {
+                        LIB_OK(hpcdnn_ft_sgemm_opt(n, n, K, a, K, b, n, c, n, alpha, beta, 0.f, &opt, nullptr, ft_ws, ft_ws_bytes, nullptr));
+                    });
+                    break;
+                }
                 default:
                     perf = timed_gflops(flop, kNumTests, [&] {
                         LIB_OK(hpcdnn_ft_sgemm_ex(n, n, K, a, K, b, n, c, n, alpha, beta, 0.f, nullptr, nullptr, ft_ws, ft_ws_bytes, sr.tile, nullptr));

@@ -29,14 +29,16 @@ def test_ft_sgemm_series_lines():
     series = dict(re.findall(r"^(\w+) = th\.as_tensor\(\[(.*)\]\)$", out, flags=re.M))
     assert list(series) == ["hpcdnn_sgemm", "kernel_sgemm_small", "kernel_sgemm_medium", "kernel_sgemm_large",
                             "kernel_sgemm_tall", "kernel_sgemm_wide", "kernel_sgemm_huge", "abft_baseline",
-                            "abft_kernel_large", "abft_kernel_wide", "abft_kernel_huge", "abft_kernel_huge_workspace",
+                            "abft_kernel_medium", "abft_kernel_large", "abft_kernel_tall", "abft_kernel_wide",
+                            "abft_kernel_huge", "warp_abft_kernel", "abft_kernel_huge_workspace",
                             "abft_kernel_large_workspace", "abft_kernel_wide_workspace"]
     for name, body in series.items():
         vals = _floats(body)
         assert len(vals) == 3 and all(v > 0 for v in vals), (name, body)
     # a sub-range of series, as the reference's <st_kernel> <end_kernel> arguments select
     out = _run("ft_sgemm", 256, 256, 256, 10, 16)
-    assert re.findall(r"^(\w+) = th", out, flags=re.M) == ["abft_baseline", "abft_kernel_large", "abft_kernel_wide", "abft_kernel_huge"]
+    assert re.findall(r"^(\w+) = th", out, flags=re.M) == ["abft_baseline", "abft_kernel_medium", "abft_kernel_large",
+                                                                "abft_kernel_tall", "abft_kernel_wide", "abft_kernel_huge"]
 
 
 def test_sgemm_rows():
