@@ -13,6 +13,7 @@ size sweep, rocBLAS/hipBLASLt through torch.matmul as a timed comparison only).
 from __future__ import annotations
 
 import argparse
+import re
 import json
 import os
 import statistics
@@ -24,9 +25,18 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 4 SIMD x 64 flop/clk x 2.4 GHz
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per 6144^3 SGEMM launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by what the same
-# counters read for a device copy of known size): the figures and commands are in profiles/sgemm_kernel_6144cube.md
-SGEMM_6144_TRAFFIC_BYTES = 1.812e9
+
+
+def profiled_traffic_bytes(summary):
+    """HBM bytes per launch as the rocprofv3 summary under profiles/ states them (FETCH_SIZE and WRITE_SIZE of two
+    --pmc runs, scaled by what the same counters read for a device copy of known size), or None without the file."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", summary)
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    m = re.search(r"HBM traffic per launch:.*?=\s*([0-9.]+)\s*GB", text)
+    return float(m.group(1)) * 1e9 if m else None
 
 
 def main() -> int:
@@ -169,7 +179,7 @@ def main() -> int:
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
-            "traffic": SGEMM_6144_TRAFFIC_BYTES,
+            "traffic": profiled_traffic_bytes("sgemm_kernel_6144cube.md"),
             "kernel": "sgemm_kernel (one launch = 2*6144^3 flop)",
             "kernel_ms": round(kern_ms, 4),
         },
@@ -305,6 +315,25 @@ def main() -> int:
             "ft_sgemm_gflops": round(2.0 * m * m * kk / ms_cls / 1e6, 1),
             "overhead_pct_vs_sgemm": round((ms_cls - ms_plain) / ms_plain * 100.0, 2),
             "class0_256x128_ft_sgemm_gflops": round(2.0 * m * m * kk / ms_c0 / 1e6, 1),
+        }
+        del a, b, c
+
+        # ---- ABFT on a product with few columns (one of the irregular shapes): the 64-column tile classes
+        m, n_, kk = 16384, 64, 4096
+        a, b, c = operands(m, n_, kk, 27)
+        cls = blas.ft_pick_class(m, n_, kk)
+        status_s = blas.ft_status_alloc(m, n_, tile_class=cls)
+        status_1 = blas.ft_status_alloc(m, n_, tile_class=1)
+        ft_ws_s = blas.workspace(blas.ft_workspace_bytes(m, n_, kk))
+        gws = blas.workspace(max(blas.sgemm_workspace_bytes(m, n_, kk), 4))
+        ms_plain = median_timed(lambda: blas.sgemm(m, n_, kk, a, b, c, 1.0, 0.0, ws=gws), st, wu)
+        ms_cls = median_timed(lambda: blas.ft_sgemm(m, n_, kk, a, b, c, 1.0, 0.0, status=status_s, ws=ft_ws_s, tile_class=cls), st, wu)
+        ms_c1 = median_timed(lambda: blas.ft_sgemm(m, n_, kk, a, b, c, 1.0, 0.0, status=status_1, ws=ft_ws_s, tile_class=1), st, wu)
+        extras["abft_16384x64x4096"] = {
+            "picked_tile_class": cls, "picked_tile": list(blas.ft_tile(cls)),
+            "sgemm_gflops": round(2.0 * m * n_ * kk / ms_plain / 1e6, 1),
+            "ft_sgemm_gflops": round(2.0 * m * n_ * kk / ms_cls / 1e6, 1),
+            "class1_128x128_ft_sgemm_gflops": round(2.0 * m * n_ * kk / ms_c1 / 1e6, 1),
         }
         del a, b, c
 

@@ -250,24 +250,40 @@ extern "C" int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N) {
 
 extern "C" int hpcdnn_ft_num_tiles(int M, int N) { return hpcdnn_ft_num_tiles_ex(0, M, N); }
 
-// The class with the shortest predicted run (workspace variant): rounds of tiles over the CUs times the tile area, a
-// partial last round counting for what its K split leaves of it plus the second pass over those tiles, with the
-// measured efficiency of the smaller tiles relative to the 256-row one.
+// The class with the shortest predicted run (workspace variant).  Matrix-core time: rounds of tiles over the CUs
+// times the tile's flops, a partial last round counting for what its K split leaves of it plus the second pass over
+// those tiles, with the measured efficiency of the smaller tiles relative to the 256-row one.  An operand that is
+// read once cannot arrive faster than the bytes in flight allow (two K steps of the tile's rows per resident
+// workgroup and trip to memory), which is what decides between the classes on tall products with few columns.
 extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
     // measured on squares 1024 ... 6144: the 128-row class keeps up with the 256-row one (two of its workgroups share a CU
     // and cover each other's verification), the 64-row class runs 4-5 % behind; the 64-column classes move twice the
     // operand bytes per flop and only pay where the 128-column ones would multiply empty columns
     static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 1.0, 0.955, 0.92, 0.88};
+    static const int resident_max[HPCDNN_FT_NUM_CLASSES] = {1, 2, 2, 2, 3};  // workgroups of the class a CU holds
+    constexpr double kPeakFlopsPerCu = 157.3e12 / 256.0, kTrip = 0.73e-6;
     const int cus = device_cus();
     int best = 0;
     double best_cost = 1e300;
     for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
+        const FtClass& fc = kFtClasses[c];
         const int64_t tiles = hpcdnn_ft_num_tiles_ex(c, M, N);
-        const FtTail tail = ft_tail_plan(kFtClasses[c], M, N, K);
+        const FtTail tail = ft_tail_plan(fc, M, N, K);
         double rounds = static_cast<double>(ceil_div(tiles > 0 ? tiles : 1, cus));
-        if (tail.ways >= 2)
+        int64_t groups = tiles;  // workgroups of the launch
+        if (tail.ways >= 2) {
             rounds = static_cast<double>(tiles / cus) + static_cast<double>(ceil_div(static_cast<int64_t>(tail.tiles) * tail.ways, cus)) / tail.ways + 0.06;
-        const double cost = rounds * kFtClasses[c].bm * kFtClasses[c].bn / rel_eff[c];
+            groups = tiles - tail.tiles + static_cast<int64_t>(tail.tiles) * tail.ways;
+        }
+        double cost = rounds * 2.0 * fc.bm * fc.bn * (K > 0 ? K : 1) / kPeakFlopsPerCu / rel_eff[c];
+        const double busy = static_cast<double>(groups < cus ? groups : cus);
+        double resident = static_cast<double>(ceil_div(groups > 0 ? groups : 1, cus));
+        if (resident > resident_max[c]) resident = resident_max[c];
+        const double in_flight = busy * resident * 2.0 * kGemmBK;  // k values of every tile row / column on their way
+        const double stream_a = static_cast<double>(M) * K * kTrip / (in_flight * fc.bm);
+        const double stream_b = static_cast<double>(N) * K * kTrip / (in_flight * fc.bn);
+        const double stream = stream_a > stream_b ? stream_a : stream_b;
+        if (stream > cost) cost = stream;
         if (cost < best_cost) { best_cost = cost; best = c; }
     }
     return best;
