@@ -459,3 +459,57 @@ def test_partial_last_round_is_split_along_k(blas, oracle_mod):
     ref = a3[rows].double() @ b3.double()
     den = a3[rows].abs().double() @ b3.abs().double()
     assert float(((c3[rows].double() - ref).abs() / den).max()) <= TOL
+
+
+@pytest.mark.parametrize("tile_class,M,N,K", [(0, 768, 640, 1100), (1, 512, 384, 800), (4, 300, 200, 530)])
+def test_workspace_reuse_and_graph_replay_see_fresh_operands(blas, tile_class, M, N, K):
+    """The checksum vectors in the workspace belong to one call: a workspace of unknown contents, back-to-back calls
+    that reuse it with other operands, and replays of a captured call whose operands changed in between must all
+    verify against the operands of *that* call - a stale checksum vector would flag every tile."""
+    dev = "cuda"
+    ops = []
+    for seed in (910, 920):
+        a = torch.empty(M, K, device=dev)
+        b = torch.empty(K, N, device=dev)
+        blas.fill_uniform_matrix(a, M, K, seed)
+        blas.fill_uniform_matrix(b, K, N, seed + 1)
+        ops.append((a, b, (a.double() @ b.double()).float()))
+    ws = torch.full((blas.ft_workspace_bytes(M, N, K) // 4,), float("nan"), device=dev)  # poisoned
+    tau = blas.ft_default_tau(K)
+    results = []
+    for rnd in range(3):
+        for a, b, _ in ops:  # no synchronisation between the calls
+            c = torch.empty(M, N, device=dev)
+            status = blas.ft_status_alloc(M, N, tile_class=tile_class)
+            blas.ft_sgemm(M, N, K, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ws, tile_class=tile_class)
+            results.append((c, status))
+    torch.cuda.synchronize()
+    for i, (c, status) in enumerate(results):
+        st = blas.ft_status_numpy(status)
+        assert not st["flag"].any(), (i, st["flag"])
+        assert (c - ops[i % 2][2]).abs().max().item() < 1e-3 * (K ** 0.5)
+    # a captured call, replayed with the operands it was captured with and then with new ones in the same buffers
+    a, b = ops[0][0].clone(), ops[0][1].clone()
+    c = torch.empty(M, N, device=dev)
+    status = blas.ft_status_alloc(M, N, tile_class=tile_class)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        blas.ft_sgemm(M, N, K, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ws, tile_class=tile_class)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            blas.ft_sgemm(M, N, K, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ws, tile_class=tile_class)
+    torch.cuda.synchronize()
+    for replay in range(4):
+        src = ops[replay % 2]
+        a.copy_(src[0])
+        b.copy_(src[1])
+        c.fill_(float("nan"))
+        status.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        st = blas.ft_status_numpy(status)
+        assert not st["flag"].any(), (replay, st["flag"])
+        assert (c - src[2]).abs().max().item() < 1e-3 * (K ** 0.5), replay
