@@ -45,6 +45,16 @@ def test_sgemv_alpha_beta_padded_ld_and_no_workspace(blas, oracle_mod, trans, al
     _gemv_case(blas, oracle_mod, trans, 777, 513, alpha, beta, lda=517, use_ws=False)
 
 
+@pytest.mark.parametrize("trans", [False, True])
+@pytest.mark.parametrize("M,N,lda", [(5, 3000, 3001), (130, 16384, 16384), (70, 16385, 16390), (300, 2048, 2052), (3, 4099, 4099),
+                                     (513, 6000, 6004)])
+def test_sgemv_wide_rows(blas, oracle_mod, trans, M, N, lda):
+    """Rows of 2048 ... 16384 elements take the kernels that keep x in LDS (plain product) or give every wave a strip
+    of 2048 columns (transposed product); sizes on either side of their limits, ragged last strips, padded rows."""
+    _gemv_case(blas, oracle_mod, trans, M, N, 0.75, -1.25, lda=lda)
+    _gemv_case(blas, oracle_mod, trans, M, N, 1.0, 0.0, lda=lda, use_ws=False)
+
+
 def test_sgemv_exact_sums_and_reproducible(blas):
     # small integers: every partial sum is exact in FP32, so any summation order gives the same bits
     M, N = 1500, 700
