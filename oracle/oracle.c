@@ -24,8 +24,17 @@
  *   oracle_abft_*: pinned to the checksum algebra (e^T(AB) = (e^T A)B,
  *     (AB)e = A(Be)) and to the one known-answer case the reference holds
  *     (+1.0 at tile-local (0,1), threshold 0.1 -> row 0, col 1, magnitude 1;
- *     kernel/ft_sgemm/include/ft_sgemm_huge.cuh:40,145,263,358).  Bit-level
- *     oracle_abft_relative_thresholds (data-scaled thresholds, an addition
+ *     kernel/ft_sgemm/include/ft_sgemm_huge.cuh:40,145,263,358).
+ *   oracle_tile_acc (the FP32 accumulator model of the fault campaign):
+ *     pinned to numpy float64 on a rectangular padded case, to a float
+ *     accumulation-order case and to a hand case a transposed operand fails.
+ *   oracle_ft_sgemm with tau < 0, oracle_abft_decide_lines with per-line
+ *     thresholds, oracle_ft_sgemm_checked (verification every check_interval
+ *     k with resync, ft_sgemm_huge.cuh:143,263-271): pinned to independent
+ *     compositions of the pieces above and to closed forms (faults in
+ *     different intervals are each located; a corrected fault leaves no trace
+ *     in the later intervals).
+ *   oracle_abft_relative_thresholds (data-scaled thresholds, an addition
  *     with no reference counterpart): pinned to closed forms (constant and
  *     single-entry tiles) and to its scaling laws.  Bit-level
  *     agreement with the reference's CUDA kernels or cuBLAS: parity unpinned

@@ -192,6 +192,40 @@ def test_abft_residuals_not_transposed_for_rectangular_tiles(oracle_mod):
     assert dc.tolist() == [33.0, 66.0, 99.0, 132.0, 165.0]  # column sums of A@B
 
 
+def test_abft_reference_checksums_and_observe_are_the_two_halves_of_the_residuals(oracle_mod):
+    """abft_reference_checksums ((e^T A)B and A(Be), through the operands) and abft_observe (reference minus the line
+    sums of the accumulators) are what the device campaign calls separately: the first against numpy FP64 on a
+    rectangular, padded case that a transposed operand or a swapped output would fail, the second on hand values, and
+    the pair against abft_residuals."""
+    tm, tn, K, lda, ldb = 5, 7, 11, 13, 9
+    rng = np.random.default_rng(77)
+    a = rng.standard_normal((tm, lda)).astype(np.float32)
+    b = rng.standard_normal((K, ldb)).astype(np.float32)
+    a[:, K:] = np.nan   # padding is never read
+    b[:, tn:] = np.nan
+    cr, cc = oracle_mod.abft_reference_checksums(a, lda, b, ldb, tm, tn, K)
+    a64, b64 = a[:, :K].astype(np.float64), b[:, :tn].astype(np.float64)
+    assert cr.shape == (tm,) and cc.shape == (tn,)
+    assert np.allclose(cr, a64 @ b64.sum(axis=1), rtol=0, atol=1e-12)
+    assert np.allclose(cc, a64.sum(axis=0) @ b64, rtol=0, atol=1e-12)
+    # observe: residual = reference - observed line sum, rows and columns kept apart, padded accumulator rows
+    acc = np.full((3, 6), np.nan, dtype=np.float32)
+    acc[:, :4] = np.array([[1, 2, 3, 4], [10, 20, 30, 40], [0.5, 0.25, 0.125, 0]], dtype=np.float32)
+    dr, dc = oracle_mod.abft_observe(acc, 6, np.array([10.0, 90.0, 1.0]), np.array([11.5, 22.25, 33.0, 50.0]))
+    assert dr.tolist() == [0.0, -10.0, 0.125]
+    assert dc.tolist() == [0.0, 0.0, -0.125, 6.0]
+    # the composition is abft_residuals
+    acc2 = (a64 @ b64).astype(np.float32)
+    dr2, dc2 = oracle_mod.abft_observe(acc2, tn, cr, cc)
+    dr3, dc3 = oracle_mod.abft_residuals(a, lda, b, ldb, acc2, tn, tm, tn, K)
+    assert np.array_equal(dr2, dr3) and np.array_equal(dc2, dc3)
+
+
+def test_num_threads_reports_the_openmp_pool(oracle_mod):
+    import os
+    assert 1 <= oracle_mod.num_threads() <= max(os.cpu_count(), 1) * 4
+
+
 def test_abft_reference_known_answer(oracle_mod):
     """The one case the reference holds: +1.0 at tile-local (m=0, n=1) of a 128x128 tile, threshold 0.1
     -> row 0 and column 1 flagged, magnitude 1 removed (ft_sgemm_huge.cuh:40,145,263,358)."""
