@@ -1,6 +1,6 @@
-// SGEMV (row-major, both orientations) and the offline ABFT baseline composed from the library's own
-// SGEMM + SGEMV + SAXPY + SDOT, the way the reference composes its baseline from cuBLAS calls
-// (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:1-34).
+// SGEMV (row-major, both orientations; the counterpart of the cublasSgemv calls of the reference's offline ABFT
+// baseline) and the offline ABFT baseline itself (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:1-34): the library's
+// SGEMM per K panel plus two launches that do what the reference's six SGEMV, two SAXPY and two SDOT calls do.
 #include "common.h"
 
 namespace hpcdnn {

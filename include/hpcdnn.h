@@ -140,7 +140,7 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * `ws`/`ws_bytes`: optional DEVICE scratch of
  * hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM,M,N,K) bytes, 16-byte aligned, no
  * initialisation needed.  With it the checksum vectors of A and B are formed
- * once per tile row / tile column by two small kernels ahead of the GEMM
+ * once per tile row / tile column by a small kernel ahead of the GEMM
  * (faster); with ws == NULL each workgroup forms them in its main loop, as the
  * reference does.  Detection, location and correction are the same in both.
  * The size the query returns also has room for the K slices of a partial last
@@ -283,11 +283,12 @@ int hpcdnn_ft_sgemm_static(int M, int N, int K, const float* A, int lda, const f
 int hpcdnn_sgemv(int trans, int M, int N, float alpha, const float* A, int lda, const float* x, float beta, float* y,
                  void* ws, size_t ws_bytes, void* stream);
 
-/* Offline (panel-wise) ABFT SGEMM composed from hpcdnn_sgemm, hpcdnn_sgemv,
- * hpcdnn_saxpy and hpcdnn_sdot: C = alpha*A*B + beta*C is formed one K panel of
- * HPCDNN_OFFLINE_FT_PANEL_K at a time, and after every panel the row and
- * column sums of C are compared with checksums carried through the operands
- * (e^T A_p) B_p and A_p (B_p e), accumulated over the panels.
+/* Offline (panel-wise) ABFT SGEMM: C = alpha*A*B + beta*C is formed one K panel
+ * of HPCDNN_OFFLINE_FT_PANEL_K at a time (hpcdnn_sgemm), and after every panel
+ * the row and column sums of C (one pass over C) are compared with checksums
+ * carried through the operands, (e^T A_p) B_p and A_p (B_p e), accumulated over
+ * the panels (three launches per panel where the reference issues a GEMM, six
+ * SGEMV, two SAXPY and two SDOT calls).
  * `residuals`: DEVICE array of 2*ceil(K/panel) floats; [2p] = sum over the
  * columns of (column sums of C - reference), [2p+1] = the same over the rows,
  * after panel p.  Fault-free both are rounding noise; a soft error of size d
