@@ -47,7 +47,8 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline SGEMM line only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--ft-launches", type=int, default=1000, help="launches of the ABFT fault campaign")
-    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "sgemm_1024", "ft_sgemm", "saxpy", "sdot", "copy", "sgemv_n", "sgemv_t"],
+    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "sgemm_1024", "ft_sgemm", "ft_sgemm_fused", "ft_sgemm_wave", "offline_ft", "saxpy", "sdot", "copy",
+                             "sgemv_n", "sgemv_t"],
                     help="run one kernel only for --steps launches (for profiling with rocprofv3) and print a short line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -102,6 +103,22 @@ def main() -> int:
             status = blas.ft_status_alloc(m, m)
             ft_ws = blas.workspace(blas.ft_workspace_bytes(m, m, m))
             fn = lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=blas.ft_default_tau(m), status=status, ws=ft_ws)
+            work, unit = 2.0 * m ** 3, "GFLOP/s"
+        elif args.kernel in ("ft_sgemm_fused", "ft_sgemm_wave"):
+            m = 4096
+            a, b, c = operands(m, m, m, 20)
+            wave = args.kernel == "ft_sgemm_wave"
+            status = blas.ft_status_alloc(m, m, granularity=1 if wave else 0)
+            ft_ws = blas.workspace(blas.ft_workspace_bytes(m, m, m)) if wave else None
+            fn = lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=blas.ft_default_tau(m), status=status, ws=ft_ws,
+                                       granularity=1 if wave else 0)
+            work, unit = 2.0 * m ** 3, "GFLOP/s"
+        elif args.kernel == "offline_ft":
+            m = 4096
+            a, b, c = operands(m, m, m, 20)
+            ows = blas.workspace(blas.offline_ft_workspace_bytes(m, m, m))
+            res = torch.zeros(2 * (m // 256), device=dev)
+            fn = lambda: blas.offline_ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, res, ows)
             work, unit = 2.0 * m ** 3, "GFLOP/s"
         elif args.kernel in ("sgemv_n", "sgemv_t"):
             mv = 16384

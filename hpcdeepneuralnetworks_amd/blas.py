@@ -113,7 +113,7 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
              tile_class: int = 0, granularity: int = 0, check_interval: int = 0, faults=None) -> None:
     """ABFT GEMM; ``fault`` = (tile, row, col, delta) or None; ``status`` = int32 tensor of 8*ft_num_check_tiles words;
     ``ws`` = optional scratch tensor of ``ft_workspace_bytes(M, N, K)`` bytes (checksum vectors are then formed
-    by a pre-pass instead of inside the main loop); ``tile_class`` selects the ABFT tile (0 = 256x128, 1 = 128x128,
+    by a pre-pass instead of inside the main loop); ``tile_class`` selects the ABFT tile (0 = 256x128, 1 = 128x128, 3 = 128x64, 4 = 64x64,
     2 = 64x128).  ``granularity`` FT_GRAN_TILE keeps one checksum pair, verification and status record per tile of the
     class, FT_GRAN_WAVE one per wave tile (``ft_check_tile``); ``check_interval`` > 0 also verifies every that many
     values of k inside the K loop, with re-synchronised references; ``faults`` = up to four
