@@ -420,7 +420,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     float* const s_dump = s_br + 2 * BK + tid;                      // where the lanes that publish nothing write
     // destinations of this lane's publishes (parity 0); strides and the parity distance are the same for the
     // publishing lanes and the dump, so every write is base + immediate offset
-    float* const pub_a = (lane < 4) ? s_apart + (4 * (tid & 3)) * kParts + wave : s_dump;
+    // (after the transposing reduction lane l < 16 of a wave holds the wave's column sum of k = 4 * (l % 4) + l / 4)
+    float* const pub_a = (lane < 16) ? s_apart + (4 * (tid & 3) + (lane >> 2)) * kParts + wave : s_dump;
     float* const pub_b = (tid % B_V4_PER_ROW < B_SLOTS) ? s_br + tid / B_V4_PER_ROW + kHalfWaves * (tid % B_V4_PER_ROW) : s_dump;
     const int x32_addr = (lane ^ 32) * 4;  // ds_bpermute address of the partner lane in the other half wave
     // With wave-tile checksums a thread keeps one column sum per wave row gm (its columns lie in one wave column)
@@ -469,19 +470,27 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
             for (int e = 0; e < 4; ++e) HPCDNN_PIN(e_pa[e]);
         } else if constexpr (E == 1) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) e_pa[e] += dpp_mov<kDppRor4>(e_pa[e]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) HPCDNN_PIN(e_pa[e]);
+            // The four k values of a lane are summed over the 16 lanes of the wave that hold the same k group (lane
+            // bits 2 .. 5) by a transposing reduction: lane bit 2 decides which value of a pair stays and which
+            // travels to lane ^ 4, bit 3 likewise for the two that are left, then plain exchanges with lane ^ 16 and
+            // lane ^ 32.  One value per lane is left after two stages, so the whole costs 5 additions and 6 selects
+            // where four separate reductions cost 16 additions.
+            const bool up = lane & 4;
+            const float s0 = up ? e_pa[0] : e_pa[1], s1 = up ? e_pa[2] : e_pa[3];
+            e_pa[0] = up ? e_pa[1] : e_pa[0];
+            e_pa[1] = up ? e_pa[3] : e_pa[2];
+            e_sw[0] = lane_xor<4>(s0);
+            e_sw[1] = lane_xor<4>(s1);
         } else if constexpr (E == 2) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) e_pa[e] += dpp_mov<kDppRor8>(e_pa[e]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) HPCDNN_PIN(e_pa[e]);
+            e_pa[0] += e_sw[0];
+            e_pa[1] += e_sw[1];
+            const bool up = lane & 8;
+            const float s0 = up ? e_pa[0] : e_pa[1];
+            e_pa[0] = up ? e_pa[1] : e_pa[0];
+            e_sw[0] = lane_xor<8>(s0);
         } else if constexpr (E == 3) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                e_sw[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pa[e]), 0x401F));
+            e_pa[0] += e_sw[0];
+            e_sw[0] = lane_xor<16>(e_pa[0]);
         } else if constexpr (E == 4) {
             // row sums of B: in-thread over the 4 columns, first butterfly step for each staged k row ...
             e_pb0 = (rb[S][0].x + rb[S][0].y) + (rb[S][0].z + rb[S][0].w);
@@ -508,22 +517,17 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             // a k row of a 64-column tile lies in one row of 16 lanes and is complete here
             if constexpr (B_V4_PER_ROW == 32) e_swb = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pk), 0x401F));
         } else if constexpr (E == 8) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                e_pa[e] += e_sw[e];
-                e_sw[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(x32_addr, __builtin_bit_cast(int, e_pa[e])));
-            }
+            e_pa[0] += e_sw[0];
+            e_sw[0] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(x32_addr, __builtin_bit_cast(int, e_pa[0])));
             if constexpr (B_V4_PER_ROW == 32) e_pk += e_swb;
             HPCDNN_PIN(e_pk);
         } else if constexpr (E == 9) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { e_pa[e] += e_sw[e]; HPCDNN_PIN(e_pa[e]); }  // sum over the whole wave
+            e_pa[0] += e_sw[0];  // sum over the whole wave
+            HPCDNN_PIN(e_pa[0]);
         } else {
-            // lanes 0..3 of each wave publish the four k groups, lanes 0 (and 1) of each half wave the row sums; the other
-            // lanes write to their dump word, which keeps the loop free of branches
-            float* da = pub_a + par * (BK * kParts);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) da[e * kParts] = e_pa[e];
+            // lanes 0..15 of each wave publish the 16 column sums, the first lane (or two) of each k row of B its row sum;
+            // the other lanes write to their dump word, which keeps the loop free of branches
+            *(pub_a + par * (BK * kParts)) = e_pa[0];
             *(pub_b + par * BK) = e_pk;
         }
     };
