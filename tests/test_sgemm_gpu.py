@@ -190,6 +190,16 @@ def test_split_k_forced_matches_and_is_deterministic(blas, oracle_mod):
     assert np.array_equal(outs[-1][:, :N], again[:, :N])
 
 
+@pytest.mark.parametrize("M,N,K,split", [(200, 136, 4200, 13), (200, 136, 4200, 32), (77, 132, 9000, 64), (200, 138, 4200, 16)])
+def test_split_k_many_slices(blas, oracle_mod, M, N, K, split):
+    """More than eight slices are added by the reduction whose lanes share the slices of a group of elements (N a
+    multiple of 4; 138 columns take the other one): ragged element counts, beta != 0, padded ldc, same bits twice."""
+    ws = blas.workspace(M * N * split * 4)
+    first = _check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=4, split_k=split, ws=ws, ldc=N + 8)
+    again = _check(oracle_mod, blas, M, N, K, 1.5, -1.0, tile=4, split_k=split, ws=ws, ldc=N + 8)
+    assert np.array_equal(first[:, :N], again[:, :N])
+
+
 def test_tail_split_forced_matches_and_is_deterministic(blas, oracle_mod):
     """Only the tiles left over after the last full round of CUs are split along K (split_k < -1)."""
     M, N, K = 1088, 1024, 520  # 64x64 tiles: 17 x 16 = 272 = 256 + 16 leftover tiles; ragged K
