@@ -46,6 +46,7 @@ EXPORTS = (
     "hpcdnn_ft_default_tau",
     "hpcdnn_sgemv",
     "hpcdnn_offline_ft_sgemm",
+    "hpcdnn_offline_ft_sgemm_scalar",
     "hpcdnn_saxpy",
     "hpcdnn_sdot",
     "hpcdnn_workspace_bytes",
@@ -141,6 +142,8 @@ def lib():
     L.hpcdnn_sgemv.argtypes = [i, i, i, f, fp, i, fp, f, fp, vp, sz, vp]
     L.hpcdnn_offline_ft_sgemm.restype = i
     L.hpcdnn_offline_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, C.POINTER(Fault), fp, vp, sz, vp]
+    L.hpcdnn_offline_ft_sgemm_scalar.restype = i
+    L.hpcdnn_offline_ft_sgemm_scalar.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, C.POINTER(Fault), fp, vp, sz, vp]
     L.hpcdnn_saxpy.restype = i
     L.hpcdnn_saxpy.argtypes = [i64, f, fp, fp, vp]
     L.hpcdnn_sdot.restype = i

@@ -199,24 +199,29 @@ def sgemv_workspace_bytes(M: int, N: int) -> int:
 
 
 def offline_ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float,
-                     beta: float, residuals: torch.Tensor, ws: torch.Tensor, fault=None) -> None:
+                     beta: float, residuals: torch.Tensor, ws: torch.Tensor, fault=None, scalar: bool = False) -> None:
     """Panel-wise (offline) ABFT GEMM; ``residuals`` = float32 tensor of ``2*ceil(K/256)`` elements (column-side and
-    row-side residual sums per panel); ``fault`` = (panel, row, col, delta) with global row/col, or None.
+    row-side residual sums per panel), or of ``ceil(K/256)`` with ``scalar=True`` (one scalar checksum per panel:
+    total of C against the reference carried through the operands); ``fault`` = (panel, row, col, delta) with global
+    row/col, or None.
 
-    Counterpart of ``baseline_ft_sgemm(...)`` (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:1-34).
+    Counterpart of ``baseline_ft_sgemm(...)`` (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:1-34) and, with
+    ``scalar=True``, of ``offline_ft_sgemm(...)`` (:36-91).
     """
     pa, lda = _matrix(A, M, K, "A")
     pb, ldb = _matrix(B, K, N, "B")
     pc, ldc = _matrix(Cm, M, N, "C")
     panels = -(-K // _lib.OFFLINE_FT_PANEL_K)
+    need = panels if scalar else 2 * panels
     pr = _dev(residuals, "residuals")
-    if residuals.numel() < 2 * panels or not residuals.is_contiguous():
-        raise HpcdnnError(f"residuals must be a contiguous float32 GPU tensor with >= {2 * panels} elements")
+    if residuals.numel() < need or not residuals.is_contiguous():
+        raise HpcdnnError(f"residuals must be a contiguous float32 GPU tensor with >= {need} elements")
     f = None
     if fault is not None:
         f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
-    check(_lib.lib().hpcdnn_offline_ft_sgemm(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, f, pr, ws.data_ptr(),
-                                             ws.numel() * ws.element_size(), _stream()), "hpcdnn_offline_ft_sgemm")
+    fn = _lib.lib().hpcdnn_offline_ft_sgemm_scalar if scalar else _lib.lib().hpcdnn_offline_ft_sgemm
+    check(fn(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, f, pr, ws.data_ptr(), ws.numel() * ws.element_size(), _stream()),
+          "hpcdnn_offline_ft_sgemm_scalar" if scalar else "hpcdnn_offline_ft_sgemm")
 
 
 def offline_ft_workspace_bytes(M: int, N: int, K: int) -> int:

@@ -443,11 +443,24 @@ struct OfflineArgs {
     int c_blocks, a_blocks, b_blocks;  // roles of the sums launch, in this order; one more block when res_out is set
     int row_blocks, col_blocks;        // 64-row blocks of C, 1024-column blocks of C
     int carry_col_blocks;              // 256-column blocks of the carry launch (after its row_blocks row blocks)
+    // one scalar checksum per panel (hpcdnn_offline_ft_sgemm_scalar): the running reference total, and how many
+    // col_slots the finishing block adds to it (0: the row / column residual sums above)
+    double* scalar_ref;
+    int scalar;
 };
 
 // residual sums of a panel: the block partials added in block order
 __device__ __forceinline__ void finish_residuals(const OfflineArgs& p) {
     if (threadIdx.x != 0) return;
+    if (p.scalar) {
+        // total of C (block partials in block order) against the reference carried through the operands
+        double total = 0.0;
+        for (int b = 0; b < p.row_blocks; ++b) total += p.row_slots[b];
+        const double ref = *p.scalar_ref + p.col_slots[0];
+        *p.scalar_ref = ref;
+        p.res_out[0] = static_cast<float>(total - ref);
+        return;
+    }
     double sc = 0.0, sr = 0.0;
     for (int b = 0; b < p.carry_col_blocks; ++b) sc += p.col_slots[b];
     for (int b = 0; b < p.row_blocks; ++b) sr += p.row_slots[b];
@@ -587,6 +600,41 @@ __global__ __launch_bounds__(kGemvThreads) void offline_carry_kernel(const Offli
     if (tid == 0) p.col_slots[cbk] = s;
 }
 
+// One scalar checksum per panel.  Blocks 0 .. row_blocks-1: the sum of C over 64 rows, from the row sums of the sums
+// pass (column-block partials in order, rows in order within a thread, threads by block_sum_f64).  The last block:
+// alpha * sum_k a_col[k] * b_row[k], the panel's contribution to e^T (A B) e.
+__global__ __launch_bounds__(kGemvThreads) void offline_scalar_kernel(const OfflineArgs p) {
+    constexpr int pk = HPCDNN_OFFLINE_FT_PANEL_K;
+    __shared__ double red[kGemvWaves];
+    const int tid = threadIdx.x;
+    if (static_cast<int>(blockIdx.x) < p.row_blocks) {
+        const int r = blockIdx.x * kSumRows + tid;
+        double d = 0.0;
+        if (tid < kSumRows && r < p.M) d = static_cast<double>(strided_sum(p.rowpart + r, p.M, p.col_blocks));
+        const double s = block_sum_f64(d, red);
+        if (tid == 0) p.row_slots[blockIdx.x] = s;
+        return;
+    }
+    double d = 0.0;
+    if (tid < p.kp) {
+        const float ak = strided_sum(p.apart + tid, pk, p.row_blocks), bk = strided_sum(p.bpart + tid, pk, p.col_blocks);
+        d = static_cast<double>(ak) * static_cast<double>(bk);
+    }
+    const double s = block_sum_f64(d, red);
+    if (tid == 0) p.col_slots[0] = static_cast<double>(p.alpha) * s;
+}
+
+// the running scalar reference before the first panel: beta times the total of the C that is there (its row sums
+// from a sums pass), or zero
+__global__ __launch_bounds__(kGemvThreads) void offline_scalar_init_kernel(const OfflineArgs p, float beta) {
+    __shared__ double red[kGemvWaves];
+    double d = 0.0;
+    if (beta != 0.f)
+        for (int r = threadIdx.x; r < p.M; r += kGemvThreads) d += static_cast<double>(strided_sum(p.rowpart + r, p.M, p.col_blocks));
+    const double s = block_sum_f64(d, red);
+    if (threadIdx.x == 0) *p.scalar_ref = static_cast<double>(beta) * s;
+}
+
 // running references before the first panel: beta times the sums of the C that is there, or zeros
 __global__ __launch_bounds__(kGemvThreads) void offline_init_kernel(const OfflineArgs p, float beta) {
     const int i = blockIdx.x * kGemvThreads + threadIdx.x;
@@ -618,7 +666,7 @@ static OfflineWs offline_layout(int M, int N) {
     w.bpart = off; off += align64(cb * pk);
     w.ref_row = off; off += align64(M);
     w.ref_col = off; off += align64(N);
-    w.slots = off; off += align64(2 * (rb + static_cast<size_t>(ceil_div(N, kCarryCols))));  // doubles
+    w.slots = off; off += align64(2 * (rb + static_cast<size_t>(ceil_div(N, kCarryCols)) + 1));  // doubles; the last one is the scalar reference
     w.total = off;
     return w;
 }
@@ -637,13 +685,14 @@ extern "C" int hpcdnn_sgemv(int trans, int M, int N, float alpha, const float* A
     return run_sgemv(trans, M, N, alpha, A, lda, x, beta, y, ws, ws_bytes, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
-                                       int ldc, float alpha, float beta, const hpcdnn_fault* inject, float* residuals,
-                                       void* ws, size_t ws_bytes, void* stream) {
+static int run_offline_ft_sgemm(bool scalar, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                                int ldc, float alpha, float beta, const hpcdnn_fault* inject, float* residuals, void* ws,
+                                size_t ws_bytes, void* stream) {
     if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
     constexpr int pk = HPCDNN_OFFLINE_FT_PANEL_K;
     const int panels = K > 0 ? static_cast<int>(ceil_div(K, pk)) : 0;
+    const int per_panel = scalar ? 1 : 2;  // residuals per panel
     if (panels > 0 && !residuals) return HPCDNN_ERR_INVALID_VALUE;
     if (inject && (inject->tile < 0 || inject->tile >= panels || inject->row < 0 || inject->row >= M || inject->col < 0 ||
                    inject->col >= N))
@@ -667,6 +716,8 @@ extern "C" int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int 
     a.carry_col_blocks = static_cast<int>(ceil_div(N, kCarryCols));
     a.row_slots = reinterpret_cast<double*>(base + w.slots);
     a.col_slots = a.row_slots + a.row_blocks;
+    a.scalar_ref = a.col_slots + a.carry_col_blocks;
+    a.scalar = scalar ? 1 : 0;
     a.c_blocks = a.row_blocks * a.col_blocks;
     int rc = HPCDNN_OK;
     // running reference checksums start from what C already holds (nothing when beta == 0: C is not read then)
@@ -675,8 +726,12 @@ extern "C" int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int 
         first.a_blocks = first.b_blocks = 0;
         offline_sums_kernel<<<first.c_blocks, kGemvThreads, 0, s>>>(first);
     }
-    const int most = M > N ? M : N;
-    offline_init_kernel<<<static_cast<int>(ceil_div(most, kGemvThreads)), kGemvThreads, 0, s>>>(a, beta);
+    if (scalar) {
+        offline_scalar_init_kernel<<<1, kGemvThreads, 0, s>>>(a, beta);
+    } else {
+        const int most = M > N ? M : N;
+        offline_init_kernel<<<static_cast<int>(ceil_div(most, kGemvThreads)), kGemvThreads, 0, s>>>(a, beta);
+    }
     rc = launch_status();
     if (rc != HPCDNN_OK) return rc;
     for (int p = 0; p < panels; ++p) {
@@ -690,18 +745,35 @@ extern "C" int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int 
         if (inject && inject->tile == p)
             add_to_element_kernel<<<1, 1, 0, s>>>(C + static_cast<int64_t>(inject->row) * ldc + inject->col, inject->delta);
         // row and column sums of C, column sums of the A panel, row sums of the B panel (:8-17); one more block
-        // finishes the residual sums of the panel before
+        // finishes the residuals of the panel before
         a.a_blocks = a.row_blocks;
         a.b_blocks = static_cast<int>(ceil_div(kp, kSumRows)) * a.col_blocks;
-        a.res_out = p > 0 ? residuals + 2 * (p - 1) : nullptr;
+        a.res_out = p > 0 ? residuals + per_panel * (p - 1) : nullptr;
         offline_sums_kernel<<<a.c_blocks + a.a_blocks + a.b_blocks + (p > 0 ? 1 : 0), kGemvThreads, 0, s>>>(a);
-        // checksums carried through the operands into the running references, residual vectors and their block sums
-        // (:20-30)
-        offline_carry_kernel<<<a.row_blocks + a.carry_col_blocks, kGemvThreads, 0, s>>>(a);
+        if (scalar) {
+            // the total of C and the panel's carried scalar (:42-54)
+            offline_scalar_kernel<<<a.row_blocks + 1, kGemvThreads, 0, s>>>(a);
+        } else {
+            // checksums carried through the operands into the running references, residual vectors and their block
+            // sums (:20-30)
+            offline_carry_kernel<<<a.row_blocks + a.carry_col_blocks, kGemvThreads, 0, s>>>(a);
+        }
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;
     }
-    a.res_out = residuals + 2 * (panels - 1);
+    a.res_out = residuals + per_panel * (panels - 1);
     offline_finish_kernel<<<1, kWave, 0, s>>>(a);
     return launch_status();
+}
+
+extern "C" int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                                       int ldc, float alpha, float beta, const hpcdnn_fault* inject, float* residuals,
+                                       void* ws, size_t ws_bytes, void* stream) {
+    return run_offline_ft_sgemm(false, M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, inject, residuals, ws, ws_bytes, stream);
+}
+
+extern "C" int hpcdnn_offline_ft_sgemm_scalar(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                                              int ldc, float alpha, float beta, const hpcdnn_fault* inject, float* residuals,
+                                              void* ws, size_t ws_bytes, void* stream) {
+    return run_offline_ft_sgemm(true, M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, inject, residuals, ws, ws_bytes, stream);
 }

@@ -306,6 +306,24 @@ int hpcdnn_offline_ft_sgemm(int M, int N, int K, const float* A, int lda, const 
                             float alpha, float beta, const hpcdnn_fault* inject, float* residuals, void* ws,
                             size_t ws_bytes, void* stream);
 
+/* The same with one scalar checksum per panel: after every panel the total of C
+ * is compared with a reference carried through the operands,
+ *   e^T (A_p B_p) e = sum_k (e^T A_p)_k (B_p e)_k,
+ * accumulated over the panels (no second pass over the panels, a single
+ * residual per panel).  `residuals`: DEVICE array of ceil(K/panel) floats,
+ * [p] = total of C - reference after panel p; it equals residuals[2p] of
+ * hpcdnn_offline_ft_sgemm up to rounding.  Same workspace, `inject` and
+ * contract otherwise.
+ * Restates offline_ft_sgemm(num_tests, M, N, K, handle, dA, dB, dC, dE, dRes,
+ * dcheck_*..., alpha, beta, negative_1)
+ * (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:36-91), which forms the total
+ * of C, of the A panel's column sums and of the B panel's row sums after each
+ * panel product (twice over, each into the same scalar) and uses none of them:
+ * the identity above is what makes those sums a check. */
+int hpcdnn_offline_ft_sgemm_scalar(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                                   int ldc, float alpha, float beta, const hpcdnn_fault* inject, float* residuals,
+                                   void* ws, size_t ws_bytes, void* stream);
+
 /* y = alpha*x + y, one fused multiply-add per element, any n >= 0, any 4-byte
  * aligned x and y.  Replaces saxpy/saxpy3/_saxpy <<<ceil(n/4/tpb),tpb>>>
  * (N,alpha,x,y) (kernel/saxpy/saxpy.cu:15-48, launch :110-114). */

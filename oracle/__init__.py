@@ -109,6 +109,9 @@ def _load():
     lib.oracle_offline_ft_sgemm.restype = None
     lib.oracle_offline_ft_sgemm.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
                                             C.c_float, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, dp]
+    lib.oracle_offline_ft_sgemm_scalar.restype = None
+    lib.oracle_offline_ft_sgemm_scalar.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
+                                            C.c_float, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, dp]
     _lib = lib
     return lib
 
@@ -281,6 +284,17 @@ def offline_ft_sgemm(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, panel, fault=
     _load().oracle_offline_ft_sgemm(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, panel, int(fp_), int(fr),
                                     int(fc), float(fd), _d(res))
     return res[:2 * panels]
+
+
+def offline_ft_sgemm_scalar(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, panel, fault=None) -> np.ndarray:
+    """FP64 model of the panel-wise ABFT GEMM with one scalar checksum per panel; updates ``c`` in place and returns
+    the ceil(K/panel) residuals."""
+    panels = -(-K // panel)
+    res = np.zeros(max(panels, 1), np.float64)
+    fp_, fr, fc, fd = (-1, 0, 0, 0.0) if fault is None else fault
+    _load().oracle_offline_ft_sgemm_scalar(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, panel, int(fp_), int(fr),
+                                           int(fc), float(fd), _d(res))
+    return res[:panels]
 
 
 def abft_relative_thresholds(acc: np.ndarray, K: int, factor: float = 1.0):

@@ -21,6 +21,10 @@
  *     fault).  The reference computes these sums and never checks or prints
  *     them (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:26-30), so it holds
  *     no expected values: bit-level agreement with cuBLAS is parity unpinned.
+ *   oracle_offline_ft_sgemm_scalar (one scalar checksum per panel,
+ *     baseline_ft_sgemm.cuh:36-91): pinned to numpy float64 (total of C minus
+ *     the carried scalar, computed from whole-matrix sums) and to the same
+ *     closed form.
  *   oracle_abft_*: pinned to the checksum algebra (e^T(AB) = (e^T A)B,
  *     (AB)e = A(Be)) and to the one known-answer case the reference holds
  *     (+1.0 at tile-local (0,1), threshold 0.1 -> row 0, col 1, magnitude 1;
@@ -595,3 +599,51 @@ void oracle_offline_ft_sgemm(int M, int N, int K, const float* A, int lda, const
         for (int n = 0; n < N; ++n) C[(size_t)m * ldc + n] = (float)acc[(size_t)m * N + n];
     free(acc); free(ref_row); free(ref_col); free(a_col); free(b_row);
 }
+
+/* Offline ABFT with one scalar checksum per panel: the reference's second offline routine forms, after every panel
+ * product, the total of C (row sums of C dotted with ones), the total of the A panel's column sums and the total of
+ * the B panel's row sums, twice over, and leaves them unused (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:36-91).
+ * The identity that turns those sums into a check is e^T (A_p B_p) e = sum_k (e^T A_p)_k (B_p e)_k:
+ *   res[p] = (sum of all of C after panel p) - (beta * sum of C before + alpha * sum over the panels so far of
+ *            sum_k a_col[k] * b_row[k]).
+ * FP64 throughout; C receives the rounded product (with the uncorrected fault). */
+void oracle_offline_ft_sgemm_scalar(int M, int N, int K, const float* A, int lda, const float* B, int ldb,
+                                    float* C, int ldc, float alpha, float beta, int panel, int fault_panel,
+                                    int fault_row, int fault_col, float fault_delta, double* res) {
+    double* acc = (double*)calloc((size_t)M * N, sizeof(double));
+    double ref = 0.0;
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            double c0 = (beta != 0.0f) ? (double)beta * (double)C[(size_t)m * ldc + n] : 0.0;
+            acc[(size_t)m * N + n] = c0;
+            ref += c0;
+        }
+    int panels = (K + panel - 1) / panel;
+    for (int p = 0; p < panels; ++p) {
+        int k0 = p * panel, kp = (K - k0 < panel) ? K - k0 : panel;
+        #pragma omp parallel for schedule(static)
+        for (int m = 0; m < M; ++m)
+            for (int k = 0; k < kp; ++k) {
+                double a = (double)alpha * (double)A[(size_t)m * lda + k0 + k];
+                const float* brow = B + (size_t)(k0 + k) * ldb;
+                double* crow = acc + (size_t)m * N;
+                for (int n = 0; n < N; ++n) crow[n] += a * (double)brow[n];
+            }
+        if (p == fault_panel) acc[(size_t)fault_row * N + fault_col] += (double)fault_delta;
+        double carried = 0.0;
+        for (int k = 0; k < kp; ++k) {
+            double s = 0.0, t = 0.0;
+            for (int m = 0; m < M; ++m) s += (double)A[(size_t)m * lda + k0 + k];
+            for (int n = 0; n < N; ++n) t += (double)B[(size_t)(k0 + k) * ldb + n];
+            carried += s * t;
+        }
+        ref += (double)alpha * carried;
+        double total = 0.0;
+        for (size_t i = 0; i < (size_t)M * N; ++i) total += acc[i];
+        res[p] = total - ref;
+    }
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) C[(size_t)m * ldc + n] = (float)acc[(size_t)m * N + n];
+    free(acc);
+}
+

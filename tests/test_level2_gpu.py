@@ -142,3 +142,34 @@ def test_offline_ft_bad_arguments(blas):
     assert L.hpcdnn_offline_ft_sgemm(64, 64, 64, p, 64, p, 64, p, 64, 1.0, 0.0, C.byref(bad), p, ws.data_ptr(), ws.numel() * 4, None) == 1
     bad = _lib.Fault(0, 64, 0, 1.0)
     assert L.hpcdnn_offline_ft_sgemm(64, 64, 64, p, 64, p, 64, p, 64, 1.0, 0.0, C.byref(bad), p, ws.data_ptr(), ws.numel() * 4, None) == 1
+
+
+@pytest.mark.parametrize("M,N,K,alpha,beta,fault", [(512, 384, 1024, 1.0, 0.0, None), (300, 200, 700, 1.5, -0.5, (1, 299, 0, 6.0)),
+                                                    (1024, 1024, 256, 1.0, 1.0, (0, 17, 1000, -4.0))])
+def test_offline_ft_scalar_checksum(blas, oracle_mod, M, N, K, alpha, beta, fault):
+    """One scalar checksum per panel (baseline_ft_sgemm.cuh:36-91): residuals against the FP64 model within the noise
+    of adding M*N FP32-rounded entries, C as for SGEMM, and equal to residual [2p] of the row/column variant up to
+    the same noise."""
+    a = oracle_mod.fill_uniform_matrix(M, K, 850, ld=K + 4)
+    b = oracle_mod.fill_uniform_matrix(K, N, 851, ld=N + 4)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, 852, ld=N + 8)
+    da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+    panels = -(-K // 256)
+    res = torch.full((panels,), float("nan"), device="cuda")
+    ws = torch.full((blas.offline_ft_workspace_bytes(M, N, K) // 4,), float("nan"), device="cuda")  # poisoned
+    blas.offline_ft_sgemm(M, N, K, da, db, dc, alpha, beta, res, ws, fault=fault, scalar=True)
+    c_model = c0.copy()
+    res_model = oracle_mod.offline_ft_sgemm_scalar(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, alpha, beta, 256, fault)
+    got = res.cpu().numpy().astype(np.float64)
+    assert np.abs(got - res_model).max() < 0.05, (got, res_model)
+    ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, K + 4, b, N + 4, c0, N + 8, alpha, beta)
+    if fault is not None:
+        ref[fault[1], fault[2]] += fault[3]
+        den[fault[1], fault[2]] += abs(fault[3])
+    assert oracle_mod.gemm_max_err(N, dc.cpu().numpy(), N + 8, ref, den) <= TOL
+    # the row/column variant's column-side residual is the same quantity
+    dc2 = torch.from_numpy(c0).cuda()
+    res2 = torch.full((2 * panels,), float("nan"), device="cuda")
+    blas.offline_ft_sgemm(M, N, K, da, db, dc2, alpha, beta, res2, ws, fault=fault)
+    assert np.abs(got - res2.cpu().numpy()[0::2]).max() < 0.05
+

@@ -650,3 +650,31 @@ def test_golden_fixtures_pin_rng_saxpy_and_the_reference_fault_case(oracle_mod):
     for name in ("flag", "row", "col", "n_bad_rows", "n_bad_cols"):
         assert st[name] == k["expect"][name], name
     assert fix == k["expect"]["correction"]
+
+
+def test_offline_scalar_checksum_model(oracle_mod):
+    """One scalar checksum per panel: against whole-matrix numpy FP64 sums (a route that shares no loop with the
+    model: total of the product so far minus beta * total of C0 minus alpha * (column sums of A) . (row sums of B)
+    over the k range done), against the closed form (0 before the faulted panel, delta from it on), and against
+    residual [2p] of the row/column model, which it equals."""
+    M, N, K, panel = 37, 29, 610, 256
+    rng = np.random.default_rng(123)
+    a = rng.standard_normal((M, K + 3)).astype(np.float32)
+    b = rng.standard_normal((K, N + 5)).astype(np.float32)
+    c0 = rng.standard_normal((M, N + 2)).astype(np.float32)
+    alpha, beta = 1.25, -0.75
+    for fault in (None, (1, 5, 7, 3.5), (2, 36, 28, -2.0)):
+        c = c0.copy()
+        res = oracle_mod.offline_ft_sgemm_scalar(M, N, K, a, K + 3, b, N + 5, c, N + 2, alpha, beta, panel, fault)
+        assert res.shape == (3,)
+        a64, b64, c64 = a[:, :K].astype(np.float64), b[:, :N].astype(np.float64), c0[:, :N].astype(np.float64)
+        for p in range(3):
+            k1 = min(K, (p + 1) * panel)
+            total = (beta * c64 + alpha * a64[:, :k1] @ b64[:k1]).sum() + (fault[3] if fault and fault[0] <= p else 0.0)
+            ref = beta * c64.sum() + alpha * float(a64[:, :k1].sum(axis=0) @ b64[:k1].sum(axis=1))
+            assert abs(res[p] - (total - ref)) < 1e-9
+            assert abs(res[p] - (fault[3] if fault and fault[0] <= p else 0.0)) < 1e-9
+        c2 = c0.copy()
+        both = oracle_mod.offline_ft_sgemm(M, N, K, a, K + 3, b, N + 5, c2, N + 2, alpha, beta, panel, fault)
+        assert np.allclose(res, both[0::2], atol=1e-9) and np.array_equal(c, c2)
+
