@@ -28,6 +28,17 @@ inline int ft_sgemm(int M, int N, int K, const float* A, const float* B, float* 
                     size_t ws_bytes = 0) {
     return hpcdnn_ft_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, 0.0f, inject, status, ws, ws_bytes, nullptr);
 }
+// the two offline routines of kernel/ft_sgemm/include/baseline_ft_sgemm.cuh (:1-34 and :36-91): their cuBLAS handle and
+// eleven scratch vectors become one workspace of hpcdnn_workspace_bytes(HPCDNN_OP_OFFLINE_FT_SGEMM, M, N, K) bytes,
+// `residuals` receives what the reference leaves in dRes (2 values per K panel of 256, 1 for the scalar routine)
+inline int baseline_ft_sgemm(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta,
+                             float* residuals, void* ws, size_t ws_bytes) {
+    return hpcdnn_offline_ft_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, nullptr, residuals, ws, ws_bytes, nullptr);
+}
+inline int offline_ft_sgemm(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta,
+                            float* residuals, void* ws, size_t ws_bytes) {
+    return hpcdnn_offline_ft_sgemm_scalar(M, N, K, A, K, B, N, C, N, alpha, beta, nullptr, residuals, ws, ws_bytes, nullptr);
+}
 inline int saxpy(int N, float alpha, const float* x, float* y) { return hpcdnn_saxpy(N, alpha, x, y, nullptr); }
 // `ws` from hpcdnn_workspace_bytes(HPCDNN_OP_SDOT, ...) / hpcdnn_workspace_init
 inline int sdot(int N, const float* x, const float* y, float* out, void* ws, size_t ws_bytes) {
