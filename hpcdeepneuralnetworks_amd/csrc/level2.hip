@@ -326,19 +326,23 @@ static int run_sgemv(int trans, int M, int N, float alpha, const float* A, int l
     return launch_status();
 }
 
-// ---- offline ABFT (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:3-31), three launches per K panel behind the GEMM:
-//   sums   one pass over C for its row *and* column sums (partial per 1024-column / 64-row block), the column sums
-//          of the A panel and the row sums of the B panel, all in one grid;
-//   carry  the checksums carried through the operands, added to the running references, and next to them the
-//          residual vectors (sums of C minus references) reduced to one partial per block;
-//   the residual sums of panel p are finished by one extra block of the sums launch of panel p + 1 (a last small
-//   launch after the loop finishes the last panel's).
-// Every sum is formed in a fixed order: lanes, then waves, then blocks by index.
+// ---- offline ABFT (kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:3-31), two launches per K panel behind the GEMM:
+//   sums    one grid whose blocks (a) pass over C once for its row *and* column sums (partial per 512-column /
+//           64-row block), (b) form the column sums of the A panel and the row sums of the B panel of the *next* K
+//           panel (they depend on nothing the GEMM computes, so they are ready a launch ahead), (c) carry this panel's
+//           sums through its operands: rowcarry[m] = sum_k A_p[m][k] b_row[k], colcarry[chunk][n] = sum over a chunk
+//           of 64 k of a_col[k] B_p[k][n], and (d) one block that adds up the residual block sums of the panel before;
+//   finish  one thread per row and per column: running reference += alpha * carried value, sum of C's row / column
+//           from its block partials, residual, block sum of the residuals.
+// A last small launch after the loop adds up the last panel's block sums.  Every sum is formed in a fixed order: lanes,
+// then waves, then blocks by index.
 constexpr int kSumRows = 64;            // rows of one block of the sums pass: 16 per wave
 constexpr int kSumPieceCols = 4 * kWave;  // one 16-byte load per lane
 constexpr int kSumPieces = 2;           // 1 KiB pieces of a row per block: 512 columns
 constexpr int kSumCols = kSumPieces * kSumPieceCols;
-constexpr int kCarryCols = 256;         // columns per block of the carried column checksum
+constexpr int kCarryCols = 256;         // columns per block of the carried column checksum and of the finish launch
+constexpr int kCarryChunk = 64;         // k values per block of the carried column checksum
+constexpr int kCarryChunks = HPCDNN_OFFLINE_FT_PANEL_K / kCarryChunk;
 
 // rows [r0, r0 + 64) x columns [c0, c0 + PIECES * 256) of a row-major matrix: rowsum[r] = sum over the block's
 // columns of row r (lane partials combined by DPP), colsum[c] = sum over the block's rows of column c (in-lane over
@@ -401,10 +405,10 @@ __device__ __forceinline__ void sums_block(const float* __restrict__ mat, int ld
     }
 }
 
-// base[0] + base[stride] + ... (count terms, added in index order): sixteen loads are in flight before the first
+// base[0] + base[stride] + ... (count terms, added in index order): 32 loads are in flight before the first
 // addition waits, instead of one trip to memory per term
 __device__ __forceinline__ float strided_sum(const float* __restrict__ base, size_t stride, int count) {
-    constexpr int kBatch = 16;
+    constexpr int kBatch = 32;
     float s = 0.f;
     int i = 0;
     for (; i + kBatch <= count; i += kBatch) {
@@ -426,25 +430,32 @@ struct OfflineArgs {
     int M, N, kp;  // kp: columns of the A panel = rows of the B panel (<= HPCDNN_OFFLINE_FT_PANEL_K)
     const float* C;
     int ldc;
-    const float* Ap;
+    const float* Ap;  // this panel's operands (carry roles)
     int lda;
     const float* Bp;
     int ldb;
+    const float* An;  // the next panel's operands (panel-sum roles) and its width, 0 when there is none
+    const float* Bn;
+    int kn;
     float alpha;
-    float* rowpart;  // [col blocks of C][M]   row sums of C per 1024-column block
-    float* colpart;  // [row blocks of C][N]   column sums of C per 64-row block
-    float* apart;    // [row blocks][panel]    column sums of the A panel per 64-row block
-    float* bpart;    // [col blocks][panel]    row sums of the B panel per 1024-column block
-    float* ref_row;  // [M] running reference row checksum
-    float* ref_col;  // [N] running reference column checksum
-    double* row_slots;  // [row blocks]        sum of (row sums of C - reference) per carry block
-    double* col_slots;  // [N / 256]           the same for the column sums
-    float* res_out;     // where the residual sums of the panel before this one go (sums launch), or nullptr
-    int c_blocks, a_blocks, b_blocks;  // roles of the sums launch, in this order; one more block when res_out is set
-    int row_blocks, col_blocks;        // 64-row blocks of C, 1024-column blocks of C
-    int carry_col_blocks;              // 256-column blocks of the carry launch (after its row_blocks row blocks)
-    // one scalar checksum per panel (hpcdnn_offline_ft_sgemm_scalar): the running reference total, and how many
-    // col_slots the finishing block adds to it (0: the row / column residual sums above)
+    float* rowpart;     // [col blocks of C][M]   row sums of C per 512-column block
+    float* colpart;     // [row blocks of C][N]   column sums of C per 64-row block
+    float* apart;       // [row blocks][panel]    column sums of this panel of A per 64-row block
+    float* bpart;       // [col blocks][panel]    row sums of this panel of B per 512-column block
+    float* apart_next;  // the same for the next panel, written by the sums launch
+    float* bpart_next;
+    float* rowcarry;    // [M]                    sum_k A_p[m][k] * b_row[k]
+    float* colcarry;    // [kCarryChunks][N]      sum over 64 k of a_col[k] * B_p[k][n]
+    float* ref_row;     // [M] running reference row checksum
+    float* ref_col;     // [N] running reference column checksum
+    double* row_slots;  // residual block sums of the finish launch (256 rows each); scalar variant: totals of C per 64 rows
+    double* col_slots;  // [N / 256]           the same for the column sums; scalar variant: [0] = the carried scalar
+    float* res_out;     // where the residuals of the panel before this one go (sums launch), or nullptr
+    // roles of the sums launch, in this order; one more block when res_out is set
+    int c_blocks, a_blocks, b_blocks, rc_blocks, cc_blocks;
+    int row_blocks, col_blocks;        // 64-row blocks of C, 512-column blocks of C
+    int fin_row_blocks, fin_col_blocks;  // 256-row / 256-column blocks of the finish launch
+    // one scalar checksum per panel (hpcdnn_offline_ft_sgemm_scalar): the running reference total
     double* scalar_ref;
     int scalar;
 };
@@ -462,34 +473,10 @@ __device__ __forceinline__ void finish_residuals(const OfflineArgs& p) {
         return;
     }
     double sc = 0.0, sr = 0.0;
-    for (int b = 0; b < p.carry_col_blocks; ++b) sc += p.col_slots[b];
-    for (int b = 0; b < p.row_blocks; ++b) sr += p.row_slots[b];
+    for (int b = 0; b < p.fin_col_blocks; ++b) sc += p.col_slots[b];
+    for (int b = 0; b < p.fin_row_blocks; ++b) sr += p.row_slots[b];
     p.res_out[0] = static_cast<float>(sc);
     p.res_out[1] = static_cast<float>(sr);
-}
-
-__global__ __launch_bounds__(kGemvThreads) void offline_sums_kernel(const OfflineArgs p) {
-    __shared__ v4f part[kGemvWaves][kSumPieces][kWave];
-    int b = blockIdx.x;
-    if (b < p.c_blocks) {
-        const int rb = b / p.col_blocks, cb = b % p.col_blocks;
-        sums_block<kSumPieces, true, true>(p.C, p.ldc, p.M, p.N, rb * kSumRows, cb * kSumCols, p.rowpart + static_cast<size_t>(cb) * p.M,
-                                           p.colpart + static_cast<size_t>(rb) * p.N, part);
-        return;
-    }
-    b -= p.c_blocks;
-    if (b < p.a_blocks) {  // column sums of the A panel (M x kp): one 256-column piece
-        sums_block<1, false, true>(p.Ap, p.lda, p.M, p.kp, b * kSumRows, 0, nullptr, p.apart + static_cast<size_t>(b) * HPCDNN_OFFLINE_FT_PANEL_K, part);
-        return;
-    }
-    b -= p.a_blocks;
-    if (b < p.b_blocks) {  // row sums of the B panel (kp x N)
-        const int rb = b / p.col_blocks, cb = b % p.col_blocks;
-        sums_block<kSumPieces, true, false>(p.Bp, p.ldb, p.kp, p.N, rb * kSumRows, cb * kSumCols,
-                                            p.bpart + static_cast<size_t>(cb) * HPCDNN_OFFLINE_FT_PANEL_K, nullptr, part);
-        return;
-    }
-    finish_residuals(p);
 }
 
 // sum of a double over the block, valid in thread 0 (wave partials added in wave order)
@@ -504,80 +491,65 @@ __device__ __forceinline__ double block_sum_f64(double v, double* lds) {
     return s;
 }
 
-// Blocks 0 .. row_blocks-1: ref_row[m] += alpha * sum_k A_p[m][k] * b_row[k] for 64 rows (b_row = the B panel's row
-// sums, its column-block partials added in order), then the row residuals c_row[m] - ref_row[m] of those rows, summed.
-// The other blocks: ref_col[n] += alpha * sum_k a_col[k] * B_p[k][n] for 256 columns (a_col likewise from its
-// row-block partials), and the column residuals.  (baseline_ft_sgemm.cuh:20-30)
-__global__ __launch_bounds__(kGemvThreads) void offline_carry_kernel(const OfflineArgs p) {
+// rowcarry[m] = sum_k A_p[m][k] * b_row[k] for the 64 rows of block rb (b_row = the B panel's row sums, its
+// column-block partials added in order): one wave per row, the row's 256 values in one load.  (baseline_ft_sgemm.cuh:23)
+__device__ __forceinline__ void carry_rows_block(const OfflineArgs& p, int rb, float* vec) {
     constexpr int pk = HPCDNN_OFFLINE_FT_PANEL_K;
     static_assert(pk == kGemvThreads && pk == kSumPieceCols, "one thread per k of a panel, one piece per panel row of A");
-    __shared__ float vec[pk];
-    __shared__ v4f part[kGemvWaves][kWave];
-    __shared__ float colsum[kCarryCols];  // carried sums of the block's columns (or of its 64 rows)
-    __shared__ double red[kGemvWaves];
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-    if (static_cast<int>(blockIdx.x) < p.row_blocks) {
-        vec[tid] = tid < p.kp ? strided_sum(p.bpart + tid, pk, p.col_blocks) : 0.f;
-        __syncthreads();
-        const v4f bv = *reinterpret_cast<const v4f*>(vec + lane * 4);
-        const int r0 = blockIdx.x * kSumRows;
-        constexpr int kUnroll = 8;
-        for (int i = 0; i < kSumRows / kGemvWaves; i += kUnroll) {
-            v4f a[kUnroll];
+    vec[tid] = tid < p.kp ? strided_sum(p.bpart + tid, pk, p.col_blocks) : 0.f;
+    __syncthreads();
+    const v4f bv = *reinterpret_cast<const v4f*>(vec + lane * 4);
+    const int r0 = rb * kSumRows;
+    constexpr int kUnroll = 16;
+    static_assert(kSumRows / kGemvWaves == kUnroll, "all rows of a wave in one batch");
+    v4f a[kUnroll];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const int r = r0 + wave + kGemvWaves * (i + u);
-                const bool valid = r < p.M;
-                a[u] = buffer_load_v4f(make_rsrc(p.Ap + static_cast<int64_t>(valid ? r : r0) * p.lda, valid ? static_cast<int64_t>(p.kp) * 4 : 0), lane * 16);
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                float s = __builtin_fmaf(a[u].x, bv.x, 0.f);
-                s = __builtin_fmaf(a[u].y, bv.y, s);
-                s = __builtin_fmaf(a[u].z, bv.z, s);
-                s = __builtin_fmaf(a[u].w, bv.w, s);
-                s = wave_sum_lane63(s);
-                if (lane == kWave - 1) colsum[wave + kGemvWaves * (i + u)] = s;  // row number inside the block
-            }
-        }
-        __syncthreads();
-        // one thread per row: reference, sum of C's row from its column-block partials, residual
-        double d = 0.0;
-        const int r = r0 + tid;
-        if (tid < kSumRows && r < p.M) {
-            const float ref = __builtin_fmaf(p.alpha, colsum[tid], p.ref_row[r]);
-            p.ref_row[r] = ref;
-            const float c = strided_sum(p.rowpart + r, p.M, p.col_blocks);
-            d = static_cast<double>(c - ref);
-        }
-        const double s = block_sum_f64(d, red);
-        if (tid == 0) p.row_slots[blockIdx.x] = s;
-        return;
+    for (int u = 0; u < kUnroll; ++u) {
+        const int r = r0 + wave + kGemvWaves * u;
+        const bool valid = r < p.M;
+        a[u] = buffer_load_v4f(make_rsrc(p.Ap + static_cast<int64_t>(valid ? r : r0) * p.lda, valid ? static_cast<int64_t>(p.kp) * 4 : 0), lane * 16);
     }
-    const int cbk = blockIdx.x - p.row_blocks, c0 = cbk * kCarryCols;
-    vec[tid] = tid < p.kp ? strided_sum(p.apart + tid, pk, p.row_blocks) : 0.f;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int r = r0 + wave + kGemvWaves * u;
+        float s = __builtin_fmaf(a[u].x, bv.x, 0.f);
+        s = __builtin_fmaf(a[u].y, bv.y, s);
+        s = __builtin_fmaf(a[u].z, bv.z, s);
+        s = __builtin_fmaf(a[u].w, bv.w, s);
+        s = wave_sum_lane63(s);
+        if (lane == kWave - 1 && r < p.M) p.rowcarry[r] = s;
+    }
+}
+
+// colcarry[chunk][n] = sum over the 64 k of the chunk of a_col[k] * B_p[k][n] for the 256 columns of block cbk (a_col
+// from its row-block partials): wave w takes rows w, w + 4, ... of the chunk, all sixteen in flight; the four wave
+// partials are added in wave order.  (baseline_ft_sgemm.cuh:20)
+__device__ __forceinline__ void carry_cols_block(const OfflineArgs& p, int cbk, int chunk, float* vec, v4f (*part)[kWave]) {
+    constexpr int pk = HPCDNN_OFFLINE_FT_PANEL_K;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int c0 = cbk * kCarryCols, k0 = chunk * kCarryChunk;
+    if (tid < kCarryChunk) vec[tid] = (k0 + tid < p.kp) ? strided_sum(p.apart + k0 + tid, pk, p.row_blocks) : 0.f;
     __syncthreads();
     const int64_t row_bytes = static_cast<int64_t>(p.N - c0) * 4;
+    constexpr int kUnroll = kCarryChunk / kGemvWaves;
+    v4f bq[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int kk = k0 + wave + u * kGemvWaves;
+        const bool valid = kk < p.kp;
+        bq[u] = buffer_load_v4f(make_rsrc(p.Bp + static_cast<int64_t>(valid ? kk : 0) * p.ldb + c0, valid ? row_bytes : 0), lane * 16);
+    }
     v4f acc = {0.f, 0.f, 0.f, 0.f};
-    constexpr int kUnroll = 8;
-    for (int k = wave; k < p.kp; k += kUnroll * kGemvWaves) {
-        v4f bq[kUnroll];
-        float av[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int kk = k + u * kGemvWaves;
-            const bool valid = kk < p.kp;
-            bq[u] = buffer_load_v4f(make_rsrc(p.Bp + static_cast<int64_t>(valid ? kk : 0) * p.ldb + c0, valid ? row_bytes : 0), lane * 16);
-            av[u] = valid ? vec[kk] : 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            acc.x = __builtin_fmaf(bq[u].x, av[u], acc.x);
-            acc.y = __builtin_fmaf(bq[u].y, av[u], acc.y);
-            acc.z = __builtin_fmaf(bq[u].z, av[u], acc.z);
-            acc.w = __builtin_fmaf(bq[u].w, av[u], acc.w);
-        }
+    for (int u = 0; u < kUnroll; ++u) {
+        const float av = vec[wave + u * kGemvWaves];
+        acc.x = __builtin_fmaf(bq[u].x, av, acc.x);
+        acc.y = __builtin_fmaf(bq[u].y, av, acc.y);
+        acc.z = __builtin_fmaf(bq[u].z, av, acc.z);
+        acc.w = __builtin_fmaf(bq[u].w, av, acc.w);
     }
     part[wave][lane] = acc;
     __syncthreads();
@@ -585,19 +557,78 @@ __global__ __launch_bounds__(kGemvThreads) void offline_carry_kernel(const Offli
         v4f t = part[0][lane];
 #pragma unroll
         for (int w = 1; w < kGemvWaves; ++w) t += part[w][lane];
-        *reinterpret_cast<v4f*>(colsum + lane * 4) = t;
+        const float tv[4] = {t.x, t.y, t.z, t.w};
+        float* dst = p.colcarry + static_cast<size_t>(chunk) * p.N;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (c0 + lane * 4 + e < p.N) dst[c0 + lane * 4 + e] = tv[e];
     }
-    __syncthreads();
-    const int n = c0 + tid;
+}
+
+__global__ __launch_bounds__(kGemvThreads) void offline_sums_kernel(const OfflineArgs p) {
+    __shared__ v4f part[kGemvWaves][kSumPieces][kWave];
+    __shared__ float vec[HPCDNN_OFFLINE_FT_PANEL_K];
+    int b = blockIdx.x;
+    if (b < p.c_blocks) {
+        const int rb = b / p.col_blocks, cb = b % p.col_blocks;
+        sums_block<kSumPieces, true, true>(p.C, p.ldc, p.M, p.N, rb * kSumRows, cb * kSumCols, p.rowpart + static_cast<size_t>(cb) * p.M,
+                                           p.colpart + static_cast<size_t>(rb) * p.N, part);
+        return;
+    }
+    b -= p.c_blocks;
+    if (b < p.a_blocks) {  // column sums of the next A panel (M x kn): one 256-column piece
+        sums_block<1, false, true>(p.An, p.lda, p.M, p.kn, b * kSumRows, 0, nullptr, p.apart_next + static_cast<size_t>(b) * HPCDNN_OFFLINE_FT_PANEL_K, part);
+        return;
+    }
+    b -= p.a_blocks;
+    if (b < p.b_blocks) {  // row sums of the next B panel (kn x N)
+        const int rb = b / p.col_blocks, cb = b % p.col_blocks;
+        sums_block<kSumPieces, true, false>(p.Bn, p.ldb, p.kn, p.N, rb * kSumRows, cb * kSumCols,
+                                            p.bpart_next + static_cast<size_t>(cb) * HPCDNN_OFFLINE_FT_PANEL_K, nullptr, part);
+        return;
+    }
+    b -= p.b_blocks;
+    if (b < p.rc_blocks) {
+        carry_rows_block(p, b, vec);
+        return;
+    }
+    b -= p.rc_blocks;
+    if (b < p.cc_blocks) {
+        carry_cols_block(p, b / kCarryChunks, b % kCarryChunks, vec, reinterpret_cast<v4f(*)[kWave]>(&part[0][0][0]));
+        return;
+    }
+    finish_residuals(p);
+}
+
+// One thread per row (blocks 0 .. fin_row_blocks-1) or per column: the carried value goes into the running reference,
+// the row / column sum of C is put together from its block partials, and the residuals of the block's 256 lines are
+// summed.  (baseline_ft_sgemm.cuh:26-30)
+__global__ __launch_bounds__(kGemvThreads) void offline_finish_lines_kernel(const OfflineArgs p) {
+    __shared__ double red[kGemvWaves];
+    const int tid = threadIdx.x;
     double d = 0.0;
+    if (static_cast<int>(blockIdx.x) < p.fin_row_blocks) {
+        const int r = blockIdx.x * kGemvThreads + tid;
+        if (r < p.M) {
+            const float ref = __builtin_fmaf(p.alpha, p.rowcarry[r], p.ref_row[r]);
+            p.ref_row[r] = ref;
+            d = static_cast<double>(strided_sum(p.rowpart + r, p.M, p.col_blocks) - ref);
+        }
+        const double s = block_sum_f64(d, red);
+        if (tid == 0) p.row_slots[blockIdx.x] = s;
+        return;
+    }
+    const int cb = blockIdx.x - p.fin_row_blocks, n = cb * kCarryCols + tid;
     if (n < p.N) {
-        const float ref = __builtin_fmaf(p.alpha, colsum[tid], p.ref_col[n]);
+        float carried = p.colcarry[n];
+#pragma unroll
+        for (int ch = 1; ch < kCarryChunks; ++ch) carried += p.colcarry[static_cast<size_t>(ch) * p.N + n];
+        const float ref = __builtin_fmaf(p.alpha, carried, p.ref_col[n]);
         p.ref_col[n] = ref;
-        const float c = strided_sum(p.colpart + n, p.N, p.row_blocks);
-        d = static_cast<double>(c - ref);
+        d = static_cast<double>(strided_sum(p.colpart + n, p.N, p.row_blocks) - ref);
     }
     const double s = block_sum_f64(d, red);
-    if (tid == 0) p.col_slots[cbk] = s;
+    if (tid == 0) p.col_slots[cb] = s;
 }
 
 // One scalar checksum per panel.  Blocks 0 .. row_blocks-1: the sum of C over 64 rows, from the row sums of the sums
@@ -650,7 +681,8 @@ __global__ void offline_finish_kernel(const OfflineArgs p) { finish_residuals(p)
 
 // ---- workspace carving (sizes in floats, each region 64-float aligned)
 struct OfflineWs {
-    size_t rowpart, colpart, apart, bpart, ref_row, ref_col, slots, total;
+    size_t rowpart, colpart, apart, bpart, rowcarry, colcarry, ref_row, ref_col, slots, total;
+    size_t apart_len, bpart_len;  // one of the two panel-sum buffers each
 };
 
 static size_t align64(size_t v) { return (v + 63) & ~static_cast<size_t>(63); }
@@ -662,8 +694,12 @@ static OfflineWs offline_layout(int M, int N) {
     size_t off = 0;
     w.rowpart = off; off += align64(cb * M);
     w.colpart = off; off += align64(rb * N);
-    w.apart = off; off += align64(rb * pk);
-    w.bpart = off; off += align64(cb * pk);
+    w.apart_len = align64(rb * pk);
+    w.bpart_len = align64(cb * pk);
+    w.apart = off; off += 2 * w.apart_len;  // this panel's and the next one's
+    w.bpart = off; off += 2 * w.bpart_len;
+    w.rowcarry = off; off += align64(M);
+    w.colcarry = off; off += align64(static_cast<size_t>(kCarryChunks) * N);
     w.ref_row = off; off += align64(M);
     w.ref_col = off; off += align64(N);
     w.slots = off; off += align64(2 * (rb + static_cast<size_t>(ceil_div(N, kCarryCols)) + 1));  // doubles; the last one is the scalar reference
@@ -709,22 +745,33 @@ static int run_offline_ft_sgemm(bool scalar, int M, int N, int K, const float* A
     a.M = M; a.N = N;
     a.C = C; a.ldc = ldc; a.lda = lda; a.ldb = ldb;
     a.alpha = alpha;
-    a.rowpart = base + w.rowpart; a.colpart = base + w.colpart; a.apart = base + w.apart; a.bpart = base + w.bpart;
+    a.rowpart = base + w.rowpart; a.colpart = base + w.colpart;
+    a.rowcarry = base + w.rowcarry; a.colcarry = base + w.colcarry;
     a.ref_row = base + w.ref_row; a.ref_col = base + w.ref_col;
     a.row_blocks = static_cast<int>(ceil_div(M, kSumRows));
     a.col_blocks = static_cast<int>(ceil_div(N, kSumCols));
-    a.carry_col_blocks = static_cast<int>(ceil_div(N, kCarryCols));
+    a.fin_row_blocks = static_cast<int>(ceil_div(M, kGemvThreads));
+    a.fin_col_blocks = static_cast<int>(ceil_div(N, kCarryCols));
     a.row_slots = reinterpret_cast<double*>(base + w.slots);
     a.col_slots = a.row_slots + a.row_blocks;
-    a.scalar_ref = a.col_slots + a.carry_col_blocks;
+    a.scalar_ref = a.col_slots + a.fin_col_blocks;
     a.scalar = scalar ? 1 : 0;
-    a.c_blocks = a.row_blocks * a.col_blocks;
+    float* apart[2] = {base + w.apart, base + w.apart + w.apart_len};
+    float* bpart[2] = {base + w.bpart, base + w.bpart + w.bpart_len};
     int rc = HPCDNN_OK;
-    // running reference checksums start from what C already holds (nothing when beta == 0: C is not read then)
-    if (beta != 0.f) {
+    // running reference checksums start from what C already holds (nothing when beta == 0: C is not read then); the
+    // same launch forms the sums of the first panels of A and B
+    {
         OfflineArgs first = a;
-        first.a_blocks = first.b_blocks = 0;
-        offline_sums_kernel<<<first.c_blocks, kGemvThreads, 0, s>>>(first);
+        first.c_blocks = beta != 0.f ? a.row_blocks * a.col_blocks : 0;
+        first.An = A;
+        first.Bn = B;
+        first.kn = K < pk ? K : pk;
+        first.apart_next = apart[0];
+        first.bpart_next = bpart[0];
+        first.a_blocks = a.row_blocks;
+        first.b_blocks = static_cast<int>(ceil_div(first.kn, kSumRows)) * a.col_blocks;
+        offline_sums_kernel<<<first.c_blocks + first.a_blocks + first.b_blocks, kGemvThreads, 0, s>>>(first);
     }
     if (scalar) {
         offline_scalar_init_kernel<<<1, kGemvThreads, 0, s>>>(a, beta);
@@ -734,29 +781,39 @@ static int run_offline_ft_sgemm(bool scalar, int M, int N, int K, const float* A
     }
     rc = launch_status();
     if (rc != HPCDNN_OK) return rc;
+    a.c_blocks = a.row_blocks * a.col_blocks;
     for (int p = 0; p < panels; ++p) {
         const int k0 = p * pk, kp = (K - k0 < pk) ? K - k0 : pk;
         a.kp = kp;
         a.Ap = A + k0;
         a.Bp = B + static_cast<int64_t>(k0) * ldb;
+        a.apart = apart[p & 1];
+        a.bpart = bpart[p & 1];
         // the panel's product (baseline_ft_sgemm.cuh:5)
         rc = hpcdnn_sgemm(M, N, kp, a.Ap, lda, a.Bp, ldb, C, ldc, alpha, p == 0 ? beta : 1.f, nullptr, 0, stream);
         if (rc != HPCDNN_OK) return rc;
         if (inject && inject->tile == p)
             add_to_element_kernel<<<1, 1, 0, s>>>(C + static_cast<int64_t>(inject->row) * ldc + inject->col, inject->delta);
-        // row and column sums of C, column sums of the A panel, row sums of the B panel (:8-17); one more block
-        // finishes the residuals of the panel before
-        a.a_blocks = a.row_blocks;
-        a.b_blocks = static_cast<int>(ceil_div(kp, kSumRows)) * a.col_blocks;
+        // row and column sums of C (:8-11), the next panel's sums (:14-17), this panel's sums carried through its
+        // operands (:20-23); one more block finishes the residuals of the panel before
+        const int kn = p + 1 < panels ? ((K - k0 - pk < pk) ? K - k0 - pk : pk) : 0;
+        a.kn = kn;
+        a.An = A + k0 + pk;
+        a.Bn = B + static_cast<int64_t>(k0 + pk) * ldb;
+        a.apart_next = apart[(p + 1) & 1];
+        a.bpart_next = bpart[(p + 1) & 1];
+        a.a_blocks = kn > 0 ? a.row_blocks : 0;
+        a.b_blocks = kn > 0 ? static_cast<int>(ceil_div(kn, kSumRows)) * a.col_blocks : 0;
+        a.rc_blocks = scalar ? 0 : a.row_blocks;
+        a.cc_blocks = scalar ? 0 : a.fin_col_blocks * kCarryChunks;
         a.res_out = p > 0 ? residuals + per_panel * (p - 1) : nullptr;
-        offline_sums_kernel<<<a.c_blocks + a.a_blocks + a.b_blocks + (p > 0 ? 1 : 0), kGemvThreads, 0, s>>>(a);
+        offline_sums_kernel<<<a.c_blocks + a.a_blocks + a.b_blocks + a.rc_blocks + a.cc_blocks + (p > 0 ? 1 : 0), kGemvThreads, 0, s>>>(a);
         if (scalar) {
             // the total of C and the panel's carried scalar (:42-54)
             offline_scalar_kernel<<<a.row_blocks + 1, kGemvThreads, 0, s>>>(a);
         } else {
-            // checksums carried through the operands into the running references, residual vectors and their block
-            // sums (:20-30)
-            offline_carry_kernel<<<a.row_blocks + a.carry_col_blocks, kGemvThreads, 0, s>>>(a);
+            // running references, residual vectors and their block sums (:26-30)
+            offline_finish_lines_kernel<<<a.fin_row_blocks + a.fin_col_blocks, kGemvThreads, 0, s>>>(a);
         }
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;

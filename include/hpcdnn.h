@@ -287,8 +287,8 @@ int hpcdnn_sgemv(int trans, int M, int N, float alpha, const float* A, int lda, 
  * of HPCDNN_OFFLINE_FT_PANEL_K at a time (hpcdnn_sgemm), and after every panel
  * the row and column sums of C (one pass over C) are compared with checksums
  * carried through the operands, (e^T A_p) B_p and A_p (B_p e), accumulated over
- * the panels (three launches per panel where the reference issues a GEMM, six
- * SGEMV, two SAXPY and two SDOT calls).
+ * the panels (the GEMM and two more launches per panel where the reference
+ * issues a GEMM, six SGEMV, two SAXPY and two SDOT calls).
  * `residuals`: DEVICE array of 2*ceil(K/panel) floats; [2p] = sum over the
  * columns of (column sums of C - reference), [2p+1] = the same over the rows,
  * after panel p.  Fault-free both are rounding noise; a soft error of size d
