@@ -270,11 +270,15 @@ def main() -> int:
         status_w = blas.ft_status_alloc(m, m, granularity=blas.FT_GRAN_WAVE)
         ms_wave = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status_w, ws=ft_ws,
                                                      granularity=blas.FT_GRAN_WAVE), st, wu)
+        status_w1 = blas.ft_status_alloc(m, m, tile_class=1, granularity=blas.FT_GRAN_WAVE)  # 64x64 wave tiles of the 128x128 class
+        ms_wave1 = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status_w1, ws=ft_ws, tile_class=1,
+                                                      granularity=blas.FT_GRAN_WAVE), st, wu)
         ms_cad = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ft_ws, check_interval=256), st, wu)
         ms_cad_fused = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, check_interval=256), st, wu)
         pct = lambda t: round((t - ms_plain) / ms_plain * 100.0, 2)
         extras["abft_granularity_4096"] = {
             "tile_256x128_overhead_pct": pct(ms_ft), "wave_tile_128x32_overhead_pct": pct(ms_wave),
+            "wave_tile_64x64_of_128x128_class_overhead_pct": pct(ms_wave1),
             "tile_verify_every_256k_overhead_pct": pct(ms_cad), "tile_verify_every_256k_no_workspace_overhead_pct": pct(ms_cad_fused),
             "wave_tile_gflops": round(2.0 * m ** 3 / ms_wave / 1e6, 1),
             "reference_T4_block_warp_thread_overhead_pct": [13.49, 27.52, 45.13],    # 4761.49 / {4195.57, 3733.88, 3280.92} - 1

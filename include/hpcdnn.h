@@ -196,6 +196,8 @@ int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
  * verified, located and corrected on its own, so one fault per wave tile is
  * correctable where tile granularity reports two faults in one 256x128 tile
  * as uncorrectable.  Needs the workspace (HPCDNN_ERR_WORKSPACE without one).
+ * Class 1 is the cheapest carrier of this granularity (4096^3: +13 % over plain
+ * SGEMM, class 0: +19 %).
  * The wave tile is the finest granularity on this hardware: a matrix-core
  * instruction spreads its 32x32 result over all 64 lanes, so there is no
  * per-thread tile to keep checksums for.
