@@ -55,8 +55,8 @@ static const FtClass kFtClasses[HPCDNN_FT_NUM_CLASSES] = {
      HPCDNN_FT_KERNEL(256, 2, 4, 2, 0, true), abft_encode_kernel<256, 128>, abft_encode_kernel<128, 32>},
     // 1 large
     {128, 128, 2, 2, HPCDNN_FT_KERNEL(128, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(128, 2, 2, 2, 0, false),
-     HPCDNN_FT_KERNEL(128, 2, 2, 2, 1, false), HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<128, 128>,
-     abft_encode_kernel<64, 64>},
+     HPCDNN_FT_KERNEL(128, 2, 2, 2, 1, false), HPCDNN_FT_KERNEL(128, 2, 2, 1, 0, true), HPCDNN_FT_KERNEL(128, 2, 2, 2, 0, true),
+     abft_encode_kernel<128, 128>, abft_encode_kernel<64, 64>},
     // 2 wide
     {64, 128, 2, 2, HPCDNN_FT_KERNEL(64, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(64, 2, 2, 2, 0, false),
      HPCDNN_FT_KERNEL(64, 2, 2, 2, 1, false), HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<64, 128>,

@@ -211,7 +211,7 @@ int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
  * record of a check tile merges its verifications: bad-line counts add up,
  * flag 2 if any verification could not locate its fault, else 1 if any
  * corrected an element; row, col and the residuals are those of the first
- * correction.  Tile granularity, class 0 only.
+ * correction.  Tile granularity, classes 0 and 1.
  *
  * Check tiles are numbered row-major over the matrix,
  * t = (i / cm) * ceil(N / cn) + (j / cn); `status` holds

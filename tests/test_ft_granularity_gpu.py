@@ -157,6 +157,23 @@ def test_verification_cadence_corrects_one_fault_per_interval(blas, oracle_mod, 
     assert np.array_equal(c_cad[:, :N], plain.cpu().numpy()[:, :N])
 
 
+@pytest.mark.parametrize("mode", ["fused", "workspace"])
+def test_verification_cadence_on_the_128x128_class(blas, oracle_mod, mode):
+    """The same on 128 x 128 tiles (tile numbers, rows and columns of the faults are those of that class)."""
+    M, N, K = 300, 260, 900      # 3 x 3 tiles, 4 verifications (k = 256, 512, 768, 900)
+    tau = blas.ft_default_tau(K)
+    a, b, c0 = _problem(oracle_mod, M, N, K, 1350)
+    ws = _ws(blas, M, N, K) if mode == "workspace" else None
+    for faults in ([], [(4, 100, 30, 0.75, 1), (4, 7, 2, -12.0, 3)], [(8, 43, 3, 2.0, 0), (0, 127, 127, -0.5, 2), (0, 1, 1, 1.0, 2)]):
+        c, st = _device_run(blas, a, b, c0, M, N, K, 1.5, -1.0, tau, ws, tile_class=1, check_interval=256, faults=faults)
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm_checked(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, 128, 128, tau, 256, faults)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (faults, f, st[f], st_model[f])
+        if not np.any(st["flag"] == 2):
+            _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.5, -1.0)
+
+
 def test_cadence_with_data_scaled_threshold_and_interval_edge_cases(blas, oracle_mod):
     M, N, K = 300, 200, 700
     a, b, c0 = _problem(oracle_mod, M, N, K, 1400)
@@ -179,8 +196,8 @@ def test_option_errors(blas):
     ws = torch.zeros(1 << 20, device="cuda")
     with pytest.raises(blas.HpcdnnError):   # wave-tile checksums come from the workspace
         blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, granularity=blas.FT_GRAN_WAVE)
-    with pytest.raises(blas.HpcdnnError):   # the cadence kernels exist for the 256 x 128 class
-        blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, tile_class=1, check_interval=64, ws=ws)
+    with pytest.raises(blas.HpcdnnError):   # the cadence kernels exist for the 256 x 128 and 128 x 128 classes
+        blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, tile_class=2, check_interval=64, ws=ws)
     with pytest.raises(blas.HpcdnnError):   # a multiple of the K step
         blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, check_interval=100, ws=ws)
     with pytest.raises(blas.HpcdnnError):   # wave tile 128 x 32: column 32 does not exist
