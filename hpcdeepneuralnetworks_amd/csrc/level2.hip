@@ -320,7 +320,10 @@ static int run_sgemv(int trans, int M, int N, float alpha, const float* A, int l
         const dim3 grid(static_cast<unsigned>(ceil_div(N, kGemvColsPerBlock)), chunks);
         sgemv_t_kernel<8><<<grid, kGemvThreads, 0, s>>>(M, N, rows_per_chunk, alpha, A, lda, x, beta, y, partial);
     }
-    if (chunks > 1)
+    if (chunks > 8 && N % 4 == 0 && (reinterpret_cast<uintptr_t>(partial) & 15u) == 0)
+        // many chunks: the reduction that keeps all of a lane's slices in flight (y as a 1 x N matrix)
+        splitk_reduce_wide_kernel<><<<static_cast<int>(ceil_div(N, 256)), 256, 0, s>>>(1, N, chunks, partial, y, N, alpha, beta);
+    else if (chunks > 1)
         sgemv_t_finish_kernel<<<static_cast<int>(ceil_div(N, kGemvThreads)), kGemvThreads, 0, s>>>(N, chunks, alpha, partial,
                                                                                                   beta, y);
     return launch_status();

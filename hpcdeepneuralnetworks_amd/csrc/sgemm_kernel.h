@@ -1137,49 +1137,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
     }
 }
 
-// The same for many slices (N a multiple of 4, 16-byte aligned partials): four lanes share a group of four
-// consecutive elements, each adds a quarter of the slices in slice order (up to sixteen 16-byte loads in flight, so
-// 64 slices cost one trip to memory where the kernel above makes eight), and the four partial sums are combined as
-// (q0 + q1) + (q2 + q3) by exchanges with lane ^ 16 and lane ^ 32: a fixed order, the same bits on every run.
-// A wave covers 16 groups (256 contiguous bytes per slice) x 4 quarters.
-template <int kUnused = 0>
-__global__ __launch_bounds__(256) void splitk_reduce_wide_kernel(int M, int N, int splits, const float* __restrict__ ws,
-                                                                 float* __restrict__ C, int ldc, float alpha, float beta) {
-    const int64_t total = static_cast<int64_t>(M) * N;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int q = lane >> 4;
-    const int64_t e = (static_cast<int64_t>(blockIdx.x) * 64 + (threadIdx.x / kWave) * 16 + (lane & 15)) * 4;
-    const int per = (splits + 3) / 4;
-    const int z0 = q * per, z1 = (z0 + per < splits) ? z0 + per : splits;
-    v4f s = {0.f, 0.f, 0.f, 0.f};
-    if (e < total) {
-        constexpr int kBatch = 16;
-        for (int z = z0; z < z1; z += kBatch) {
-            v4f t[kBatch];
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u)
-                t[u] = (z + u < z1) ? *reinterpret_cast<const v4f*>(ws + static_cast<size_t>(z + u) * total + e) : v4f{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) s += t[u];
-        }
-    }
-    float sv[4] = {s.x, s.y, s.z, s.w};
-    const int x32_addr = (lane ^ 32) * 4;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        sv[c] += lane_xor<16>(sv[c]);
-        sv[c] += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(x32_addr, __builtin_bit_cast(int, sv[c])));
-    }
-    if (q == 0 && e < total) {
-        const int64_t r = e / N, c0 = e - r * N;
-        float* dst = C + r * ldc + c0;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const float t = alpha * sv[c];
-            dst[c] = (beta == 0.f) ? t : __builtin_fmaf(beta, dst[c], t);
-        }
-    }
-}
+// (splitk_reduce_wide_kernel, the variant for many slices, lives in common.h: the transposed SGEMV shares it)
 
 // Fixed-order second phase of the tail split: for the tiles after the first full_tiles, C = alpha * (slice 0 +
 // slice 1 + ...) + beta*C.  grid = (tail tiles, bm / 32): one block adds 32 rows of one tile, 4 columns per thread.
