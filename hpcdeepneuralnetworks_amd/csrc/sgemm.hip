@@ -1,6 +1,7 @@
 // SGEMM / ABFT-SGEMM entry points: argument checks, tile + split-K choice, launch.
 #include "gemm_host.h"
 #include "sgemm_small_kernel.h"
+#include "sgemm_persistent_kernel.h"
 
 namespace hpcdnn {
 
@@ -14,25 +15,34 @@ struct TileConfig {
     float eff;  // fitted steady-state fraction of the FP32 MFMA peak of one CU
     bool wave_split_k;  // small-problem kernel: the waves of a workgroup split K (other summation order, no tail split)
     int nslot;          // K steps a workgroup keeps on their way from memory (0: not modelled)
+    // persistent variants for several rounds of whole tiles (beta == 0, beta != 0), or nullptr
+    void (*persistent)(const GemmArgs);
+    void (*persistent_beta)(const GemmArgs);
 };
 
-#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, EFF)                                                          \
+#define HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, PERSISTENT, PERSISTENT_BETA)                                                        \
     {                                                                                                    \
         BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
-            sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC>, EFF, false, 2 \
+            sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC>, EFF, false, 2, \
+            PERSISTENT, PERSISTENT_BETA                                                                          \
     }
+
+#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, EFF) HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, nullptr, nullptr)
+#define HPCDNN_TILE_PERSISTENT(BM, BN, WGM, WGN, OCC, EFF) \
+    HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false>),       \
+                 (sgemm_persistent_kernel<BM, BN, WGM, WGN, true>))
 
 #define HPCDNN_TILE_DEEP(BM, BN, WGM, WGN, OCC, EFF, NSLOT)                                               \
     {                                                                                                    \
         BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
             sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC, NSLOT>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC, NSLOT>, EFF, \
-            false, NSLOT                                                                                 \
+            false, NSLOT, nullptr, nullptr                                                               \
     }
 
 #define HPCDNN_SMALL_TILE(TMB, OCC, EFF)                                                                  \
     {                                                                                                    \
         32 * TMB, 32, kSmallBK, kSmallThreads, OCC, small_lds_bytes<TMB>(), sgemm_small_kernel<TMB, false, OCC>, \
-            sgemm_small_kernel<TMB, true, OCC>, EFF, true, 0                                             \
+            sgemm_small_kernel<TMB, true, OCC>, EFF, true, 0, nullptr, nullptr                           \
     }
 
 // The counterpart of the reference's small/medium/large/tall/wide/huge shape table
@@ -40,14 +50,14 @@ struct TileConfig {
 // workgroup.  EFF comes from a least-squares fit of plan_cost() below to measured times of every tile over
 // squares 256..6144 with K = n, 1024 and 256 and a set of skinny shapes on an MI355X.
 static const TileConfig kTiles[] = {
-    HPCDNN_TILE(256, 128, 2, 2, 2, 0.978f),  // 0 huge (the ABFT tile)
+    HPCDNN_TILE_PERSISTENT(256, 128, 2, 2, 2, 0.978f),  // 0 huge (the ABFT tile)
     HPCDNN_TILE(128, 128, 2, 2, 2, 0.970f),  // 1 large
     HPCDNN_TILE(128, 64, 2, 2, 2, 0.945f),   // 2 tall
     HPCDNN_TILE(64, 128, 2, 2, 2, 0.939f),   // 3 wide
     HPCDNN_TILE(64, 64, 2, 2, 4, 0.900f),    // 4 medium
     HPCDNN_TILE(192, 256, 2, 2, 1, 0.964f),  // 5 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
     HPCDNN_TILE(256, 192, 2, 2, 1, 0.946f),  // 6
-    HPCDNN_TILE(128, 256, 2, 2, 2, 0.987f),  // 7
+    HPCDNN_TILE_PERSISTENT(128, 256, 2, 2, 2, 0.987f),  // 7
     HPCDNN_TILE(256, 256, 2, 4, 1, 1.000f),  // 8 giant, eight waves
     HPCDNN_TILE(256, 128, 4, 2, 1, 1.000f),  // 9 huge, eight waves
     HPCDNN_TILE(256, 256, 4, 2, 1, 1.000f),  // 10 giant, eight waves (4 x 2)
@@ -85,11 +95,21 @@ constexpr double kStreamLatency = 0.73e-6;     // trip to HBM under load, fitted
 constexpr double kReduceFixed = 2.5e-6;        // second launch of split-K
 constexpr double kReduceBytesPerSec = 8e12;    // partials written once and read once, C written once
 
-static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int cus) {
+constexpr double kPersistGain = 0.975;         // persistent kernel against the tile-per-workgroup kernel of the same tile (measured 0.95 .. 0.99)
+
+// The persistent kernel takes unsplit problems of more than one round of whole tiles with an even number of K steps,
+// enough of them to spread a tile's stores over.
+static int persistent_grid(const TileConfig& t, int M, int N, int K, int cus) {
+    const int grid = cus / kXcds * kXcds;
+    if (!t.persistent || (M % t.bm) || (N % t.bn) || (K % (2 * t.bk)) || K / t.bk < kPersistDripSteps + 2) return 0;
+    return static_cast<int64_t>(M / t.bm) * (N / t.bn) > grid ? grid : 0;
+}
+
+static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int cus, bool count_persistent = true) {
     const double tiles = static_cast<double>(ceil_div(M, t.bm)) * ceil_div(N, t.bn) * split;
-    const double n = ceil(tiles / cus);
     const double k_slice = ceil(static_cast<double>(ceil_div(K, split)) / t.bk) * t.bk;
     const bool edge = (M % t.bm) || (N % t.bn) || (K % t.bk);
+    const double n = ceil(tiles / cus);
     double eff = t.eff;
     const double resident = t.blocks_per_cu < n ? t.blocks_per_cu : n;
     // tiles whose waves own one or two 32x32 blocks (two staging sets): alone on a SIMD a wave cannot hide its waits
@@ -111,6 +131,7 @@ static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int
         if (stream > cost) cost = stream;
     }
     if (split > 1) cost += kReduceFixed + (2.0 * split + 1.0) * M * static_cast<double>(N) * 4.0 / kReduceBytesPerSec;
+    if (count_persistent && split == 1 && persistent_grid(t, M, N, K, cus) > 0) cost *= kPersistGain;
     return cost;
 }
 
@@ -228,7 +249,8 @@ static RowSplit choose_row_split(int M, int N, int K, int cus) {
             const int64_t tile_rows = k * cus / tiles_n;
             const int64_t rows1 = tile_rows * cfg.bm;
             if (tile_rows < 1 || rows1 >= M) continue;
-            const double c1 = plan_cost(cfg, static_cast<int>(rows1), N, K, 1, cus);
+            // (without the persistent kernel's gain: a second launch has to pay for itself on round counting alone)
+            const double c1 = plan_cost(cfg, static_cast<int>(rows1), N, K, 1, cus, false);
             double c2 = 0.0;
             const Plan rest = choose_plan(M - static_cast<int>(rows1), N, K, false, 0, false, &c2, true);
             const double c = c1 + c2 + kSecondLaunch;
@@ -327,10 +349,17 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     }
     const bool edge = needs_edge(a, cfg.bm, cfg.bn, cfg.bk);
     void (*fn)(const GemmArgs) = edge ? cfg.edge : cfg.plain;
+    dim3 grid(a.full_tiles + tail_tiles * a.tail_split, 1, split);
+    // Several rounds of whole tiles written straight to C: one persistent workgroup per CU walks its tiles as one
+    // stream of K steps (same bits; see sgemm_persistent_kernel.h for what it saves)
+    const int persistent = (split == 1 && tail_tiles == 0 && ldc <= kMaxLdc) ? persistent_grid(cfg, M, N, K, device_cus()) : 0;
+    if (persistent > 0) {
+        fn = beta == 0.f ? cfg.persistent : cfg.persistent_beta;
+        grid = dim3(persistent, 1, 1);
+    }
     rc = enable_lds(fn, cfg.lds_bytes);
     if (rc != HPCDNN_OK) return rc;
 
-    dim3 grid(a.full_tiles + tail_tiles * a.tail_split, 1, split);
     hipLaunchKernelGGL(fn, grid, dim3(cfg.threads), cfg.lds_bytes, stream, a);
     rc = launch_status();
     if (rc != HPCDNN_OK) return rc;
