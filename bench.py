@@ -47,7 +47,7 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline SGEMM line only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--ft-launches", type=int, default=1000, help="launches of the ABFT fault campaign")
-    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "sgemm_1024", "ft_sgemm", "ft_sgemm_fused", "ft_sgemm_wave", "offline_ft", "saxpy", "sdot", "copy",
+    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "sgemm_1024", "sgemm_lowk", "ft_sgemm", "ft_sgemm_fused", "ft_sgemm_wave", "offline_ft", "saxpy", "sdot", "copy",
                              "sgemv_n", "sgemv_t"],
                     help="run one kernel only for --steps launches (for profiling with rocprofv3) and print a short line")
     args = ap.parse_args()
@@ -97,6 +97,12 @@ def main() -> int:
             a, b, c = operands(m, m, m, 10)
             fn = lambda: blas.sgemm(m, m, m, a, b, c, 1.0, 0.0)
             work, unit = 2.0 * m ** 3, "GFLOP/s"
+        elif args.kernel == "sgemm_lowk":
+            # the low-K shape of the irregular set: 2048 tiles of 128x256, eight per persistent workgroup
+            mm, kk = 8192, 256
+            a, b, c = operands(mm, mm, kk, 10)
+            fn = lambda: blas.sgemm(mm, mm, kk, a, b, c, 1.0, 0.0)
+            work, unit = 2.0 * mm * mm * kk, "GFLOP/s"
         elif args.kernel == "ft_sgemm":
             m = 4096
             a, b, c = operands(m, m, m, 20)
