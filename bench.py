@@ -78,7 +78,13 @@ def main() -> int:
         return e0.elapsed_time(e1) / steps
 
     def median_timed(fn, steps, warmup, batches=5):
-        return statistics.median(timed(fn, steps, warmup if b == 0 else 1) for b in range(batches))
+        """Median over batches.  Short kernels get more calls: the clock sags within milliseconds of idling (allocating
+        and filling the next operands is enough), so every measurement is preceded by at least 25 ms of the same
+        call and each batch covers at least 8 ms."""
+        per_call = max(timed(fn, 3, warmup), 1e-3)
+        steps = min(max(steps, int(8.0 / per_call) + 1), 4000)
+        lead = min(max(warmup, int(25.0 / per_call) + 1), 8000)
+        return statistics.median(timed(fn, steps, lead if b == 0 else 1) for b in range(batches))
 
     def operands(M, N, K, seed):
         a = torch.empty(M, K, device=dev)
