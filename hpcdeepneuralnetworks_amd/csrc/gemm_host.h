@@ -9,7 +9,7 @@ namespace hpcdnn {
 
 constexpr int kMaxLda = (1 << 21) - 64;    // 256 * lda * 4 < 2^31
 constexpr int kMaxLdb = (1 << 25) - 1024;  // 16 * ldb * 4 + row < 2^31
-constexpr int kMaxLdc = (1 << 21) - 64;    // persistent kernel only: 256 * ldc * 4 + row < 2^31
+constexpr int kMaxLdc = (1 << 21) - 64;    // 256 * ldc * 4 + row < 2^31
 
 inline int check_gemm_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
     if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
@@ -18,8 +18,8 @@ inline int check_gemm_args(int M, int N, int K, const float* A, int lda, const f
     if (M > 0 && N > 0 && K > 0 && (!A || !B)) return HPCDNN_ERR_INVALID_VALUE;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) & 3u)
         return HPCDNN_ERR_INVALID_VALUE;
-    // byte offsets inside one tile are 32-bit: 256 rows of A, 16 rows of B
-    if (lda > kMaxLda || ldb > kMaxLdb) return HPCDNN_ERR_INVALID_VALUE;
+    // byte offsets inside one tile are 32-bit: 256 rows of A and of C, 16 rows of B
+    if (lda > kMaxLda || ldb > kMaxLdb || ldc > kMaxLdc) return HPCDNN_ERR_INVALID_VALUE;
     return HPCDNN_OK;
 }
 

@@ -1090,6 +1090,40 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // the 256x128 tiles measured 0.2 % slower with it and keep the plain store).
     constexpr bool kStreamC = BM * BN <= 128 * 128;
     const float alpha = p.alpha, beta = p.beta;
+    if constexpr (EDGE) {
+        // Ragged tiles: a buffer descriptor from the tile's corner to the last element of C inside the tile, so the
+        // hardware drops stores to rows >= M (and returns 0 for loads there); the row offset has to be part of the
+        // vector offset for that (a scalar offset is not range-checked).  Columns >= N would land in the next row:
+        // they are switched off once per block column.  A compare, a branch and a 64-bit multiply per store, which
+        // is what the pointer form compiles to, cost a 64x64 tile 3200 cycles here.
+        const int64_t c_bytes = (static_cast<int64_t>(p.M - 1 - m0) * p.ldc + (p.N - n0)) * 4;
+        const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.C + static_cast<int64_t>(m0) * p.ldc + n0, c_bytes);
+        const int ldc_bytes = p.ldc * 4;  // BM * ldc * 4 < 2^31 (host check)
+        const int lane_off = (wm * WM + lh * 4) * ldc_bytes + (wn * WN + lr) * 4;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if (col_base + j * 32 >= p.N) continue;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                float old[16];
+                if (beta != 0.f) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        old[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                     c_rsrc, lane_off + j * 128 + (i * 32 + 8 * (v / 4) + (v % 4)) * ldc_bytes, 0, 0));
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const float t = alpha * acc[i][j][v];
+                    const float out = (beta == 0.f) ? t : __builtin_fmaf(beta, old[v], t);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), c_rsrc,
+                                                          lane_off + j * 128 + (i * 32 + 8 * (v / 4) + (v % 4)) * ldc_bytes, 0,
+                                                          kStreamC ? 2 : 0);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1101,19 +1135,16 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int r = 8 * (v / 4) + (v % 4);
-                    const bool ok = !EDGE || (row_base + i * 32 + r < p.M && col < p.N);
-                    old[v] = ok ? cbase[static_cast<size_t>(r) * p.ldc] : 0.f;
+                    old[v] = cbase[static_cast<size_t>(r) * p.ldc];
                 }
             }
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int r = 8 * (v / 4) + (v % 4);
-                if (!EDGE || (row_base + i * 32 + r < p.M && col < p.N)) {
-                    const float t = alpha * acc[i][j][v];
-                    const float out = (beta == 0.f) ? t : __builtin_fmaf(beta, old[v], t);
-                    if constexpr (kStreamC) __builtin_nontemporal_store(out, &cbase[static_cast<size_t>(r) * p.ldc]);
-                    else cbase[static_cast<size_t>(r) * p.ldc] = out;
-                }
+                const float t = alpha * acc[i][j][v];
+                const float out = (beta == 0.f) ? t : __builtin_fmaf(beta, old[v], t);
+                if constexpr (kStreamC) __builtin_nontemporal_store(out, &cbase[static_cast<size_t>(r) * p.ldc]);
+                else cbase[static_cast<size_t>(r) * p.ldc] = out;
             }
         }
 }

@@ -81,7 +81,7 @@ const char* hpcdnn_version(void);
 const char* hpcdnn_error_string(int code);
 
 /* C = alpha*A*B + beta*C, A is MxK, B is KxN, C is MxN, any M,N,K >= 0 and any
- * lda >= K, ldb >= N, ldc >= N with lda <= 2^21 - 64 and ldb <= 2^25 - 1024 (byte
+ * lda >= K, ldb >= N, ldc >= N with lda, ldc <= 2^21 - 64 and ldb <= 2^25 - 1024 (byte
  * offsets inside one tile are 32-bit; larger values return
  * HPCDNN_ERR_INVALID_VALUE).  A, B and C are 4-byte aligned.  C is not read
  * when beta == 0.

@@ -82,6 +82,7 @@ def test_bad_arguments_are_rejected_without_a_gpu(L):
     # leading dimensions beyond the 32-bit tile offsets
     assert L.hpcdnn_sgemm(4, 4, 4, dummy, (1 << 21) - 63, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
     assert L.hpcdnn_sgemm(4, 4, 4, dummy, 4, dummy, (1 << 25) - 1023, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
+    assert L.hpcdnn_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, (1 << 21) - 63, 1.0, 0.0, None, 0, None) == INVALID
     from hpcdeepneuralnetworks_amd._lib import Fault
 
     bad = Fault(5, 0, 0, 1.0)  # only one tile exists

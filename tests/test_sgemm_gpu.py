@@ -444,9 +444,9 @@ def test_host_threads_on_their_own_streams(blas, oracle_mod):
 
 
 def test_maximum_leading_dimensions(blas):
-    """lda and ldb at the documented limits (32-bit byte offsets inside one tile), for every kernel family; one more
-    is refused."""
-    lda, ldb = (1 << 21) - 64, (1 << 25) - 1024
+    """lda, ldb and ldc at the documented limits (32-bit byte offsets inside one tile), for every kernel family; one
+    more is refused."""
+    lda, ldb, ldc = (1 << 21) - 64, (1 << 25) - 1024, (1 << 21) - 64
     M, N, K = 300, 100, 40
     abuf = torch.empty(M * lda, device="cuda")
     bbuf = torch.empty(K * ldb + 8, device="cuda")
@@ -457,10 +457,16 @@ def test_maximum_leading_dimensions(blas):
     ref = a.double() @ b.double()
     den = a.abs().double() @ b.abs().double()
     small = [t for t, shape in enumerate(blas.tile_table()) if shape[:2] == (32, 32)][0]
+    cbuf = torch.empty(M * ldc, device="cuda")
+    c = cbuf.view(M, ldc)[:, :N]
+    c0 = torch.rand(M, N, device="cuda", generator=gen) * 2 - 1
     for tile in (-1, 0, 4, 8, small, len(blas.tile_table()) - 1):
-        c = torch.zeros(M, N, device="cuda")
-        blas.sgemm(M, N, K, a, b, c, 1.0, 0.0, tile=tile, split_k=0 if tile < 0 else 1)
-        assert float(((c.double() - ref).abs() / den).max()) <= TOL, tile
+        for beta in (0.0, -1.5):
+            c.copy_(c0)
+            blas.sgemm(M, N, K, a, b, c, 1.0, beta, tile=tile, split_k=0 if tile < 0 else 1)
+            assert float(((c.double() - ref - beta * c0.double()).abs() / (den + abs(beta) * c0.abs().double())).max()) <= TOL, (tile, beta)
+    with pytest.raises(blas.HpcdnnError):
+        blas.sgemm(8, N, K, a, b, cbuf[:7 * (ldc + 1) + N].as_strided((8, N), (ldc + 1, 1)), 1.0, 0.0)
     with pytest.raises(blas.HpcdnnError):
         blas.sgemm(M, N, K, a, bbuf[:(K - 1) * (ldb + 1) + N].as_strided((K, N), (ldb + 1, 1)), torch.zeros(M, N, device="cuda"), 1.0, 0.0)
     with pytest.raises(blas.HpcdnnError):
