@@ -178,6 +178,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr bool kShortStep = FT == 0 && NMG <= 8;  // one or two 32x32 blocks per wave: little to hide latencies behind
     constexpr bool kNoBounds = kShortStep && !EDGE;
     constexpr bool kEarlyStore = kShortStep && NSLOT > 2;
+    // Plain SGEMM on ragged tiles: the loads of every K step but the slice's last touch nothing outside the
+    // matrices once rows m >= M are folded onto row M - 1 (what they read only reaches accumulators that are never
+    // stored), so those steps run with unbounded descriptors and plain pointer steps; the byte counts that the range
+    // checks need are formed only for the steps at the end of the slice.
+    constexpr bool kLazyBounds = EDGE && FT == 0;
 
     extern __shared__ __align__(16) float smem[];
     float* const As = smem;
@@ -202,6 +207,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     }
     tile_of_block(tile_id, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+    // (a tile that hangs over the last column reads B past the ends of its rows: into the next row, which must exist
+    // and be long enough for that to stay inside the matrix)
+    const bool lazy_ok = n0 + BN <= p.N || p.ldb >= BN;
     // the K range of one pass of the pipeline: the slice, or one verification interval of it
     int kbeg = k_slice * k_chunk;
     int kend = (p.K - kbeg < k_chunk) ? p.K : kbeg + k_chunk;
@@ -221,8 +229,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
     for (int s = 0; s < A_SLOTS; ++s) {
         const int idx = tid + s * kGemmThreads;
-        const int row = idx / A_V4_PER_ROW;
+        int row = idx / A_V4_PER_ROW;
         a_kc[s] = (idx % A_V4_PER_ROW) * 4;
+        if constexpr (kLazyBounds) row = row < p.M - m0 ? row : p.M - 1 - m0;
         a_voff[s] = (row * p.lda + a_kc[s]) * 4;
         a_lds[s] = row * AS + a_kc[s];
     }
@@ -262,10 +271,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     int enc_off = kbeg * 4;
     float g_ac[2][GM][B_SLOTS];
     v4f g_br[2][GN];
-    auto gload1 = [&](auto slot, auto part) {
+    auto gload1 = [&](auto slot, auto part, auto bulk) {  // bulk: this K step is not the slice's last (kLazyBounds)
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P == 0) k_slot[S] = k_loaded;
-        if constexpr (kNoBounds) {
+        if constexpr (kNoBounds || (kLazyBounds && decltype(bulk)::value)) {
             if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc_unbounded(a_base), a_voff[P]);
             else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc_unbounded(b_base), b_voff[P - A_SLOTS]);
         } else {
@@ -320,6 +329,16 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // After the last part of a K step: move to the next one, unless that would leave the slice; then the
     // descriptors are emptied, so the fetches that run ahead past the end all return 0 (never multiplied, and
     // neutral for the checksums).
+    auto gload_advance_bulk = [&]() {  // kLazyBounds, a step that is not the slice's last: no end to look out for
+        a_base += BK;
+        b_base += b_step;
+        k_loaded += BK;
+    };
+    // kLazyBounds, at the end of the bulk steps: the byte counts from the current bases to the ends of A and B
+    auto bounds_from_position = [&]() {
+        a_left = (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - k_loaded)) * 4;
+        b_left = (static_cast<int64_t>(p.K - 1 - k_loaded) * p.ldb + (p.N - n0)) * 4;
+    };
     auto gload_advance = [&]() {
         const bool more = k_loaded + BK < kend;
         a_base += more ? BK : 0;
@@ -332,6 +351,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // The same in two parts, so that the short-step schedule can place them apart.  Its full tiles keep no bounds at
     // all: nothing they fetch lies outside the matrix, and past the end of the slice they fetch its last K step
     // again instead of zeros.
+    auto gload_advance_a_bulk = [&]() { a_base += BK; };
+    auto gload_advance_b_bulk = [&]() {
+        b_base += b_step;
+        k_loaded += BK;
+    };
     auto gload_advance_a = [&]() {
         const bool more = k_loaded + BK < kend;
         a_base += more ? BK : 0;
@@ -632,8 +656,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     //                (+ consume the checksum partials of step kt+1)
     // Work past the end of the slice (kt+1, kt+2 >= nkt) moves duplicate data that is never multiplied, which
     // keeps the loop free of branches (and lets the loads stay two steps ahead).
-    auto step_in = [&](auto sl_next, auto sl_free, auto stage, auto flush, auto masked) {
+    auto step_in = [&](auto sl_next, auto sl_free, auto stage, auto flush, auto masked, auto bulk) {
         constexpr int st = decltype(stage)::value;
+        constexpr bool kBulk = kLazyBounds && decltype(bulk)::value;
         constexpr int NMASK = (EDGE && decltype(masked)::value) ? (FT ? NGL : A_SLOTS) : 0;
         constexpr int NS0 = NRD + NMASK + NPROD + 2 * NGL;
         constexpr int NS1 = NRD + NCONS;
@@ -658,7 +683,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     if constexpr (o < NRD) fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
                     else if constexpr (o < NRD + NMASK) gmask1(sl_next, std::integral_constant<int, o - NRD>{});
                     else if constexpr (o < NRD + NMASK + NGL) lstore1(sl_next, std::integral_constant<int, o - NRD - NMASK>{}, st ^ 1);
-                    else gload1(sl_free, std::integral_constant<int, o - NRD - NMASK - NGL>{});
+                    else gload1(sl_free, std::integral_constant<int, o - NRD - NMASK - NGL>{}, bulk);
                 } else if constexpr (o < NRD) {
                     fread1(S1{}, std::integral_constant<int, o>{}, st, 1);
                 } else if constexpr (o < NRD + NMASK) {
@@ -666,8 +691,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 } else if constexpr (o < NRD + NMASK + NPROD) {
                     produce1(sl_next, std::integral_constant<int, o - NRD - NMASK>{}, st ^ 1);
                 } else if constexpr (o < NRD + NMASK + NPROD + NGL) {
-                    gload1(sl_free, std::integral_constant<int, o - NRD - NMASK - NPROD>{});
-                    if constexpr (o == NRD + NMASK + NPROD + NGL - 1 && !kShortStep) gload_advance();
+                    gload1(sl_free, std::integral_constant<int, o - NRD - NMASK - NPROD>{}, bulk);
+                    if constexpr (o == NRD + NMASK + NPROD + NGL - 1 && !kShortStep) {
+                        if constexpr (kBulk) gload_advance_bulk();
+                        else gload_advance();
+                    }
                 } else {
                     lstore1(sl_next, std::integral_constant<int, o - NRD - NMASK - NPROD - NGL>{}, st ^ 1);
                 }
@@ -681,8 +709,14 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             mfma1(S1{}, m);
             if constexpr (kShortStep) {
                 if constexpr (Mi == 0) static_for<NRD>([&](auto o) { fread1(S0{}, o, st ^ 1, 0); });
-                if constexpr (Mi == 1) gload_advance_a();
-                if constexpr (Mi == 2) gload_advance_b();
+                if constexpr (Mi == 1) {
+                    if constexpr (kBulk) gload_advance_a_bulk();
+                    else gload_advance_a();
+                }
+                if constexpr (Mi == 2) {
+                    if constexpr (kBulk) gload_advance_b_bulk();
+                    else gload_advance_b();
+                }
             } else {
                 constexpr int k_lo = (Mi * NS1 + NMG - 1) / NMG, k_hi = ((Mi + 1) * NS1 + NMG - 1) / NMG;
                 static_for<k_hi - k_lo>([&](auto d) {
@@ -697,29 +731,29 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     };
 
     // with two staging sets steps alternate between (next = slot 1, LDS stage 0) and (next = slot 0, LDS stage 1)
-    auto step = [&](auto sl_next, auto sl_free, auto flush, auto masked) {
-        step_in(sl_next, sl_free, std::integral_constant<int, (decltype(sl_next)::value == 1) ? 0 : 1>{}, flush, masked);
+    auto step = [&](auto sl_next, auto sl_free, auto flush, auto masked, auto bulk) {
+        step_in(sl_next, sl_free, std::integral_constant<int, (decltype(sl_next)::value == 1) ? 0 : 1>{}, flush, masked, bulk);
     };
     // step number kt with kt % NSLOT == phase: its successor waits in slot (phase + 1) % NSLOT, slot phase is free
-    auto step_at = [&](auto phase, auto masked) {
+    auto step_at = [&](auto phase, auto masked, auto bulk) {
         constexpr int Ph = decltype(phase)::value;
         step_in(std::integral_constant<int, (Ph + 1) % NSLOT>{}, std::integral_constant<int, Ph % NSLOT>{},
-                std::integral_constant<int, Ph % 2>{}, std::false_type{}, masked);
+                std::integral_constant<int, Ph % 2>{}, std::false_type{}, masked, bulk);
     };
 
     // One pass of the software pipeline over [kbeg, kend).
     auto run_k_range = [&]() {
     if (nkt > 0) {
         // prologue: step 0 -> LDS stage 0, step 1 -> staging slot 1, first-half fragments of step 0 -> buffer 0
-        static_for<NGL>([&](auto s) { gload1(S0{}, s); });
+        static_for<NGL>([&](auto s) { gload1(S0{}, s, std::false_type{}); });
         gload_advance();
         if constexpr (EDGE) static_for<NGL>([&](auto s) { gmask1(S0{}, s); });
         static_for<NGL>([&](auto s) { lstore1(S0{}, s, 0); });
         static_for<NPROD>([&](auto e) { produce1(S0{}, e, 0); });
-        static_for<NGL>([&](auto s) { gload1(S1{}, s); });
+        static_for<NGL>([&](auto s) { gload1(S1{}, s, std::false_type{}); });
         gload_advance();
         static_for<NSLOT - 2>([&](auto extra) {  // steps 2 .. NSLOT-1 -> their slots
-            static_for<NGL>([&](auto s) { gload1(std::integral_constant<int, decltype(extra)::value + 2>{}, s); });
+            static_for<NGL>([&](auto s) { gload1(std::integral_constant<int, decltype(extra)::value + 2>{}, s, std::false_type{}); });
             gload_advance();
         });
         __syncthreads();
@@ -730,28 +764,40 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             // whole groups of NSLOT steps; on a ragged tile only the slice's last K step can be partial, and it is
             // step nkt - 2 that moves it to LDS, so the steps before that one run without the masks
             const int bulk_end = EDGE ? nkt - 2 : nkt;
+            if constexpr (kLazyBounds) {
+                // groups whose loads (NSLOT steps ahead) all stay before the slice's last K step
+                for (; lazy_ok && kt + 2 * NSLOT + 1 <= nkt; kt += NSLOT)
+                    static_for<NSLOT>([&](auto ph) { step_at(ph, std::false_type{}, std::true_type{}); });
+                if (kt > 0) bounds_from_position();
+            }
             for (; kt + NSLOT <= bulk_end; kt += NSLOT)
-                static_for<NSLOT>([&](auto ph) { step_at(ph, std::false_type{}); });
+                static_for<NSLOT>([&](auto ph) { step_at(ph, std::false_type{}, std::false_type{}); });
             // what is left (fewer than a group, plus the two last steps of a ragged tile), one step at a time
             static_for<NSLOT + (EDGE ? 1 : -1)>([&](auto i) {
-                if (kt + decltype(i)::value < nkt) step_at(std::integral_constant<int, decltype(i)::value % NSLOT>{}, std::true_type{});
+                if (kt + decltype(i)::value < nkt) step_at(std::integral_constant<int, decltype(i)::value % NSLOT>{}, std::true_type{}, std::false_type{});
             });
         } else {
             if constexpr (EDGE && FT == 0) {
                 // plain SGEMM on a ragged tile: only the last K step can be partial, and step kt consumes the staged
                 // data of step kt+1, so every step before kt = nkt-2 runs without the masks
+                // pairs whose loads (two steps ahead) both stay before the slice's last K step
+                for (; lazy_ok && kt + 4 < nkt; kt += 2) {
+                    step(S1{}, S0{}, std::false_type{}, std::false_type{}, std::true_type{});
+                    step(S0{}, S1{}, std::false_type{}, std::false_type{}, std::true_type{});
+                }
+                if (kt > 0) bounds_from_position();
                 for (; kt + 3 < nkt; kt += 2) {
-                    step(S1{}, S0{}, std::false_type{}, std::false_type{});
-                    step(S0{}, S1{}, std::false_type{}, std::false_type{});
+                    step(S1{}, S0{}, std::false_type{}, std::false_type{}, std::false_type{});
+                    step(S0{}, S1{}, std::false_type{}, std::false_type{}, std::false_type{});
                 }
             }
             for (; kt + 1 < nkt; kt += 2) {
-                step(S1{}, S0{}, std::false_type{}, std::true_type{});
+                step(S1{}, S0{}, std::false_type{}, std::true_type{}, std::false_type{});
                 flush_now = ((kt & 14) == 14) || (kt + 2 >= nkt);
-                step(S0{}, S1{}, std::true_type{}, std::true_type{});
+                step(S0{}, S1{}, std::true_type{}, std::true_type{}, std::false_type{});
             }
             flush_now = true;
-            if (kt < nkt) step(S1{}, S0{}, std::true_type{}, std::true_type{});
+            if (kt < nkt) step(S1{}, S0{}, std::true_type{}, std::true_type{}, std::false_type{});
         }
         __syncthreads();  // every wave is done with the staging buffers (the verification below reuses them)
     }
