@@ -247,7 +247,7 @@ def main() -> int:
 
         # irregular / skinny shapes (split-K with a caller-provided workspace where the library chooses it)
         irregular = {}
-        for (M, N, K) in ((8192, 8192, 256), (16384, 64, 4096), (128, 128, 65536), (6000, 6000, 6000), (3001, 3001, 3001)):
+        for (M, N, K) in ((8192, 8192, 256), (16384, 64, 4096), (128, 128, 65536), (6000, 6000, 6000), (3001, 3001, 3001), (1000, 1000, 1000)):
             a, b, c = operands(M, N, K, 15)
             ws = blas.workspace(max(blas.sgemm_workspace_bytes(M, N, K), 4))
             ms = median_timed(lambda: blas.sgemm(M, N, K, a, b, c, 1.0, 0.0, ws=ws), st, wu)

@@ -1116,6 +1116,26 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     }
     if (p.partial) {
         float* out = p.partial + static_cast<size_t>(blockIdx.z) * p.M * p.N;
+        if constexpr (EDGE) {
+            // (ragged tiles: through a descriptor that ends with the slice's last element of this tile, as for C below)
+            const __amdgpu_buffer_rsrc_t o_rsrc = make_rsrc(out + static_cast<int64_t>(m0) * p.N + n0,
+                                                            (static_cast<int64_t>(p.M - 1 - m0) * p.N + (p.N - n0)) * 4);
+            const int ld_bytes = p.N * 4;
+            const int lane_off = (wm * WM + lh * 4) * ld_bytes + (wn * WN + lr) * 4;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if (col_base + j * 32 >= p.N) continue;
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const float value = acc[i][j][v];
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), o_rsrc,
+                                                              lane_off + j * 128 + (i * 32 + 8 * (v / 4) + (v % 4)) * ld_bytes, 0, 0);
+                    }
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1124,7 +1144,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 for (int v = 0; v < 16; ++v) {
                     const int row = row_base + i * 32 + 8 * (v / 4) + (v % 4);
                     const int col = col_base + j * 32;
-                    if (!EDGE || (row < p.M && col < p.N)) out[static_cast<size_t>(row) * p.N + col] = acc[i][j][v];
+                    out[static_cast<size_t>(row) * p.N + col] = acc[i][j][v];
                 }
         return;
     }
