@@ -791,6 +791,18 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     step(S0{}, S1{}, std::false_type{}, std::false_type{}, std::false_type{});
                 }
             }
+            if constexpr (EDGE && FT != 0) {
+                // ABFT on a ragged problem: a tile that does not hang over the last column needs the masks only where
+                // plain SGEMM does, in the slice's last two K steps (its checksums want zeros in columns k >= kend of
+                // A and rows k >= kend of B; the columns n >= N that the other steps would have to clear do not exist)
+                if (n0 + BN <= p.N) {
+                    for (; kt + 3 < nkt; kt += 2) {
+                        step(S1{}, S0{}, std::false_type{}, std::false_type{}, std::false_type{});
+                        flush_now = (kt & 14) == 14;
+                        step(S0{}, S1{}, std::true_type{}, std::false_type{}, std::false_type{});
+                    }
+                }
+            }
             for (; kt + 1 < nkt; kt += 2) {
                 step(S1{}, S0{}, std::false_type{}, std::true_type{}, std::false_type{});
                 flush_now = ((kt & 14) == 14) || (kt + 2 >= nkt);
