@@ -95,7 +95,12 @@ constexpr double kStreamLatency = 0.73e-6;     // trip to HBM under load, fitted
 constexpr double kReduceFixed = 2.5e-6;        // second launch of split-K
 constexpr double kReduceBytesPerSec = 8e12;    // partials written once and read once, C written once
 
-constexpr double kPersistGain = 0.975;         // persistent kernel against the tile-per-workgroup kernel of the same tile (measured 0.95 .. 0.99)
+// Persistent kernel against the tile-per-workgroup kernel of the same tile.  What it saves is a fixed time per tile,
+// so the gain shrinks with K (measured 5 % at K = 256, 3 % at 512, 1-2.5 % at 1024, 0.5-1 % at 4096): that is the
+// estimate a split plan has to beat.  Among unsplit plans a flat 2.5 % ranks better (it also stands for the
+// eight-wave tiles' efficiency being fitted a little high): 4096 x 4096 x 1024 runs 2 % faster on the persistent
+// 128 x 256 tile than on the 256 x 256 tile that the K-dependent figure would pick.
+constexpr double kPersistGainK = 12.8, kPersistGainMax = 0.05, kPersistRankGain = 0.025;
 
 // The persistent kernel takes unsplit problems of more than one round of whole tiles with an even number of K steps,
 // enough of them to spread a tile's stores over.
@@ -131,34 +136,41 @@ static double plan_cost(const TileConfig& t, int M, int N, int K, int split, int
         if (stream > cost) cost = stream;
     }
     if (split > 1) cost += kReduceFixed + (2.0 * split + 1.0) * M * static_cast<double>(N) * 4.0 / kReduceBytesPerSec;
-    if (count_persistent && split == 1 && persistent_grid(t, M, N, K, cus) > 0) cost *= kPersistGain;
+    if (count_persistent && split == 1 && persistent_grid(t, M, N, K, cus) > 0) cost *= 1.0 - kPersistRankGain;
     return cost;
 }
 
 // Tail split: with T tiles on `cus` CUs the last T % cus tiles keep only some CUs busy for a whole tile time.
 // Splitting just those tiles s ways along K turns that round into ceil(r*s/cus) rounds of 1/s tile time each, at the
-// price of writing and re-reading r*s raw tiles.  Returns the cost, and the chosen s through *ways (0 = no gain).
+// price of writing and re-reading r*s raw tiles.  Returns the cost of the best s in 2..16 (slices of at least 8 K
+// steps, partials that fit the workspace), and that s through *ways (0 = nothing to split or nothing fits).
 static double tail_plan_cost(const TileConfig& t, int M, int N, int K, int cus, size_t ws_bytes, int* ways) {
     *ways = 0;
     const int64_t tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
     const int64_t r = tiles % cus, full = tiles - r;
-    if (full == 0 || r == 0 || 2 * r > cus) return 1e300;
-    int64_t s = cus / r;
-    const int64_t most = K / (8 * t.bk);  // at least 8 K steps per slice
-    if (s > most) s = most;
-    if (s > 16) s = 16;
-    const size_t tile_bytes = static_cast<size_t>(t.bm) * t.bn * sizeof(float);
-    while (s >= 2 && static_cast<size_t>(r * s) * tile_bytes > ws_bytes) --s;
-    if (s < 2) return 1e300;
+    if (full == 0 || r == 0) return 1e300;
+    // (more left-over tiles than half the CUs: only the tiles of 128 x 128 and up have slices long enough to pay;
+    // measured at 1280^3, where the model promised the 64 x 64 tile 9 % and the split ran 3 % slower)
+    if (2 * r > cus && t.bm * t.bn < 128 * 128) return 1e300;
     const bool edge = (M % t.bm) || (N % t.bn) || (K % t.bk);
     const double per_tile = 2.0 * t.bm * t.bn * K / (kPeakFlopsPerCu * t.eff) * (edge ? kEdgePenalty : 1.0);
     const double n_full = static_cast<double>(full / cus);
     const double fixed = kFixedBase + kFixedPer32K * t.bm * t.bn / 32768.0;
     const double n = n_full + 1.0;
     const double exposed = t.blocks_per_cu == 1 ? n : 1.0 + kCoveredFraction * (n - 1.0);
-    *ways = static_cast<int>(s);
-    return n_full * per_tile + ceil(static_cast<double>(r * s) / cus) * per_tile / s + exposed * fixed + kReduceFixed +
-           (2.0 * s + 1.0) * r * static_cast<double>(tile_bytes) / kReduceBytesPerSec;
+    const size_t tile_bytes = static_cast<size_t>(t.bm) * t.bn * sizeof(float);
+    const int64_t most = K / (8 * t.bk);
+    double best = 1e300;
+    for (int64_t s = 2; s <= 16 && s <= most; ++s) {
+        if (static_cast<size_t>(r * s) * tile_bytes > ws_bytes) break;
+        const double c = n_full * per_tile + ceil(static_cast<double>(r * s) / cus) * per_tile / s + exposed * fixed + kReduceFixed +
+                         (2.0 * s + 1.0) * r * static_cast<double>(tile_bytes) / kReduceBytesPerSec;
+        if (c < best) {
+            best = c;
+            *ways = static_cast<int>(s);
+        }
+    }
+    return best;
 }
 
 static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, bool allow_tail = true,
@@ -196,9 +208,18 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
     // A split has to promise more than the model's error on it (measured: predicted gains below 2-3 % turned out
     // as losses of about 1 %): if some unsplit plan is within 2.5 % of the best, only unsplit plans compete.
     double best_unsplit = 1e300;
+    int best_unsplit_tile = -1;
     for (int i = 0; i < n_cand; ++i)
-        if (cand[i].plan.split == 1 && cand[i].cost < best_unsplit) best_unsplit = cand[i].cost;
-    if (best_unsplit <= best_cost * 1.025) {
+        if (cand[i].plan.split == 1 && cand[i].cost < best_unsplit) {
+            best_unsplit = cand[i].cost;
+            best_unsplit_tile = cand[i].plan.tile;
+        }
+    double unsplit_to_beat = best_unsplit;
+    if (best_unsplit_tile >= 0 && persistent_grid(kTiles[best_unsplit_tile], M, N, K, cus) > 0) {
+        const double gain = kPersistGainK / K;
+        unsplit_to_beat *= (1.0 - (gain < kPersistGainMax ? gain : kPersistGainMax)) / (1.0 - kPersistRankGain);
+    }
+    if (unsplit_to_beat <= best_cost * 1.025 || best_unsplit <= best_cost) {
         best_cost = best_unsplit;
         int kept = 0;
         for (int i = 0; i < n_cand; ++i)
