@@ -18,7 +18,11 @@
 //            banks for that read.
 //   B stage: [16][BN + 8]   n contiguous, as in memory; lane (col c, half h)
 //            reads B[8g+4h+q][c] with ds_read_b32.  Stride BN+8 puts the two
-//            half-waves (rows 4 apart) on disjoint banks.
+//            half-waves (rows 4 apart) on disjoint banks.  128- and 192-column
+//            tiles use stride 264 (same banks): with rows less than 256 words
+//            apart the compiler pairs the reads into ds_read2_b32, whose 8-bit
+//            offsets cannot hold the stage and block offsets, and adds those to
+//            the address with vector-ALU instructions inside the K loop.
 // The MFMA k index is a permutation of the memory k index (lane half h of
 // k-step q in group g carries k = 8g+4h+q); A and B use the same permutation,
 // so the contraction is unchanged.
@@ -84,6 +88,12 @@ constexpr int kGemmBK = 16;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tiles share A and B panels
 
+// Row stride (floats) of the staged B tile.
+template <int BN>
+constexpr int b_stage_stride() {
+    return (BN == 128 || BN == 192) ? 264 : BN + 8;
+}
+
 // LDS the ABFT verification needs (it reuses the staging buffers once the K loop has drained): FP64 partials of the
 // reference checksums, observed line sums and their absolute counterparts per wave row / wave column, one residual
 // per line, one record per check tile, per-wave sums of |acc| per check tile.  GM x GN check tiles per workgroup tile.
@@ -100,7 +110,7 @@ constexpr size_t gemm_lds_bytes() {
     // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x one column
     // sum per wave, 16 row sums) and a dump area for the branch-free predicated writes of the lanes that
     // publish nothing (one word per thread plus the reach of the strided writes)
-    constexpr size_t staging = sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * (BN + 8)) +
+    constexpr size_t staging = sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * b_stage_stride<BN>()) +
            (FT == 1 ? sizeof(float) * (2 * (kGemmBK * (THREADS / 64) + kGemmBK) + THREADS + 2 * kGemmBK * (THREADS / 64)) : 0);
     constexpr size_t verify = FT ? ft_verify_lds_bytes<BM, BN, WGM, WGN, GRAN ? WGM : 1, GRAN ? WGN : 1>() : 0;
     return staging > verify ? staging : verify;
@@ -165,7 +175,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 32, TN = WN / 32;
     static_assert(TM >= 1 && TN >= 1 && WM % 32 == 0 && WN % 32 == 0, "wave tile is made of 32x32 blocks");
-    constexpr int AS = BK + 4, BS = BN + 8;
+    constexpr int AS = BK + 4, BS = b_stage_stride<BN>();
     constexpr int A_STAGE = BM * AS, B_STAGE = BK * BS;
     constexpr int A_V4_PER_ROW = BK / 4, B_V4_PER_ROW = BN / 4;
     constexpr int A_SLOTS = BM * BK / 4 / kGemmThreads, B_SLOTS = BK * BN / 4 / kGemmThreads;

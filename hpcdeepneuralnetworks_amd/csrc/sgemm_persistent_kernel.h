@@ -30,7 +30,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, 1) void sgemm_persistent_kernel(
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 32, TN = WN / 32;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile is made of 32x32 blocks");
-    constexpr int AS = BK + 4, BS = BN + 8;
+    constexpr int AS = BK + 4, BS = b_stage_stride<BN>();
     constexpr int A_STAGE = BM * AS, B_STAGE = BK * BS;
     constexpr int A_V4_PER_ROW = BK / 4, B_V4_PER_ROW = BN / 4;
     constexpr int A_SLOTS = BM * BK / 4 / kThreads, B_SLOTS = BK * BN / 4 / kThreads;
