@@ -88,10 +88,12 @@ constexpr int kGemmBK = 16;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;  // tile rows swept together so that co-resident tiles share A and B panels
 
-// Row stride (floats) of the staged B tile.
-template <int BN>
+// Row stride (floats) of the staged B tile (see the LDS layout above).  The 64-column tiles take the wide stride in
+// the ABFT kernels only: four plain 64 x 64 workgroups per CU would not fit in LDS with it, and their loops have the
+// registers to keep the paired reads' addresses.
+template <int BN, int FT = 0>
 constexpr int b_stage_stride() {
-    return (BN == 128 || BN == 192) ? 264 : BN + 8;
+    return (BN == 128 || BN == 192 || (BN == 64 && FT != 0)) ? 264 : BN + 8;
 }
 
 // LDS the ABFT verification needs (it reuses the staging buffers once the K loop has drained): FP64 partials of the
@@ -110,7 +112,7 @@ constexpr size_t gemm_lds_bytes() {
     // two stages of the A and B tiles; the ABFT kernel adds two stages of checksum partials (16 k x one column
     // sum per wave, 16 row sums) and a dump area for the branch-free predicated writes of the lanes that
     // publish nothing (one word per thread plus the reach of the strided writes)
-    constexpr size_t staging = sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * b_stage_stride<BN>()) +
+    constexpr size_t staging = sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * b_stage_stride<BN, FT>()) +
            (FT == 1 ? sizeof(float) * (2 * (kGemmBK * (THREADS / 64) + kGemmBK) + THREADS + 2 * kGemmBK * (THREADS / 64)) : 0);
     constexpr size_t verify = FT ? ft_verify_lds_bytes<BM, BN, WGM, WGN, GRAN ? WGM : 1, GRAN ? WGN : 1>() : 0;
     return staging > verify ? staging : verify;
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 32, TN = WN / 32;
     static_assert(TM >= 1 && TN >= 1 && WM % 32 == 0 && WN % 32 == 0, "wave tile is made of 32x32 blocks");
-    constexpr int AS = BK + 4, BS = b_stage_stride<BN>();
+    constexpr int AS = BK + 4, BS = b_stage_stride<BN, FT>();
     constexpr int A_STAGE = BM * AS, B_STAGE = BK * BS;
     constexpr int A_V4_PER_ROW = BK / 4, B_V4_PER_ROW = BN / 4;
     constexpr int A_SLOTS = BM * BK / 4 / kGemmThreads, B_SLOTS = BK * BN / 4 / kGemmThreads;
