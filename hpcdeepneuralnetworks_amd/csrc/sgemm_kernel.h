@@ -1128,7 +1128,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int col_base = n0 + wn * WN + lr;      // + j*32
 
     if (FT != 1 && tail_out) {
-        // whole tile, no bounds: rows and columns past the matrix hold zeros (their operands read as zeros)
+        // whole tile, no bounds: the reduction that reads these images skips rows and columns past the matrix
         float* out = tail_out + (wm * WM + lh * 4) * BN + wn * WN + lr;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
