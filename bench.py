@@ -208,8 +208,8 @@ def main() -> int:
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
-            "traffic": profiled_traffic_bytes("sgemm_kernel_6144cube.md"),
-            "kernel": "sgemm_kernel (one launch = 2*6144^3 flop)",
+            "traffic": profiled_traffic_bytes("sgemm_persistent_kernel_6144cube.md"),
+            "kernel": "sgemm_persistent_kernel<192,256> (one launch = 2*6144^3 flop)",
             "kernel_ms": round(kern_ms, 4),
         },
     }

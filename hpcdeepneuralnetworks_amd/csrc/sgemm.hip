@@ -32,6 +32,10 @@ struct TileConfig {
     HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false>),       \
                  (sgemm_persistent_kernel<BM, BN, WGM, WGN, true>))
 
+// (192 accumulators per lane: 64 of a finished tile's stores go out at the tile boundary, no beta != 0 variant)
+#define HPCDNN_TILE_PERSISTENT_BIG(BM, BN, WGM, WGN, OCC, EFF) \
+    HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false, 64>), nullptr)
+
 #define HPCDNN_TILE_DEEP(BM, BN, WGM, WGN, OCC, EFF, NSLOT)                                               \
     {                                                                                                    \
         BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
@@ -55,7 +59,7 @@ static const TileConfig kTiles[] = {
     HPCDNN_TILE(128, 64, 2, 2, 2, 0.945f),   // 2 tall
     HPCDNN_TILE(64, 128, 2, 2, 2, 0.939f),   // 3 wide
     HPCDNN_TILE(64, 64, 2, 2, 4, 0.900f),    // 4 medium
-    HPCDNN_TILE(192, 256, 2, 2, 1, 0.964f),  // 5 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
+    HPCDNN_TILE_PERSISTENT_BIG(192, 256, 2, 2, 1, 0.964f),  // 5 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
     HPCDNN_TILE(256, 192, 2, 2, 1, 0.946f),  // 6
     HPCDNN_TILE_PERSISTENT(128, 256, 2, 2, 2, 0.987f),  // 7
     HPCDNN_TILE(256, 256, 2, 4, 1, 1.000f),  // 8 giant, eight waves
@@ -374,7 +378,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     // Several rounds of whole tiles written straight to C: one persistent workgroup per CU walks its tiles as one
     // stream of K steps (same bits; see sgemm_persistent_kernel.h for what it saves)
     const int persistent = (split == 1 && tail_tiles == 0 && ldc <= kMaxLdc) ? persistent_grid(cfg, M, N, K, device_cus()) : 0;
-    if (persistent > 0) {
+    if (persistent > 0 && (beta == 0.f ? cfg.persistent : cfg.persistent_beta)) {
         fn = beta == 0.f ? cfg.persistent : cfg.persistent_beta;
         grid = dim3(persistent, 1, 1);
     }

@@ -13,6 +13,8 @@
 //     time behind the MFMAs of the next tile's first eight K steps, like the other side instructions of the loop;
 //     the last tile's stores go out after the loop.  With beta != 0 (template flag BETA; C is not read without
 //     it) each group of stores is preceded, one K step earlier, by the loads of the old values it needs.
+//     A tile whose accumulators leave too few registers for a full second set (192 x 256: 192 of 512) stores the
+//     first IMM values of a finished tile at the boundary itself and hands out the rest (beta == 0 only).
 // Same LDS layout, fragment layout, accumulator layout and K-step schedule as sgemm_kernel.h; the summation order
 // of every element of C is the same as there, so both kernels give the same bits.
 #pragma once
@@ -23,7 +25,7 @@ namespace hpcdnn {
 
 constexpr int kPersistDripSteps = 8;  // K steps over which a finished tile's stores are spread
 
-template <int BM, int BN, int WGM, int WGN, bool BETA>
+template <int BM, int BN, int WGM, int WGN, bool BETA, int IMM = 0>
 __global__ __launch_bounds__(WGM * WGN * kWave, 1) void sgemm_persistent_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
     constexpr int kThreads = WGM * WGN * kWave;
@@ -39,8 +41,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, 1) void sgemm_persistent_kernel(
     constexpr int NRD = TM + TN;            // fragment read groups per half K step
     constexpr int NMG = 4 * TM * TN;        // MFMAs per half K step
     constexpr int kStores = TM * TN * 16;   // stores per lane per tile
-    constexpr int NPST = kStores / kPersistDripSteps;
-    static_assert(kStores % kPersistDripSteps == 0, "the stores of a tile split evenly over the drip steps");
+    constexpr int kDrip = kStores - IMM;    // of them handed out during the next tile
+    constexpr int NPST = kDrip / kPersistDripSteps;
+    static_assert(kDrip % kPersistDripSteps == 0, "the deferred stores of a tile split evenly over the drip steps");
+    static_assert(!(BETA && IMM != 0), "stores at the boundary would wait for the old values of C");
     // K steps at the start of a tile that carry stores; with BETA group g is loaded in step g and stored in step g + 1
     constexpr int kDripSection = BETA ? kPersistDripSteps + 2 : kPersistDripSteps;
 
@@ -119,16 +123,16 @@ __global__ __launch_bounds__(WGM * WGN * kWave, 1) void sgemm_persistent_kernel(
     };
 
     // ---- LDS -> fragment registers -> MFMA
-    v16f acc[TM][TN], done[TM][TN];  // the tile being multiplied; the finished tile (times alpha) whose stores are going out
+    v16f acc[TM][TN];   // the tile being multiplied
+    float done[kDrip];  // the finished tile (times alpha), less its first IMM values: the stores that are going out
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                acc[i][j][v] = 0.f;
-                done[i][j][v] = 0.f;
-            }
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+#pragma unroll
+    for (int e = 0; e < kDrip; ++e) done[e] = 0.f;
     v4f fa[2][TM];
     float fb[2][TN][4];
     const int a_frag_off = (wm * WM + lr) * AS + lh * 4;
@@ -164,19 +168,19 @@ __global__ __launch_bounds__(WGM * WGN * kWave, 1) void sgemm_persistent_kernel(
         return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<float*>(static_cast<uint64_t>(done_hi) << 32 | done_lo), 0,
                                                  done_bytes, 0x00020000);
     };
-    // store number E of the tile: element v of block (i, j)
+    // deferred store number E of the tile: element v of block (i, j), which is store IMM + E of all of them
     auto pload1 = [&](auto idx) {
-        constexpr int E = decltype(idx)::value;
-        constexpr int j = E % TN, v = (E / TN) % 16, i = E / (TN * 16);
+        constexpr int E = decltype(idx)::value, Q = E + IMM;
+        constexpr int j = Q % TN, v = (Q / TN) % 16, i = Q / (TN * 16);
         constexpr int r = i * 32 + 8 * (v / 4) + (v % 4);
         old[(E / NPST) & 1][E % NPST] =
             __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(done_rsrc(), lane_off + j * 128, r * ldc_bytes, 0));
     };
     auto pstore1 = [&](auto idx) {
-        constexpr int E = decltype(idx)::value;
-        constexpr int j = E % TN, v = (E / TN) % 16, i = E / (TN * 16);
+        constexpr int E = decltype(idx)::value, Q = E + IMM;
+        constexpr int j = Q % TN, v = (Q / TN) % 16, i = Q / (TN * 16);
         constexpr int r = i * 32 + 8 * (v / 4) + (v % 4);
-        float value = done[i][j][v];  // (a bit cast applied to the vector element itself reads element 0)
+        float value = done[E];
         if constexpr (BETA) value = __builtin_fmaf(beta, old[(E / NPST) & 1][E % NPST], value);
         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), done_rsrc(), lane_off + j * 128,
                                               r * ldc_bytes, 0);
@@ -249,19 +253,28 @@ __global__ __launch_bounds__(WGM * WGN * kWave, 1) void sgemm_persistent_kernel(
             step(S0{}, S1{}, S1{}, std::integral_constant<int, -1>{});
         }
         // tile boundary: the stream is already inside the next tile (its step 0 is in LDS, step 1 in flight)
+        const uint64_t corner = reinterpret_cast<uint64_t>(p.C + static_cast<int64_t>(m0) * p.ldc + n0);
+        done_lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(corner));
+        done_hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(corner >> 32));
+        done_bytes = -1;
+        static_for<kStores>([&](auto q) {
+            constexpr int Q = decltype(q)::value;
+            constexpr int j = Q % TN, v = (Q / TN) % 16, i = Q / (TN * 16);
+            const float scaled = alpha * acc[i][j][v];
+            if constexpr (Q < IMM) {
+                constexpr int r = i * 32 + 8 * (v / 4) + (v % 4);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, scaled), done_rsrc(), lane_off + j * 128,
+                                                      r * ldc_bytes, 0);
+            } else {
+                done[Q - IMM] = scaled;
+            }
+        });
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    done[i][j][v] = alpha * acc[i][j][v];
-                    acc[i][j][v] = 0.f;
-                }
-        const uint64_t corner = reinterpret_cast<uint64_t>(p.C + static_cast<int64_t>(m0) * p.ldc + n0);
-        done_lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(corner));
-        done_hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(corner >> 32));
-        done_bytes = -1;
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
         tile += stride;
         if (tile >= total) break;
         origin(tile, m0, n0);
