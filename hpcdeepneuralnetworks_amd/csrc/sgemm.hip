@@ -18,35 +18,40 @@ struct TileConfig {
     // persistent variants for several rounds of whole tiles (beta == 0, beta != 0), or nullptr
     void (*persistent)(const GemmArgs);
     void (*persistent_beta)(const GemmArgs);
+    int persistent_per_cu;  // workgroups of the persistent kernel per CU
 };
 
-#define HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, PERSISTENT, PERSISTENT_BETA)                                                        \
+#define HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, PERSISTENT, PERSISTENT_BETA, PER_CU)                                                        \
     {                                                                                                    \
         BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
             sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC>, EFF, false, 2, \
-            PERSISTENT, PERSISTENT_BETA                                                                          \
+            PERSISTENT, PERSISTENT_BETA, PER_CU                                                                        \
     }
 
-#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, EFF) HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, nullptr, nullptr)
+#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, EFF) HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, nullptr, nullptr, 1)
 #define HPCDNN_TILE_PERSISTENT(BM, BN, WGM, WGN, OCC, EFF) \
     HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false>),       \
-                 (sgemm_persistent_kernel<BM, BN, WGM, WGN, true>))
+                 (sgemm_persistent_kernel<BM, BN, WGM, WGN, true>), 1)
+// (the 128 x 128 tile: 64 accumulators per lane, two persistent workgroups per CU)
+#define HPCDNN_TILE_PERSISTENT_TWO(BM, BN, WGM, WGN, OCC, EFF) \
+    HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false, 0, 2>),  \
+                 (sgemm_persistent_kernel<BM, BN, WGM, WGN, true, 0, 2>), 2)
 
 // (192 accumulators per lane: 64 of a finished tile's stores go out at the tile boundary, no beta != 0 variant)
 #define HPCDNN_TILE_PERSISTENT_BIG(BM, BN, WGM, WGN, OCC, EFF) \
-    HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false, 64>), nullptr)
+    HPCDNN_TILE_(BM, BN, WGM, WGN, OCC, EFF, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false, 64>), nullptr, 1)
 
 #define HPCDNN_TILE_DEEP(BM, BN, WGM, WGN, OCC, EFF, NSLOT)                                               \
     {                                                                                                    \
         BM, BN, kGemmBK, WGM * WGN * kWave, OCC, gemm_lds_bytes<BM, BN>(),                               \
             sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC, NSLOT>, sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC, NSLOT>, EFF, \
-            false, NSLOT, nullptr, nullptr                                                               \
+            false, NSLOT, nullptr, nullptr, 1                                                             \
     }
 
 #define HPCDNN_SMALL_TILE(TMB, OCC, EFF)                                                                  \
     {                                                                                                    \
         32 * TMB, 32, kSmallBK, kSmallThreads, OCC, small_lds_bytes<TMB>(), sgemm_small_kernel<TMB, false, OCC>, \
-            sgemm_small_kernel<TMB, true, OCC>, EFF, true, 0, nullptr, nullptr                           \
+            sgemm_small_kernel<TMB, true, OCC>, EFF, true, 0, nullptr, nullptr, 1                         \
     }
 
 // The counterpart of the reference's small/medium/large/tall/wide/huge shape table
@@ -55,7 +60,7 @@ struct TileConfig {
 // squares 256..6144 with K = n, 1024 and 256 and a set of skinny shapes on an MI355X.
 static const TileConfig kTiles[] = {
     HPCDNN_TILE_PERSISTENT(256, 128, 2, 2, 2, 0.978f),  // 0 huge (the ABFT tile)
-    HPCDNN_TILE(128, 128, 2, 2, 2, 0.970f),  // 1 large
+    HPCDNN_TILE_PERSISTENT_TWO(128, 128, 2, 2, 2, 0.970f),  // 1 large
     HPCDNN_TILE(128, 64, 2, 2, 2, 0.945f),   // 2 tall
     HPCDNN_TILE(64, 128, 2, 2, 2, 0.939f),   // 3 wide
     HPCDNN_TILE(64, 64, 2, 2, 4, 0.900f),    // 4 medium
@@ -109,7 +114,7 @@ constexpr double kPersistGainK = 12.8, kPersistGainMax = 0.05, kPersistRankGain 
 // The persistent kernel takes unsplit problems of more than one round of whole tiles with an even number of K steps,
 // enough of them to spread a tile's stores over.
 static int persistent_grid(const TileConfig& t, int M, int N, int K, int cus) {
-    const int grid = cus / kXcds * kXcds;
+    const int grid = cus / kXcds * kXcds * t.persistent_per_cu;
     if (!t.persistent || (M % t.bm) || (N % t.bn) || (K % (2 * t.bk)) || K / t.bk < kPersistDripSteps + 2) return 0;
     return static_cast<int64_t>(M / t.bm) * (N / t.bn) > grid ? grid : 0;
 }

@@ -6,7 +6,7 @@
 // the matrix cores idle while every CU waits for its first loads or for its stores.  On a short K (8192 x 8192 x
 // 256: sixteen K steps per tile) that is a sixth of the run.
 //
-// Here one workgroup per CU walks the tiles id, id + grid, id + 2 grid, ... as one stream of K steps:
+// Here one workgroup per CU (two of the 128 x 128 tile, which has the registers for it) walks the tiles id, id + grid, id + 2 grid, ... as one stream of K steps:
 //   * the loads that run two K steps ahead cross over to the next tile's first steps, so the pipeline never
 //     drains and a tile boundary costs only the move of the accumulators;
 //   * the finished tile (times alpha) moves to a second register set, and its stores are handed out a few at a
@@ -25,8 +25,8 @@ namespace hpcdnn {
 
 constexpr int kPersistDripSteps = 8;  // K steps over which a finished tile's stores are spread
 
-template <int BM, int BN, int WGM, int WGN, bool BETA, int IMM = 0>
-__global__ __launch_bounds__(WGM * WGN * kWave, 1) void sgemm_persistent_kernel(const GemmArgs p) {
+template <int BM, int BN, int WGM, int WGN, bool BETA, int IMM = 0, int PER_CU = 1>
+__global__ __launch_bounds__(WGM * WGN * kWave, PER_CU) void sgemm_persistent_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
     constexpr int kThreads = WGM * WGN * kWave;
     constexpr int WM = BM / WGM, WN = BN / WGN;

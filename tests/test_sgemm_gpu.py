@@ -356,15 +356,16 @@ def test_row_split_gives_the_same_bits_as_one_launch(blas, oracle_mod):
 
 
 @pytest.mark.parametrize("M,N,K,tile", [(2176, 4608, 320, 7), (4352, 2304, 192, 0), (4096, 4096, 160, 7), (4096, 2048, 256, 0),
-                                        (3264, 4608, 320, 5), (3072, 4096, 512, 5)])
+                                        (3264, 4608, 320, 5), (3072, 4096, 512, 5), (2176, 4608, 320, 1), (4096, 4096, 160, 1)])
 @pytest.mark.parametrize("alpha,beta", [(1.5, 0.0), (1.0, -1.5)])
 def test_persistent_kernel_on_several_rounds_of_whole_tiles(blas, oracle_mod, M, N, K, tile, alpha, beta):
     """More tiles than CUs, every tile whole, an even number (>= 10) of K steps: the 256x128 and 128x256 tiles run as
     one persistent workgroup per CU that stores a finished tile while it multiplies the next.  Checked against the
-    FP64 criterion (sampled rows + Freivalds over all of C), for the same bits as the 128x128 tile-per-workgroup
+    FP64 criterion (sampled rows + Freivalds over all of C), for the same bits as the 128x64 tile-per-workgroup
     kernel, with a padded ldc whose padding stays untouched, and with NaN in C when beta == 0.  306 tiles leave a
     partial last round, 512 tiles give every workgroup two, 256 tiles (one round) take the ordinary kernel.  The 192x256
-    tile stores a third of a finished tile at the tile boundary and has no beta != 0 variant (the ordinary kernel runs)."""
+    tile stores a third of a finished tile at the tile boundary and has no beta != 0 variant (the ordinary kernel runs).
+    The 128x128 tile runs two persistent workgroups per CU, so it takes more than 512 tiles."""
     _sampled_check(oracle_mod, blas, M, N, K, alpha, beta, nrows=12, seed=700 + tile, tile=tile, split_k=1)
     dev = "cuda"
     ldc = N + 24
@@ -376,7 +377,7 @@ def test_persistent_kernel_on_several_rounds_of_whole_tiles(blas, oracle_mod, M,
         c0[:, :N] = torch.rand(M, N, device=dev) * 2 - 1
     c1, c2 = c0.clone(), c0.clone()
     blas.sgemm(M, N, K, da, db, c1, alpha, beta, tile=tile, split_k=1)  # ldc = the row stride of c1
-    blas.sgemm(M, N, K, da, db, c2, alpha, beta, tile=1, split_k=1)
+    blas.sgemm(M, N, K, da, db, c2, alpha, beta, tile=2, split_k=1)
     assert torch.equal(c1[:, :N], c2[:, :N])
     assert not torch.isnan(c1[:, :N]).any()
     assert torch.isnan(c1[:, N:]).all()
