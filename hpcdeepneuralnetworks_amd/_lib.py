@@ -29,6 +29,9 @@ EXPORTS = (
     "hpcdnn_error_string",
     "hpcdnn_sgemm",
     "hpcdnn_sgemm_ex",
+    "hpcdnn_sgemm_tn",
+    "hpcdnn_sgemm_tn_ex",
+    "hpcdnn_sgemm_cm_nt",
     "hpcdnn_sgemm_num_tiles",
     "hpcdnn_sgemm_tile_info",
     "hpcdnn_sgemm_plan",
@@ -108,6 +111,12 @@ def lib():
     L.hpcdnn_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, vp, sz, vp]
     L.hpcdnn_sgemm_ex.restype = i
     L.hpcdnn_sgemm_ex.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, vp, sz, i, i, vp]
+    L.hpcdnn_sgemm_tn.restype = i
+    L.hpcdnn_sgemm_tn.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, vp, sz, vp]
+    L.hpcdnn_sgemm_tn_ex.restype = i
+    L.hpcdnn_sgemm_tn_ex.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, vp, sz, i, i, vp]
+    L.hpcdnn_sgemm_cm_nt.restype = i
+    L.hpcdnn_sgemm_cm_nt.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, vp, sz, vp]
     L.hpcdnn_sgemm_num_tiles.restype = i
     L.hpcdnn_sgemm_num_tiles.argtypes = []
     L.hpcdnn_sgemm_tile_info.restype = i

@@ -108,6 +108,34 @@ def sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Te
     check(rc, "hpcdnn_sgemm")
 
 
+def sgemm_tn(M: int, N: int, K: int, At: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
+             ws: torch.Tensor | None = None, tile: int = -1, split_k: int = 0) -> None:
+    """In place ``C = alpha*At.T@B + beta*C`` with ``At`` the K x M row-major transpose of the left operand."""
+    pa, lda = _matrix(At, K, M, "At")
+    pb, ldb = _matrix(B, K, N, "B")
+    pc, ldc = _matrix(Cm, M, N, "C")
+    wsp, wsb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
+    L = _lib.lib()
+    if tile < 0 and split_k == 0:
+        rc = L.hpcdnn_sgemm_tn(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, wsp, wsb, _stream())
+    else:
+        rc = L.hpcdnn_sgemm_tn_ex(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, wsp, wsb, tile, split_k, _stream())
+    check(rc, "hpcdnn_sgemm_tn")
+
+
+def sgemm_cm_nt(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
+                ws: torch.Tensor | None = None) -> None:
+    """Column-major ``C (M x N) = alpha*A (M x K) @ B (N x K).T + beta*C``, the layout of the reference's
+    ``sgemm_<shape><<<...>>>(M, N, K, A, B, C, alpha, beta)`` (kernel/ft_sgemm/include/sgemm_huge.cuh:14) and of the cuBLAS
+    call beside it (kernel/ft_sgemm/sgemm.cu:111).  The tensors hold the column-major matrices as their row-major
+    transposes: ``A`` is K x M, ``B`` is K x N, ``C`` is N x M; their row strides are the leading dimensions."""
+    pa, lda = _matrix(A, K, M, "A")
+    pb, ldb = _matrix(B, K, N, "B")
+    pc, ldc = _matrix(Cm, N, M, "C")
+    wsp, wsb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
+    check(_lib.lib().hpcdnn_sgemm_cm_nt(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, wsp, wsb, _stream()), "hpcdnn_sgemm_cm_nt")
+
+
 def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
              tau: float = 0.0, fault=None, status: torch.Tensor | None = None, ws: torch.Tensor | None = None,
              tile_class: int = 0, granularity: int = 0, check_interval: int = 0, faults=None) -> None:

@@ -11,15 +11,18 @@ constexpr int kMaxLda = (1 << 21) - 64;    // 256 * lda * 4 < 2^31
 constexpr int kMaxLdb = (1 << 25) - 1024;  // 16 * ldb * 4 + row < 2^31
 constexpr int kMaxLdc = (1 << 21) - 64;    // 256 * ldc * 4 + row < 2^31
 
-inline int check_gemm_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+// ta: A is given transposed, K rows of M floats (row length lda >= M, at most kMaxLdb: a K step is 16 of its rows)
+inline int check_gemm_args(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                           bool ta = false) {
     if (M < 0 || N < 0 || K < 0) return HPCDNN_ERR_INVALID_VALUE;
-    if (lda < (K > 1 ? K : 1) || ldb < (N > 1 ? N : 1) || ldc < (N > 1 ? N : 1)) return HPCDNN_ERR_INVALID_VALUE;
+    const int a_cols = ta ? M : K;
+    if (lda < (a_cols > 1 ? a_cols : 1) || ldb < (N > 1 ? N : 1) || ldc < (N > 1 ? N : 1)) return HPCDNN_ERR_INVALID_VALUE;
     if (M > 0 && N > 0 && !C) return HPCDNN_ERR_INVALID_VALUE;
     if (M > 0 && N > 0 && K > 0 && (!A || !B)) return HPCDNN_ERR_INVALID_VALUE;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) & 3u)
         return HPCDNN_ERR_INVALID_VALUE;
     // byte offsets inside one tile are 32-bit: 256 rows of A and of C, 16 rows of B
-    if (lda > kMaxLda || ldb > kMaxLdb || ldc > kMaxLdc) return HPCDNN_ERR_INVALID_VALUE;
+    if (lda > (ta ? kMaxLdb : kMaxLda) || ldb > kMaxLdb || ldc > kMaxLdc) return HPCDNN_ERR_INVALID_VALUE;
     return HPCDNN_OK;
 }
 
@@ -44,6 +47,10 @@ inline GemmArgs make_args(int M, int N, int K, const float* A, int lda, const fl
 inline bool needs_edge(const GemmArgs& a, int bm, int bn, int bk) {
     return !(a.M % bm == 0 && a.N % bn == 0 && a.K % bk == 0);
 }
+
+// The kernel of tile `tile` (bm x bn, as a cross-check of the index) for a transposed left operand, or nullptr when
+// the tile has none (sgemm_ta.hip).
+void (*sgemm_ta_kernel(int tile, int bm, int bn, bool edge))(const GemmArgs);
 
 // Kernels that use more than the default 64 KiB of LDS must opt in once per device.
 inline int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {

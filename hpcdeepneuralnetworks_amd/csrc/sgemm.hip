@@ -290,11 +290,15 @@ static RowSplit choose_row_split(int M, int N, int K, int cus) {
     return best;
 }
 
+// ta: A is given transposed (K x M row-major).  Those kernels exist for every tile but the 32 x 32 one and have no
+// persistent variant; everything else (plans, splits, reductions) is shared.
 static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
-                     float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split, hipStream_t stream) {
-    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
+                     float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split, hipStream_t stream,
+                     bool ta = false) {
+    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc, ta);
     if (rc != HPCDNN_OK) return rc;
     if (tile >= kNumTiles || split == -1) return HPCDNN_ERR_INVALID_VALUE;
+    if (ta && tile >= 0 && kTiles[tile].wave_split_k) return HPCDNN_ERR_INVALID_VALUE;
     if (tile >= 0 && kTiles[tile].wave_split_k && split < -1) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
 
@@ -304,7 +308,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         struct Decision {
             int M, N, K, cus;
             size_t ws_bytes;
-            bool ws_aligned, valid;
+            bool ws_aligned, valid, ta;
             Plan plan;
             RowSplit rows;
         };
@@ -314,9 +318,9 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         const size_t usable = ws ? ws_bytes : 0;
         const int cus = device_cus();  // of the current device: the plan depends on it
         if (!(memo.valid && memo.M == M && memo.N == N && memo.K == K && memo.cus == cus && memo.ws_bytes == usable &&
-              memo.ws_aligned == ws_aligned)) {
+              memo.ws_aligned == ws_aligned && memo.ta == ta)) {
             double cost = 0.0;
-            memo.plan = choose_plan(M, N, K, ws != nullptr, usable, ws_aligned, &cost);
+            memo.plan = choose_plan(M, N, K, ws != nullptr, usable, ws_aligned, &cost, ta);
             memo.rows = RowSplit{-1, 0, -1, 1e300};
             if (K > 0) {
                 const RowSplit rs = choose_row_split(M, N, K, cus);
@@ -325,6 +329,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
             memo.M = M; memo.N = N; memo.K = K; memo.cus = cus;
             memo.ws_bytes = usable;
             memo.ws_aligned = ws_aligned;
+            memo.ta = ta;
             memo.valid = true;
         }
         Plan plan = memo.plan;
@@ -332,10 +337,10 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         if (tile < 0 && split < -1) plan = choose_plan(M, N, K, false, 0, false, nullptr, true);
         const RowSplit rs = memo.rows;  // copied: the nested calls below do not touch the memo, but keep it simple
         if (tile < 0 && split == 0 && rs.tile1 >= 0) {
-            rc = run_sgemm(rs.rows1, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, rs.tile1, 1, stream);
+            rc = run_sgemm(rs.rows1, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, rs.tile1, 1, stream, ta);
             if (rc != HPCDNN_OK) return rc;
-            return run_sgemm(M - rs.rows1, N, K, A + static_cast<int64_t>(rs.rows1) * lda, lda, B, ldb,
-                             C + static_cast<int64_t>(rs.rows1) * ldc, ldc, alpha, beta, nullptr, 0, rs.tile2, 1, stream);
+            return run_sgemm(M - rs.rows1, N, K, A + (ta ? rs.rows1 : static_cast<int64_t>(rs.rows1) * lda), lda, B, ldb,
+                             C + static_cast<int64_t>(rs.rows1) * ldc, ldc, alpha, beta, nullptr, 0, rs.tile2, 1, stream, ta);
         }
         if (tile < 0) {
             tile = plan.tile;
@@ -378,11 +383,12 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         if (split > 1) a.partial = static_cast<float*>(ws);
     }
     const bool edge = needs_edge(a, cfg.bm, cfg.bn, cfg.bk);
-    void (*fn)(const GemmArgs) = edge ? cfg.edge : cfg.plain;
+    void (*fn)(const GemmArgs) = ta ? sgemm_ta_kernel(tile, cfg.bm, cfg.bn, edge) : edge ? cfg.edge : cfg.plain;
+    if (!fn) return HPCDNN_ERR_INVALID_VALUE;
     dim3 grid(a.full_tiles + tail_tiles * a.tail_split, 1, split);
     // Several rounds of whole tiles written straight to C: one persistent workgroup per CU walks its tiles as one
     // stream of K steps (same bits; see sgemm_persistent_kernel.h for what it saves)
-    const int persistent = (split == 1 && tail_tiles == 0 && ldc <= kMaxLdc) ? persistent_grid(cfg, M, N, K, device_cus()) : 0;
+    const int persistent = (split == 1 && tail_tiles == 0 && ldc <= kMaxLdc && !ta) ? persistent_grid(cfg, M, N, K, device_cus()) : 0;
     if (persistent > 0 && (beta == 0.f ? cfg.persistent : cfg.persistent_beta)) {
         fn = beta == 0.f ? cfg.persistent : cfg.persistent_beta;
         grid = dim3(persistent, 1, 1);
@@ -428,6 +434,25 @@ extern "C" int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, con
                                float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split_k, void* stream) {
     return run_sgemm(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, ws, ws_bytes, tile, split_k,
                      static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hpcdnn_sgemm_tn(int M, int N, int K, const float* At, int ldat, const float* B, int ldb, float* C, int ldc,
+                               float alpha, float beta, void* ws, size_t ws_bytes, void* stream) {
+    return run_sgemm(M, N, K, At, ldat, B, ldb, C, ldc, alpha, beta, ws, ws_bytes, -1, 0, static_cast<hipStream_t>(stream), true);
+}
+
+extern "C" int hpcdnn_sgemm_tn_ex(int M, int N, int K, const float* At, int ldat, const float* B, int ldb, float* C, int ldc,
+                                  float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split_k, void* stream) {
+    return run_sgemm(M, N, K, At, ldat, B, ldb, C, ldc, alpha, beta, ws, ws_bytes, tile, split_k,
+                     static_cast<hipStream_t>(stream), true);
+}
+
+// Column-major C (M x N) = alpha * A (M x K) * B (N x K)^T + beta * C is, read row by row, the N x M matrix
+// C^T = alpha * (B^T)^T * A^T + beta * C^T with B^T = the memory of B as K rows of N and A^T = the memory of A as K
+// rows of M: the transposed-left-operand product with the operands swapped.
+extern "C" int hpcdnn_sgemm_cm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                                  float alpha, float beta, void* ws, size_t ws_bytes, void* stream) {
+    return run_sgemm(N, M, K, B, ldb, A, lda, C, ldc, alpha, beta, ws, ws_bytes, -1, 0, static_cast<hipStream_t>(stream), true);
 }
 
 extern "C" int hpcdnn_sgemm_num_tiles(void) { return kNumTiles; }

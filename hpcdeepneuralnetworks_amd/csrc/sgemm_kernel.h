@@ -163,9 +163,18 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
 // CADENCE (ABFT only): the K loop runs in intervals of p.check_interval; after each interval the pipeline drains,
 // the accumulators are verified against the references of the k range done so far, and the references are
 // re-synchronised, as the reference kernel does every 256 k (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:143,263-271).
-template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS, int NSLOT = 2, int GRAN = 0, bool CADENCE = false>
+//
+// TA (plain SGEMM only): the left operand is given transposed, p.A = A^T as a K x M row-major matrix with row length
+// p.lda >= M, which is how the operands of a column-major C = A * B^T lie in memory
+// (kernel/ft_sgemm/include/sgemm_huge.cuh:14, cublasSgemm(N, T, ...) in kernel/ft_sgemm/sgemm.cu:111).  A K step of
+// the tile is then 16 rows of BM floats, like B's; a lane fetches four consecutive m of one k and writes them as four
+// words into the same [m][k] staging layout, so everything from the fragment reads on is the code of the untransposed
+// case and every element of C sums its products in the same order.
+template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS, int NSLOT = 2, int GRAN = 0, bool CADENCE = false,
+          bool TA = false>
 __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
+    static_assert(!TA || FT == 0, "the ABFT kernels take A row by row");
     static_assert(NSLOT == 2 || (FT == 0 && NSLOT % 2 == 0), "the ABFT loop is written for two staging sets");
     static_assert(FT != 0 || (GRAN == 0 && !CADENCE), "granularity and cadence belong to the ABFT kernels");
     static_assert(GRAN == 0 || FT == 2, "wave-tile checksums come from the pre-encoded vectors");
@@ -221,7 +230,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     // (a tile that hangs over the last column reads B past the ends of its rows: into the next row, which must exist
     // and be long enough for that to stay inside the matrix)
-    const bool lazy_ok = n0 + BN <= p.N || p.ldb >= BN;
+    const bool lazy_ok = (n0 + BN <= p.N || p.ldb >= BN) && (!TA || m0 + BM <= p.M || p.lda >= BM);
     // the K range of one pass of the pipeline: the slice, or one verification interval of it
     int kbeg = k_slice * k_chunk;
     int kend = (p.K - kbeg < k_chunk) ? p.K : kbeg + k_chunk;
@@ -230,10 +239,17 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // ---- global -> register staging: which 16-byte groups of the A and B tiles this thread moves.
     // Descriptors start at the tile's first element of the current K step and end with the matrix, so that
     // rows m >= M of A and rows k >= K of B read as 0; the base moves forward by one K step per load.
-    const float* a_base = p.A + static_cast<int64_t>(m0) * p.lda + kbeg;
+    // (TA: A^T is walked like B, rows k >= K read as 0, and columns m >= M, the next row or padding, only reach
+    // accumulators of rows m >= M, which are never stored)
+    auto a_origin = [&](int k) { return TA ? p.A + static_cast<int64_t>(k) * p.lda + m0 : p.A + static_cast<int64_t>(m0) * p.lda + k; };
+    auto a_bytes_left = [&](int k) {  // bytes from a_origin(k) to the end of A
+        return TA ? (static_cast<int64_t>(p.K - 1 - k) * p.lda + (p.M - m0)) * 4 : (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - k)) * 4;
+    };
+    const float* a_base = a_origin(kbeg);
     const float* b_base = p.B + static_cast<int64_t>(kbeg) * p.ldb + n0;
-    int64_t a_left = (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - kbeg)) * 4;  // bytes from a_base to the end of A
+    int64_t a_left = a_bytes_left(kbeg);
     int64_t b_left = (static_cast<int64_t>(p.K - 1 - kbeg) * p.ldb + (p.N - n0)) * 4;
+    const int64_t a_step = TA ? static_cast<int64_t>(BK) * p.lda : BK;
     const int64_t b_step = static_cast<int64_t>(BK) * p.ldb;
 
     int a_voff[A_SLOTS], a_lds[A_SLOTS], a_kc[A_SLOTS];
@@ -241,11 +257,21 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
     for (int s = 0; s < A_SLOTS; ++s) {
         const int idx = tid + s * kGemmThreads;
-        int row = idx / A_V4_PER_ROW;
-        a_kc[s] = (idx % A_V4_PER_ROW) * 4;
-        if constexpr (kLazyBounds) row = row < p.M - m0 ? row : p.M - 1 - m0;
-        a_voff[s] = (row * p.lda + a_kc[s]) * 4;
-        a_lds[s] = row * AS + a_kc[s];
+        if constexpr (TA) {
+            // four neighbouring lanes take 64 contiguous bytes of one row of A^T (one request to the vector cache,
+            // as in the untransposed case), the sixteen quads of a wave the sixteen k; a wave's word writes of one
+            // of a lane's four m land in 64 different LDS banks (80 q + k for q = 0..3, k = 0..15)
+            const int k = (idx / 4) % BK, m = ((idx / (4 * BK)) * 4 + idx % 4) * 4;
+            a_kc[s] = k;
+            a_voff[s] = (k * p.lda + m) * 4;
+            a_lds[s] = m * AS + k;
+        } else {
+            int row = idx / A_V4_PER_ROW;
+            a_kc[s] = (idx % A_V4_PER_ROW) * 4;
+            if constexpr (kLazyBounds) row = row < p.M - m0 ? row : p.M - 1 - m0;
+            a_voff[s] = (row * p.lda + a_kc[s]) * 4;
+            a_lds[s] = row * AS + a_kc[s];
+        }
     }
 #pragma unroll
     for (int s = 0; s < B_SLOTS; ++s) {
@@ -319,7 +345,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // run over the whole tile width) force them to 0 as well.
     auto gmask1 = [&](auto slot, auto part) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
-        if constexpr (P < A_SLOTS) {
+        if constexpr (P < A_SLOTS && TA) {
+            // nothing to force: rows k >= K of A^T read as 0, and a K slice ends on a K step unless it ends with K
+        } else if constexpr (P < A_SLOTS) {
             const int left = kend - (k_slot[S] + a_kc[P]);
             v4f v = ra[S][P];
             v.x = left > 0 ? v.x : 0.f;
@@ -342,20 +370,28 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // descriptors are emptied, so the fetches that run ahead past the end all return 0 (never multiplied, and
     // neutral for the checksums).
     auto gload_advance_bulk = [&]() {  // kLazyBounds, a step that is not the slice's last: no end to look out for
-        a_base += BK;
+        a_base += a_step;
         b_base += b_step;
         k_loaded += BK;
     };
     // kLazyBounds, at the end of the bulk steps: the byte counts from the current bases to the ends of A and B
     auto bounds_from_position = [&]() {
-        a_left = (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - k_loaded)) * 4;
+        a_left = a_bytes_left(k_loaded);
         b_left = (static_cast<int64_t>(p.K - 1 - k_loaded) * p.ldb + (p.N - n0)) * 4;
     };
     auto gload_advance = [&]() {
         const bool more = k_loaded + BK < kend;
-        a_base += more ? BK : 0;
-        a_left = more ? a_left - BK * 4 : 0;
-        b_base += more ? b_step : 0;
+        if constexpr (TA) {
+            // the bases move on regardless (an emptied descriptor returns 0 wherever it starts): with both steps
+            // held in registers the compiler would otherwise branch around the updates, and the branch would cut
+            // the K step's instruction schedule in two
+            a_base += a_step;
+            b_base += b_step;
+        } else {
+            a_base += more ? a_step : 0;
+            b_base += more ? b_step : 0;
+        }
+        a_left = more ? a_left - a_step * 4 : 0;
         b_left = more ? b_left - b_step * 4 : 0;
         k_loaded += more ? BK : 0;
         if constexpr (FT == 2) enc_off += BK * 4;
@@ -363,15 +399,15 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // The same in two parts, so that the short-step schedule can place them apart.  Its full tiles keep no bounds at
     // all: nothing they fetch lies outside the matrix, and past the end of the slice they fetch its last K step
     // again instead of zeros.
-    auto gload_advance_a_bulk = [&]() { a_base += BK; };
+    auto gload_advance_a_bulk = [&]() { a_base += a_step; };
     auto gload_advance_b_bulk = [&]() {
         b_base += b_step;
         k_loaded += BK;
     };
     auto gload_advance_a = [&]() {
         const bool more = k_loaded + BK < kend;
-        a_base += more ? BK : 0;
-        if constexpr (!kNoBounds) a_left = more ? a_left - BK * 4 : 0;
+        a_base += more ? a_step : 0;
+        if constexpr (!kNoBounds) a_left = more ? a_left - a_step * 4 : 0;
     };
     auto gload_advance_b = [&]() {
         const bool more = k_loaded + BK < kend;
@@ -381,7 +417,13 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     };
     auto lstore1 = [&](auto slot, auto part, int stage) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
-        if constexpr (P < A_SLOTS)
+        if constexpr (P < A_SLOTS && TA) {
+            float* const dst = As + stage * A_STAGE + a_lds[P];
+            dst[0] = ra[S][P].x;
+            dst[AS] = ra[S][P].y;
+            dst[2 * AS] = ra[S][P].z;
+            dst[3 * AS] = ra[S][P].w;
+        } else if constexpr (P < A_SLOTS)
             *reinterpret_cast<v4f*>(As + stage * A_STAGE + a_lds[P]) = ra[S][P];
         else
             *reinterpret_cast<v4f*>(Bs + stage * B_STAGE + b_lds[P - A_SLOTS]) = rb[S][P - A_SLOTS];
@@ -389,9 +431,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 
     // CADENCE: point the staging state at the start of the next verification interval [kbeg, kend)
     auto k_range_reset = [&]() {
-        a_base = p.A + static_cast<int64_t>(m0) * p.lda + kbeg;
+        a_base = a_origin(kbeg);
         b_base = p.B + static_cast<int64_t>(kbeg) * p.ldb + n0;
-        a_left = (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - kbeg)) * 4;
+        a_left = a_bytes_left(kbeg);
         b_left = (static_cast<int64_t>(p.K - 1 - kbeg) * p.ldb + (p.N - n0)) * 4;
         k_loaded = kbeg;
 #pragma unroll

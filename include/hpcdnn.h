@@ -108,6 +108,32 @@ int hpcdnn_sgemm(int M, int N, int K, const float* A, int lda, const float* B, i
 int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                     float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split_k, void* stream);
 
+/* The same product with the left operand given transposed: C (M x N, row-major)
+ * = alpha * At^T * B + beta * C, where At is K x M row-major with row length
+ * ldat >= M (ldat <= 2^25 - 1024); everything else as hpcdnn_sgemm.  Every
+ * element of C sums its products in the order hpcdnn_sgemm uses, so the result
+ * has the bits of hpcdnn_sgemm on the explicitly transposed operand.  This is the
+ * operand layout of the reference's column-major family (below).  The _ex form
+ * pins tile and split as hpcdnn_sgemm_ex does; the 32 x 32 tile is not available
+ * (HPCDNN_ERR_INVALID_VALUE). */
+int hpcdnn_sgemm_tn(int M, int N, int K, const float* At, int ldat, const float* B, int ldb, float* C, int ldc,
+                    float alpha, float beta, void* ws, size_t ws_bytes, void* stream);
+int hpcdnn_sgemm_tn_ex(int M, int N, int K, const float* At, int ldat, const float* B, int ldb, float* C, int ldc,
+                       float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split_k, void* stream);
+
+/* COLUMN-MAJOR C (M x N, ldc >= M) = alpha * A (M x K, lda >= M) * B (N x K,
+ * ldb >= N)^T + beta * C: the buffers, argument order and meaning of
+ * sgemm_{small,medium,large,tall,wide,huge}<<<...>>>(M,N,K,A,B,C,alpha,beta)
+ * (kernel/ft_sgemm/include/sgemm_huge.cuh:14, launched at
+ * kernel/ft_sgemm/sgemm.cu:114-157) and of the cuBLAS call they are checked
+ * against, cublasSgemm(handle, CUBLAS_OP_N, CUBLAS_OP_T, M, N, K, &alpha, dA, M,
+ * dB, N, &beta, dC, M) (kernel/ft_sgemm/sgemm.cu:111), taken as they are.  Read
+ * row by row the same memory is C^T (N x M) = B^T^T * A^T, which is what runs:
+ * hpcdnn_sgemm_tn(N, M, K, B, ldb, A, lda, C, ldc, ...).  Workspace as for
+ * hpcdnn_sgemm with M and N exchanged; lda, ldb <= 2^25 - 1024, ldc <= 2^21 - 64. */
+int hpcdnn_sgemm_cm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                       float alpha, float beta, void* ws, size_t ws_bytes, void* stream);
+
 /* Number of tile configurations, and the shape of entry `tile` (returns 0, or
  * HPCDNN_ERR_INVALID_VALUE when out of range).  Counterpart of the reference's
  * shape table (kernel/ft_sgemm/code_gen/main.py:8-16). */

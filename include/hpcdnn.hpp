@@ -23,6 +23,11 @@ inline int sgemm(int N, const float* A, const float* B, float* C, float alpha, f
 inline int sgemm(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta) {
     return hpcdnn_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, nullptr, 0, nullptr);
 }
+// the same family on its own column-major buffers: C (M x N) = alpha * A (M x K) * B (N x K)^T + beta * C with
+// lda = M, ldb = N, ldc = M, as the driver hands them to cuBLAS (kernel/ft_sgemm/sgemm.cu:111)
+inline int sgemm_cm_nt(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta) {
+    return hpcdnn_sgemm_cm_nt(M, N, K, A, M, B, N, C, M, alpha, beta, nullptr, 0, nullptr);
+}
 inline int ft_sgemm(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta,
                     hpcdnn_ft_status* status = nullptr, const hpcdnn_fault* inject = nullptr, void* ws = nullptr,
                     size_t ws_bytes = 0) {

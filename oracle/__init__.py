@@ -75,6 +75,9 @@ def _load():
     lib.oracle_gemm_f64_rows.restype = None
     lib.oracle_gemm_f64_rows.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int,
                                          C.c_float, C.c_float, ip, C.c_int, dp, dp]
+    lib.oracle_gemm_cm_nt_f64.restype = None
+    lib.oracle_gemm_cm_nt_f64.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int,
+                                          C.c_float, C.c_float, dp, dp]
     lib.oracle_gemm_max_err.restype = C.c_double
     lib.oracle_gemm_max_err.argtypes = [C.c_int, fp, C.c_int, ip, C.c_int, dp, dp]
     lib.oracle_saxpy.restype = None
@@ -166,6 +169,17 @@ def gemm_f64_rows(M, N, K, a, lda, b, ldb, c0, ldc, alpha, beta, rows=None):
     den = np.empty((nrows, N), dtype=np.float64)
     c0p = _f(c0) if c0 is not None else None
     _load().oracle_gemm_f64_rows(M, N, K, _f(a), lda, _f(b), ldb, c0p, ldc, alpha, beta, rp, nrows, _d(ref), _d(den))
+    return ref, den
+
+
+def gemm_cm_nt_f64(M, N, K, a, lda, b, ldb, c0, ldc, alpha, beta):
+    """FP64 reference and denominators of column-major C = alpha*A*B^T + beta*C (kernel/ft_sgemm/sgemm.cu:111).
+    ``a``, ``b``, ``c0`` are the flat column-major buffers (any array whose memory is that buffer); the results are
+    returned as N x M row-major arrays, i.e. the column-major M x N matrix as it lies in memory with ld = M."""
+    ref = np.empty((N, M), dtype=np.float64)
+    den = np.empty((N, M), dtype=np.float64)
+    c0p = _f(c0) if c0 is not None else None
+    _load().oracle_gemm_cm_nt_f64(M, N, K, _f(a), lda, _f(b), ldb, c0p, ldc, alpha, beta, _d(ref), _d(den))
     return ref, den
 
 

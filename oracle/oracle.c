@@ -13,6 +13,10 @@
  *
  * Parity status:
  *   oracle_cpu_gemm, oracle_gemm_f64, oracle_saxpy, oracle_sdot_*: pinned.
+ *   oracle_gemm_cm_nt_f64 (the column-major A*B^T of the ft_sgemm family):
+ *     pinned to numpy float64 on the operands viewed column-major, with
+ *     padded leading dimensions, and to a hand case that an untransposed B,
+ *     a transposed A or a row-major C each fail.
  *   oracle_sgemv_f64: pinned (numpy float64 matrix-vector products, both
  *     orientations, padded leading dimension).
  *   oracle_offline_ft_sgemm: pinned to the closed form (residual sums are 0
@@ -145,6 +149,31 @@ void oracle_gemm_f64_rows(int M, int N, int K, const float* A, int lda, const fl
             }
         }
         free(acc);
+    }
+}
+
+/* The product of the reference's column-major family in FP64:
+ *   C[m + n*ldc] = alpha * sum_k A[m + k*lda] * B[n + k*ldb] + beta * C0[m + n*ldc]
+ * (C = alpha*A*B^T + beta*C with A M x K, B N x K, C M x N, all column-major:
+ * the operand indexing of kernel/ft_sgemm/include/sgemm_huge.cuh:14-60 and the
+ * cuBLAS call cublasSgemm(N, T, M, N, K, dA, M, dB, N, dC, M) that the driver
+ * checks it against, kernel/ft_sgemm/sgemm.cu:111).  ref and denom are packed
+ * column-major M x N (ld = M): ref[m + n*M]; denom as in oracle_gemm_f64_rows. */
+void oracle_gemm_cm_nt_f64(int M, int N, int K, const float* A, int lda, const float* B, int ldb,
+                           const float* C0, int ldc, float alpha, float beta, double* ref, double* denom) {
+    #pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; ++n) {
+        for (int m = 0; m < M; ++m) {
+            double acc = 0.0, accabs = 0.0;
+            for (int k = 0; k < K; ++k) {
+                double a = (double)A[(size_t)m + (size_t)k * lda], b = (double)B[(size_t)n + (size_t)k * ldb];
+                acc += a * b;
+                accabs += fabs(a) * fabs(b);
+            }
+            double c0 = (beta != 0.0f && C0) ? (double)C0[(size_t)m + (size_t)n * ldc] : 0.0;
+            ref[(size_t)m + (size_t)n * M] = (double)alpha * acc + (double)beta * c0;
+            if (denom) denom[(size_t)m + (size_t)n * M] = fabs((double)alpha) * accabs + fabs((double)beta) * fabs(c0);
+        }
     }
 }
 

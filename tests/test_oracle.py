@@ -102,6 +102,40 @@ def test_gemm_f64_rows_matches_numpy(oracle_mod, M, N, K, lda, ldb, ldc):
     assert np.array_equal(ref2, ref[rows]) and np.array_equal(den2, den[rows])
 
 
+@pytest.mark.parametrize("M,N,K,lda,ldb,ldc", [(17, 9, 33, 20, 12, 19), (8, 24, 5, 8, 24, 8), (1, 1, 1, 1, 1, 1)])
+def test_gemm_cm_nt_matches_numpy_on_column_major_views(oracle_mod, M, N, K, lda, ldb, ldc):
+    """The column-major A*B^T of the reference's ft_sgemm family (kernel/ft_sgemm/sgemm.cu:111) against numpy float64 on
+    Fortran-ordered views of the same buffers, leading dimensions padded with NaN."""
+    rng = np.random.default_rng(4)
+    abuf = np.full((K, lda), np.nan, np.float32)   # column k of A is row k of the buffer
+    bbuf = np.full((K, ldb), np.nan, np.float32)
+    cbuf = np.full((N, ldc), np.nan, np.float32)
+    abuf[:, :M] = rng.uniform(-1, 1, (K, M))
+    bbuf[:, :N] = rng.uniform(-1, 1, (K, N))
+    cbuf[:, :M] = rng.uniform(-1, 1, (N, M))
+    A = np.ndarray((M, K), np.float32, abuf, strides=(4, 4 * lda)).astype(np.float64)   # A[m, k] = buffer[m + k*lda]
+    B = np.ndarray((N, K), np.float32, bbuf, strides=(4, 4 * ldb)).astype(np.float64)
+    C0 = np.ndarray((M, N), np.float32, cbuf, strides=(4, 4 * ldc)).astype(np.float64)
+    alpha, beta = 1.5, -0.5
+    ref, den = oracle_mod.gemm_cm_nt_f64(M, N, K, abuf, lda, bbuf, ldb, cbuf, ldc, alpha, beta)
+    want = alpha * (A @ B.T) + beta * C0                                               # M x N
+    assert np.allclose(ref.T, want, rtol=0, atol=1e-12)                                 # ref holds it column-major
+    assert np.allclose(den.T, abs(alpha) * (np.abs(A) @ np.abs(B).T) + abs(beta) * np.abs(C0), rtol=0, atol=1e-12)
+
+
+def test_gemm_cm_nt_hand_case_fails_every_transposition_mistake(oracle_mod):
+    """A = [[1,2],[3,4],[5,6]] (3 x 2), B = [[1,0],[0,1],[1,1],[2,0]] (4 x 2): A*B^T = [[1,2,3,2],[3,4,7,6],[5,6,11,10]].
+    A*B is not even defined, A^T, B untransposed or a row-major C give other numbers."""
+    A = np.array([[1, 2], [3, 4], [5, 6]], np.float32)
+    B = np.array([[1, 0], [0, 1], [1, 1], [2, 0]], np.float32)
+    abuf = np.asfortranarray(A).ravel(order="K")   # column-major memory
+    bbuf = np.asfortranarray(B).ravel(order="K")
+    ref, _ = oracle_mod.gemm_cm_nt_f64(3, 4, 2, abuf, 3, bbuf, 4, None, 3, 1.0, 0.0)
+    want = np.array([[1, 2, 3, 2], [3, 4, 7, 6], [5, 6, 11, 10]], np.float64)
+    assert np.array_equal(ref, want.T)                                                  # memory order: column by column
+    assert np.array_equal(ref.ravel(), [1, 3, 5, 2, 4, 6, 3, 7, 11, 2, 6, 10])
+
+
 def test_gemm_max_err_is_the_componentwise_criterion(oracle_mod):
     M = N = 4
     ref = np.ones((M, N))
