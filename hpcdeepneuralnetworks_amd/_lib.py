@@ -16,6 +16,7 @@ CSRC = os.path.join(_PKG, "csrc")
 OP_SGEMM = 0
 OP_SDOT = 1
 OP_FT_SGEMM = 2
+OP_FT_SGEMM_CM_NT = 5
 OP_SGEMV = 3
 OP_OFFLINE_FT_SGEMM = 4
 OFFLINE_FT_PANEL_K = 256
@@ -41,6 +42,7 @@ EXPORTS = (
     "hpcdnn_ft_sgemm_ex",
     "hpcdnn_ft_sgemm_static",
     "hpcdnn_ft_sgemm_opt",
+    "hpcdnn_ft_sgemm_cm_nt",
     "hpcdnn_ft_check_tile_info",
     "hpcdnn_ft_num_check_tiles",
     "hpcdnn_ft_tile_info",
@@ -129,6 +131,8 @@ def lib():
     L.hpcdnn_ft_sgemm.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp, sz, vp]
     L.hpcdnn_ft_sgemm_static.restype = i
     L.hpcdnn_ft_sgemm_static.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(Fault), vp, vp]
+    L.hpcdnn_ft_sgemm_cm_nt.restype = i
+    L.hpcdnn_ft_sgemm_cm_nt.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(FtOptions), vp, vp, sz, vp]
     L.hpcdnn_ft_sgemm_opt.restype = i
     L.hpcdnn_ft_sgemm_opt.argtypes = [i, i, i, fp, i, fp, i, fp, i, f, f, f, C.POINTER(FtOptions), vp, vp, sz, vp]
     L.hpcdnn_ft_check_tile_info.restype = i

@@ -183,6 +183,40 @@ FT_GRAN_TILE, FT_GRAN_WAVE = _lib.FT_GRAN_TILE, _lib.FT_GRAN_WAVE
 FT_STATIC_SCRATCH_BYTES = 4 << 20
 
 
+def ft_cm_nt_workspace_bytes(M: int, N: int, K: int) -> int:
+    return int(_lib.lib().hpcdnn_workspace_bytes(_lib.OP_FT_SGEMM_CM_NT, M, N, K))
+
+
+def ft_sgemm_cm_nt(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
+                   ws: torch.Tensor, tau: float = 0.0, status: torch.Tensor | None = None, tile_class: int = 0,
+                   granularity: int = 0, check_interval: int = 0, faults=None) -> None:
+    """ABFT GEMM on the column-major buffers of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)``
+    (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21): ``C (M x N) = alpha*A (M x K) @ B (N x K).T + beta*C``.  The tensors hold
+    the column-major matrices as their row-major transposes (``A`` K x M, ``B`` K x N, ``C`` N x M).  Tiles, status
+    records and fault coordinates are those of ``ft_sgemm(N, M, K, ...)`` on the row-major ``C^T``.  ``ws`` (required):
+    ``ft_cm_nt_workspace_bytes(M, N, K)`` bytes."""
+    pa, lda = _matrix(A, K, M, "A")
+    pb, ldb = _matrix(B, K, N, "B")
+    pc, ldc = _matrix(Cm, N, M, "C")
+    L = _lib.lib()
+    sp = None
+    if status is not None:
+        need = 8 * L.hpcdnn_ft_num_check_tiles(tile_class, granularity, N, M)
+        if not (status.is_cuda and status.dtype == torch.int32 and status.numel() >= need and status.is_contiguous()):
+            raise HpcdnnError(f"status must be a contiguous int32 GPU tensor with >= {need} elements")
+        sp = status.data_ptr()
+    every = list(faults or [])
+    if len(every) > _lib.FT_MAX_FAULTS:
+        raise HpcdnnError(f"at most {_lib.FT_MAX_FAULTS} faults per call")
+    opt = _lib.FtOptions()
+    opt.tile_class, opt.granularity, opt.check_interval, opt.n_faults = tile_class, granularity, check_interval, len(every)
+    for i, fl in enumerate(every):
+        opt.faults[i] = _lib.FaultAt(int(fl[0]), int(fl[1]), int(fl[2]), float(fl[3]), int(fl[4]) if len(fl) > 4 else 0)
+    wp, wb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
+    check(L.hpcdnn_ft_sgemm_cm_nt(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, C.byref(opt), sp, wp, wb, _stream()),
+          "hpcdnn_ft_sgemm_cm_nt")
+
+
 def ft_sgemm_static(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
                     tau: float = 0.0, fault=None, status: torch.Tensor | None = None) -> None:
     """``ft_sgemm`` with the library's own fixed scratch array instead of a workspace: allocates nothing; refuses

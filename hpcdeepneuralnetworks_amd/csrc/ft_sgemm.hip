@@ -328,6 +328,94 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
     return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws, ws_bytes, 0, stream);
 }
 
+// ---- ABFT SGEMM on the reference family's own column-major buffers.  Read row by row, column-major
+// C = alpha * A * B^T + beta * C is C^T (N x M) = (B^T)^T * A^T with both operands K-major; the ABFT kernels take their
+// left operand row by row (their checksum arithmetic works on its staging registers), so that operand, the memory of
+// B seen as K rows of N, is first transposed into the workspace: one pass over B, 8 N K bytes of traffic beside the
+// product's 2 M N K flop.
+// dst (cols x rows) = src (rows x cols)^T, 64 x 64 blocks through LDS.  VEC: every row of src and dst starts on a
+// 16-byte boundary, so both sides move 16 bytes per lane (a wave covers four 256-byte row segments per instruction);
+// otherwise one float per lane.  block[r][c] with a row stride of 65 words keeps the transposed reads (and the word
+// writes of the 16-byte loads) on 64 different banks.
+template <bool VEC>
+__global__ __launch_bounds__(256) void transpose_kernel(int rows, int cols, const float* __restrict__ src, int ld_src,
+                                                        float* __restrict__ dst, int ld_dst) {
+    __shared__ float block[64][65];
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    if constexpr (VEC) {
+        const int g = threadIdx.x & 15, q = threadIdx.x >> 4;  // 16 groups of four columns, 16 rows per pass
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = q + 16 * i, c = 4 * g;
+            v4f v = {0.f, 0.f, 0.f, 0.f};
+            if (r0 + r < rows && c0 + c < cols) {  // cols % 4 == 0: a group is inside or outside as a whole
+                v = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src + static_cast<int64_t>(r0 + r) * ld_src + c0 + c));
+            }
+            block[r][c] = v.x;
+            block[r][c + 1] = v.y;
+            block[r][c + 2] = v.z;
+            block[r][c + 3] = v.w;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = q + 16 * i, r = 4 * g;  // row c of dst, its columns r .. r + 3
+            if (c0 + c < cols && r0 + r < rows) {
+                const v4f v = {block[r][c], block[r + 1][c], block[r + 2][c], block[r + 3][c]};
+                *reinterpret_cast<v4f*>(dst + static_cast<int64_t>(c0 + c) * ld_dst + r0 + r) = v;
+            }
+        }
+    } else {
+        const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int r = r0 + ty + 4 * i, c = c0 + tx;
+            block[ty + 4 * i][tx] = (r < rows && c < cols) ? __builtin_nontemporal_load(src + static_cast<int64_t>(r) * ld_src + c) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = c0 + ty + 4 * i, r = r0 + tx;
+            if (c < cols && r < rows) dst[static_cast<int64_t>(c) * ld_dst + r] = block[tx][ty + 4 * i];
+        }
+    }
+}
+
+namespace hpcdnn {
+static size_t round_up_256(size_t b) { return (b + 255) / 256 * 256; }
+size_t ft_cm_nt_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return round_up_256(static_cast<size_t>(N) * K * sizeof(float)) + ft_workspace_bytes(N, M, K);
+}
+}  // namespace hpcdnn
+
+extern "C" int hpcdnn_ft_sgemm_cm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                                     float alpha, float beta, float tau, const hpcdnn_ft_options* opt, hpcdnn_ft_status* status,
+                                     void* ws, size_t ws_bytes, void* stream) {
+    // the row-major problem: C^T (N x M, ldc) = Bt^T (N x K) * At (K x M, lda), Bt = the memory of B (K x N, ldb)
+    int rc = check_gemm_args(N, M, K, B, ldb, A, lda, C, ldc, true);
+    if (rc != HPCDNN_OK) return rc;
+    if (M == 0 || N == 0) return HPCDNN_OK;
+    hpcdnn_ft_options none{};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (K == 0) return run_ft_sgemm(N, M, 0, nullptr, 1, nullptr, M, C, ldc, alpha, beta, tau, opt ? *opt : none, status, nullptr, 0, s);
+    const size_t copy_bytes = round_up_256(static_cast<size_t>(N) * K * sizeof(float));
+    if (!ws || ws_bytes < copy_bytes) return HPCDNN_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(ws) & 15u) return HPCDNN_ERR_INVALID_VALUE;
+    float* bt = static_cast<float*>(ws);
+    const dim3 blocks(static_cast<unsigned>(ceil_div(N, 64)), static_cast<unsigned>(ceil_div(K, 64)));
+    // (src: K rows of N, dst: N rows of K in the 16-byte aligned workspace)
+    if (N % 4 == 0 && K % 4 == 0 && ldb % 4 == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0)
+        transpose_kernel<true><<<blocks, 256, 0, s>>>(K, N, B, ldb, bt, K);
+    else
+        transpose_kernel<false><<<blocks, 256, 0, s>>>(K, N, B, ldb, bt, K);
+    rc = launch_status();
+    if (rc != HPCDNN_OK) return rc;
+    const size_t rest = ws_bytes - copy_bytes;
+    return run_ft_sgemm(N, M, K, bt, K, A, lda, C, ldc, alpha, beta, tau, opt ? *opt : none, status,
+                        rest ? static_cast<unsigned char*>(ws) + copy_bytes : nullptr, rest, s);
+}
+
 // ---- ABFT SGEMM for callers that can neither allocate nor pass a workspace: the checksum vectors (and, when they
 // fit, the K slices of a partial last round) live in a fixed device array of this library.  Every device the
 // library runs on holds its own copy of the array at its own address, looked up once per device.

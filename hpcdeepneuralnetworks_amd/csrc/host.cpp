@@ -8,6 +8,7 @@ namespace hpcdnn {
 size_t sdot_workspace_bytes();
 size_t sgemm_workspace_bytes(int M, int N, int K);
 size_t ft_workspace_bytes(int M, int N, int K);
+size_t ft_cm_nt_workspace_bytes(int M, int N, int K);
 size_t sgemv_workspace_bytes(int M, int N);
 size_t offline_ft_workspace_bytes(int M, int N, int K);
 }  // namespace hpcdnn
@@ -28,6 +29,7 @@ extern "C" size_t hpcdnn_workspace_bytes(int op, int M, int N, int K) {
         case HPCDNN_OP_SGEMM: return hpcdnn::sgemm_workspace_bytes(M, N, K);
         case HPCDNN_OP_SDOT: return hpcdnn::sdot_workspace_bytes();
         case HPCDNN_OP_FT_SGEMM: return hpcdnn::ft_workspace_bytes(M, N, K);
+        case HPCDNN_OP_FT_SGEMM_CM_NT: return hpcdnn::ft_cm_nt_workspace_bytes(M, N, K);
         case HPCDNN_OP_SGEMV: return hpcdnn::sgemv_workspace_bytes(M, N);
         case HPCDNN_OP_OFFLINE_FT_SGEMM: return hpcdnn::offline_ft_workspace_bytes(M, N, K);
         default: return 0;

@@ -49,6 +49,7 @@ extern "C" {
 #define HPCDNN_OP_FT_SGEMM 2
 #define HPCDNN_OP_SGEMV 3            /* M, N as passed to hpcdnn_sgemv; only trans = 1 uses a workspace */
 #define HPCDNN_OP_OFFLINE_FT_SGEMM 4
+#define HPCDNN_OP_FT_SGEMM_CM_NT 5     /* M, N, K as passed to hpcdnn_ft_sgemm_cm_nt */
 
 /* K panel of hpcdnn_offline_ft_sgemm (the reference checks every 256 columns,
  * kernel/ft_sgemm/include/baseline_ft_sgemm.cuh:3). */
@@ -266,6 +267,25 @@ typedef struct hpcdnn_ft_options {
 int hpcdnn_ft_sgemm_opt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                         float alpha, float beta, float tau, const hpcdnn_ft_options* opt, hpcdnn_ft_status* status,
                         void* ws, size_t ws_bytes, void* stream);
+/* hpcdnn_ft_sgemm_opt on the reference family's own COLUMN-MAJOR buffers:
+ * C (M x N, ldc >= M) = alpha * A (M x K, lda >= M) * B (N x K, ldb >= N)^T +
+ * beta * C, the buffers, argument order and meaning of
+ * ft_sgemm_huge<<<...>>>(M,N,K,A,B,C,alpha,beta)
+ * (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21, launched at
+ * kernel/ft_sgemm/sgemm.cu:159-165).  It runs as the row-major problem
+ * C^T (N x M) = (B^T)^T * A^T: tiles, check tiles, status records and fault
+ * coordinates are those of hpcdnn_ft_sgemm_opt(N, M, K, ...), i.e. `row` counts
+ * along N (the columns of the column-major C) and `col` along M; use
+ * hpcdnn_ft_num_check_tiles(tile_class, granularity, N, M) records.  `ws` is
+ * REQUIRED (K > 0): hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM_CM_NT, M, N, K)
+ * bytes, 16-byte aligned, no initialisation; its first N*K floats receive the
+ * transposed copy of B that the ABFT kernels read row by row, the rest is the
+ * workspace of hpcdnn_ft_sgemm_opt.  At least the copy must fit
+ * (HPCDNN_ERR_WORKSPACE otherwise); with no room beyond it the checksum
+ * vectors are formed in the main loop.  `opt` may be NULL. */
+int hpcdnn_ft_sgemm_cm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                          float alpha, float beta, float tau, const hpcdnn_ft_options* opt, hpcdnn_ft_status* status,
+                          void* ws, size_t ws_bytes, void* stream);
 int hpcdnn_ft_check_tile_info(int tile_class, int granularity, int* cm, int* cn);
 int hpcdnn_ft_num_check_tiles(int tile_class, int granularity, int M, int N);
 int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N);
