@@ -255,6 +255,25 @@ def main() -> int:
             del a, b, c, ws
         extras["sgemm_irregular_gflops"] = irregular
 
+        # the reference family's column-major C = A * B^T (kernel/ft_sgemm/sgemm.cu:111) on its own buffers: plain SGEMM
+        # reads the K-major operands in place, the ABFT entry point first transposes one of them into its workspace
+        cm = {}
+        for m in (1024, 4096, 6144):
+            a, b, c = operands(m, m, m, 17)   # square: the same tensors serve as the K x M, K x N and N x M buffers
+            ws = blas.workspace(max(blas.sgemm_workspace_bytes(m, m, m), 4))
+            ms = median_timed(lambda: blas.sgemm_cm_nt(m, m, m, a, b, c, 1.0, 0.0, ws=ws), st, wu)
+            ms_lt = median_timed(lambda: torch.matmul(b.t(), a, out=c), st, wu)   # C^T = B^T^T A^T on the same memory
+            cm[str(m)] = {"sgemm_cm_nt_gflops": round(2.0 * m ** 3 / ms / 1e6, 1), "hipblaslt_via_torch_tn_gflops": round(2.0 * m ** 3 / ms_lt / 1e6, 1)}
+            if m == 4096:
+                ft_ws_cm = blas.workspace(blas.ft_cm_nt_workspace_bytes(m, m, m))
+                status_cm = blas.ft_status_alloc(m, m)
+                ms_ft = median_timed(lambda: blas.ft_sgemm_cm_nt(m, m, m, a, b, c, 1.0, 0.0, ft_ws_cm, status=status_cm), st, wu)
+                cm[str(m)]["ft_sgemm_cm_nt_gflops"] = round(2.0 * m ** 3 / ms_ft / 1e6, 1)
+                cm[str(m)]["ft_overhead_pct_vs_sgemm_cm_nt"] = round((ms_ft - ms) / ms * 100.0, 2)
+                del ft_ws_cm, status_cm
+            del a, b, c, ws
+        extras["column_major_a_bt"] = cm
+
         # ---- ABFT at 4096^3: overhead vs plain SGEMM and the seeded single-fault campaign
         m = 4096
         a, b, c = operands(m, m, m, 20)

@@ -51,6 +51,8 @@ inline bool needs_edge(const GemmArgs& a, int bm, int bn, int bk) {
 // The kernel of tile `tile` (bm x bn, as a cross-check of the index) for a transposed left operand, or nullptr when
 // the tile has none (sgemm_ta.hip).
 void (*sgemm_ta_kernel(int tile, int bm, int bn, bool edge))(const GemmArgs);
+// Its persistent kernel (beta == 0 or beta != 0 variant), or nullptr; only tiles whose untransposed kernel has one
+void (*sgemm_ta_persistent_kernel(int tile, int bm, int bn, bool beta))(const GemmArgs);
 
 // Kernels that use more than the default 64 KiB of LDS must opt in once per device.
 inline int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {

@@ -290,8 +290,8 @@ static RowSplit choose_row_split(int M, int N, int K, int cus) {
     return best;
 }
 
-// ta: A is given transposed (K x M row-major).  Those kernels exist for every tile but the 32 x 32 one and have no
-// persistent variant; everything else (plans, splits, reductions) is shared.
+// ta: A is given transposed (K x M row-major).  Those kernels exist for every tile but the 32 x 32 one (sgemm_ta.hip);
+// everything else (plans, splits, reductions) is shared.
 static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                      float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split, hipStream_t stream,
                      bool ta = false) {
@@ -388,9 +388,11 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     dim3 grid(a.full_tiles + tail_tiles * a.tail_split, 1, split);
     // Several rounds of whole tiles written straight to C: one persistent workgroup per CU walks its tiles as one
     // stream of K steps (same bits; see sgemm_persistent_kernel.h for what it saves)
-    const int persistent = (split == 1 && tail_tiles == 0 && ldc <= kMaxLdc && !ta) ? persistent_grid(cfg, M, N, K, device_cus()) : 0;
-    if (persistent > 0 && (beta == 0.f ? cfg.persistent : cfg.persistent_beta)) {
-        fn = beta == 0.f ? cfg.persistent : cfg.persistent_beta;
+    const int persistent = (split == 1 && tail_tiles == 0 && ldc <= kMaxLdc) ? persistent_grid(cfg, M, N, K, device_cus()) : 0;
+    void (*const pfn)(const GemmArgs) = ta ? sgemm_ta_persistent_kernel(tile, cfg.bm, cfg.bn, beta != 0.f)
+                                           : beta == 0.f ? cfg.persistent : cfg.persistent_beta;
+    if (persistent > 0 && pfn) {
+        fn = pfn;
         grid = dim3(persistent, 1, 1);
     }
     rc = enable_lds(fn, cfg.lds_bytes);

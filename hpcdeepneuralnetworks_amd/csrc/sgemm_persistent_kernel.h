@@ -25,7 +25,8 @@ namespace hpcdnn {
 
 constexpr int kPersistDripSteps = 8;  // K steps over which a finished tile's stores are spread
 
-template <int BM, int BN, int WGM, int WGN, bool BETA, int IMM = 0, int PER_CU = 1>
+// TA: the left operand is given transposed (K x M row-major), staged as in sgemm_kernel.h's TA kernels.
+template <int BM, int BN, int WGM, int WGN, bool BETA, int IMM = 0, int PER_CU = 1, bool TA = false>
 __global__ __launch_bounds__(WGM * WGN * kWave, PER_CU) void sgemm_persistent_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
     constexpr int kThreads = WGM * WGN * kWave;
@@ -71,8 +72,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, PER_CU) void sgemm_persistent_ke
     origin(tile, m0, n0);
 
     // ---- global -> register staging (two sets: K step t+1 waits in one while t+2 is on its way)
+    const int64_t a_step = TA ? static_cast<int64_t>(BK) * p.lda : BK;
     const int64_t b_step = static_cast<int64_t>(BK) * p.ldb;
-    const float* a_base = p.A + static_cast<int64_t>(m0) * p.lda;  // of the K step the next load fetches
+    auto a_origin = [&](int m) { return TA ? p.A + m : p.A + static_cast<int64_t>(m) * p.lda; };
+    const float* a_base = a_origin(m0);  // of the K step the next load fetches
     const float* b_base = p.B + n0;
     const float* a_next = a_base;  // where the stream goes on after this tile's last K step (itself: harmless re-reads)
     const float* b_next = b_base;
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, PER_CU) void sgemm_persistent_ke
         if (t < total) {
             int nm0, nn0;
             origin(t, nm0, nn0);
-            a_next = p.A + static_cast<int64_t>(nm0) * p.lda;
+            a_next = a_origin(nm0);
             b_next = p.B + nn0;
         }
     };
@@ -92,9 +95,15 @@ __global__ __launch_bounds__(WGM * WGN * kWave, PER_CU) void sgemm_persistent_ke
 #pragma unroll
     for (int s = 0; s < A_SLOTS; ++s) {
         const int idx = tid + s * kThreads;
-        const int row = idx / A_V4_PER_ROW, kc = (idx % A_V4_PER_ROW) * 4;
-        a_voff[s] = (row * p.lda + kc) * 4;
-        a_lds[s] = row * AS + kc;
+        if constexpr (TA) {
+            const int k = (idx / 4) % BK, m = ((idx / (4 * BK)) * 4 + idx % 4) * 4;  // four m of one k (sgemm_kernel.h)
+            a_voff[s] = (k * p.lda + m) * 4;
+            a_lds[s] = m * AS + k;
+        } else {
+            const int row = idx / A_V4_PER_ROW, kc = (idx % A_V4_PER_ROW) * 4;
+            a_voff[s] = (row * p.lda + kc) * 4;
+            a_lds[s] = row * AS + kc;
+        }
     }
 #pragma unroll
     for (int s = 0; s < B_SLOTS; ++s) {
@@ -112,14 +121,23 @@ __global__ __launch_bounds__(WGM * WGN * kWave, PER_CU) void sgemm_persistent_ke
     // after the loads of a K step: on to the next one, which after the tile's last step is the next tile's first
     auto gload_advance = [&]() {
         const bool more = k_loaded + BK < p.K;
-        a_base = more ? a_base + BK : a_next;
+        a_base = more ? a_base + a_step : a_next;
         b_base = more ? b_base + b_step : b_next;
         k_loaded = more ? k_loaded + BK : 0;
     };
     auto lstore1 = [&](auto slot, auto part, int stage) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
-        if constexpr (P < A_SLOTS) *reinterpret_cast<v4f*>(As + stage * A_STAGE + a_lds[P]) = ra[S][P];
-        else *reinterpret_cast<v4f*>(Bs + stage * B_STAGE + b_lds[P - A_SLOTS]) = rb[S][P - A_SLOTS];
+        if constexpr (P < A_SLOTS && TA) {
+            float* const dst = As + stage * A_STAGE + a_lds[P];
+            dst[0] = ra[S][P].x;
+            dst[AS] = ra[S][P].y;
+            dst[2 * AS] = ra[S][P].z;
+            dst[3 * AS] = ra[S][P].w;
+        } else if constexpr (P < A_SLOTS) {
+            *reinterpret_cast<v4f*>(As + stage * A_STAGE + a_lds[P]) = ra[S][P];
+        } else {
+            *reinterpret_cast<v4f*>(Bs + stage * B_STAGE + b_lds[P - A_SLOTS]) = rb[S][P - A_SLOTS];
+        }
     };
 
     // ---- LDS -> fragment registers -> MFMA

@@ -134,6 +134,36 @@ def test_large_whole_tile_shape_matches_untransposed_bits(blas, oracle_mod):
     assert oracle_mod.gemm_max_err(N, got, N, ref, den) <= TOL
 
 
+@pytest.mark.parametrize("M,N,K,tile", [(2176, 4608, 320, 7), (4352, 2304, 192, 0), (3264, 4608, 320, 5), (2176, 4608, 320, 1)])
+@pytest.mark.parametrize("alpha,beta", [(1.5, 0.0), (1.0, -1.5)])
+def test_persistent_kernels_on_several_rounds_of_whole_tiles(blas, oracle_mod, M, N, K, tile, alpha, beta):
+    """More whole tiles than CUs and an even number (>= 10) of K steps: the persistent kernels of the 256x128, 128x256,
+    192x256 (beta == 0 only) and 128x128 tiles run, here with the transposed staging.  Same bits as the 128x64
+    tile-per-workgroup kernel on the untransposed operand; padded ldat / ldc with NaN padding, NaN in C when beta == 0."""
+    dev = "cuda"
+    ldat, ldc = M + 8, N + 24
+    da, db = torch.empty(M, K, device=dev), torch.empty(K, N, device=dev)
+    blas.fill_uniform_matrix(da, M, K, 51)
+    blas.fill_uniform_matrix(db, K, N, 52)
+    dat = torch.full((K, ldat), float("nan"), device=dev)
+    dat[:, :M] = da.t()
+    c0 = torch.full((M, ldc), float("nan"), device=dev)
+    if beta != 0.0:
+        c0[:, :N] = torch.rand(M, N, device=dev) * 2 - 1
+    c1, c2 = c0.clone(), c0.clone()
+    blas.sgemm_tn(M, N, K, dat, db, c1, alpha, beta, tile=tile, split_k=1)
+    blas.sgemm(M, N, K, da, db, c2, alpha, beta, tile=2, split_k=1)
+    assert torch.equal(c1[:, :N], c2[:, :N])
+    assert not torch.isnan(c1[:, :N]).any()
+    assert torch.isnan(c1[:, N:]).all()
+    rows = np.array([0, 1, M // 2 + 3, M - 1], np.int32)
+    a, b = oracle_mod.fill_uniform_matrix(M, K, 51), oracle_mod.fill_uniform_matrix(K, N, 52)
+    c0h = np.ascontiguousarray(c0[:, :N].cpu().numpy()) if beta != 0.0 else None
+    ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, K, b, N, c0h, N, alpha, beta, rows=rows)
+    got = np.ascontiguousarray(c1[torch.from_numpy(rows).long().cuda(), :N].cpu().numpy())
+    assert oracle_mod.gemm_max_err(N, got, N, ref, den) <= TOL
+
+
 @pytest.mark.parametrize("M,N,K,pad", [(128, 128, 128, (0, 0, 0)), (1024, 1024, 1024, (0, 0, 0)), (300, 170, 90, (4, 7, 2)), (17, 400, 33, (1, 0, 5)),
                                       (1, 1, 1, (0, 0, 0)), (513, 64, 2050, (3, 3, 3))])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, -1.5)])
