@@ -117,7 +117,8 @@ int run_sgemm(int start, int end, int gap) {
 struct Series {
     int number;        // the reference's kernel_number (kernel/ft_sgemm/sgemm.cu:186)
     const char* name;  // the reference's series name (:187-188) where a counterpart exists
-    int kind;          // 0 plain SGEMM, 1 offline ABFT, 2 ABFT without workspace, 3 ABFT with workspace, 4 wave-tile ABFT
+    int kind;          // 0 plain SGEMM, 1 offline ABFT, 2 ABFT without workspace, 3 ABFT with workspace, 4 wave-tile ABFT,
+                       // 5 / 6 plain SGEMM / ABFT on column-major operands
     int tile;          // plain SGEMM: row of the tile table, -1 = chosen by the library; ABFT: tile class
 };
 
@@ -143,6 +144,10 @@ const Series kSeries[] = {
     {19, "abft_kernel_huge_workspace", 3, 0},
     {20, "abft_kernel_large_workspace", 3, 1},
     {21, "abft_kernel_wide_workspace", 3, 2},
+    // the reference's own operand layout, column-major C = A * B^T (kernel/ft_sgemm/sgemm.cu:111): the same device
+    // buffers read as the column-major n x K, n x K and n x n matrices
+    {22, "hpcdnn_sgemm_column_major", 5, -1},
+    {23, "abft_kernel_huge_column_major", 6, 0},
 };
 
 int run_ft_sgemm(int start, int end, int gap, int first, int last) {
@@ -160,6 +165,10 @@ int run_ft_sgemm(int start, int end, int gap, int first, int last) {
         const size_t o = hpcdnn_workspace_bytes(HPCDNN_OP_OFFLINE_FT_SGEMM, n, n, K);
         if (f > ft_ws_bytes) ft_ws_bytes = f;
         if (o > off_ws_bytes) off_ws_bytes = o;
+    }
+    for (int n = start; n <= end; n += gap) {  // the column-major ABFT series adds room for its transposed operand
+        const size_t f = hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM_CM_NT, n, n, K);
+        if (f > ft_ws_bytes) ft_ws_bytes = f;
     }
     void *ft_ws = nullptr, *off_ws = nullptr;
     HIP_OK(hipMalloc(&ft_ws, ft_ws_bytes ? ft_ws_bytes : 16));
@@ -225,6 +234,19 @@ int run_ft_sgemm(int start, int end, int gap, int first, int last) {
                     opt.granularity = HPCDNN_FT_GRAN_WAVE;
                     perf = timed_gflops(flop, kNumTests, [&] {
                         LIB_OK(hpcdnn_ft_sgemm_opt(n, n, K, a, K, b, n, c, n, alpha, beta, 0.f, &opt, nullptr, ft_ws, ft_ws_bytes, nullptr));
+                    });
+                    break;
+                }
+                case 5:
+                    perf = timed_gflops(flop, kNumTests, [&] {
+                        LIB_OK(hpcdnn_sgemm_cm_nt(n, n, K, a, n, b, n, c, n, alpha, beta, gemm_ws, gemm_ws_bytes, nullptr));
+                    });
+                    break;
+                case 6: {
+                    hpcdnn_ft_options opt{};
+                    opt.tile_class = sr.tile;
+                    perf = timed_gflops(flop, kNumTests, [&] {
+                        LIB_OK(hpcdnn_ft_sgemm_cm_nt(n, n, K, a, n, b, n, c, n, alpha, beta, 0.f, &opt, nullptr, ft_ws, ft_ws_bytes, nullptr));
                     });
                     break;
                 }

@@ -23,7 +23,7 @@ def _floats(text):
 
 
 def test_ft_sgemm_series_lines():
-    out = _run("ft_sgemm", 256, 768, 256, 0, 21)
+    out = _run("ft_sgemm", 256, 768, 256, 0, 23)
     assert out.startswith("     256|     512|     768|")
     assert "finish verified!" in out
     series = dict(re.findall(r"^(\w+) = th\.as_tensor\(\[(.*)\]\)$", out, flags=re.M))
@@ -31,7 +31,8 @@ def test_ft_sgemm_series_lines():
                             "kernel_sgemm_tall", "kernel_sgemm_wide", "kernel_sgemm_huge", "abft_baseline",
                             "abft_kernel_medium", "abft_kernel_large", "abft_kernel_tall", "abft_kernel_wide",
                             "abft_kernel_huge", "warp_abft_kernel", "abft_kernel_huge_workspace",
-                            "abft_kernel_large_workspace", "abft_kernel_wide_workspace"]
+                            "abft_kernel_large_workspace", "abft_kernel_wide_workspace",
+                            "hpcdnn_sgemm_column_major", "abft_kernel_huge_column_major"]
     for name, body in series.items():
         vals = _floats(body)
         assert len(vals) == 3 and all(v > 0 for v in vals), (name, body)
