@@ -47,7 +47,7 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline SGEMM line only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--ft-launches", type=int, default=1000, help="launches of the ABFT fault campaign")
-    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "sgemm_1024", "sgemm_lowk", "ft_sgemm", "ft_sgemm_fused", "ft_sgemm_wave", "offline_ft", "saxpy", "sdot", "copy",
+    ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "sgemm_1024", "sgemm_lowk", "sgemm_cm_nt", "ft_sgemm_cm_nt", "ft_sgemm", "ft_sgemm_fused", "ft_sgemm_wave", "offline_ft", "saxpy", "sdot", "copy",
                              "sgemv_n", "sgemv_t"],
                     help="run one kernel only for --steps launches (for profiling with rocprofv3) and print a short line")
     args = ap.parse_args()
@@ -109,6 +109,20 @@ def main() -> int:
             a, b, c = operands(mm, mm, kk, 10)
             fn = lambda: blas.sgemm(mm, mm, kk, a, b, c, 1.0, 0.0)
             work, unit = 2.0 * mm * mm * kk, "GFLOP/s"
+        elif args.kernel == "sgemm_cm_nt":
+            # the reference family's column-major C = A * B^T at the headline size (square: the tensors serve as the
+            # K x M, K x N and N x M buffers)
+            m = 6144
+            a, b, c = operands(m, m, m, 10)
+            fn = lambda: blas.sgemm_cm_nt(m, m, m, a, b, c, 1.0, 0.0)
+            work, unit = 2.0 * m ** 3, "GFLOP/s"
+        elif args.kernel == "ft_sgemm_cm_nt":
+            m = 4096
+            a, b, c = operands(m, m, m, 20)
+            status = blas.ft_status_alloc(m, m)
+            ft_ws = blas.workspace(blas.ft_cm_nt_workspace_bytes(m, m, m))
+            fn = lambda: blas.ft_sgemm_cm_nt(m, m, m, a, b, c, 1.0, 0.0, ft_ws, tau=blas.ft_default_tau(m), status=status)
+            work, unit = 2.0 * m ** 3, "GFLOP/s"
         elif args.kernel == "ft_sgemm":
             m = 4096
             a, b, c = operands(m, m, m, 20)
