@@ -20,12 +20,6 @@ size_t ft_workspace_bytes(int M, int N, int K);
 //
 // Wave-tile granularity (the counterpart of ft_sgemm_huge_warp.cuh / ft_sgemm_huge_thread.cuh) runs the FT = 2 kernel
 // with one checksum pair per wave tile: the tile a wave of the workspace kernel owns, (bm / wgm) x (bn / wgn).
-struct FtKernel {
-    void (*plain)(const GemmArgs);
-    void (*edge)(const GemmArgs);
-    int threads;
-    size_t lds;
-};
 typedef void (*EncodeFn)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int, int);
 struct FtClass {
     int bm, bn;
@@ -113,10 +107,12 @@ static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
     return tile_mode > wave_mode ? tile_mode : wave_mode;
 }
 
+// ta: A is given transposed (K x M row-major, lda >= M); those kernels read the checksum vectors from the workspace,
+// which is then required
 static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                         float alpha, float beta, float tau, const hpcdnn_ft_options& opt, hpcdnn_ft_status* status, void* ws,
-                        size_t ws_bytes, hipStream_t s) {
-    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
+                        size_t ws_bytes, hipStream_t s, bool ta = false) {
+    int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc, ta);
     if (rc != HPCDNN_OK) return rc;
     if (opt.tile_class < 0 || opt.tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
     if (opt.granularity != HPCDNN_FT_GRAN_TILE && opt.granularity != HPCDNN_FT_GRAN_WAVE) return HPCDNN_ERR_INVALID_VALUE;
@@ -129,7 +125,7 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     const bool cadence = opt.check_interval > 0 && opt.check_interval < K;
     if (cadence && (wave || !fc.pre_cad.plain)) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
-    if (wave && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
+    if ((wave || ta) && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
 
     GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, fc.bm, fc.bn);
     // tau > 0: absolute; tau == 0: the absolute default for unit-range data; tau < 0: scaled to the data, the
@@ -177,11 +173,22 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         a.enc_b = enc_b;
         const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
         const int b_blocks = static_cast<int>(ceil_div(N, 128));  // the pre-pass walks B in blocks of 128 columns
-        hipLaunchKernelGGL(wave ? fc.encode_wave : fc.encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(1024), 0, s, M, N, K,
-                           A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
+        if (ta) {
+            // the B half of the pre-pass as it is (no row groups), the A half by the kernel that walks A^T
+            const EncodeAtFn enc_at = ft_ta_encode(cm);
+            if (!enc_at) return HPCDNN_ERR_INVALID_VALUE;
+            hipLaunchKernelGGL(enc_at, dim3(static_cast<unsigned>(ceil_div(a.enc_ld, 64)), row_groups), dim3(256), 0, s, M, K, A, lda,
+                               enc_a, a.enc_ld);
+            rc = launch_status();
+            if (rc != HPCDNN_OK) return rc;
+        }
+        hipLaunchKernelGGL(wave ? fc.encode_wave : fc.encode, dim3(k_blocks * ((ta ? 0 : row_groups) + b_blocks)), dim3(1024), 0, s, M, N, K,
+                           A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, ta ? 0 : row_groups, col_groups);
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;
-        const FtKernel& k = wave ? fc.wave : (cadence ? fc.pre_cad : fc.pre);
+        const FtKernel ta_k = ta ? ft_ta_kernel(opt.tile_class, fc.bm, fc.bn, wave ? 1 : (cadence ? 2 : 0)) : FtKernel{nullptr, nullptr, 0, 0};
+        if (ta && !ta_k.plain) return HPCDNN_ERR_INVALID_VALUE;
+        const FtKernel& k = ta ? ta_k : wave ? fc.wave : (cadence ? fc.pre_cad : fc.pre);
         void (*fn)(const GemmArgs) = edge ? k.edge : k.plain;
         rc = enable_lds(fn, k.lds);
         if (rc != HPCDNN_OK) return rc;
@@ -329,91 +336,18 @@ extern "C" int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, con
 }
 
 // ---- ABFT SGEMM on the reference family's own column-major buffers.  Read row by row, column-major
-// C = alpha * A * B^T + beta * C is C^T (N x M) = (B^T)^T * A^T with both operands K-major; the ABFT kernels take their
-// left operand row by row (their checksum arithmetic works on its staging registers), so that operand, the memory of
-// B seen as K rows of N, is first transposed into the workspace: one pass over B, 8 N K bytes of traffic beside the
-// product's 2 M N K flop.
-// dst (cols x rows) = src (rows x cols)^T, 64 x 64 blocks through LDS.  VEC: every row of src and dst starts on a
-// 16-byte boundary, so both sides move 16 bytes per lane (a wave covers four 256-byte row segments per instruction);
-// otherwise one float per lane.  block[r][c] with a row stride of 65 words keeps the transposed reads (and the word
-// writes of the 16-byte loads) on 64 different banks.
-template <bool VEC>
-__global__ __launch_bounds__(256) void transpose_kernel(int rows, int cols, const float* __restrict__ src, int ld_src,
-                                                        float* __restrict__ dst, int ld_dst) {
-    __shared__ float block[64][65];
-    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    if constexpr (VEC) {
-        const int g = threadIdx.x & 15, q = threadIdx.x >> 4;  // 16 groups of four columns, 16 rows per pass
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = q + 16 * i, c = 4 * g;
-            v4f v = {0.f, 0.f, 0.f, 0.f};
-            if (r0 + r < rows && c0 + c < cols) {  // cols % 4 == 0: a group is inside or outside as a whole
-                v = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src + static_cast<int64_t>(r0 + r) * ld_src + c0 + c));
-            }
-            block[r][c] = v.x;
-            block[r][c + 1] = v.y;
-            block[r][c + 2] = v.z;
-            block[r][c + 3] = v.w;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = q + 16 * i, r = 4 * g;  // row c of dst, its columns r .. r + 3
-            if (c0 + c < cols && r0 + r < rows) {
-                const v4f v = {block[r][c], block[r + 1][c], block[r + 2][c], block[r + 3][c]};
-                *reinterpret_cast<v4f*>(dst + static_cast<int64_t>(c0 + c) * ld_dst + r0 + r) = v;
-            }
-        }
-    } else {
-        const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int r = r0 + ty + 4 * i, c = c0 + tx;
-            block[ty + 4 * i][tx] = (r < rows && c < cols) ? __builtin_nontemporal_load(src + static_cast<int64_t>(r) * ld_src + c) : 0.f;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int c = c0 + ty + 4 * i, r = r0 + tx;
-            if (c < cols && r < rows) dst[static_cast<int64_t>(c) * ld_dst + r] = block[tx][ty + 4 * i];
-        }
-    }
-}
-
+// C = alpha * A * B^T + beta * C is C^T (N x M) = (B^T)^T * A^T with both operands K-major: the row-major problem with
+// its left operand, the memory of B seen as K rows of N, given transposed.
 namespace hpcdnn {
-static size_t round_up_256(size_t b) { return (b + 255) / 256 * 256; }
-size_t ft_cm_nt_workspace_bytes(int M, int N, int K) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return round_up_256(static_cast<size_t>(N) * K * sizeof(float)) + ft_workspace_bytes(N, M, K);
-}
+size_t ft_cm_nt_workspace_bytes(int M, int N, int K) { return ft_workspace_bytes(N, M, K); }
 }  // namespace hpcdnn
 
 extern "C" int hpcdnn_ft_sgemm_cm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                                      float alpha, float beta, float tau, const hpcdnn_ft_options* opt, hpcdnn_ft_status* status,
                                      void* ws, size_t ws_bytes, void* stream) {
-    // the row-major problem: C^T (N x M, ldc) = Bt^T (N x K) * At (K x M, lda), Bt = the memory of B (K x N, ldb)
-    int rc = check_gemm_args(N, M, K, B, ldb, A, lda, C, ldc, true);
-    if (rc != HPCDNN_OK) return rc;
-    if (M == 0 || N == 0) return HPCDNN_OK;
     hpcdnn_ft_options none{};
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (K == 0) return run_ft_sgemm(N, M, 0, nullptr, 1, nullptr, M, C, ldc, alpha, beta, tau, opt ? *opt : none, status, nullptr, 0, s);
-    const size_t copy_bytes = round_up_256(static_cast<size_t>(N) * K * sizeof(float));
-    if (!ws || ws_bytes < copy_bytes) return HPCDNN_ERR_WORKSPACE;
-    if (reinterpret_cast<uintptr_t>(ws) & 15u) return HPCDNN_ERR_INVALID_VALUE;
-    float* bt = static_cast<float*>(ws);
-    const dim3 blocks(static_cast<unsigned>(ceil_div(N, 64)), static_cast<unsigned>(ceil_div(K, 64)));
-    // (src: K rows of N, dst: N rows of K in the 16-byte aligned workspace)
-    if (N % 4 == 0 && K % 4 == 0 && ldb % 4 == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0)
-        transpose_kernel<true><<<blocks, 256, 0, s>>>(K, N, B, ldb, bt, K);
-    else
-        transpose_kernel<false><<<blocks, 256, 0, s>>>(K, N, B, ldb, bt, K);
-    rc = launch_status();
-    if (rc != HPCDNN_OK) return rc;
-    const size_t rest = ws_bytes - copy_bytes;
-    return run_ft_sgemm(N, M, K, bt, K, A, lda, C, ldc, alpha, beta, tau, opt ? *opt : none, status,
-                        rest ? static_cast<unsigned char*>(ws) + copy_bytes : nullptr, rest, s);
+    return run_ft_sgemm(N, M, K, B, ldb, A, lda, C, ldc, alpha, beta, tau, opt ? *opt : none, status, ws, ws_bytes,
+                        static_cast<hipStream_t>(stream), true);
 }
 
 // ---- ABFT SGEMM for callers that can neither allocate nor pass a workspace: the checksum vectors (and, when they

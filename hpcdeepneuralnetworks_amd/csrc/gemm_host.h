@@ -54,6 +54,21 @@ void (*sgemm_ta_kernel(int tile, int bm, int bn, bool edge))(const GemmArgs);
 // Its persistent kernel (beta == 0 or beta != 0 variant), or nullptr; only tiles whose untransposed kernel has one
 void (*sgemm_ta_persistent_kernel(int tile, int bm, int bn, bool beta))(const GemmArgs);
 
+// An ABFT kernel: full-tile and ragged-tile instantiation, its workgroup size and LDS need
+struct FtKernel {
+    void (*plain)(const GemmArgs);
+    void (*edge)(const GemmArgs);
+    int threads;
+    size_t lds;
+};
+// The ABFT kernels of a tile class for a transposed left operand (ft_sgemm_ta.hip); they read the checksum vectors
+// from the workspace.  kind 0: one checksum pair per workgroup tile; 1: per wave tile; 2: per workgroup tile with a
+// verification every check_interval k.  {nullptr, ...} where the class has no such kernel.
+FtKernel ft_ta_kernel(int tile_class, int bm, int bn, int kind);
+// Its enc_a pre-pass (row groups of `rows` rows of the product), or nullptr
+typedef void (*EncodeAtFn)(int, int, const float*, int, float*, int);
+EncodeAtFn ft_ta_encode(int rows);
+
 // Kernels that use more than the default 64 KiB of LDS must opt in once per device.
 inline int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {
     if (bytes <= 64 * 1024) return HPCDNN_OK;

@@ -164,17 +164,18 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
 // the accumulators are verified against the references of the k range done so far, and the references are
 // re-synchronised, as the reference kernel does every 256 k (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:143,263-271).
 //
-// TA (plain SGEMM only): the left operand is given transposed, p.A = A^T as a K x M row-major matrix with row length
+// TA (plain SGEMM, and ABFT with pre-encoded checksum vectors): the left operand is given transposed, p.A = A^T as a K x M row-major matrix with row length
 // p.lda >= M, which is how the operands of a column-major C = A * B^T lie in memory
 // (kernel/ft_sgemm/include/sgemm_huge.cuh:14, cublasSgemm(N, T, ...) in kernel/ft_sgemm/sgemm.cu:111).  A K step of
 // the tile is then 16 rows of BM floats, like B's; a lane fetches four consecutive m of one k and writes them as four
 // words into the same [m][k] staging layout, so everything from the fragment reads on is the code of the untransposed
-// case and every element of C sums its products in the same order.
+// case and every element of C sums its products in the same order.  The ABFT loop, whose row checksums work on a
+// lane's four k of one row, reads those back from the LDS stage that the transposed writes have just filled.
 template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS, int NSLOT = 2, int GRAN = 0, bool CADENCE = false,
           bool TA = false>
 __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
-    static_assert(!TA || FT == 0, "the ABFT kernels take A row by row");
+    static_assert(!TA || FT == 0 || FT == 2, "with a transposed A the checksum vectors come from the pre-pass");
     static_assert(NSLOT == 2 || (FT == 0 && NSLOT % 2 == 0), "the ABFT loop is written for two staging sets");
     static_assert(FT != 0 || (GRAN == 0 && !CADENCE), "granularity and cadence belong to the ABFT kernels");
     static_assert(GRAN == 0 || FT == 2, "wave-tile checksums come from the pre-encoded vectors");
@@ -253,6 +254,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int64_t b_step = static_cast<int64_t>(BK) * p.ldb;
 
     int a_voff[A_SLOTS], a_lds[A_SLOTS], a_kc[A_SLOTS];
+    int a_nvalid[A_SLOTS];  // TA: columns of the slot's group of four m inside the matrix (may be <= 0 or >= 4)
+    int a_lds_rows[A_SLOTS];  // TA ABFT: where the untransposed staging keeps this thread's row and k group
     int b_voff[B_SLOTS], b_lds[B_SLOTS], b_row[B_SLOTS], b_nvalid[B_SLOTS];
 #pragma unroll
     for (int s = 0; s < A_SLOTS; ++s) {
@@ -265,6 +268,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             a_kc[s] = k;
             a_voff[s] = (k * p.lda + m) * 4;
             a_lds[s] = m * AS + k;
+            a_nvalid[s] = p.M - (m0 + m);
+            a_lds_rows[s] = (idx / A_V4_PER_ROW) * AS + (idx % A_V4_PER_ROW) * 4;
         } else {
             int row = idx / A_V4_PER_ROW;
             a_kc[s] = (idx % A_V4_PER_ROW) * 4;
@@ -346,7 +351,17 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     auto gmask1 = [&](auto slot, auto part) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P < A_SLOTS && TA) {
-            // nothing to force: rows k >= K of A^T read as 0, and a K slice ends on a K step unless it ends with K
+            // rows k >= K of A^T read as 0, and a K slice ends on a K step unless it ends with K; columns m >= M
+            // (the next row or padding) matter to the ABFT kernels only, whose column sums run over the whole tile
+            if constexpr (FT != 0) {
+                const int nv = a_nvalid[P];
+                v4f v = ra[S][P];
+                v.x = nv > 0 ? v.x : 0.f;
+                v.y = nv > 1 ? v.y : 0.f;
+                v.z = nv > 2 ? v.z : 0.f;
+                v.w = nv > 3 ? v.w : 0.f;
+                ra[S][P] = v;
+            }
         } else if constexpr (P < A_SLOTS) {
             const int left = kend - (k_slot[S] + a_kc[P]);
             v4f v = ra[S][P];
@@ -528,6 +543,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             for (int e = 0; e < 4; ++e) cr_lo[gn][sl][e] = 0.f;
     float e_pa[4], e_sw[4];
     v4f e_t[kPartV4 * B_SLOTS], e_brv[GN];
+    v4f e_a[TA ? A_SLOTS : 1];  // TA: this thread's rows of the staged K step (four k each), read back from LDS
     float e_pb0, e_pb1, e_pk, e_swb, e_ac[GM][B_SLOTS];
     const int e_hw = tid / B_V4_PER_ROW;  // first k row this thread stages of B (a half wave per row of a 128-column tile)
     const int e_class = tid & 3;         // k group (4 k values) this thread stages of A
@@ -623,6 +639,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     for (int sl = 0; sl < B_SLOTS; ++sl) e_ac[gm][sl] = g_ac[S][gm][sl];
 #pragma unroll
                 for (int gn = 0; gn < GN; ++gn) e_brv[gn] = g_br[S][gn];
+                // (the barrier before the second half has made stage `par`, which holds this K step, complete)
+                if constexpr (TA) {
+#pragma unroll
+                    for (int sl = 0; sl < A_SLOTS; ++sl) e_a[sl] = *reinterpret_cast<const v4f*>(As + par * A_STAGE + a_lds_rows[sl]);
+                }
             }
         } else if constexpr (E == 0) {
 #pragma unroll
@@ -662,10 +683,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             constexpr int lo = GRAN ? 0 : (piece == 0 ? 0 : A_SLOTS / 2), hi = GRAN ? A_SLOTS : (piece == 0 ? A_SLOTS / 2 : A_SLOTS);
 #pragma unroll
             for (int sl = lo; sl < hi; ++sl) {
-                cr_lo[gn][sl][0] = __builtin_fmaf(ra[S][sl].x, e_brv[gn].x, cr_lo[gn][sl][0]);
-                cr_lo[gn][sl][1] = __builtin_fmaf(ra[S][sl].y, e_brv[gn].y, cr_lo[gn][sl][1]);
-                cr_lo[gn][sl][2] = __builtin_fmaf(ra[S][sl].z, e_brv[gn].z, cr_lo[gn][sl][2]);
-                cr_lo[gn][sl][3] = __builtin_fmaf(ra[S][sl].w, e_brv[gn].w, cr_lo[gn][sl][3]);
+                const v4f av = TA ? e_a[TA ? sl : 0] : ra[S][sl];
+                cr_lo[gn][sl][0] = __builtin_fmaf(av.x, e_brv[gn].x, cr_lo[gn][sl][0]);
+                cr_lo[gn][sl][1] = __builtin_fmaf(av.y, e_brv[gn].y, cr_lo[gn][sl][1]);
+                cr_lo[gn][sl][2] = __builtin_fmaf(av.z, e_brv[gn].z, cr_lo[gn][sl][2]);
+                cr_lo[gn][sl][3] = __builtin_fmaf(av.w, e_brv[gn].w, cr_lo[gn][sl][3]);
             }
 #pragma unroll
             for (int sl = lo; sl < hi; ++sl)
@@ -849,7 +871,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 // ABFT on a ragged problem: a tile that does not hang over the last column needs the masks only where
                 // plain SGEMM does, in the slice's last two K steps (its checksums want zeros in columns k >= kend of
                 // A and rows k >= kend of B; the columns n >= N that the other steps would have to clear do not exist)
-                if (n0 + BN <= p.N) {
+                if (n0 + BN <= p.N && (!TA || m0 + BM <= p.M)) {
                     for (; kt + 3 < nkt; kt += 2) {
                         step(S1{}, S0{}, std::false_type{}, std::false_type{}, std::false_type{});
                         flush_now = (kt & 14) == 14;
@@ -1474,6 +1496,37 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
             const int k = kb + half + kHalves * in_group;
             // (the last block of 128 columns may reach past the last column group)
             if (k < enc_ld && group < col_groups) enc_b[static_cast<int64_t>(group) * enc_ld + k] = out;
+        }
+    }
+}
+
+// The enc_a half of the pre-pass for a transposed left operand: enc_a[g][k] = sum over the rows m of row group g
+// (RM rows, m < M) of At[k][m], in the layout above (zeros for K <= k < enc_ld; k and k + 8 of a K step side by side).
+// A row of At holds a group's RM values side by side: the 16 lanes of a DPP row read them 16 at a time (64 contiguous
+// bytes, the four rows of a wave four different k) and add their partial sums across the row; a block of four waves
+// covers 64 values of k of one row group.
+template <int RM>
+__global__ __launch_bounds__(256) void abft_encode_at_kernel(int M, int K, const float* __restrict__ At, int ldat,
+                                                             float* __restrict__ enc_a, int enc_ld) {
+    static_assert(RM % 16 == 0, "a row group is read 16 values at a time");
+    const int l16 = threadIdx.x & 15, krow = threadIdx.x >> 4;  // 16 rows of k per pass
+    const int group = blockIdx.y, m0 = group * RM;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const int k = blockIdx.x * 64 + pass * 16 + krow;
+        float t = 0.f;
+        if (k < K) {
+            const float* row = At + static_cast<int64_t>(k) * ldat + m0;
+            float v[RM / 16];
+#pragma unroll
+            for (int j = 0; j < RM / 16; ++j) v[j] = (m0 + l16 + 16 * j < M) ? row[l16 + 16 * j] : 0.f;
+#pragma unroll
+            for (int j = 0; j < RM / 16; ++j) t += v[j];
+        }
+        t = row16_allsum(t);
+        if (l16 == 0 && k < enc_ld) {
+            const int q = k & 15;
+            enc_a[static_cast<int64_t>(group) * enc_ld + (k & ~15) + (q & 7) * 2 + (q >> 3)] = t;
         }
     }
 }
