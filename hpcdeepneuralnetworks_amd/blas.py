@@ -188,13 +188,13 @@ def ft_cm_nt_workspace_bytes(M: int, N: int, K: int) -> int:
 
 
 def ft_sgemm_cm_nt(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
-                   ws: torch.Tensor, tau: float = 0.0, status: torch.Tensor | None = None, tile_class: int = 0,
+                   ws: torch.Tensor | None, tau: float = 0.0, status: torch.Tensor | None = None, tile_class: int = 0,
                    granularity: int = 0, check_interval: int = 0, faults=None) -> None:
     """ABFT GEMM on the column-major buffers of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)``
     (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21): ``C (M x N) = alpha*A (M x K) @ B (N x K).T + beta*C``.  The tensors hold
     the column-major matrices as their row-major transposes (``A`` K x M, ``B`` K x N, ``C`` N x M).  Tiles, status
-    records and fault coordinates are those of ``ft_sgemm(N, M, K, ...)`` on the row-major ``C^T``.  ``ws`` (required):
-    ``ft_cm_nt_workspace_bytes(M, N, K)`` bytes."""
+    records and fault coordinates are those of ``ft_sgemm(N, M, K, ...)`` on the row-major ``C^T``.  ``ws``: optional
+    scratch of ``ft_cm_nt_workspace_bytes(M, N, K)`` bytes, as for ``ft_sgemm``."""
     pa, lda = _matrix(A, K, M, "A")
     pb, ldb = _matrix(B, K, N, "B")
     pc, ldc = _matrix(Cm, N, M, "C")

@@ -107,8 +107,7 @@ static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
     return tile_mode > wave_mode ? tile_mode : wave_mode;
 }
 
-// ta: A is given transposed (K x M row-major, lda >= M); those kernels read the checksum vectors from the workspace,
-// which is then required
+// ta: A is given transposed (K x M row-major, lda >= M)
 static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                         float alpha, float beta, float tau, const hpcdnn_ft_options& opt, hpcdnn_ft_status* status, void* ws,
                         size_t ws_bytes, hipStream_t s, bool ta = false) {
@@ -125,7 +124,7 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     const bool cadence = opt.check_interval > 0 && opt.check_interval < K;
     if (cadence && (wave || !fc.pre_cad.plain)) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
-    if ((wave || ta) && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
+    if (wave && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
 
     GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, fc.bm, fc.bn);
     // tau > 0: absolute; tau == 0: the absolute default for unit-range data; tau < 0: scaled to the data, the
@@ -215,7 +214,9 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
                                                                                         a.full_tiles, a.tail_status, status);
         return launch_status();
     }
-    const FtKernel& k = cadence ? fc.fused_cad : fc.fused;
+    const FtKernel ta_k = ta ? ft_ta_kernel(opt.tile_class, fc.bm, fc.bn, cadence ? 4 : 3) : FtKernel{nullptr, nullptr, 0, 0};
+    if (ta && !ta_k.plain) return HPCDNN_ERR_INVALID_VALUE;
+    const FtKernel& k = ta ? ta_k : cadence ? fc.fused_cad : fc.fused;
     void (*fn)(const GemmArgs) = edge ? k.edge : k.plain;
     rc = enable_lds(fn, k.lds);
     if (rc != HPCDNN_OK) return rc;

@@ -61,9 +61,10 @@ struct FtKernel {
     int threads;
     size_t lds;
 };
-// The ABFT kernels of a tile class for a transposed left operand (ft_sgemm_ta.hip); they read the checksum vectors
-// from the workspace.  kind 0: one checksum pair per workgroup tile; 1: per wave tile; 2: per workgroup tile with a
-// verification every check_interval k.  {nullptr, ...} where the class has no such kernel.
+// The ABFT kernels of a tile class for a transposed left operand (ft_sgemm_ta.hip).  Checksum vectors from the
+// workspace: kind 0, one checksum pair per workgroup tile; 1, per wave tile; 2, per workgroup tile with a verification
+// every check_interval k.  Checksum vectors formed in the main loop: kind 3, per workgroup tile; 4, with the
+// verification cadence.  {nullptr, ...} where the class has no such kernel.
 FtKernel ft_ta_kernel(int tile_class, int bm, int bn, int kind);
 // Its enc_a pre-pass (row groups of `rows` rows of the product), or nullptr
 typedef void (*EncodeAtFn)(int, int, const float*, int, float*, int);

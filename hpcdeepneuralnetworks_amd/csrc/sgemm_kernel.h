@@ -164,7 +164,7 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
 // the accumulators are verified against the references of the k range done so far, and the references are
 // re-synchronised, as the reference kernel does every 256 k (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:143,263-271).
 //
-// TA (plain SGEMM, and ABFT with pre-encoded checksum vectors): the left operand is given transposed, p.A = A^T as a K x M row-major matrix with row length
+// TA: the left operand is given transposed, p.A = A^T as a K x M row-major matrix with row length
 // p.lda >= M, which is how the operands of a column-major C = A * B^T lie in memory
 // (kernel/ft_sgemm/include/sgemm_huge.cuh:14, cublasSgemm(N, T, ...) in kernel/ft_sgemm/sgemm.cu:111).  A K step of
 // the tile is then 16 rows of BM floats, like B's; a lane fetches four consecutive m of one k and writes them as four
@@ -175,7 +175,6 @@ template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS, i
           bool TA = false>
 __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
-    static_assert(!TA || FT == 0 || FT == 2, "with a transposed A the checksum vectors come from the pre-pass");
     static_assert(NSLOT == 2 || (FT == 0 && NSLOT % 2 == 0), "the ABFT loop is written for two staging sets");
     static_assert(FT != 0 || (GRAN == 0 && !CADENCE), "granularity and cadence belong to the ABFT kernels");
     static_assert(GRAN == 0 || FT == 2, "wave-tile checksums come from the pre-encoded vectors");
@@ -514,7 +513,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // destinations of this lane's publishes (parity 0); strides and the parity distance are the same for the
     // publishing lanes and the dump, so every write is base + immediate offset
     // (after the transposing reduction lane l < 16 of a wave holds the wave's column sum of k = 4 * (l % 4) + l / 4)
-    float* const pub_a = (lane < 16) ? s_apart + (4 * (tid & 3) + (lane >> 2)) * kParts + wave : s_dump;
+    // (TA: a lane stages four m of k = lane / 4, so the first lane of each quad ends up with the wave's sum of that k)
+    float* const pub_a = TA ? ((lane & 3) == 0 ? s_apart + (lane >> 2) * kParts + wave : s_dump)
+                            : (lane < 16) ? s_apart + (4 * (tid & 3) + (lane >> 2)) * kParts + wave : s_dump;
     float* const pub_b = (tid % B_V4_PER_ROW < B_SLOTS) ? s_br + tid / B_V4_PER_ROW + kHalfWaves * (tid % B_V4_PER_ROW) : s_dump;
     const int x32_addr = (lane ^ 32) * 4;  // ds_bpermute address of the partner lane in the other half wave
     // With wave-tile checksums a thread keeps one column sum per wave row gm (its columns lie in one wave column)
@@ -556,7 +557,23 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 
     auto produce1 = [&](auto slot, auto piece, int par) {
         constexpr int S = decltype(slot)::value, E = decltype(piece)::value;
-        if constexpr (E == 0) {
+        if constexpr (TA && E <= 3) {
+            // column sums of A^T's staged K step: a lane holds four m of one k per slot, the four lanes of a quad
+            // the wave's sixteen m-groups of that k between them
+            if constexpr (E == 0) {
+                v4f t = ra[S][0];
+#pragma unroll
+                for (int sl = 1; sl < A_SLOTS; ++sl) t += ra[S][sl];
+                e_pa[0] = (t.x + t.y) + (t.z + t.w);
+                HPCDNN_PIN(e_pa[0]);
+            } else if constexpr (E == 1) {
+                e_pa[0] += dpp_mov<kDppXor1>(e_pa[0]);
+                HPCDNN_PIN(e_pa[0]);
+            } else if constexpr (E == 2) {
+                e_pa[0] += dpp_mov<kDppXor2>(e_pa[0]);
+                HPCDNN_PIN(e_pa[0]);
+            }
+        } else if constexpr (E == 0) {
             v4f t = ra[S][0];
 #pragma unroll
             for (int sl = 1; sl < A_SLOTS; ++sl) t += ra[S][sl];
@@ -611,12 +628,14 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             // a k row of a 64-column tile lies in one row of 16 lanes and is complete here
             if constexpr (B_V4_PER_ROW == 32) e_swb = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, e_pk), 0x401F));
         } else if constexpr (E == 8) {
-            e_pa[0] += e_sw[0];
-            e_sw[0] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(x32_addr, __builtin_bit_cast(int, e_pa[0])));
+            if constexpr (!TA) {
+                e_pa[0] += e_sw[0];
+                e_sw[0] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(x32_addr, __builtin_bit_cast(int, e_pa[0])));
+            }
             if constexpr (B_V4_PER_ROW == 32) e_pk += e_swb;
             HPCDNN_PIN(e_pk);
         } else if constexpr (E == 9) {
-            e_pa[0] += e_sw[0];  // sum over the whole wave
+            if constexpr (!TA) e_pa[0] += e_sw[0];  // sum over the whole wave
             HPCDNN_PIN(e_pa[0]);
         } else {
             // lanes 0..15 of each wave publish the 16 column sums, the first lane (or two) of each k row of B its row sum;
@@ -653,6 +672,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 for (int v = 0; v < kPartV4; ++v) e_t[kPartV4 * sl + v] = *reinterpret_cast<const v4f*>(row + 4 * v);
             }
             e_brv[0] = *reinterpret_cast<const v4f*>(br + 4 * e_class);
+            if constexpr (TA) {
+#pragma unroll
+                for (int sl = 0; sl < A_SLOTS; ++sl) e_a[sl] = *reinterpret_cast<const v4f*>(As + par * A_STAGE + a_lds_rows[sl]);
+            }
         } else if constexpr (E == 1) {
 #pragma unroll
             for (int sl = 0; sl < B_SLOTS; ++sl) {

@@ -277,11 +277,10 @@ int hpcdnn_ft_sgemm_opt(int M, int N, int K, const float* A, int lda, const floa
  * coordinates are those of hpcdnn_ft_sgemm_opt(N, M, K, ...), i.e. `row` counts
  * along N (the columns of the column-major C) and `col` along M; use
  * hpcdnn_ft_num_check_tiles(tile_class, granularity, N, M) records.  Both
- * operands are read where they lie (no transposed copy).  `ws` is REQUIRED
- * (K > 0): hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM_CM_NT, M, N, K) bytes (=
- * that of HPCDNN_OP_FT_SGEMM for N, M, K), 16-byte aligned, no initialisation:
- * these kernels take the checksum vectors from the pre-pass
- * (HPCDNN_ERR_WORKSPACE without it).  `opt` may be NULL. */
+ * operands are read where they lie (no transposed copy).  `ws`: optional
+ * scratch of hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM_CM_NT, M, N, K) bytes (=
+ * that of HPCDNN_OP_FT_SGEMM for N, M, K), with the meaning and rules it has
+ * for hpcdnn_ft_sgemm_opt.  `opt` may be NULL. */
 int hpcdnn_ft_sgemm_cm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                           float alpha, float beta, float tau, const hpcdnn_ft_options* opt, hpcdnn_ft_status* status,
                           void* ws, size_t ws_bytes, void* stream);

@@ -18,6 +18,12 @@ TOL = 1e-5
 DECISION_FIELDS = ("flag", "row", "col", "n_bad_rows", "n_bad_cols")
 
 
+@pytest.fixture(params=["fused", "workspace"])
+def ft_mode(request):
+    """Checksum vectors formed in the main loop (no workspace) or by the pre-pass kernels (with workspace)."""
+    return request.param
+
+
 def _buffers(oracle_mod, M, N, K, pad, seed):
     lda, ldb, ldc = M + pad[0], N + pad[1], M + pad[2]
     abuf = oracle_mod.fill_uniform_matrix(K, M, seed, ld=lda)       # column k of A = row k of the buffer
@@ -32,12 +38,13 @@ def _ws(blas, M, N, K):
     return torch.full((max(nbytes // 4, 4),), float("nan"), dtype=torch.float32, device="cuda")   # poisoned
 
 
-def _run(blas, oracle_mod, M, N, K, alpha, beta, tau, faults=None, pad=(0, 0, 0), seed=600, **opts):
+def _run(blas, oracle_mod, M, N, K, alpha, beta, tau, faults=None, pad=(0, 0, 0), seed=600, mode="workspace", **opts):
     abuf, bbuf, cbuf = _buffers(oracle_mod, M, N, K, pad, seed)
     da, db, dc = torch.from_numpy(abuf).cuda(), torch.from_numpy(bbuf).cuda(), torch.from_numpy(cbuf).cuda()
     tile_class, gran = opts.get("tile_class", 0), opts.get("granularity", 0)
     status = blas.ft_status_alloc(N, M, tile_class=tile_class, granularity=gran)
-    blas.ft_sgemm_cm_nt(M, N, K, da, db, dc, alpha, beta, _ws(blas, M, N, K), tau=tau, status=status, faults=faults, **opts)
+    ws = _ws(blas, M, N, K) if mode == "workspace" else None
+    blas.ft_sgemm_cm_nt(M, N, K, da, db, dc, alpha, beta, ws, tau=tau, status=status, faults=faults, **opts)
     c = dc.cpu().numpy()
     ref, den = oracle_mod.gemm_cm_nt_f64(M, N, K, abuf, abuf.shape[1], bbuf, bbuf.shape[1], cbuf, cbuf.shape[1], alpha, beta)
     err = oracle_mod.gemm_max_err(M, c, c.shape[1], ref, den)
@@ -49,22 +56,23 @@ def _run(blas, oracle_mod, M, N, K, alpha, beta, tau, faults=None, pad=(0, 0, 0)
 @pytest.mark.parametrize("M,N,K,pad", [(128, 256, 64, (0, 0, 0)), (384, 512, 320, (0, 0, 0)), (200, 300, 100, (4, 8, 12)), (1, 1, 1, (0, 0, 0)),
                                       (129, 257, 17, (3, 1, 2)), (1024, 1024, 1024, (0, 0, 0))])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, -1.5)])
-def test_fault_free_values_and_clean_records(blas, oracle_mod, M, N, K, pad, alpha, beta):
+def test_fault_free_values_and_clean_records(blas, oracle_mod, ft_mode, M, N, K, pad, alpha, beta):
     tau = blas.ft_default_tau(K)
-    *_, st, _ = _run(blas, oracle_mod, M, N, K, alpha, beta, tau, pad=pad)
+    *_, st, _ = _run(blas, oracle_mod, M, N, K, alpha, beta, tau, pad=pad, mode=ft_mode)
     assert np.all(st["flag"] == 0) and np.all(st["row"] == -1) and np.all(st["col"] == -1)
     assert st["max_clean_residual"].max() < 0.6 * tau
 
 
 @pytest.mark.parametrize("fault", [None, (1, 5, 7, 3.0)])
-def test_against_the_row_major_call_on_a_transposed_copy(blas, oracle_mod, fault):
+def test_against_the_row_major_call_on_a_transposed_copy(blas, oracle_mod, ft_mode, fault):
     M, N, K = 300, 520, 272
     tau = blas.ft_default_tau(K)
-    abuf, bbuf, cbuf, c, st, status = _run(blas, oracle_mod, M, N, K, 1.0, 1.0, tau, faults=[fault] if fault else None, pad=(4, 8, 4))
+    abuf, bbuf, cbuf, c, st, status = _run(blas, oracle_mod, M, N, K, 1.0, 1.0, tau, faults=[fault] if fault else None, pad=(4, 8, 4),
+                                           mode=ft_mode)
     bt = torch.from_numpy(np.ascontiguousarray(bbuf[:, :N].T)).cuda()        # N x K row-major
     dc = torch.from_numpy(cbuf).cuda()
     status2 = blas.ft_status_alloc(N, M)
-    ws = torch.full((max(blas.ft_workspace_bytes(N, M, K) // 4, 4),), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.full((max(blas.ft_workspace_bytes(N, M, K) // 4, 4),), float("nan"), dtype=torch.float32, device="cuda") if ft_mode == "workspace" else None
     blas.ft_sgemm(N, M, K, bt, torch.from_numpy(abuf).cuda(), dc, 1.0, 1.0, tau=tau, fault=fault, status=status2, ws=ws)
     c2, st2 = dc.cpu().numpy(), blas.ft_status_numpy(status2)
     for f in DECISION_FIELDS:
@@ -79,12 +87,12 @@ def test_against_the_row_major_call_on_a_transposed_copy(blas, oracle_mod, fault
         assert abs(c2[5, 128 + 7] - c[5, 128 + 7]) < 1e-3
 
 
-def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod):
+def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod, ft_mode):
     """The reference's only fault experiment: +1.0 into local element (0, 1) of a tile, threshold 0.1
     (ft_sgemm_huge.cuh:30,40,145) -> located and removed."""
     M, N, K = 256, 512, 256                      # C^T is 512 x 256: two tiles of 256 x 128 down, two across
     for tile in range(4):
-        *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, 0.1, faults=[(tile, 0, 1, 1.0)])
+        *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, 0.1, faults=[(tile, 0, 1, 1.0)], mode=ft_mode)
         exp = [0, 0, 0, 0]
         exp[tile] = 1
         assert st["flag"].tolist() == exp
@@ -92,7 +100,7 @@ def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod):
         assert abs(st["row_residual"][tile] + 1.0) < 1e-3 and abs(st["col_residual"][tile] + 1.0) < 1e-3
 
 
-def test_seeded_faults_decisions_equal_cpu_model(blas, oracle_mod):
+def test_seeded_faults_decisions_equal_cpu_model(blas, oracle_mod, ft_mode):
     M, N, K = 300, 600, 512                       # C^T: 600 x 300 -> 3 x 3 tiles, last row / column of tiles clipped
     tau = blas.ft_default_tau(K)
     rng = np.random.default_rng(17)
@@ -104,7 +112,7 @@ def test_seeded_faults_decisions_equal_cpu_model(blas, oracle_mod):
         i, j = int(rng.integers(tm)), int(rng.integers(tn))
         delta = float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-1, 2)))
         abuf, bbuf, cbuf, c, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 1.0, tau, faults=[(tile, i, j, delta)],
-                                          pad=(4, 4, 8), seed=700 + trial)
+                                          pad=(4, 4, 8), seed=700 + trial, mode=ft_mode)
         # the CPU model on the row-major problem C^T (N x M) = Bt^T (N x K) * At (K x M)
         bt = np.ascontiguousarray(bbuf[:, :N].T)
         c_model = cbuf.copy()
@@ -122,19 +130,20 @@ def test_other_classes_granularity_and_cadence(blas, oracle_mod):
     assert st["flag"][0] == 1 and (st["row"][0], st["col"][0]) == (3, 4)
     *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, tau, faults=[(1, 3, 4, 2.0)], granularity=blas.FT_GRAN_WAVE)
     assert st["flag"][1] == 1 and (st["row"][1], st["col"][1]) == (3, 4)
-    *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, tau, faults=[(0, 3, 4, 2.0, 1)], check_interval=256)
-    assert st["flag"][0] == 1 and (st["row"][0], st["col"][0]) == (3, 4)
+    for mode in ("workspace", "fused"):
+        *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, tau, faults=[(0, 3, 4, 2.0, 1)], check_interval=256, mode=mode)
+        assert st["flag"][0] == 1 and (st["row"][0], st["col"][0]) == (3, 4)
 
 
-def test_workspace_is_required(blas, oracle_mod):
+def test_workspace_rules(blas, oracle_mod):
     from hpcdeepneuralnetworks_amd.blas import HpcdnnError
     M, N, K = 200, 300, 128
     abuf, bbuf, cbuf = _buffers(oracle_mod, M, N, K, (0, 0, 0), 800)
     da, db = torch.from_numpy(abuf).cuda(), torch.from_numpy(bbuf).cuda()
-    with pytest.raises(HpcdnnError):
-        blas.ft_sgemm_cm_nt(M, N, K, da, db, torch.from_numpy(cbuf).cuda(), 1.0, 0.0, None)
-    with pytest.raises(HpcdnnError):   # too small for the checksum vectors
+    with pytest.raises(HpcdnnError):   # a workspace too small for the checksum vectors is an error, not a silent fallback
         blas.ft_sgemm_cm_nt(M, N, K, da, db, torch.from_numpy(cbuf).cuda(), 1.0, 0.0, torch.empty(64, device="cuda"))
+    with pytest.raises(HpcdnnError):   # wave-tile checksums come from the pre-pass
+        blas.ft_sgemm_cm_nt(M, N, K, da, db, torch.from_numpy(cbuf).cuda(), 1.0, 0.0, None, granularity=blas.FT_GRAN_WAVE)
     # K = 0: C = beta * C, nothing else needed
     dc = torch.full((N, M), 2.0, device="cuda")
     blas.ft_sgemm_cm_nt(M, N, 0, da, db, dc, 1.0, 0.5, None)
@@ -142,11 +151,11 @@ def test_workspace_is_required(blas, oracle_mod):
 
 
 @pytest.mark.parametrize("tile_class", [0, 1, 2, 3, 4])
-def test_every_tile_class_on_a_ragged_problem(blas, oracle_mod, tile_class):
+def test_every_tile_class_on_a_ragged_problem(blas, oracle_mod, ft_mode, tile_class):
     """Ragged in M, N and K with padded leading dimensions: the columns m >= M of the K-major operand (the next row
     or NaN padding) must not reach the column checksums.  One seeded fault per class, located and corrected."""
     M, N, K = 333, 270, 203
     tau = blas.ft_default_tau(K)
-    *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, -1.5, tau, faults=[(0, 9, 3, -4.0)], pad=(5, 2, 3), tile_class=tile_class)
+    *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, -1.5, tau, faults=[(0, 9, 3, -4.0)], pad=(5, 2, 3), tile_class=tile_class, mode=ft_mode)
     assert st["flag"][0] == 1 and (st["row"][0], st["col"][0]) == (9, 3)
     assert np.all(st["flag"][1:] == 0)
