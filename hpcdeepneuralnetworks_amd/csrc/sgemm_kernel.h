@@ -249,7 +249,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const float* b_base = p.B + static_cast<int64_t>(kbeg) * p.ldb + n0;
     int64_t a_left = a_bytes_left(kbeg);
     int64_t b_left = (static_cast<int64_t>(p.K - 1 - kbeg) * p.ldb + (p.N - n0)) * 4;
-    const int64_t a_step = TA ? static_cast<int64_t>(BK) * p.lda : BK;
+    const int64_t a_step = static_cast<int64_t>(BK) * p.lda;  // TA only (the untransposed A moves on by BK floats)
     const int64_t b_step = static_cast<int64_t>(BK) * p.ldb;
 
     int a_voff[A_SLOTS], a_lds[A_SLOTS], a_kc[A_SLOTS];
@@ -384,7 +384,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // descriptors are emptied, so the fetches that run ahead past the end all return 0 (never multiplied, and
     // neutral for the checksums).
     auto gload_advance_bulk = [&]() {  // kLazyBounds, a step that is not the slice's last: no end to look out for
-        a_base += a_step;
+        if constexpr (TA) a_base += a_step;
+        else a_base += BK;
         b_base += b_step;
         k_loaded += BK;
     };
@@ -401,27 +402,39 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             // the K step's instruction schedule in two
             a_base += a_step;
             b_base += b_step;
+            a_left = more ? a_left - a_step * 4 : 0;
+            b_left = more ? b_left - b_step * 4 : 0;
         } else {
-            a_base += more ? a_step : 0;
+            // (statement for statement what the untransposed kernels were tuned with: whether the compiler keeps
+            // these as scalar selects or branches around them hangs on their exact form)
+            a_base += more ? BK : 0;
+            a_left = more ? a_left - BK * 4 : 0;
             b_base += more ? b_step : 0;
+            b_left = more ? b_left - b_step * 4 : 0;
         }
-        a_left = more ? a_left - a_step * 4 : 0;
-        b_left = more ? b_left - b_step * 4 : 0;
         k_loaded += more ? BK : 0;
         if constexpr (FT == 2) enc_off += BK * 4;
     };
     // The same in two parts, so that the short-step schedule can place them apart.  Its full tiles keep no bounds at
     // all: nothing they fetch lies outside the matrix, and past the end of the slice they fetch its last K step
     // again instead of zeros.
-    auto gload_advance_a_bulk = [&]() { a_base += a_step; };
+    auto gload_advance_a_bulk = [&]() {
+        if constexpr (TA) a_base += a_step;
+        else a_base += BK;
+    };
     auto gload_advance_b_bulk = [&]() {
         b_base += b_step;
         k_loaded += BK;
     };
     auto gload_advance_a = [&]() {
         const bool more = k_loaded + BK < kend;
-        a_base += more ? a_step : 0;
-        if constexpr (!kNoBounds) a_left = more ? a_left - a_step * 4 : 0;
+        if constexpr (TA) {
+            a_base += more ? a_step : 0;
+            if constexpr (!kNoBounds) a_left = more ? a_left - a_step * 4 : 0;
+        } else {
+            a_base += more ? BK : 0;
+            if constexpr (!kNoBounds) a_left = more ? a_left - BK * 4 : 0;
+        }
     };
     auto gload_advance_b = [&]() {
         const bool more = k_loaded + BK < kend;
