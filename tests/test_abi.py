@@ -82,6 +82,12 @@ def test_bad_arguments_are_rejected_without_a_gpu(L):
     assert L.hpcdnn_sgemm_cm_nt(8, 4, 4, dummy, 7, dummy, 4, dummy, 8, 1.0, 0.0, None, 0, None) == INVALID
     assert L.hpcdnn_sgemm_cm_nt(8, 4, 4, dummy, 8, dummy, 3, dummy, 8, 1.0, 0.0, None, 0, None) == INVALID
     assert L.hpcdnn_sgemm_cm_nt(8, 4, 4, dummy, 8, dummy, 4, dummy, 7, 1.0, 0.0, None, 0, None) == INVALID
+    # ... and its ABFT counterpart (same leading-dimension rules; empty problems need nothing)
+    assert L.hpcdnn_ft_sgemm_cm_nt(8, 4, 4, dummy, 7, dummy, 4, dummy, 8, 1.0, 0.0, 0.0, None, None, None, 0, None) == INVALID
+    assert L.hpcdnn_ft_sgemm_cm_nt(8, 4, 4, dummy, 8, dummy, 3, dummy, 8, 1.0, 0.0, 0.0, None, None, None, 0, None) == INVALID
+    assert L.hpcdnn_ft_sgemm_cm_nt(8, 4, 4, dummy, 8, dummy, 4, dummy, 7, 1.0, 0.0, 0.0, None, None, None, 0, None) == INVALID
+    assert L.hpcdnn_ft_sgemm_cm_nt(0, 4, 4, None, 1, None, 4, None, 1, 1.0, 0.0, 0.0, None, None, None, 0, None) == 0
+    assert L.hpcdnn_workspace_bytes(5, 300, 200, 100) == L.hpcdnn_workspace_bytes(2, 200, 300, 100) > 0
     assert L.hpcdnn_sgemm_ex(4, 4, 4, dummy, 4, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, 99, 1, None) == INVALID
     assert L.hpcdnn_sgemm_ex(4, 4, 64, dummy, 64, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, 0, 2, None) == WORKSPACE
     # the 32 x 32 tile has no tail split (its waves split K among themselves)
