@@ -20,7 +20,6 @@ size_t ft_workspace_bytes(int M, int N, int K);
 //
 // Wave-tile granularity (the counterpart of ft_sgemm_huge_warp.cuh / ft_sgemm_huge_thread.cuh) runs the FT = 2 kernel
 // with one checksum pair per wave tile: the tile a wave of the workspace kernel owns, (bm / wgm) x (bn / wgn).
-typedef void (*EncodeFn)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int, int);
 struct FtClass {
     int bm, bn;
     int wgm, wgn;        // wave layout of the workspace kernels
@@ -172,17 +171,11 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         a.enc_b = enc_b;
         const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
         const int b_blocks = static_cast<int>(ceil_div(N, 128));  // the pre-pass walks B in blocks of 128 columns
-        if (ta) {
-            // the B half of the pre-pass as it is (no row groups), the A half by the kernel that walks A^T
-            const EncodeAtFn enc_at = ft_ta_encode(cm);
-            if (!enc_at) return HPCDNN_ERR_INVALID_VALUE;
-            hipLaunchKernelGGL(enc_at, dim3(static_cast<unsigned>(ceil_div(a.enc_ld, 64)), row_groups), dim3(256), 0, s, M, K, A, lda,
-                               enc_a, a.enc_ld);
-            rc = launch_status();
-            if (rc != HPCDNN_OK) return rc;
-        }
-        hipLaunchKernelGGL(wave ? fc.encode_wave : fc.encode, dim3(k_blocks * ((ta ? 0 : row_groups) + b_blocks)), dim3(1024), 0, s, M, N, K,
-                           A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, ta ? 0 : row_groups, col_groups);
+        // (ta: the same launch, with the blocks of the A half walking A^T)
+        const EncodeFn encode = ta ? ft_ta_encode(cm, cn) : wave ? fc.encode_wave : fc.encode;
+        if (!encode) return HPCDNN_ERR_INVALID_VALUE;
+        hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(1024), 0, s, M, N, K,
+                           A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;
         const FtKernel ta_k = ta ? ft_ta_kernel(opt.tile_class, fc.bm, fc.bn, wave ? 1 : (cadence ? 2 : 0)) : FtKernel{nullptr, nullptr, 0, 0};

@@ -43,14 +43,16 @@ FtKernel ft_ta_kernel(int tile_class, int bm, int bn, int kind) {
     return c.kind[kind];
 }
 
-EncodeAtFn ft_ta_encode(int rows) {
-    switch (rows) {
-        case 256: return abft_encode_at_kernel<256>;
-        case 128: return abft_encode_at_kernel<128>;
-        case 64: return abft_encode_at_kernel<64>;
-        case 32: return abft_encode_at_kernel<32>;
-        default: return nullptr;
-    }
+EncodeFn ft_ta_encode(int rows, int cols) {
+    // the check tiles of the classes above, at either granularity
+    if (rows == 256 && cols == 128) return abft_encode_kernel<256, 128, true>;
+    if (rows == 128 && cols == 32) return abft_encode_kernel<128, 32, true>;
+    if (rows == 128 && cols == 128) return abft_encode_kernel<128, 128, true>;
+    if (rows == 64 && cols == 64) return abft_encode_kernel<64, 64, true>;
+    if (rows == 64 && cols == 128) return abft_encode_kernel<64, 128, true>;
+    if (rows == 32 && cols == 64) return abft_encode_kernel<32, 64, true>;
+    if (rows == 128 && cols == 64) return abft_encode_kernel<128, 64, true>;
+    return nullptr;
 }
 
 }  // namespace hpcdnn

@@ -66,9 +66,9 @@ struct FtKernel {
 // every check_interval k.  Checksum vectors formed in the main loop: kind 3, per workgroup tile; 4, with the
 // verification cadence.  {nullptr, ...} where the class has no such kernel.
 FtKernel ft_ta_kernel(int tile_class, int bm, int bn, int kind);
-// Its enc_a pre-pass (row groups of `rows` rows of the product), or nullptr
-typedef void (*EncodeAtFn)(int, int, const float*, int, float*, int);
-EncodeAtFn ft_ta_encode(int rows);
+// Its pre-pass over both operands (row groups of `rows` rows, column groups of `cols` columns of the product), or nullptr
+typedef void (*EncodeFn)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int, int);
+EncodeFn ft_ta_encode(int rows, int cols);
 
 // Kernels that use more than the default 64 KiB of LDS must opt in once per device.
 inline int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {

@@ -1449,7 +1449,11 @@ __global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int 
 // enc_b[g][k] = sum over the columns n of column group g (n < N) of B[k][n]; zero for K <= k < enc_ld.  A half
 // wave reads 128 columns of one k row (32 lanes x 4 columns) and owns 8 of the block's 256 rows; CN / 4 neighbouring
 // lanes share a column group.
-template <int RM, int CN>
+//
+// TA: A is given transposed (K rows of M floats, row length lda).  A row then holds a group's RM values side by side:
+// the 16 lanes of a DPP row read them 16 at a time (64 contiguous bytes; the four rows of a wave four different k) and
+// add their partial sums across the row; a block covers 256 values of k of one row group, 64 per pass.
+template <int RM, int CN, bool TA = false>
 __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
                                                            const float* __restrict__ B, int ldb,
                                                            float* __restrict__ enc_a, float* __restrict__ enc_b,
@@ -1462,7 +1466,29 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
     static_assert(kRowsPerHalf <= kGroupLanes, "every k row of a half wave has a lane of each group to write it");
     __shared__ v4f part[kWaves][kWave];
     const int a_blocks = k_blocks * row_groups;
-    if (static_cast<int>(blockIdx.x) < a_blocks) {
+    if (TA && static_cast<int>(blockIdx.x) < a_blocks) {
+        static_assert(RM % 16 == 0, "a row group is read 16 values at a time");
+        const int l16 = threadIdx.x & 15, krow = threadIdx.x >> 4;  // 64 rows of k per pass
+        const int group = blockIdx.x / k_blocks, m0 = group * RM;
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int k = (blockIdx.x % k_blocks) * 256 + pass * 64 + krow;
+            float t = 0.f;
+            if (k < K) {
+                const float* row = A + static_cast<int64_t>(k) * lda + m0;
+                float v[RM / 16];
+#pragma unroll
+                for (int j = 0; j < RM / 16; ++j) v[j] = (m0 + l16 + 16 * j < M) ? row[l16 + 16 * j] : 0.f;
+#pragma unroll
+                for (int j = 0; j < RM / 16; ++j) t += v[j];
+            }
+            t = row16_allsum(t);
+            if (l16 == 0 && k < enc_ld) {
+                const int q = k & 15;  // k and k + 8 of a K step side by side, as below
+                enc_a[static_cast<int64_t>(group) * enc_ld + (k & ~15) + (q & 7) * 2 + (q >> 3)] = t;
+            }
+        }
+    } else if (static_cast<int>(blockIdx.x) < a_blocks) {
         const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
         const int group = blockIdx.x / k_blocks, m0 = group * RM;
         const int k = ((blockIdx.x % k_blocks) * kWave + lane) * 4;
@@ -1532,37 +1558,6 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
             const int k = kb + half + kHalves * in_group;
             // (the last block of 128 columns may reach past the last column group)
             if (k < enc_ld && group < col_groups) enc_b[static_cast<int64_t>(group) * enc_ld + k] = out;
-        }
-    }
-}
-
-// The enc_a half of the pre-pass for a transposed left operand: enc_a[g][k] = sum over the rows m of row group g
-// (RM rows, m < M) of At[k][m], in the layout above (zeros for K <= k < enc_ld; k and k + 8 of a K step side by side).
-// A row of At holds a group's RM values side by side: the 16 lanes of a DPP row read them 16 at a time (64 contiguous
-// bytes, the four rows of a wave four different k) and add their partial sums across the row; a block of four waves
-// covers 64 values of k of one row group.
-template <int RM>
-__global__ __launch_bounds__(256) void abft_encode_at_kernel(int M, int K, const float* __restrict__ At, int ldat,
-                                                             float* __restrict__ enc_a, int enc_ld) {
-    static_assert(RM % 16 == 0, "a row group is read 16 values at a time");
-    const int l16 = threadIdx.x & 15, krow = threadIdx.x >> 4;  // 16 rows of k per pass
-    const int group = blockIdx.y, m0 = group * RM;
-#pragma unroll
-    for (int pass = 0; pass < 4; ++pass) {
-        const int k = blockIdx.x * 64 + pass * 16 + krow;
-        float t = 0.f;
-        if (k < K) {
-            const float* row = At + static_cast<int64_t>(k) * ldat + m0;
-            float v[RM / 16];
-#pragma unroll
-            for (int j = 0; j < RM / 16; ++j) v[j] = (m0 + l16 + 16 * j < M) ? row[l16 + 16 * j] : 0.f;
-#pragma unroll
-            for (int j = 0; j < RM / 16; ++j) t += v[j];
-        }
-        t = row16_allsum(t);
-        if (l16 == 0 && k < enc_ld) {
-            const int q = k & 15;
-            enc_a[static_cast<int64_t>(group) * enc_ld + (k & ~15) + (q & 7) * 2 + (q >> 3)] = t;
         }
     }
 }
