@@ -33,6 +33,12 @@ inline int ft_sgemm(int M, int N, int K, const float* A, const float* B, float* 
                     size_t ws_bytes = 0) {
     return hpcdnn_ft_sgemm(M, N, K, A, K, B, N, C, N, alpha, beta, 0.0f, inject, status, ws, ws_bytes, nullptr);
 }
+// ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta) on its own column-major buffers (lda = M, ldb = N, ldc = M;
+// kernel/ft_sgemm/sgemm.cu:159-165); status records are those of the row-major N x M matrix C^T
+inline int ft_sgemm_cm_nt(int M, int N, int K, const float* A, const float* B, float* C, float alpha, float beta,
+                          hpcdnn_ft_status* status = nullptr, void* ws = nullptr, size_t ws_bytes = 0) {
+    return hpcdnn_ft_sgemm_cm_nt(M, N, K, A, M, B, N, C, M, alpha, beta, 0.0f, nullptr, status, ws, ws_bytes, nullptr);
+}
 // the two offline routines of kernel/ft_sgemm/include/baseline_ft_sgemm.cuh (:1-34 and :36-91): their cuBLAS handle and
 // eleven scratch vectors become one workspace of hpcdnn_workspace_bytes(HPCDNN_OP_OFFLINE_FT_SGEMM, M, N, K) bytes,
 // `residuals` receives what the reference leaves in dRes (2 values per K panel of 256, 1 for the scalar routine)
