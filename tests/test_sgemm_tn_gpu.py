@@ -184,6 +184,35 @@ def test_column_major_a_b_transposed(blas, oracle_mod, M, N, K, pad, alpha, beta
     assert np.all(np.isnan(c[:, M:]))
 
 
+def test_maximum_leading_dimensions(blas):
+    """ldat and ldb at the documented limit of the K-major operands (a K step is 16 of their rows; byte offsets inside one
+    tile are 32-bit) and ldc at its own, for several kernel families and for the ABFT entry point; one more is refused."""
+    ldat, ldb, ldc = (1 << 25) - 1024, (1 << 25) - 1024, (1 << 21) - 64
+    M, N, K = 300, 100, 40
+    atbuf = torch.empty(K * ldat + 8, device="cuda")
+    bbuf = torch.empty(K * ldb + 8, device="cuda")
+    at, b = atbuf[:K * ldat].view(K, ldat)[:, :M], bbuf[:K * ldb].view(K, ldb)[:, :N]
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    at.copy_(torch.rand(K, M, device="cuda", generator=gen) * 2 - 1)
+    b.copy_(torch.rand(K, N, device="cuda", generator=gen) * 2 - 1)
+    ref = at.double().t() @ b.double()
+    den = at.abs().double().t() @ b.abs().double()
+    cbuf = torch.empty(M * ldc, device="cuda")
+    c = cbuf.view(M, ldc)[:, :N]
+    c0 = torch.rand(M, N, device="cuda", generator=gen) * 2 - 1
+    for tile in (-1, 0, 4, 8, len(blas.tile_table()) - 1):
+        for beta in (0.0, -1.5):
+            c.copy_(c0)
+            blas.sgemm_tn(M, N, K, at, b, c, 1.0, beta, tile=tile, split_k=0 if tile < 0 else 1)
+            assert float(((c.double() - ref - beta * c0.double()).abs() / (den + abs(beta) * c0.abs().double())).max()) <= TOL, (tile, beta)
+    # the column-major ABFT entry point on the same buffers: A (M x K, lda = ldat), B (N x K, ldb), C (M x N) held as N x M
+    ccm = torch.zeros(N, M, device="cuda")
+    blas.ft_sgemm_cm_nt(M, N, K, at, b, ccm, 1.0, 0.0, None)
+    assert float(((ccm.double() - ref.t()).abs() / den.t()).max()) <= TOL
+    with pytest.raises(blas.HpcdnnError):
+        blas.sgemm_tn(M, N, 8, atbuf[:7 * (ldat + 1) + M].as_strided((8, M), (ldat + 1, 1)), b, torch.zeros(M, N, device="cuda"), 1.0, 0.0)
+
+
 def test_bad_arguments(blas):
     from hpcdeepneuralnetworks_amd.blas import HpcdnnError
     x = torch.zeros(64, 64, device="cuda")
