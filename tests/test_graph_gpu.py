@@ -31,6 +31,13 @@ def test_captured_sequence_replays_like_eager(blas):
     ws_dot = blas.workspace(64 + 8 * 4096)
     ws_gv = blas.workspace(max(blas.sgemv_workspace_bytes(M, N), 4))
     fault = (3, 17, 33, 2.5)
+    # the same product on column-major operands: A as its K x M row-major transpose, B (N x K) = the memory of b, C as N x M
+    a_t = a.t().contiguous()
+    c_cm = torch.zeros(N, M, device=dev)
+    c_ftcm = torch.zeros(N, M, device=dev)
+    status_cm = blas.ft_status_alloc(N, M)
+    ws_ftcm = blas.workspace(blas.ft_cm_nt_workspace_bytes(M, N, K))
+    fault_cm = (2, 5, 9, 1.5)
 
     def sequence():
         blas.sgemm(M, N, K, a, b, c_plain, 1.0, 0.0)
@@ -39,6 +46,8 @@ def test_captured_sequence_replays_like_eager(blas):
         blas.saxpy(nv, 0.5, x, y)
         blas.sdot(nv, x, y, dot, ws=ws_dot)
         blas.sgemv(True, M, N, 1.0, c_plain, x[:M], 0.0, gv, ws=ws_gv)
+        blas.sgemm_cm_nt(M, N, K, a_t, b, c_cm, 1.0, 0.0)
+        blas.ft_sgemm_cm_nt(M, N, K, a_t, b, c_ftcm, 1.0, 0.0, ws_ftcm, status=status_cm, faults=[fault_cm])
 
     # eager reference (y accumulates: replay r leaves y = y0 + 0.5 * (r + 1) * x applied step by step)
     sequence()
@@ -46,6 +55,10 @@ def test_captured_sequence_replays_like_eager(blas):
     ref_plain, ref_split, ref_ft = c_plain.clone(), c_split.clone(), c_ft.clone()
     ref_status = blas.ft_status_numpy(status).copy()
     ref_gv = gv.clone()
+    ref_cm, ref_ftcm = c_cm.clone(), c_ftcm.clone()
+    ref_status_cm = blas.ft_status_numpy(status_cm).copy()
+    assert ref_status_cm["flag"][2] == 1 and (ref_status_cm["row"][2], ref_status_cm["col"][2]) == (5, 9)
+    assert torch.allclose(ref_cm.t(), ref_plain, rtol=0, atol=1e-3)
     assert ref_status["flag"][3] == 1 and (ref_status["row"][3], ref_status["col"][3]) == (17, 33)
 
     y.copy_(y0)
@@ -62,9 +75,10 @@ def test_captured_sequence_replays_like_eager(blas):
 
     y_eager = y0.clone()
     for replay in range(4):
-        for t in (c_plain, c_split, c_ft, gv):
+        for t in (c_plain, c_split, c_ft, gv, c_cm, c_ftcm):
             t.fill_(float("nan"))          # eager work between replays: results must come from the replay itself
         status.zero_()
+        status_cm.zero_()
         dot.fill_(float("nan"))
         torch.cuda.synchronize()
         graph.replay()
@@ -75,6 +89,8 @@ def test_captured_sequence_replays_like_eager(blas):
         torch.cuda.synchronize()
         assert torch.equal(c_plain, ref_plain) and torch.equal(c_split, ref_split) and torch.equal(c_ft, ref_ft), replay
         assert torch.equal(gv, ref_gv), replay
+        assert torch.equal(c_cm, ref_cm) and torch.equal(c_ftcm, ref_ftcm), replay
+        assert np.array_equal(blas.ft_status_numpy(status_cm)["flag"], ref_status_cm["flag"]), replay
         assert torch.equal(y, y_eager), replay
         assert torch.equal(dot, dot_eager), replay
         st = blas.ft_status_numpy(status)
