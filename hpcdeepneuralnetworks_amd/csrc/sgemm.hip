@@ -2,6 +2,7 @@
 #include "gemm_host.h"
 #include "sgemm_small_kernel.h"
 #include "sgemm_persistent_kernel.h"
+#include "sgemm_tiles.h"
 
 namespace hpcdnn {
 
@@ -54,31 +55,7 @@ struct TileConfig {
             sgemm_small_kernel<TMB, true, OCC>, EFF, true, 0, nullptr, nullptr, 1                         \
     }
 
-// The counterpart of the reference's small/medium/large/tall/wide/huge shape table
-// (kernel/ft_sgemm/code_gen/main.py:8-16), re-derived for 32x32 MFMA blocks and four or eight 64-lane waves per
-// workgroup.  EFF comes from a least-squares fit of plan_cost() below to measured times of every tile over
-// squares 256..6144 with K = n, 1024 and 256 and a set of skinny shapes on an MI355X.
-static const TileConfig kTiles[] = {
-    HPCDNN_TILE_PERSISTENT(256, 128, 2, 2, 2, 0.978f),  // 0 huge (the ABFT tile)
-    HPCDNN_TILE_PERSISTENT_TWO(128, 128, 2, 2, 2, 0.970f),  // 1 large
-    HPCDNN_TILE(128, 64, 2, 2, 2, 0.945f),   // 2 tall
-    HPCDNN_TILE(64, 128, 2, 2, 2, 0.939f),   // 3 wide
-    HPCDNN_TILE(64, 64, 2, 2, 4, 0.900f),    // 4 medium
-    HPCDNN_TILE_PERSISTENT_BIG(192, 256, 2, 2, 1, 0.964f),  // 5 6144-friendly: 32 x 24 tiles = 3 full rounds of 256 CUs
-    HPCDNN_TILE(256, 192, 2, 2, 1, 0.946f),  // 6
-    HPCDNN_TILE_PERSISTENT(128, 256, 2, 2, 2, 0.987f),  // 7
-    HPCDNN_TILE(256, 256, 2, 4, 1, 1.000f),  // 8 giant, eight waves
-    HPCDNN_TILE(256, 128, 4, 2, 1, 1.000f),  // 9 huge, eight waves
-    HPCDNN_TILE(256, 256, 4, 2, 1, 1.000f),  // 10 giant, eight waves (4 x 2)
-    // 11 small: 32 x 32, K split between the four waves.  Every lane fetches its own operands, so the rate is set by
-    // the vector memory path, about half the matrix peak: for problems with too few 64 x 64 tiles to go round
-    HPCDNN_SMALL_TILE(1, 4, 0.50f),
-    // 12 medium with its loads four K steps ahead: a 64-row tile moves 64 bytes per row and K step, and with one
-    // workgroup per CU two steps in flight do not cover the trip to HBM when A is long and read once.  Staged data
-    // is so old when it is needed that the LDS writes lead the step and are done long before the barrier.
-    HPCDNN_TILE_DEEP(64, 64, 2, 2, 4, 0.905f, 4),
-    HPCDNN_TILE(192, 192, 2, 2, 1, 0.943f),  // 13 3072-friendly: 16 x 16 tiles = one full round of 256 CUs
-};
+static const TileConfig kTiles[] = {HPCDNN_SGEMM_TILE_LIST};
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 struct Plan {

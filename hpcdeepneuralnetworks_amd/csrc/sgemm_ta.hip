@@ -1,8 +1,9 @@
 // SGEMM kernels for a transposed left operand (A^T given as a K x M row-major matrix), in a translation unit of their
-// own so that they compile beside the others.  Row i of the table is tile i of the table in sgemm.hip; the 32 x 32
-// tile, whose lanes fetch their own operands, has no such variant.
+// own so that they compile beside the others.  The table is built from the same tile list as the one in sgemm.hip
+// (sgemm_tiles.h); the 32 x 32 tile, whose lanes fetch their own operands, has no such variant.
 #include "gemm_host.h"
 #include "sgemm_persistent_kernel.h"
+#include "sgemm_tiles.h"
 
 namespace hpcdnn {
 
@@ -20,34 +21,25 @@ struct TaKernels {
         BM, BN, sgemm_kernel<BM, BN, WGM, WGN, false, 0, OCC, NSLOT, 0, false, true>,            \
             sgemm_kernel<BM, BN, WGM, WGN, true, 0, OCC, NSLOT, 0, false, true>, PERSISTENT, PERSISTENT_BETA \
     }
-#define HPCDNN_TA(BM, BN, WGM, WGN, OCC, NSLOT) HPCDNN_TA_(BM, BN, WGM, WGN, OCC, NSLOT, nullptr, nullptr)
-// (IMM: stores at the tile boundary, PER_CU: persistent workgroups per CU, both as for the same tile in sgemm.hip)
-#define HPCDNN_TA_PERSISTENT(BM, BN, WGM, WGN, OCC, PER_CU)                                                          \
+// the kinds of sgemm_tiles.h (IMM: stores at the tile boundary, PER_CU: persistent workgroups per CU, as in sgemm.hip)
+#define HPCDNN_TA_PERSISTENT_(BM, BN, WGM, WGN, OCC, PER_CU)                                                         \
     HPCDNN_TA_(BM, BN, WGM, WGN, OCC, 2, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false, 0, PER_CU, true>),        \
                (sgemm_persistent_kernel<BM, BN, WGM, WGN, true, 0, PER_CU, true>))
+#define HPCDNN_TILE(BM, BN, WGM, WGN, OCC, EFF) HPCDNN_TA_(BM, BN, WGM, WGN, OCC, 2, nullptr, nullptr)
+#define HPCDNN_TILE_PERSISTENT(BM, BN, WGM, WGN, OCC, EFF) HPCDNN_TA_PERSISTENT_(BM, BN, WGM, WGN, OCC, 1)
+#define HPCDNN_TILE_PERSISTENT_TWO(BM, BN, WGM, WGN, OCC, EFF) HPCDNN_TA_PERSISTENT_(BM, BN, WGM, WGN, OCC, 2)
+#define HPCDNN_TILE_PERSISTENT_BIG(BM, BN, WGM, WGN, OCC, EFF) \
+    HPCDNN_TA_(BM, BN, WGM, WGN, OCC, 2, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false, 64, 1, true>), nullptr)
+#define HPCDNN_TILE_DEEP(BM, BN, WGM, WGN, OCC, EFF, NSLOT) HPCDNN_TA_(BM, BN, WGM, WGN, OCC, NSLOT, nullptr, nullptr)
+#define HPCDNN_SMALL_TILE(TMB, OCC, EFF) {32 * TMB, 32, nullptr, nullptr, nullptr, nullptr}
 
-const TaKernels kTaKernels[] = {
-    HPCDNN_TA_PERSISTENT(256, 128, 2, 2, 2, 1),  // 0
-    HPCDNN_TA_PERSISTENT(128, 128, 2, 2, 2, 2),  // 1
-    HPCDNN_TA(128, 64, 2, 2, 2, 2),   // 2
-    HPCDNN_TA(64, 128, 2, 2, 2, 2),   // 3
-    HPCDNN_TA(64, 64, 2, 2, 4, 2),    // 4
-    HPCDNN_TA_(192, 256, 2, 2, 1, 2, (sgemm_persistent_kernel<192, 256, 2, 2, false, 64, 1, true>), nullptr),  // 5
-    HPCDNN_TA(256, 192, 2, 2, 1, 2),  // 6
-    HPCDNN_TA_PERSISTENT(128, 256, 2, 2, 2, 1),  // 7
-    HPCDNN_TA(256, 256, 2, 4, 1, 2),  // 8
-    HPCDNN_TA(256, 128, 4, 2, 1, 2),  // 9
-    HPCDNN_TA(256, 256, 4, 2, 1, 2),  // 10
-    {32, 32, nullptr, nullptr, nullptr, nullptr},  // 11
-    HPCDNN_TA(64, 64, 2, 2, 4, 4),    // 12
-    HPCDNN_TA(192, 192, 2, 2, 1, 2),  // 13
-};
+const TaKernels kTaKernels[] = {HPCDNN_SGEMM_TILE_LIST};
 }  // namespace
 
 void (*sgemm_ta_kernel(int tile, int bm, int bn, bool edge))(const GemmArgs) {
     if (tile < 0 || tile >= static_cast<int>(sizeof(kTaKernels) / sizeof(kTaKernels[0]))) return nullptr;
     const TaKernels& k = kTaKernels[tile];
-    if (k.bm != bm || k.bn != bn) return nullptr;  // the two tables have drifted apart
+    if (k.bm != bm || k.bn != bn) return nullptr;
     return edge ? k.edge : k.plain;
 }
 
