@@ -184,6 +184,39 @@ def test_column_major_a_b_transposed(blas, oracle_mod, M, N, K, pad, alpha, beta
     assert np.all(np.isnan(c[:, M:]))
 
 
+def test_operands_that_start_four_bytes_off_a_16_byte_boundary(blas, oracle_mod):
+    """A^T, B and C as views that begin one float into their allocations, with odd leading dimensions: no row of any
+    operand starts on a 16-byte boundary, for plain SGEMM (two tile families) and for ABFT in both modes."""
+    M, N, K = 203, 149, 77
+    ldat, ldb, ldc = M + 2, N + 2, M + 4                      # column-major C: N rows of M in memory
+    a = oracle_mod.fill_uniform_matrix(K, M, 520, ld=ldat)
+    b = oracle_mod.fill_uniform_matrix(K, N, 521, ld=ldb)
+    c0 = oracle_mod.fill_uniform_matrix(N, M, 522, ld=ldc)
+    ref, den = oracle_mod.gemm_cm_nt_f64(M, N, K, a, ldat, b, ldb, c0, ldc, 1.0, -0.5)
+
+    def off_by_one(x):
+        buf = torch.full((x.size + 1,), float("nan"), device="cuda")
+        buf[1:] = torch.from_numpy(x.ravel()).cuda()
+        return buf[1:].view(x.shape)
+
+    da, db = off_by_one(a), off_by_one(b)
+    assert da.data_ptr() % 16 == 4
+    for run in ("sgemm", "ft_fused", "ft_workspace"):
+        dc = off_by_one(c0)
+        if run == "sgemm":
+            blas.sgemm_cm_nt(M, N, K, da, db, dc, 1.0, -0.5)
+        else:
+            ws = blas.workspace(blas.ft_cm_nt_workspace_bytes(M, N, K)) if run == "ft_workspace" else None
+            blas.ft_sgemm_cm_nt(M, N, K, da, db, dc, 1.0, -0.5, ws)
+        c = dc.cpu().numpy()
+        assert oracle_mod.gemm_max_err(M, c, ldc, ref, den) <= TOL, run
+        assert np.all(np.isnan(c[:, M:])), run
+    # the transposed-operand entry point with a pinned big tile on the same buffers: C^T (N x M) = B^T^T A^T
+    dc = off_by_one(c0)
+    blas.sgemm_tn(N, M, K, db, da, dc, 1.0, -0.5, tile=0, split_k=1)
+    assert oracle_mod.gemm_max_err(M, dc.cpu().numpy(), ldc, ref, den) <= TOL
+
+
 def test_maximum_leading_dimensions(blas):
     """ldat and ldb at the documented limit of the K-major operands (a K step is 16 of their rows; byte offsets inside one
     tile are 32-bit) and ldc at its own, for several kernel families and for the ABFT entry point; one more is refused."""
