@@ -267,15 +267,14 @@ static RowSplit choose_row_split(int M, int N, int K, int cus) {
     return best;
 }
 
-// ta: A is given transposed (K x M row-major).  Those kernels exist for every tile but the 32 x 32 one (sgemm_ta.hip);
-// everything else (plans, splits, reductions) is shared.
+// ta: A is given transposed (K x M row-major): the kernels of sgemm_ta.hip; everything else (plans, splits,
+// reductions) is shared.
 static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                      float alpha, float beta, void* ws, size_t ws_bytes, int tile, int split, hipStream_t stream,
                      bool ta = false) {
     int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc, ta);
     if (rc != HPCDNN_OK) return rc;
     if (tile >= kNumTiles || split == -1) return HPCDNN_ERR_INVALID_VALUE;
-    if (ta && tile >= 0 && kTiles[tile].wave_split_k) return HPCDNN_ERR_INVALID_VALUE;
     if (tile >= 0 && kTiles[tile].wave_split_k && split < -1) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
 
@@ -297,7 +296,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         if (!(memo.valid && memo.M == M && memo.N == N && memo.K == K && memo.cus == cus && memo.ws_bytes == usable &&
               memo.ws_aligned == ws_aligned && memo.ta == ta)) {
             double cost = 0.0;
-            memo.plan = choose_plan(M, N, K, ws != nullptr, usable, ws_aligned, &cost, ta);
+            memo.plan = choose_plan(M, N, K, ws != nullptr, usable, ws_aligned, &cost);
             memo.rows = RowSplit{-1, 0, -1, 1e300};
             if (K > 0) {
                 const RowSplit rs = choose_row_split(M, N, K, cus);

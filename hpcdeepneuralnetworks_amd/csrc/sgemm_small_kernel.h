@@ -11,6 +11,10 @@
 // issued before the current block's MFMAs (two register sets).  At the end the four partial tiles meet in LDS and
 // are added in wave order, so the result does not depend on timing; it does differ in the last bits from the large
 // tiles' result, which add the products of one element in a different order.
+//
+// TA: A is given transposed (K rows of M floats, row length lda >= M).  Its operands are then fetched like B's: lane
+// (half h, row i) reads At[kb + 16 h + t][m0 + i] for t = 0 .. 15, one 128-byte line per half and load; the MFMAs and
+// their order are the same, so the result has the bits of the untransposed kernel.
 #pragma once
 
 #include "sgemm_kernel.h"
@@ -26,7 +30,7 @@ constexpr size_t small_lds_bytes() {
     return sizeof(float) * kSmallWaves * (32 * TMB) * 32;
 }
 
-template <int TMB, bool EDGE, int MIN_BLOCKS>
+template <int TMB, bool EDGE, int MIN_BLOCKS, bool TA = false>
 __global__ __launch_bounds__(kSmallThreads, MIN_BLOCKS) void sgemm_small_kernel(const GemmArgs p) {
     constexpr int BM = 32 * TMB, BN = 32, BK = kSmallBK;
     constexpr int kRun = BK / 2;  // k values per lane half
@@ -48,11 +52,17 @@ __global__ __launch_bounds__(kSmallThreads, MIN_BLOCKS) void sgemm_small_kernel(
     // Descriptors start at the tile's first element of the wave's current K block and end with the matrix: rows
     // m >= M of A read as 0.  They move on by four K blocks per trip.
     const int k_first = kbeg + wave * BK;
-    const float* a_base = p.A + static_cast<int64_t>(m0) * p.lda + k_first;
+    // (TA: A^T is walked like B: rows k >= K read as 0, and columns m >= M, the next row or padding, only reach
+    // accumulators of rows that are never stored)
+    const float* a_base = TA ? p.A + static_cast<int64_t>(k_first) * p.lda + m0 : p.A + static_cast<int64_t>(m0) * p.lda + k_first;
     const float* b_base = p.B + static_cast<int64_t>(k_first) * p.ldb + n0;
-    int64_t a_left = (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - k_first)) * 4;
+    int64_t a_left = TA ? (static_cast<int64_t>(p.K - 1 - k_first) * p.lda + (p.M - m0)) * 4
+                        : (static_cast<int64_t>(p.M - 1 - m0) * p.lda + (p.K - k_first)) * 4;
     int64_t b_left = (static_cast<int64_t>(p.K - 1 - k_first) * p.ldb + (p.N - n0)) * 4;
+    const int64_t a_hop = TA ? static_cast<int64_t>(kSmallWaves * BK) * p.lda : kSmallWaves * BK;
     const int64_t b_hop = static_cast<int64_t>(kSmallWaves * BK) * p.ldb;
+    const int at_voff = static_cast<int>((static_cast<unsigned>(kRun * lh) * p.lda + li) * 4u);  // TA; < 2^32 as for B
+    const int at_row_bytes = p.lda * 4;
 
     int a_voff[TMB][4];
 #pragma unroll
@@ -80,17 +90,31 @@ __global__ __launch_bounds__(kSmallThreads, MIN_BLOCKS) void sgemm_small_kernel(
         if (EDGE && blk == nb - 1) {
             const int valid = kend - (kbeg + blk * BK);  // 1 .. 32 k values in this block
             const int mine = valid - kRun * lh;          // of this lane's run (may be <= 0)
+            if constexpr (TA) {
 #pragma unroll
-            for (int tm = 0; tm < TMB; ++tm)
+                for (int t = 0; t < kRun; ++t) {
+                    const int r = kRun * lh + t;
+                    const int rc = r < valid ? r : valid - 1;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    v4f v = buffer_load_v4f(ar, a_voff[tm][c]);
-                    v.x = (4 * c + 0 < mine) ? v.x : 0.f;
-                    v.y = (4 * c + 1 < mine) ? v.y : 0.f;
-                    v.z = (4 * c + 2 < mine) ? v.z : 0.f;
-                    v.w = (4 * c + 3 < mine) ? v.w : 0.f;
-                    ra[S][tm][c] = v;
+                    for (int tm = 0; tm < TMB; ++tm) {
+                        const float v = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                                      ar, static_cast<int>((static_cast<unsigned>(rc) * p.lda + tm * 32 + li) * 4u), 0, 0));
+                        ra[S][tm][t / 4][t % 4] = (r < valid) ? v : 0.f;
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int tm = 0; tm < TMB; ++tm)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        v4f v = buffer_load_v4f(ar, a_voff[tm][c]);
+                        v.x = (4 * c + 0 < mine) ? v.x : 0.f;
+                        v.y = (4 * c + 1 < mine) ? v.y : 0.f;
+                        v.z = (4 * c + 2 < mine) ? v.z : 0.f;
+                        v.w = (4 * c + 3 < mine) ? v.w : 0.f;
+                        ra[S][tm][c] = v;
+                    }
+            }
 #pragma unroll
             for (int t = 0; t < kRun; ++t) {
                 const int r = kRun * lh + t;
@@ -99,10 +123,22 @@ __global__ __launch_bounds__(kSmallThreads, MIN_BLOCKS) void sgemm_small_kernel(
                 rb[S][t] = (r < valid) ? v : 0.f;
             }
         } else {
+            if constexpr (TA) {
+                int soff = 0;  // one running scalar offset, as for B below
 #pragma unroll
-            for (int tm = 0; tm < TMB; ++tm)
+                for (int t = 0; t < kRun; ++t) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) ra[S][tm][c] = buffer_load_v4f(ar, a_voff[tm][c]);
+                    for (int tm = 0; tm < TMB; ++tm)
+                        ra[S][tm][t / 4][t % 4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, at_voff + tm * 128, soff, 0));
+                    soff += at_row_bytes;
+                    asm volatile("" : "+s"(soff));
+                }
+            } else {
+#pragma unroll
+                for (int tm = 0; tm < TMB; ++tm)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) ra[S][tm][c] = buffer_load_v4f(ar, a_voff[tm][c]);
+            }
             if constexpr (EDGE) {
                 // one running scalar offset instead of sixteen live ones: this variant is short of scalar registers
                 int soff = 0;
@@ -120,8 +156,13 @@ __global__ __launch_bounds__(kSmallThreads, MIN_BLOCKS) void sgemm_small_kernel(
         }
     };
     auto hop = [&]() {
-        a_base += kSmallWaves * BK;
-        a_left -= kSmallWaves * BK * 4;
+        if constexpr (TA) {
+            a_base += a_hop;
+            a_left -= a_hop * 4;
+        } else {
+            a_base += kSmallWaves * BK;
+            a_left -= kSmallWaves * BK * 4;
+        }
         b_base += b_hop;
         b_left -= b_hop * 4;
     };

@@ -1,8 +1,9 @@
 // SGEMM kernels for a transposed left operand (A^T given as a K x M row-major matrix), in a translation unit of their
 // own so that they compile beside the others.  The table is built from the same tile list as the one in sgemm.hip
-// (sgemm_tiles.h); the 32 x 32 tile, whose lanes fetch their own operands, has no such variant.
+// (sgemm_tiles.h).
 #include "gemm_host.h"
 #include "sgemm_persistent_kernel.h"
+#include "sgemm_small_kernel.h"
 #include "sgemm_tiles.h"
 
 namespace hpcdnn {
@@ -31,7 +32,8 @@ struct TaKernels {
 #define HPCDNN_TILE_PERSISTENT_BIG(BM, BN, WGM, WGN, OCC, EFF) \
     HPCDNN_TA_(BM, BN, WGM, WGN, OCC, 2, (sgemm_persistent_kernel<BM, BN, WGM, WGN, false, 64, 1, true>), nullptr)
 #define HPCDNN_TILE_DEEP(BM, BN, WGM, WGN, OCC, EFF, NSLOT) HPCDNN_TA_(BM, BN, WGM, WGN, OCC, NSLOT, nullptr, nullptr)
-#define HPCDNN_SMALL_TILE(TMB, OCC, EFF) {32 * TMB, 32, nullptr, nullptr, nullptr, nullptr}
+#define HPCDNN_SMALL_TILE(TMB, OCC, EFF) \
+    {32 * TMB, 32, sgemm_small_kernel<TMB, false, OCC, true>, sgemm_small_kernel<TMB, true, OCC, true>, nullptr, nullptr}
 
 const TaKernels kTaKernels[] = {HPCDNN_SGEMM_TILE_LIST};
 }  // namespace

@@ -115,8 +115,7 @@ int hpcdnn_sgemm_ex(int M, int N, int K, const float* A, int lda, const float* B
  * element of C sums its products in the order hpcdnn_sgemm uses, so the result
  * has the bits of hpcdnn_sgemm on the explicitly transposed operand.  This is the
  * operand layout of the reference's column-major family (below).  The _ex form
- * pins tile and split as hpcdnn_sgemm_ex does; the 32 x 32 tile is not available
- * (HPCDNN_ERR_INVALID_VALUE). */
+ * pins tile and split as hpcdnn_sgemm_ex does. */
 int hpcdnn_sgemm_tn(int M, int N, int K, const float* At, int ldat, const float* B, int ldb, float* C, int ldc,
                     float alpha, float beta, void* ws, size_t ws_bytes, void* stream);
 int hpcdnn_sgemm_tn_ex(int M, int N, int K, const float* At, int ldat, const float* B, int ldb, float* C, int ldc,

@@ -73,7 +73,7 @@ def test_bad_arguments_are_rejected_without_a_gpu(L):
     assert L.hpcdnn_sgemm(4, 4, 4, dummy, 4, dummy, 4, dummy, 3, 1.0, 0.0, None, 0, None) == INVALID
     assert L.hpcdnn_sgemm(4, 4, 4, None, 4, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
     assert L.hpcdnn_sgemm(0, 4, 4, None, 4, None, 4, None, 4, 1.0, 0.0, None, 0, None) == 0  # empty: nothing to do
-    # transposed left operand: At is K x M, so its row length must reach M (not K); the 32 x 32 tile has no such kernel
+    # transposed left operand: At is K x M, so its row length must reach M (not K)
     assert L.hpcdnn_sgemm_tn(8, 4, 4, dummy, 7, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, None) == INVALID
     assert L.hpcdnn_sgemm_tn(4, 4, 8, dummy, 4, dummy, 4, dummy, 3, 1.0, 0.0, None, 0, None) == INVALID
     assert L.hpcdnn_sgemm_tn(0, 4, 4, None, 1, None, 4, None, 4, 1.0, 0.0, None, 0, None) == 0
@@ -92,7 +92,7 @@ def test_bad_arguments_are_rejected_without_a_gpu(L):
     assert L.hpcdnn_sgemm_ex(4, 4, 64, dummy, 64, dummy, 4, dummy, 4, 1.0, 0.0, None, 0, 0, 2, None) == WORKSPACE
     # the 32 x 32 tile has no tail split (its waves split K among themselves)
     small = [t for t in range(L.hpcdnn_sgemm_num_tiles()) if _tile(L, t)[:2] == (32, 32)]
-    assert L.hpcdnn_sgemm_tn_ex(64, 64, 64, dummy, 64, dummy, 64, dummy, 64, 1.0, 0.0, None, 0, small[0], 1, None) == INVALID
+    assert L.hpcdnn_sgemm_tn_ex(256, 1056, 256, dummy, 256, dummy, 1056, dummy, 1056, 1.0, 0.0, dummy, 1 << 30, small[0], -2, None) == INVALID
     assert len(small) == 1
     assert L.hpcdnn_sgemm_ex(256, 1056, 256, dummy, 256, dummy, 1056, dummy, 1056, 1.0, 0.0, dummy, 1 << 30, small[0], -2, None) == INVALID
     # leading dimensions beyond the 32-bit tile offsets
