@@ -172,14 +172,15 @@ __device__ __forceinline__ v4f buffer_load_v4f_nt(__amdgpu_buffer_rsrc_t rsrc, i
 // 128 slices cost one trip to memory where a lane that walks them eight at a time makes eight), and the four partial
 // sums are combined as
 // (q0 + q1) + (q2 + q3) by exchanges with lane ^ 16 and lane ^ 32: a fixed order, the same bits on every run.
-// A wave covers 16 groups (256 contiguous bytes per slice) x 4 quarters.
-template <int kUnused = 0>
-__global__ __launch_bounds__(256) void splitk_reduce_wide_kernel(int M, int N, int splits, const float* __restrict__ ws,
+// A wave covers 16 groups (256 contiguous bytes per slice) x 4 quarters; a block is kWaves waves (one when there are
+// so few elements that blocks of four would leave most CUs without one).
+template <int kWaves = 4>
+__global__ __launch_bounds__(64 * kWaves) void splitk_reduce_wide_kernel(int M, int N, int splits, const float* __restrict__ ws,
                                                                  float* __restrict__ C, int ldc, float alpha, float beta) {
     const int64_t total = static_cast<int64_t>(M) * N;
     const int lane = threadIdx.x & (kWave - 1);
     const int q = lane >> 4;
-    const int64_t e = (static_cast<int64_t>(blockIdx.x) * 64 + (threadIdx.x / kWave) * 16 + (lane & 15)) * 4;
+    const int64_t e = (static_cast<int64_t>(blockIdx.x) * (16 * kWaves) + (threadIdx.x / kWave) * 16 + (lane & 15)) * 4;
     const int per = (splits + 3) / 4;
     const int z0 = q * per, z1 = (z0 + per < splits) ? z0 + per : splits;
     v4f s = {0.f, 0.f, 0.f, 0.f};
@@ -215,6 +216,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_wide_kernel(int M, int N, i
             dst[c] = (beta == 0.f) ? t : __builtin_fmaf(beta, dst[c], t);
         }
     }
+}
+
+// Launch of the kernel above: one-wave blocks while blocks of four waves would number fewer than the CUs.
+inline void launch_splitk_reduce_wide(int M, int N, int splits, const float* ws, float* C, int ldc, float alpha, float beta,
+                                      int cus, hipStream_t stream) {
+    const int64_t total = static_cast<int64_t>(M) * N;
+    if (total < static_cast<int64_t>(cus) * 256)
+        splitk_reduce_wide_kernel<1><<<static_cast<int>((total + 63) / 64), 64, 0, stream>>>(M, N, splits, ws, C, ldc, alpha, beta);
+    else
+        splitk_reduce_wide_kernel<4><<<static_cast<int>((total + 255) / 256), 256, 0, stream>>>(M, N, splits, ws, C, ldc, alpha, beta);
 }
 
 }  // namespace hpcdnn

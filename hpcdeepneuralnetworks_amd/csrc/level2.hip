@@ -322,7 +322,7 @@ static int run_sgemv(int trans, int M, int N, float alpha, const float* A, int l
     }
     if (chunks > 8 && N % 4 == 0 && (reinterpret_cast<uintptr_t>(partial) & 15u) == 0)
         // many chunks: the reduction that keeps all of a lane's slices in flight (y as a 1 x N matrix)
-        splitk_reduce_wide_kernel<><<<static_cast<int>(ceil_div(N, 256)), 256, 0, s>>>(1, N, chunks, partial, y, N, alpha, beta);
+        launch_splitk_reduce_wide(1, N, chunks, partial, y, N, alpha, beta, device_cus(), s);
     else if (chunks > 1)
         sgemv_t_finish_kernel<<<static_cast<int>(ceil_div(N, kGemvThreads)), kGemvThreads, 0, s>>>(N, chunks, alpha, partial,
                                                                                                   beta, y);

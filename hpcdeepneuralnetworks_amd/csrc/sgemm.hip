@@ -388,8 +388,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     const int64_t total = static_cast<int64_t>(M) * N;
     if (split > 8 && N % 4 == 0 && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0) {
         // many slices: four lanes per group of elements, so that all of a lane's slices are in flight at once
-        splitk_reduce_wide_kernel<><<<static_cast<int>(ceil_div(total, 256)), 256, 0, stream>>>(M, N, split, static_cast<const float*>(ws), C,
-                                                                                         ldc, alpha, beta);
+        launch_splitk_reduce_wide(M, N, split, static_cast<const float*>(ws), C, ldc, alpha, beta, device_cus(), stream);
         return launch_status();
     }
     int rgrid = static_cast<int>(ceil_div(total, 256));
