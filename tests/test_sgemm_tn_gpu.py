@@ -217,6 +217,29 @@ def test_operands_that_start_four_bytes_off_a_16_byte_boundary(blas, oracle_mod)
     assert oracle_mod.gemm_max_err(M, dc.cpu().numpy(), ldc, ref, den) <= TOL
 
 
+def test_alternating_layouts_on_one_thread(blas):
+    """The library remembers its last plan per thread; calls that alternate between the two layouts (and between shapes
+    that take two launches over row ranges, a K split and a plain launch) must not pick up each other's decision."""
+    shapes = [(3584, 3584, 256, False), (128, 128, 8192, True), (700, 300, 200, False)]
+    ops = []
+    for i, (M, N, K, use_ws) in enumerate(shapes):
+        a = torch.empty(M, K, device="cuda")
+        b = torch.empty(K, N, device="cuda")
+        blas.fill_uniform_matrix(a, M, K, 60 + i)
+        blas.fill_uniform_matrix(b, K, N, 70 + i)
+        ws = blas.workspace(max(blas.sgemm_workspace_bytes(M, N, K), 1 << 16)) if use_ws else None
+        ref = torch.empty(M, N, device="cuda")
+        blas.sgemm(M, N, K, a, b, ref, 1.0, 0.0, ws=ws)
+        ops.append((M, N, K, a, a.t().contiguous(), b, ws, ref))
+    for rep in range(3):
+        for (M, N, K, a, at, b, ws, ref) in ops:
+            c1 = torch.full((M, N), float("nan"), device="cuda")
+            c2 = torch.full((M, N), float("nan"), device="cuda")
+            blas.sgemm_tn(M, N, K, at, b, c1, 1.0, 0.0, ws=ws)
+            blas.sgemm(M, N, K, a, b, c2, 1.0, 0.0, ws=ws)
+            assert torch.equal(c1, ref) and torch.equal(c2, ref), (rep, M, N, K)
+
+
 def test_maximum_leading_dimensions(blas):
     """ldat and ldb at the documented limit of the K-major operands (a K step is 16 of their rows; byte offsets inside one
     tile are 32-bit) and ldc at its own, for several kernel families and for the ABFT entry point; one more is refused."""
