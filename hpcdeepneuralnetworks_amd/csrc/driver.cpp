@@ -196,6 +196,18 @@ int run_ft_sgemm(int start, int end, int gap, int first, int last) {
             std::printf("Failed to pass the correctness verification against plain SGEMM (max |diff| %g). Exited.\n", d);
             return 3;
         }
+        // the same on the column-major operands the reference's check uses, cublasSgemm(N, T, ...) against its kernels
+        // (kernel/ft_sgemm/sgemm.cu:111): the buffers read as the column-major n x K, n x K and n x n matrices
+        LIB_OK(hpcdnn_fill_uniform(c, static_cast<int64_t>(nn), 3, nullptr));
+        LIB_OK(hpcdnn_fill_uniform(c_ref, static_cast<int64_t>(nn), 3, nullptr));
+        LIB_OK(hpcdnn_sgemm_cm_nt(n, n, K, a, n, b, n, c_ref, n, alpha, beta, nullptr, 0, nullptr));
+        LIB_OK(hpcdnn_ft_sgemm_cm_nt(n, n, K, a, n, b, n, c, n, alpha, beta, 0.f, nullptr, nullptr, ft_ws, ft_ws_bytes, nullptr));
+        HIP_OK(hipDeviceSynchronize());
+        const double d_cm = max_abs_diff(c, c_ref, static_cast<size_t>(n) * n);
+        if (!(d_cm <= 1e-2)) {
+            std::printf("Failed to pass the correctness verification on column-major operands (max |diff| %g). Exited.\n", d_cm);
+            return 3;
+        }
         std::printf("finish verified!\n");
     }
     // the device has idled through the host-side comparison: bring its clocks back up before the first series
