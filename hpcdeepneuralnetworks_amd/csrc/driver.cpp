@@ -118,7 +118,7 @@ struct Series {
     int number;        // the reference's kernel_number (kernel/ft_sgemm/sgemm.cu:186)
     const char* name;  // the reference's series name (:187-188) where a counterpart exists
     int kind;          // 0 plain SGEMM, 1 offline ABFT, 2 ABFT without workspace, 3 ABFT with workspace, 4 wave-tile ABFT,
-                       // 5 / 6 plain SGEMM / ABFT on column-major operands
+                       // 5 / 6 plain SGEMM / ABFT on column-major operands, 7 a name without a kernel (empty list)
     int tile;          // plain SGEMM: row of the tile table, -1 = chosen by the library; ABFT: tile class
 };
 
@@ -137,8 +137,12 @@ const Series kSeries[] = {
     {14, "abft_kernel_tall", 2, 3},    // 128 x 64
     {15, "abft_kernel_wide", 2, 2},    // 64 x 128
     {16, "abft_kernel_huge", 2, 0},    // 256 x 128
+    // the thread-level kernel (kernel/ft_sgemm/sgemm.cu:188) has no counterpart on matrix cores: a matrix-core result
+    // is spread over all 64 lanes of a wave, so the finest unit with accumulators of its own is the wave tile.  The
+    // series keeps its name with an empty list, so that scripts that look the name up find it.
+    {17, "thread_abft_kernel", 7, 0},
     // one checksum pair per wave tile (128 x 32 of the 256 x 128 tile): the matrix-core counterpart of the warp-level
-    // kernel; the thread-level one (series 17) has none, a matrix-core result being spread over all lanes of a wave
+    // kernel
     {18, "warp_abft_kernel", 4, 0},
     // no reference counterpart: checksum vectors from the pre-pass
     {19, "abft_kernel_huge_workspace", 3, 0},
@@ -217,6 +221,10 @@ int run_ft_sgemm(int start, int end, int gap, int first, int last) {
         if (sr.number < first) continue;
         if (sr.number > last) break;
         std::printf("%s = th.as_tensor([", sr.name);
+        if (sr.kind == 7) {
+            std::printf("])  # no per-thread checksums on matrix cores: the wave tile is the finest granularity (warp_abft_kernel)\n");
+            continue;
+        }
         for (int n = start; n <= end; n += gap) {
             LIB_OK(hpcdnn_fill_uniform(c, static_cast<int64_t>(nn), 3, nullptr));
             const double flop = 2.0 * n * static_cast<double>(n) * K;

@@ -106,6 +106,16 @@ static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
     return tile_mode > wave_mode ? tile_mode : wave_mode;
 }
 
+// K == 0 with wave-tile granularity: there is nothing to verify, every check tile gets a clean record
+__global__ __launch_bounds__(256) void ft_clean_status_kernel(hpcdnn_ft_status* __restrict__ status, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    hpcdnn_ft_status st;
+    st.flag = 0; st.row = -1; st.col = -1; st.n_bad_rows = 0; st.n_bad_cols = 0;
+    st.row_residual = 0.f; st.col_residual = 0.f; st.max_clean_residual = 0.f;
+    status[i] = st;
+}
+
 // ta: A is given transposed (K x M row-major, lda >= M)
 static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
                         float alpha, float beta, float tau, const hpcdnn_ft_options& opt, hpcdnn_ft_status* status, void* ws,
@@ -126,11 +136,12 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     if (wave && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
 
     GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, fc.bm, fc.bn);
-    // tau > 0: absolute; tau == 0: the absolute default for unit-range data; tau < 0: scaled to the data, the
-    // threshold of a line of n elements being -tau * 4.3 FP32 rounding units * sqrt(max(K, 64)) * sqrt(n) * the larger
-    // of the line's and the check tile's mean |accumulator|
-    a.tau = (tau > 0.f) ? tau : (tau == 0.f ? hpcdnn_ft_default_tau(K) : 0.f);
-    a.tau_rel = (tau < 0.f) ? -tau * 2.56e-7f * sqrtf(static_cast<float>(K > 64 ? K : 64)) : 0.f;
+    // tau > 0: absolute; tau <= 0: scaled to the data, the threshold of a line of n elements being f * 4.3 FP32
+    // rounding units * sqrt(max(K, 64)) * sqrt(n) * the larger of the line's and the check tile's mean |accumulator|,
+    // with f = -tau, or 1 for tau == 0 (the default: a threshold that follows the size and the mean of the operands
+    // cannot flag a fault-free product the way a constant calibrated for unit-range data does)
+    a.tau = (tau > 0.f) ? tau : 0.f;
+    a.tau_rel = (tau > 0.f) ? 0.f : (tau < 0.f ? -tau : 1.f) * 2.56e-7f * sqrtf(static_cast<float>(K > 64 ? K : 64));
     a.status = status;
     a.check_interval = cadence ? opt.check_interval : 0;
     int cm = 0, cn = 0;
@@ -151,6 +162,18 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         a.faults[f].col = (scol % gn) * cn + in.col;
         a.faults[f].delta = in.delta;
         a.faults[f].check = in.check;
+    }
+    if (K == 0 && wave) {
+        // an empty product: C = beta * C through the workgroup-tile kernel below, which would lay its records out per
+        // workgroup tile, so the wave-tile records are written here (all clean; faults have nothing to hit)
+        if (status) {
+            const int n = a.status_rows * a.status_ld;
+            ft_clean_status_kernel<<<static_cast<int>(ceil_div(n, 256)), 256, 0, s>>>(status, n);
+            rc = launch_status();
+            if (rc != HPCDNN_OK) return rc;
+        }
+        a.status = nullptr;
+        a.n_faults = 0;
     }
     const bool edge = needs_edge(a, fc.bm, fc.bn, kGemmBK);
     dim3 grid(a.tiles_m * a.tiles_n, 1, 1);

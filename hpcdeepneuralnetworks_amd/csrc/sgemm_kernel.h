@@ -104,7 +104,7 @@ constexpr size_t ft_verify_lds_bytes() {
     constexpr size_t threads = static_cast<size_t>(WGM) * WGN * 64;
     constexpr size_t ccp = threads / (BN / 4), crp = kGemmBK / 4, lines = static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
     return sizeof(double) * (GM * ccp * BN + GN * crp * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + lines) +
-           32 * GM * GN + sizeof(float) * GM * GN * (threads / 64);
+           32 * GM * GN + sizeof(float) * GM * GN * (threads / 64) + 2 * sizeof(float) * GM * GN;
 }
 
 template <int BM, int BN, int FT = 0, int THREADS = 256, int WGM = 2, int WGN = 2, int GRAN = 0>
@@ -940,6 +940,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     double line_off[LPT];          // CADENCE: what re-synchronisation has taken out of each of this thread's lines
 #pragma unroll
     for (int it = 0; it < LPT; ++it) line_off[it] = 0.0;
+    const int k_first = kbeg;      // first k of this workgroup's K range (kbeg moves on from interval to interval)
     hpcdnn_ft_status rec;          // thread ct < NCT: the record of check tile ct, merged over the verifications
     rec.flag = 0; rec.row = -1; rec.col = -1; rec.n_bad_rows = 0; rec.n_bad_cols = 0;
     rec.row_residual = 0.f; rec.col_residual = 0.f; rec.max_clean_residual = 0.f;
@@ -954,6 +955,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         float* const s_dr = s_crabs + WGN * BM;                         // [kLines] residuals
         int* const s_meta = reinterpret_cast<int*>(s_dr + kLines);      // [NCT][8] nbr, nbc, bad row, bad col, max clean (float bits)
         float* const s_tsum = reinterpret_cast<float*>(s_meta + 8 * NCT);  // [NCT][waves] partial sums of |acc| over a check tile
+        float* const s_fix = s_tsum + NCT * (kGemmThreads / kWave);        // [NCT][2] recomputed element, and what it changed
         static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads, WGM, WGN, GRAN>() >= ft_verify_lds_bytes<BM, BN, WGM, WGN, GM, GN>(),
                       "verification scratch fits in the kernel's LDS");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
@@ -973,6 +975,24 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             }
         };
 
+        // the same element set to val by its owner, who also leaves (val - old value) in *change
+        auto set_at = [&](int r, int c, float val, float* change) -> float {
+            const int rr = r % 32;
+            const int fi = (r % WM) / 32, fj = (c % WN) / 32, fv = 4 * (rr / 8) + rr % 4;
+            float old = 0.f;
+            if (wm == r / WM && wn == c / WN && lr == c % 32 && lh == (rr / 4) % 2) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (i == fi && j == fj && v == fv) { old = acc[i][j][v]; acc[i][j][v] = val; }
+                *change = val - old;
+            }
+            return old;
+        };
+
         // Soft-error injection: one accumulator per fault, after the K loop (or interval), before the checks
         // (run-time form of `t[2].x += error_inject`, ft_sgemm_huge.cuh:40,145).  A fault aimed at a row or column
         // of an edge tile that lies outside the matrix is ignored.  A kernel that verifies once injects every fault
@@ -985,7 +1005,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 m0 + p.faults[f].row < p.M && n0 + p.faults[f].col < p.N)
                 add_at(p.faults[f].row, p.faults[f].col, p.faults[f].delta);
 
-        if (tid < NCT) { s_meta[8 * tid] = 0; s_meta[8 * tid + 1] = 0; s_meta[8 * tid + 2] = -1; s_meta[8 * tid + 3] = -1; s_meta[8 * tid + 4] = 0; }
+        if (tid < NCT) { s_meta[8 * tid] = 0; s_meta[8 * tid + 1] = 0; s_meta[8 * tid + 2] = -1; s_meta[8 * tid + 3] = -1; s_meta[8 * tid + 4] = 0; s_fix[2 * tid + 1] = 0.f; }
 
         // reference checksums: every thread publishes its partial sums (columns nc..nc+3 over its k rows, its
         // rows over its k group); the residual step below adds the partials in a fixed order
@@ -1148,16 +1168,68 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         }
         __syncthreads();
 
-        // locate: one faulty row x one faulty column of a check tile (ft_sgemm_huge.cuh:273-296); correct with the
-        // signed row residual (the reference's round(|residual|), :358, only fits its +1.0 test fault)
+        // locate: one faulty row x one faulty column of a check tile (ft_sgemm_huge.cuh:273-296).  Correct: the
+        // reference subtracts round(|residual|) (:352-371), which only fits its +1.0 test fault, and the signed row
+        // residual would leave the fault-free rounding noise of a whole row in one element; the located accumulator
+        // is computed again from A and B instead.  One lane walks the k range done so far with one fused multiply-add
+        // per k in the order the matrix core adds them (per K step and half step g, the pairs k = 8g + q, 8g + 4 + q
+        // for q = 0..3: a 32x32x2 FP32 MFMA is two chained FMAs, lanes 0-31's k first), so the element gets exactly
+        // the bits a fault-free run gives it.  The operand row and column are staged through the LDS the reference
+        // partials no longer need, a chunk of kFixChunk values of k at a time, by all threads (the condition is
+        // uniform over the workgroup); zeros pad the last K step.
+        bool any_fixed = false;
 #pragma unroll 1
         for (int ct = 0; ct < NCT; ++ct) {
-            const int gn = ct % GN;
             if (s_meta[8 * ct] == 1 && s_meta[8 * ct + 1] == 1) {
                 const int bad_r = s_meta[8 * ct + 2], bad_c = s_meta[8 * ct + 3];
-                add_at(bad_r, bad_c, s_dr[gn * BM + bad_r]);
+                if (m0 + bad_r >= p.M || n0 + bad_c >= p.N) continue;  // (lines outside the matrix are all zeros: not reached)
+                constexpr int kFixChunk = static_cast<int>(sizeof(double) * (GM * CCP * BN + GN * CRP * BM) / (2 * sizeof(float))) / BK * BK;
+                float* const s_fa = smem;
+                float* const s_fb = smem + kFixChunk;
+                const float* const a_src = TA ? p.A + (m0 + bad_r) : p.A + static_cast<int64_t>(m0 + bad_r) * p.lda;
+                const float* const b_src = p.B + (n0 + bad_c);
+                float fixed_val = 0.f;
+#pragma unroll 1
+                for (int kc = k_first; kc < kend; kc += kFixChunk) {
+                    const int len = (kend - kc < kFixChunk) ? kend - kc : kFixChunk;
+                    const int padded = (len + BK - 1) / BK * BK;
+#pragma unroll 1
+                    for (int i = tid; i < padded; i += kGemmThreads) {
+                        const int k = kc + i;
+                        s_fa[i] = i < len ? (TA ? a_src[static_cast<int64_t>(k) * p.lda] : a_src[k]) : 0.f;
+                        s_fb[i] = i < len ? b_src[static_cast<int64_t>(k) * p.ldb] : 0.f;
+                    }
+                    __syncthreads();
+                    if (tid == 0) {
+#pragma unroll 1
+                        for (int i = 0; i < padded; i += BK) {
+                            float av[BK], bv[BK];
+#pragma unroll
+                            for (int e = 0; e < BK; e += 4) {
+                                *reinterpret_cast<v4f*>(av + e) = *reinterpret_cast<const v4f*>(s_fa + i + e);
+                                *reinterpret_cast<v4f*>(bv + e) = *reinterpret_cast<const v4f*>(s_fb + i + e);
+                            }
+#pragma unroll
+                            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                                for (int q = 0; q < 4; ++q) {
+                                    fixed_val = __builtin_fmaf(av[8 * g + q], bv[8 * g + q], fixed_val);
+                                    fixed_val = __builtin_fmaf(av[8 * g + 4 + q], bv[8 * g + 4 + q], fixed_val);
+                                }
+                        }
+                    }
+                    __syncthreads();
+                }
+                // thread 0 hands the value to the accumulator's owner, who reports what the correction changed
+                // (the re-synchronisation takes exactly that out of the two lines' residuals)
+                if (tid == 0) s_fix[2 * ct] = fixed_val;
+                __syncthreads();
+                const float old_val = set_at(bad_r, bad_c, s_fix[2 * ct], &s_fix[2 * ct + 1]);
+                (void)old_val;
+                any_fixed = true;
             }
         }
+        if (CADENCE && any_fixed) __syncthreads();  // s_fix[2 ct + 1] = corrected - faulty value, for the resync below
         if constexpr (CADENCE) {
             // re-synchronise (ft_sgemm_huge.cuh:268-271): every line starts the next interval with what is left of
             // its residual after the correction taken out of its reference
@@ -1172,7 +1244,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     const int ct = gm * GN + gn;
                     double fixed = 0.0;
                     if (s_meta[8 * ct] == 1 && s_meta[8 * ct + 1] == 1 && idx == s_meta[8 * ct + (is_row ? 2 : 3)])
-                        fixed = static_cast<double>(s_dr[gn * BM + s_meta[8 * ct + 2]]);
+                        fixed = static_cast<double>(s_fix[2 * ct + 1]);
                     line_off[it] += d_line[it] - fixed;
                 }
             }

@@ -158,13 +158,18 @@ __global__ __launch_bounds__(kVecThreads) void sdot_kernel(int64_t n, const floa
 
     // Cross-block hand-off without cache-wide fences (a device-scope release/acquire fence writes back and
     // invalidates the whole L2 of the XCD, which costs a streaming kernel a quarter of its bandwidth).  All
-    // traffic on the partials and the ticket is device-scope atomic read-modify-write, performed at the point
-    // of coherence shared by the 8 XCDs: the ticket is drawn only after the exchange that published the
-    // partial has returned, and the last block reads the partials back with atomic adds of zero.
+    // traffic on the partials and the ticket is device-scope atomic read-modify-write.  Hardware assumption: a
+    // device-scope read-modify-write is performed at the point of coherence shared by the 8 XCDs, and its return
+    // value leaves that point only after the operation has been performed there.  The ticket's increment is made
+    // to depend on the value the exchange returned, so the ticket cannot issue before the exchange that
+    // published the partial has been performed; the last block reads the partials back with atomic adds of zero.
     if (threadIdx.x == 0) {
         const double old = __hip_atomic_exchange(&partials[blockIdx.x], block_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // data dependency on `old`: the ticket cannot issue before the exchange has completed
-        const unsigned int one = (__builtin_bit_cast(unsigned long long, old) == 0x7ff8dead0000beefull) ? 2u : 1u;
+        // zero for every bit pattern of `old`, through an instruction the compiler cannot see into: a data
+        // dependency without a special value
+        unsigned int dep = static_cast<unsigned int>(__builtin_bit_cast(unsigned long long, old));
+        asm volatile("v_and_b32 %0, 0, %0" : "+v"(dep));
+        const unsigned int one = 1u + dep;
         const unsigned int t = __hip_atomic_fetch_add(ticket, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = (t == gridDim.x - 1);
     }

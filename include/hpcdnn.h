@@ -154,13 +154,15 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * tile are accumulated from A and B inside the main loop, compared with the
  * line sums of the accumulators in the epilogue, and a single faulty element
  * per tile is located (faulty row x faulty column) and corrected before
- * alpha/beta are applied.  `tau` > 0 is an absolute residual threshold, 0
- * selects the default for inputs of magnitude <= 1 (hpcdnn_ft_default_tau),
- * and `tau` < 0 scales the threshold to the data: a line of n elements is
- * flagged when its residual exceeds -tau * 2.56e-7 * sqrt(max(K, 64)) *
+ * alpha/beta are applied.  `tau` > 0 is an absolute residual threshold
+ * (hpcdnn_ft_default_tau(K) is one calibrated for operands uniform in [-1, 1];
+ * on larger or non-zero-mean data a constant flags fault-free products), and
+ * `tau` <= 0 scales the threshold to the data: a line of n elements is
+ * flagged when its residual exceeds f * 2.56e-7 * sqrt(max(K, 64)) *
  * sqrt(n) * m, m being the larger of the mean |accumulator| of the line and
- * of the whole tile, -1 being calibrated to twice the largest fault-free
- * residual of uniform operands; `inject` is a HOST
+ * of the whole tile and f = -tau, or 1 for `tau` == 0, the default (f = 1 is
+ * calibrated to twice the largest fault-free residual of uniform operands and
+ * follows the data when it is scaled or shifted); `inject` is a HOST
  * pointer to one fault or NULL; `status` is DEVICE memory for
  * hpcdnn_ft_num_tiles(M,N) records or NULL.
  * `ws`/`ws_bytes`: optional DEVICE scratch of
@@ -176,14 +178,16 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * tile's (bad-line counts add up; the location is that of the first slice that
  * corrected something).  A workspace that only holds the checksum vectors
  * (the size without that room) runs without the split.
- * Accuracy of a corrected element: the correction is the FP32-rounded row
- * residual, so with a fault of size delta the element ends up within
- *   |fault-free row residual| + 16 * 2^-24 * |delta|
- * of its fault-free accumulator (before alpha/beta): the first term is the
- * rounding noise the threshold is calibrated against (below tau / 2 for the
- * default), the second the rounding of the FP32 line sums that contain the
- * fault.  It does not scale with (|A||B|)_ij: for K of a few tens and a large
- * delta it can exceed the 1e-5 componentwise criterion of the plain product.
+ * A corrected element: the located accumulator is computed again from its
+ * row of A and column of B, one fused multiply-add per k in the order the
+ * matrix cores add them, and replaces the faulty value; a corrected product
+ * therefore has exactly the bits of a fault-free one, whatever the size of the
+ * fault (the reference subtracts a rounded residual at this point,
+ * kernel/ft_sgemm/include/ft_sgemm_huge.cuh:352-371).  The signed residuals of
+ * the located row and column are reported in the record (minus the fault, to
+ * within the rounding of the line sums).  The recomputation costs a launch
+ * that corrects about 3 us per 1024 values of k and a fault-free launch
+ * nothing.
  * Replaces ft_sgemm_huge <<<dim3(M/128,N/128),256>>>(M,N,K,A,B,C,alpha,beta)
  * (kernel/ft_sgemm/sgemm.cu:159-165, kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21). */
 int hpcdnn_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
@@ -287,10 +291,11 @@ int hpcdnn_ft_check_tile_info(int tile_class, int granularity, int* cm, int* cn)
 int hpcdnn_ft_num_check_tiles(int tile_class, int granularity, int M, int N);
 int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N);
 int hpcdnn_ft_pick_class(int M, int N, int K);
-/* Threshold hpcdnn_ft_sgemm uses when tau == 0: 1.1e-6 * max(K, 64), twice the
- * largest fault-free residual measured for operands uniform in [-1, 1] (the
- * rounding noise of the FP32 accumulators grows linearly with K).  Scale it by
- * max|A| * max|B| for other data. */
+/* An absolute threshold for operands uniform in [-1, 1], to be passed as
+ * `tau`: 1.1e-6 * max(K, 64), twice the largest fault-free residual measured
+ * for such operands (the rounding noise of the FP32 accumulators grows
+ * linearly with K).  It is not what tau == 0 selects: that is the data-scaled
+ * threshold, which needs no knowledge of the operands. */
 float hpcdnn_ft_default_tau(int K);
 
 /* hpcdnn_ft_sgemm for callers that cannot allocate device memory or carry a

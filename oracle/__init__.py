@@ -86,6 +86,11 @@ def _load():
     lib.oracle_sdot_f64.argtypes = [C.c_int64, fp, fp]
     lib.oracle_sdot_f32.restype = C.c_float
     lib.oracle_sdot_f32.argtypes = [C.c_int64, fp, fp]
+    lib.oracle_recompute_element.restype = C.c_float
+    lib.oracle_recompute_element.argtypes = [C.c_int, C.c_int, fp, fp, C.c_int]
+    lib.oracle_sgemm_device_order.restype = None
+    lib.oracle_sgemm_device_order.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int,
+                                              C.c_float, C.c_float]
     lib.oracle_tile_acc.restype = None
     lib.oracle_tile_acc.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp]
     lib.oracle_abft_reference_checksums.restype = None
@@ -204,6 +209,18 @@ def sdot_f64(x: np.ndarray, y: np.ndarray) -> float:
 
 def sdot_f32(x: np.ndarray, y: np.ndarray) -> float:
     return float(_load().oracle_sdot_f32(x.size, _f(x), _f(y)))
+
+
+def recompute_element(a_row: np.ndarray, b_col: np.ndarray, ldb: int, k0: int, k1: int) -> float:
+    """The accumulator of one element formed again over k0 <= k < k1: a_row points at the element's row of A, b_col at
+    its column's first element of B (rows ldb apart)."""
+    return float(_load().oracle_recompute_element(k0, k1, _f(a_row), _f(b_col), ldb))
+
+
+def sgemm_device_order(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta) -> None:
+    """C = alpha*A*B + beta*C in place, in the summation order of the device's tile kernels (float accumulator,
+    one fused multiply-add per k, k permuted inside each group of 16): the bits an unsplit device product has."""
+    _load().oracle_sgemm_device_order(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta)
 
 
 def tile_acc(a_tile, lda, b_tile, ldb, tm, tn, K) -> np.ndarray:

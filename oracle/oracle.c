@@ -33,6 +33,12 @@
  *     (AB)e = A(Be)) and to the one known-answer case the reference holds
  *     (+1.0 at tile-local (0,1), threshold 0.1 -> row 0, col 1, magnitude 1;
  *     kernel/ft_sgemm/include/ft_sgemm_huge.cuh:40,145,263,358).
+ *   oracle_recompute_element (the correction: the located accumulator formed
+ *     again): pinned by K = 1 and exact-integer cases in which a corrected
+ *     product must equal the fault-free one bit for bit.
+ *   oracle_sgemm_device_order (a model of this library's own summation
+ *     order, no reference counterpart): pinned to numpy float64 within the
+ *     FP32 bound and to a hand case that k ascending fails.
  *   oracle_tile_acc (the FP32 accumulator model of the fault campaign):
  *     pinned to numpy float64 on a rectangular padded case, to a float
  *     accumulation-order case and to a hand case a transposed operand fails.
@@ -298,9 +304,11 @@ void oracle_abft_residuals(int tm, int tn, int K, const float* A, int lda, const
  * ft_sgemm_huge.cuh:263-271), locate the element where one faulty row meets
  * one faulty column (:273-296) and report the correction to apply.  The
  * reference subtracts round(sum |row residuals|) (:358), which is only right
- * for its +1.0 test fault; the sound value for any magnitude is the signed
- * row residual, added back to the accumulator (acc += dr[row]).
- * Returns the correction (0 when nothing is corrected). */
+ * for its +1.0 test fault; the signed row residual measures the fault for any
+ * magnitude, but adding it back would leave the row's fault-free rounding
+ * noise in one element, so the models below compute the located accumulator
+ * again (oracle_recompute_element) and use the residual as a report only.
+ * Returns the signed row residual of the located row (0 when nothing is located). */
 /* Per-line thresholds: tau_r[m] for row m, tau_c[n] for column n. */
 float oracle_abft_decide_lines(int tm, int tn, const double* dr, const double* dc, const double* tau_r,
                                const double* tau_c, oracle_ft_status* st) {
@@ -374,11 +382,49 @@ void oracle_abft_relative_thresholds(int tm, int tn, int K, const float* acc, in
     }
 }
 
+/* Step 6 (correct): the located accumulator computed again from row `a` of A (stride 1) and column `b` of B
+ * (stride ldb) over k0 <= k < k1, in the arithmetic of oracle_tile_acc (float accumulator, one fused multiply-add
+ * per k, k ascending).  It replaces the faulty accumulator, so a corrected product has the bits of a fault-free one
+ * (the reference's correction site, ft_sgemm_huge.cuh:352-371, subtracts a rounded residual instead). */
+float oracle_recompute_element(int k0, int k1, const float* a, const float* b, int ldb) {
+    float acc = 0.0f;
+    for (int k = k0; k < k1; ++k) acc = fmaf(a[k], b[(size_t)k * ldb], acc);
+    return acc;
+}
+
+/* Row-major SGEMM in the arithmetic of the device's tile kernels: a float accumulator per element, one fused
+ * multiply-add per k, k taken K step by K step (16 values) in the order 0,4,1,5,2,6,3,7,8,12,9,13,10,14,11,15 - the
+ * order in which the 32x32x2 FP32 matrix-core instruction (two chained FMAs, lanes 0-31's k first) meets the
+ * k-permuted operand fragments -, then C = alpha*acc + beta*C (C is not read when beta == 0).  A model of this
+ * library's kernels, not of the reference: it predicts the bits of an unsplit product. */
+void oracle_sgemm_device_order(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                               int ldc, float alpha, float beta) {
+    static const int order[16] = {0, 4, 1, 5, 2, 6, 3, 7, 8, 12, 9, 13, 10, 14, 11, 15};
+    #pragma omp parallel for schedule(static)
+    for (int m = 0; m < M; ++m) {
+        float* acc = (float*)calloc((size_t)(N > 0 ? N : 1), sizeof(float));
+        for (int k0 = 0; k0 < K; k0 += 16)
+            for (int o = 0; o < 16; ++o) {
+                int k = k0 + order[o];
+                if (k >= K) continue;
+                float a = A[(size_t)m * lda + k];
+                const float* brow = B + (size_t)k * ldb;
+                for (int n = 0; n < N; ++n) acc[n] = fmaf(a, brow[n], acc[n]);
+            }
+        for (int n = 0; n < N; ++n) {
+            float* c = &C[(size_t)m * ldc + n];
+            float v = alpha * acc[n];
+            *c = (beta == 0.0f) ? v : fmaf(beta, *c, v);
+        }
+        free(acc);
+    }
+}
+
 /* Whole-matrix model: C = alpha*acc + beta*C with acc = A*B accumulated in
  * float (k ascending), one fault (tile index in row-major tile order,
  * tile-local i, j, delta added to acc before verification) or none
  * (fault_tile < 0), tiles of tile_m x tile_n (edge tiles are clipped), tau > 0
- * absolute or tau < 0 data-scaled with factor -tau, one
+ * absolute or tau <= 0 data-scaled with factor -tau (factor 1 for tau == 0), one
  * status record per tile.  Mirrors the device entry point's contract; used on
  * sizes the CPU finishes in seconds. */
 void oracle_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
@@ -405,15 +451,18 @@ void oracle_ft_sgemm(int M, int N, int K, const float* A, int lda, const float* 
         if (t == fault_tile && fault_i < tm && fault_j < tn) acc[(size_t)fault_i * tn + fault_j] += fault_delta;
         oracle_abft_residuals(tm, tn, K, A + (size_t)m0 * lda, lda, B + n0, ldb, acc, tn, dr, dc);
         float fix;
-        if (tau < 0.0f) {
+        if (tau <= 0.0f) {
             double* thr = (double*)malloc(sizeof(double) * (size_t)(tm + tn));
-            oracle_abft_relative_thresholds(tm, tn, K, acc, tn, -tau, thr, thr + tm);
+            oracle_abft_relative_thresholds(tm, tn, K, acc, tn, tau < 0.0f ? -tau : 1.0f, thr, thr + tm);
             fix = oracle_abft_decide_lines(tm, tn, dr, dc, thr, thr + tm, &status[t]);
             free(thr);
         } else {
             fix = oracle_abft_decide(tm, tn, dr, dc, tau, &status[t]);
         }
-        if (status[t].flag == 1) acc[(size_t)status[t].row * tn + status[t].col] += fix;
+        (void)fix;
+        if (status[t].flag == 1)
+            acc[(size_t)status[t].row * tn + status[t].col] =
+                oracle_recompute_element(0, K, A + (size_t)(m0 + status[t].row) * lda, B + n0 + status[t].col, ldb);
         for (int m = 0; m < tm; ++m)
             for (int n = 0; n < tn; ++n) {
                 float* c = &C[(size_t)(m0 + m) * ldc + n0 + n];
@@ -493,16 +542,23 @@ void oracle_ft_sgemm_checked(int M, int N, int K, const float* A, int lda, const
             oracle_abft_observe(tm, tn, acc, tn, part_r, part_c, dr, dc);
             oracle_ft_status cur;
             float fix;
-            if (tau < 0.0f) {
-                oracle_abft_relative_thresholds(tm, tn, K, acc, tn, -tau, thr, thr + tm);
+            if (tau <= 0.0f) {
+                oracle_abft_relative_thresholds(tm, tn, K, acc, tn, tau < 0.0f ? -tau : 1.0f, thr, thr + tm);
                 fix = oracle_abft_decide_lines(tm, tn, dr, dc, thr, thr + tm, &cur);
             } else {
                 fix = oracle_abft_decide(tm, tn, dr, dc, tau, &cur);
             }
-            if (cur.flag == 1) acc[(size_t)cur.row * tn + cur.col] += fix;
+            (void)fix;
+            double changed = 0.0;  /* what the correction added to the located accumulator */
+            if (cur.flag == 1) {
+                float* e = &acc[(size_t)cur.row * tn + cur.col];
+                float again = oracle_recompute_element(0, k1, A + (size_t)(m0 + cur.row) * lda, B + n0 + cur.col, ldb);
+                changed = (double)again - (double)*e;
+                *e = again;
+            }
             /* re-synchronise every line with what it shows after the correction */
-            for (int m = 0; m < tm; ++m) off_r[m] += dr[m] - ((cur.flag == 1 && m == cur.row) ? (double)fix : 0.0);
-            for (int n = 0; n < tn; ++n) off_c[n] += dc[n] - ((cur.flag == 1 && n == cur.col) ? (double)fix : 0.0);
+            for (int m = 0; m < tm; ++m) off_r[m] += dr[m] - ((cur.flag == 1 && m == cur.row) ? changed : 0.0);
+            for (int n = 0; n < tn; ++n) off_c[n] += dc[n] - ((cur.flag == 1 && n == cur.col) ? changed : 0.0);
             /* merge */
             rec.n_bad_rows += cur.n_bad_rows;
             rec.n_bad_cols += cur.n_bad_cols;

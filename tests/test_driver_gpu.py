@@ -26,13 +26,15 @@ def test_ft_sgemm_series_lines():
     out = _run("ft_sgemm", 256, 768, 256, 0, 23)
     assert out.startswith("     256|     512|     768|")
     assert "finish verified!" in out
-    series = dict(re.findall(r"^(\w+) = th\.as_tensor\(\[(.*)\]\)$", out, flags=re.M))
+    series = dict(re.findall(r"^(\w+) = th\.as_tensor\(\[(.*)\]\)(?:  #.*)?$", out, flags=re.M))
     assert list(series) == ["hpcdnn_sgemm", "kernel_sgemm_small", "kernel_sgemm_medium", "kernel_sgemm_large",
                             "kernel_sgemm_tall", "kernel_sgemm_wide", "kernel_sgemm_huge", "abft_baseline",
                             "abft_kernel_medium", "abft_kernel_large", "abft_kernel_tall", "abft_kernel_wide",
-                            "abft_kernel_huge", "warp_abft_kernel", "abft_kernel_huge_workspace",
+                            "abft_kernel_huge", "thread_abft_kernel", "warp_abft_kernel", "abft_kernel_huge_workspace",
                             "abft_kernel_large_workspace", "abft_kernel_wide_workspace",
                             "hpcdnn_sgemm_column_major", "abft_kernel_huge_column_major"]
+    # the thread-level series keeps its name and is empty: matrix cores have no per-thread accumulator tile
+    assert series.pop("thread_abft_kernel") == ""
     for name, body in series.items():
         vals = _floats(body)
         assert len(vals) == 3 and all(v > 0 for v in vals), (name, body)

@@ -177,7 +177,6 @@ def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod, ft_mode):
 
     rng = np.random.default_rng(2024)
     models = {}
-    worst_err = 0.0
     for launch in range(launches):
         tile = int(rng.integers(ntiles))
         i, j = int(rng.integers(blas.FT_TILE_M)), int(rng.integers(blas.FT_TILE_N))
@@ -187,19 +186,15 @@ def test_config4_4096_cube_seeded_fault_campaign(blas, oracle_mod, ft_mode):
         assert st["flag"][tile] == 1, (launch, tile, i, j, delta, st[tile])
         assert (st["row"][tile], st["col"][tile]) == (i, j), (launch, tile, i, j, delta, st[tile])
         assert np.count_nonzero(st["flag"]) == 1, (launch, "false positive elsewhere")
-        # correction restores the fault-free result to within the checksum noise (<< 1e-5 * (|A||B|)_ij ~ 1e-2)
-        diff = (dc - c_clean).abs()
-        err = float(diff.max())
-        worst_err = max(worst_err, err)
-        assert err < 4e-3, (launch, err)
-        assert int(torch.count_nonzero(diff)) <= 1
+        # the located accumulator is computed again in the matrix cores' own order: bit-identical to the fault-free run
+        assert torch.equal(dc, c_clean), (launch, tile, i, j, delta, float((dc - c_clean).abs().max()))
         if tile not in models:
             models[tile] = _TileModel(oracle_mod, a, b, K, N, tile, blas.FT_TILE_M, blas.FT_TILE_N, ntn)
         st_model, fix_model = models[tile].decide(i, j, delta, tau)
         for f in DECISION_FIELDS:
             assert st[f][tile] == st_model[f], (launch, f, st[tile], st_model)
         assert abs(float(st["row_residual"][tile]) - fix_model) < 3e-3
-    print(f"campaign ({ft_mode}): {launches} launches, worst |C - C_clean| after correction {worst_err:.3e}, "
+    print(f"campaign ({ft_mode}): {launches} launches, every corrected C bit-identical to the fault-free one, "
           f"fault-free max residual {clean['max_clean_residual'].max():.3e}, tau {tau:.1e}")
 
 
@@ -262,6 +257,56 @@ def test_k_zero_scales_c_and_flags_nothing(blas, ft_mode):
     assert torch.equal(c, c0 * 0.5)
     st = blas.ft_status_numpy(status)
     assert np.all(st["flag"] == 0) and np.all(st["max_clean_residual"] == 0.0)
+    # wave-tile granularity has more records than workgroup tiles: every one of them must come back clean, whatever
+    # the buffer held before
+    for cls in (0, 1, 2):
+        n = blas.ft_num_check_tiles(M, N, cls, blas.FT_GRAN_WAVE)
+        status = blas.ft_status_alloc(M, N, tile_class=cls, granularity=blas.FT_GRAN_WAVE)
+        assert status.numel() * status.element_size() == 32 * n
+        status.view(torch.int32).fill_(0x7fc00001)   # stale: flag, row, col and the residuals all garbage
+        c = c0.clone()
+        blas.ft_sgemm(M, N, 0, a[:, :0], b[:0, :], c, 1.0, 0.5, status=status, ws=torch.zeros(64, device="cuda"),
+                      tile_class=cls, granularity=blas.FT_GRAN_WAVE, faults=[(0, 1, 1, 3.0, 0)])
+        assert torch.equal(c, c0 * 0.5)
+        st = blas.ft_status_numpy(status)
+        assert st.shape == (n,) and np.all(st["flag"] == 0) and np.all(st["row"] == -1) and np.all(st["col"] == -1)
+        assert np.all(st["n_bad_rows"] == 0) and np.all(st["n_bad_cols"] == 0) and np.all(st["max_clean_residual"] == 0.0)
+
+
+def test_default_threshold_follows_the_data(blas, oracle_mod, ft_mode):
+    """tau = 0, the default, is the data-scaled threshold: on operands that are neither unit-range nor zero-mean
+    (x 100 + 25) a fault-free product flags nothing, a fault of 1e-3 of the typical entry is found, and the decisions
+    are those of tau = -1 and of the CPU model."""
+    M, N, K = 512, 384, 1024
+    a = oracle_mod.fill_uniform_matrix(M, K, 920) * np.float32(100.0) + np.float32(25.0)
+    b = oracle_mod.fill_uniform_matrix(K, N, 921) * np.float32(100.0) + np.float32(25.0)
+    c0 = np.zeros((M, N), np.float32)
+    typical = float(np.abs(a[:64].astype(np.float64) @ b.astype(np.float64)).mean())
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    for fault in (None, (3, 100, 50, 1e-3 * typical), (2, 255, 127, -1e-3 * typical)):
+        results = []
+        for tau in (0.0, -1.0):
+            dc = torch.from_numpy(c0).cuda()
+            status = blas.ft_status_alloc(M, N)
+            blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=tau, fault=fault, status=status, ws=_ws(blas, ft_mode, M, N, K))
+            results.append((blas.ft_status_numpy(status), dc.cpu().numpy()))
+        (st, c), (st1, c1) = results
+        assert np.array_equal(st, st1) and np.array_equal(c, c1)
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm(M, N, K, a, K, b, N, c_model, N, 1.0, 0.0, blas.FT_TILE_M, blas.FT_TILE_N, 0.0, fault)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (fault, f, st[f], st_model[f])
+        if fault is None:
+            assert np.all(st["flag"] == 0)
+            # the constant calibrated for unit-range operands does flag this fault-free product
+            dc = torch.from_numpy(c0).cuda()
+            status = blas.ft_status_alloc(M, N)
+            blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=blas.ft_default_tau(K), status=status, ws=_ws(blas, ft_mode, M, N, K))
+            assert np.count_nonzero(blas.ft_status_numpy(status)["flag"]) > 0
+        else:
+            assert st["flag"][fault[0]] == 1 and (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3]
+            assert np.count_nonzero(st["flag"]) == 1
+        _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 0.0)
 
 
 @pytest.mark.parametrize("scale_a,scale_b,shift", [(1.0, 1.0, 0.0), (250.0, 0.004, 0.0), (1e-3, 1e-3, 0.0), (1.0, 1.0, 0.5)])
@@ -320,8 +365,7 @@ def test_fault_campaign_with_data_scaled_threshold(blas, oracle_mod):
         st = blas.ft_status_numpy(status)
         assert st["flag"][tile] == 1 and (st["row"][tile], st["col"][tile]) == (i, j), (launch, tile, i, j, delta, st[tile])
         assert np.count_nonzero(st["flag"]) == 1, launch
-        diff = (dc - c_clean).abs()
-        assert int(torch.count_nonzero(diff)) <= 1 and float(diff.max()) < 3e-4 * typical, (launch, float(diff.max()))
+        assert torch.equal(dc, c_clean), (launch, float((dc - c_clean).abs().max()))
 
 
 @pytest.mark.parametrize("M,N,K,tile_class", [(512, 129, 256, 1), (600, 1, 250, 0), (512, 384, 1, 0), (200, 129, 15, 2),
@@ -396,16 +440,15 @@ def test_seeded_random_cases_equal_the_model(blas, oracle_mod):
         if caught:
             assert (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3], what
         if fault is None or caught:   # a sub-threshold fault stays in C
-            # every element obeys the componentwise criterion; the corrected one may be off by what the correction
-            # itself carries: the row's fault-free residual (rounding noise, below half the default threshold) plus the
-            # rounding of the FP32 line sums that held the fault, 16 * 2^-24 * |delta|
+            # every element obeys the componentwise criterion, the corrected one included (it is computed again)
             ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, lda, b, ldb, c0, ldc, alpha, beta)
-            allowed = TOL * den
-            if caught:
-                gi, gj = (fault[0] // ntn) * bm + fault[1], (fault[0] % ntn) * bn + fault[2]
-                allowed[gi, gj] += abs(alpha) * (0.5 * blas.ft_default_tau(K) + 16 * 2.0 ** -24 * abs(fault[3]))
             err = np.abs(c[:, :N].astype(np.float64) - ref)
-            assert np.all(err <= allowed), (what, float((err - allowed).max()))
+            assert np.all(err <= TOL * den), (what, float((err - TOL * den).max()))
+            if K < 512:   # (from 512 on a workspace call may split tiles along K, which sums in another order)
+                # fault-free or corrected, C has the bits of the device's summation order
+                want = c0.copy()
+                oracle_mod.sgemm_device_order(M, N, K, a, lda, b, ldb, want, ldc, alpha, beta)
+                assert np.array_equal(c[:, :N], want[:, :N]), what
 
 
 def test_partial_last_round_is_split_along_k(blas, oracle_mod):

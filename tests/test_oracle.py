@@ -462,6 +462,84 @@ def test_ft_sgemm_model_detects_and_corrects(oracle_mod, fault):
         assert st["row_residual"][fault[0]] == pytest.approx(-fault[3], abs=1e-4)
 
 
+@pytest.mark.parametrize("delta", [50.0, -50.0, 1e-2, -3.0e4])
+def test_corrected_product_has_the_bits_of_the_fault_free_one(oracle_mod, delta):
+    """The correction computes the located accumulator again instead of adding the residual back: with K = 1 (where a
+    residual of a whole row of products carries the most noise relative to one element) and with a longer K the
+    corrected C equals the fault-free C bit for bit, whatever the fault's size; the record still reports the
+    residual, i.e. minus the fault to within the rounding of the line sums."""
+    for M, N, K, tm, tn, fault_tile, i, j in [(16, 24, 1, 16, 8, 2, 7, 3), (20, 12, 96, 8, 8, 3, 1, 2)]:
+        rng = np.random.default_rng(K)
+        a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+        b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        c0 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+        ntn = -(-N // tn)
+        for tau in (1e-3, -1.0):
+            clean, hit = c0.copy(), c0.copy()
+            st0 = oracle_mod.ft_sgemm(M, N, K, a, K, b, N, clean, N, 1.25, -0.5, tm, tn, tau, None)
+            st1 = oracle_mod.ft_sgemm(M, N, K, a, K, b, N, hit, N, 1.25, -0.5, tm, tn, tau, (fault_tile, i, j, delta))
+            assert not st0["flag"].any()
+            assert st1["flag"][fault_tile] == 1 and (st1["row"][fault_tile], st1["col"][fault_tile]) == (i, j)
+            assert np.array_equal(hit, clean)
+            assert st1["row_residual"][fault_tile] == pytest.approx(-delta, rel=1e-5, abs=1e-5)
+            # the element itself: one fused multiply-add per k, k ascending, from zero
+            gi, gj = (fault_tile // ntn) * tm + i, (fault_tile % ntn) * tn + j
+            acc = np.float32(0.0)
+            for k in range(K):
+                acc = np.float32(float(a[gi, k]) * float(b[k, gj]) + float(acc))  # exact in double, rounded once
+            assert oracle_mod.recompute_element(a[gi], b[:, gj:], N, 0, K) == float(acc)
+            # the cadence model corrects the same way, at whichever verification the fault shows
+            for check in range(-(-K // 32)):
+                hit2 = c0.copy()
+                st2 = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, hit2, N, 1.25, -0.5, tm, tn, tau, 32,
+                                                  [(fault_tile, i, j, delta, check)])
+                assert st2["flag"][fault_tile] == 1 and np.array_equal(hit2, clean)
+
+
+def test_recompute_element_covers_exactly_its_k_range(oracle_mod):
+    a = np.arange(1, 9, dtype=np.float32)
+    b = np.full((8, 3), np.nan, dtype=np.float32)
+    b[:, 1] = [1, 10, 100, 1000, 1e4, 1e5, 1e6, 1e7]
+    assert oracle_mod.recompute_element(a, b[:, 1:], 3, 0, 8) == 87654321.0 - 1.0  # float(87654321) rounds to ...320
+    assert oracle_mod.recompute_element(a, b[:, 1:], 3, 2, 5) == 54300.0
+    assert oracle_mod.recompute_element(a, b[:, 1:], 3, 4, 4) == 0.0
+
+
+def test_sgemm_device_order_matches_numpy_and_keeps_its_k_order(oracle_mod):
+    """The model of the device's summation order: float accumulator, one fused multiply-add per k, k taken in the
+    order 0,4,1,5,2,6,3,7,8,12,9,13,10,14,11,15 inside each group of 16."""
+    M, N, K, lda, ldb, ldc = 9, 7, 53, 60, 11, 8
+    a = oracle_mod.fill_uniform_matrix(M, K, 81, ld=lda)
+    b = oracle_mod.fill_uniform_matrix(K, N, 82, ld=ldb)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, 83, ld=ldc)
+    c = c0.copy()
+    oracle_mod.sgemm_device_order(M, N, K, a, lda, b, ldb, c, ldc, 1.5, -0.75)
+    ref = 1.5 * (a[:, :K].astype(np.float64) @ b[:, :N].astype(np.float64)) - 0.75 * c0[:, :N]
+    assert np.max(np.abs(c[:, :N] - ref)) < 5e-6 and np.all(np.isnan(c[:, N:]))
+    c = np.full((M, ldc), np.nan, dtype=np.float32)   # beta == 0: C is not read
+    oracle_mod.sgemm_device_order(M, N, K, a, lda, b, ldb, c, ldc, 1.0, 0.0)
+    assert np.max(np.abs(c[:, :N] - a[:, :K].astype(np.float64) @ b[:, :N].astype(np.float64))) < 5e-6
+    # order, by cancellation: +B and -B with B = 2^30 swallow a 1.0 that is added between them and keep one added after
+    def run(K, **terms):
+        a1 = np.zeros((1, 16), dtype=np.float32)
+        for k, v in terms.items():
+            a1[0, int(k[1:])] = v
+        b1 = np.ones((16, 1), dtype=np.float32)
+        c1 = np.full((1, 1), np.nan, dtype=np.float32)
+        oracle_mod.sgemm_device_order(1, 1, K, a1, 16, b1, 1, c1, 1, 1.0, 0.0)
+        return float(c1[0, 0]), float(oracle_mod.tile_acc(a1, 16, b1, 1, 1, 1, K)[0, 0])
+    B = 2.0**30
+    assert run(16, k4=B, k5=-B, k2=1.0) == (1.0, 0.0)     # device: 4, 1, 5, 2: the one comes last; ascending: first
+    assert run(16, k1=B, k2=-B, k4=1.0) == (0.0, 1.0)     # device: 0, 4, 1, 5, 2: the one sits between them
+    assert run(16, k8=B, k9=-B, k12=1.0) == (0.0, 1.0)    # second half of the group: 8, 12, 9
+    assert run(16, k3=B, k8=-B, k7=1.0) == (0.0, 0.0)     # 3, 7, 8 in both orders
+    assert run(16, k7=B, k8=-B, k3=1.0) == (0.0, 0.0)     # ... 3, 7 | 8: the one precedes both in both orders
+    assert run(16, k6=B, k7=-B, k3=1.0) == (0.0, 0.0) and run(16, k2=B, k3=-B, k6=1.0) == (0.0, 1.0)  # 2, 6, 3, 7
+    # a ragged last group takes the k that exist, in the same relative order
+    assert run(6, k4=B, k5=-B, k2=1.0) == (1.0, 0.0)
+    assert run(5, k4=B, k5=-B, k2=1.0) == (B, B)          # k = 5 is outside K
+
+
 def test_checked_model_with_one_verification_is_the_plain_model(oracle_mod):
     M, N, K, tm, tn = 20, 12, 64, 8, 8
     rng = np.random.default_rng(6)

@@ -67,6 +67,35 @@ def test_every_tile_config_small_and_ragged_shapes(blas, oracle_mod):
             _check(oracle_mod, blas, M, N, K, 1.0, 0.0, tile=tile, seed=200 + tile)
 
 
+def test_unsplit_products_have_the_bits_of_the_summation_order_model(blas, oracle_mod):
+    """Every tile of the LDS-staged kernel (and the persistent kernels the library picks for large products) sums each
+    element of C in one float accumulator, one fused multiply-add per k, k permuted 0,4,1,5,... inside each group of
+    16: the CPU model of that order predicts the result bit for bit - ragged shapes, padded leading dimensions,
+    alpha/beta included.  (The 32x32 small-problem tile splits K over its waves and sums in another order.)"""
+    small_tile = [i for i, t in enumerate(blas.tile_table()) if t[0] == 32 and t[1] == 32]
+    shapes = [(1, 1, 1), (33, 31, 17), (130, 70, 40), (257, 129, 100), (300, 200, 333)]
+    for tile in range(_num_tiles(blas)):
+        if tile in small_tile:
+            continue
+        for (M, N, K) in shapes:
+            for alpha, beta in ((1.0, 0.0), (1.5, -0.75)):
+                a, b, c0 = _problem(oracle_mod, M, N, K, K + 3, N + 1, N + 2, seed=900 + tile)
+                da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+                blas.sgemm(M, N, K, da, db, dc, alpha, beta, tile=tile, split_k=1)
+                want = c0.copy()
+                oracle_mod.sgemm_device_order(M, N, K, a, K + 3, b, N + 1, want, N + 2, alpha, beta)
+                got = dc.cpu().numpy()
+                assert np.array_equal(got[:, :N], want[:, :N]), (tile, M, N, K, alpha, beta)
+    # the library's own choice on a product large enough for the persistent kernel, K not a multiple of 16
+    M, N, K = 2048, 1536, 200
+    a, b, c0 = _problem(oracle_mod, M, N, K, seed=950)
+    da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+    blas.sgemm(M, N, K, da, db, dc, 1.0, 1.0)
+    want = c0.copy()
+    oracle_mod.sgemm_device_order(M, N, K, a, K, b, N, want, N, 1.0, 1.0)
+    assert np.array_equal(dc.cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (1.5, -1.0), (1.0, -1.5), (0.0, 2.0), (-0.5, 0.0)])
 def test_alpha_beta_pairs_with_padded_leading_dimensions(blas, oracle_mod, alpha, beta):
     # 1.5/-1.0 and 1.0/-1.5 are the reference drivers' values (kernel/sgemm/sgemm.cu:33-34, ft_sgemm/sgemm.cu:32-34)
