@@ -10,7 +10,10 @@ size_t ft_workspace_bytes(int M, int N, int K);
 
 // ABFT tile classes (the counterpart of the reference's abft_kernel_{huge,large,wide,...} family,
 // kernel/ft_sgemm/sgemm.cu:187-188): class 0 is the 256 x 128 tile of HPCDNN_FT_TILE_M/N; the smaller classes keep
-// more CUs busy on smaller problems.  The encode is laid out for 128-column tiles, so the classes differ in height.
+// more CUs busy on smaller problems, the 64-column classes (the reference's tall 128 x 32 and medium 32 x 32 shapes,
+// kernel/ft_sgemm/code_gen/main.py:8-16, at the size of four waves of 32 x 32 matrix-core blocks) serve products with
+// few columns.  Geometry in gemm_host.h (kFtGeom), kernels in ft_kernels.hip, one translation unit per class and
+// operand layout.
 //
 // Without a workspace (FT = 1) four waves: on this part every VALU instruction takes its issue cycles away from the
 // FP32 matrix pipe of the same SIMD, whichever wave it comes from, so more waves do not hide the checksum arithmetic;
@@ -20,47 +23,39 @@ size_t ft_workspace_bytes(int M, int N, int K);
 //
 // Wave-tile granularity (the counterpart of ft_sgemm_huge_warp.cuh / ft_sgemm_huge_thread.cuh) runs the FT = 2 kernel
 // with one checksum pair per wave tile: the tile a wave of the workspace kernel owns, (bm / wgm) x (bn / wgn).
-struct FtClass {
-    int bm, bn;
-    int wgm, wgn;        // wave layout of the workspace kernels
-    FtKernel fused;      // checksum vectors formed in the main loop, one pair per workgroup tile
-    FtKernel pre;        // checksum vectors from the workspace, one pair per workgroup tile
-    FtKernel wave;       // checksum vectors from the workspace, one pair per wave tile
-    FtKernel fused_cad;  // the first two with a verification every check_interval k (class 0 only)
-    FtKernel pre_cad;
-    EncodeFn encode, encode_wave;
-};
+typedef FtGeom FtClass;
+static const FtClass* const kFtClasses = kFtGeom;
 
-#define HPCDNN_FT_KERNEL_N(BM, BN, WM_, WN_, FT, GRAN, CAD)                                                \
-    FtKernel {                                                                                             \
-        sgemm_kernel<BM, BN, WM_, WN_, false, FT, 1, 2, GRAN, CAD>,                                        \
-            sgemm_kernel<BM, BN, WM_, WN_, true, FT, 1, 2, GRAN, CAD>, WM_ * WN_ * kWave,                  \
-            gemm_lds_bytes<BM, BN, FT, WM_ * WN_ * kWave, WM_, WN_, GRAN>()                                \
+static FtKernel ft_kernel(int tile_class, bool ta, int kind) {
+    switch (tile_class * 2 + (ta ? 1 : 0)) {
+        case 0: return ft_kernel_c0_ta0(kind);
+        case 1: return ft_kernel_c0_ta1(kind);
+        case 2: return ft_kernel_c1_ta0(kind);
+        case 3: return ft_kernel_c1_ta1(kind);
+        case 4: return ft_kernel_c2_ta0(kind);
+        case 5: return ft_kernel_c2_ta1(kind);
+        case 6: return ft_kernel_c3_ta0(kind);
+        case 7: return ft_kernel_c3_ta1(kind);
+        case 8: return ft_kernel_c4_ta0(kind);
+        case 9: return ft_kernel_c4_ta1(kind);
+        default: return FtKernel{nullptr, nullptr, 0, 0};
     }
-#define HPCDNN_FT_KERNEL(BM, WM_, WN_, FT, GRAN, CAD) HPCDNN_FT_KERNEL_N(BM, 128, WM_, WN_, FT, GRAN, CAD)
-#define HPCDNN_FT_NO_KERNEL \
-    FtKernel { nullptr, nullptr, 0, 0 }
-
-static const FtClass kFtClasses[HPCDNN_FT_NUM_CLASSES] = {
-    // 0 huge
-    {256, 128, 2, 4, HPCDNN_FT_KERNEL(256, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(256, 2, 4, 2, 0, false),
-     HPCDNN_FT_KERNEL(256, 2, 4, 2, 1, false), HPCDNN_FT_KERNEL(256, 2, 2, 1, 0, true),
-     HPCDNN_FT_KERNEL(256, 2, 4, 2, 0, true), abft_encode_kernel<256, 128>, abft_encode_kernel<128, 32>},
-    // 1 large
-    {128, 128, 2, 2, HPCDNN_FT_KERNEL(128, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(128, 2, 2, 2, 0, false),
-     HPCDNN_FT_KERNEL(128, 2, 2, 2, 1, false), HPCDNN_FT_KERNEL(128, 2, 2, 1, 0, true), HPCDNN_FT_KERNEL(128, 2, 2, 2, 0, true),
-     abft_encode_kernel<128, 128>, abft_encode_kernel<64, 64>},
-    // 2 wide
-    {64, 128, 2, 2, HPCDNN_FT_KERNEL(64, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL(64, 2, 2, 2, 0, false),
-     HPCDNN_FT_KERNEL(64, 2, 2, 2, 1, false), HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<64, 128>,
-     abft_encode_kernel<32, 64>},
-    // 3 tall, 4 medium: 64 columns wide, for products with few columns (the reference's tall 128 x 32 and medium
-    // 32 x 32 shapes, kernel/ft_sgemm/code_gen/main.py:8-16, at the size of four waves of 32 x 32 matrix-core blocks)
-    {128, 64, 2, 2, HPCDNN_FT_KERNEL_N(128, 64, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL_N(128, 64, 2, 2, 2, 0, false),
-     HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<128, 64>, nullptr},
-    {64, 64, 2, 2, HPCDNN_FT_KERNEL_N(64, 64, 2, 2, 1, 0, false), HPCDNN_FT_KERNEL_N(64, 64, 2, 2, 2, 0, false),
-     HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, HPCDNN_FT_NO_KERNEL, abft_encode_kernel<64, 64>, nullptr},
-};
+}
+static EncodeFn ft_encode(int tile_class, bool ta, bool wave) {
+    switch (tile_class * 2 + (ta ? 1 : 0)) {
+        case 0: return ft_encode_c0_ta0(wave);
+        case 1: return ft_encode_c0_ta1(wave);
+        case 2: return ft_encode_c1_ta0(wave);
+        case 3: return ft_encode_c1_ta1(wave);
+        case 4: return ft_encode_c2_ta0(wave);
+        case 5: return ft_encode_c2_ta1(wave);
+        case 6: return ft_encode_c3_ta0(wave);
+        case 7: return ft_encode_c3_ta1(wave);
+        case 8: return ft_encode_c4_ta0(wave);
+        case 9: return ft_encode_c4_ta1(wave);
+        default: return nullptr;
+    }
+}
 
 // check tile of a class at a granularity: the unit that has a checksum pair, a verification and a status record
 static void check_tile(const FtClass& fc, int granularity, int* cm, int* cn) {
@@ -71,21 +66,27 @@ static void check_tile(const FtClass& fc, int granularity, int* cm, int* cn) {
 // ABFT with a workspace splits the tiles of a partial last round of CUs along K, like plain SGEMM's tail split: every
 // slice is a workgroup that verifies (and corrects) its own partial product - the checksums are linear in K - and
 // writes it raw; tail_reduce_kernel adds the slices, ft_tail_status_kernel merges their records.  With fewer tiles
-// than half the CUs every tile is split.  Returns the number of ways (1: no split) and the tiles it applies to.
+// than half the CUs every tile is split.  A slice is a multiple of `unit` values of k long: the K step, or the
+// verification interval, so that every slice of a cadence kernel verifies whole intervals of the K range.  Returns
+// the number of ways (1: no split), the tiles it applies to and the slice length.
 struct FtTail {
-    int ways, tiles;
+    int ways, tiles, k_chunk;
 };
-static FtTail ft_tail_plan(const FtClass& fc, int M, int N, int K) {
+static FtTail ft_tail_plan(const FtClass& fc, int M, int N, int K, int unit = kGemmBK) {
+    const FtTail none{1, 0, 0};
     const int cus = device_cus();
     const int64_t tiles = ceil_div(M, fc.bm) * ceil_div(N, fc.bn);
     const int64_t r = tiles % cus;
-    if (r == 0 || 2 * r > cus) return FtTail{1, 0};
+    if (r == 0 || 2 * r > cus) return none;
     int64_t s = cus / r;
     const int64_t most = K / (16 * kGemmBK);  // at least 16 K steps per slice: each slice pays a verification
     if (s > most) s = most;
     if (s > 8) s = 8;
-    if (s < 2) return FtTail{1, 0};
-    return FtTail{static_cast<int>(s), static_cast<int>(r)};
+    if (s < 2) return none;
+    const int k_chunk = static_cast<int>(ceil_div(ceil_div(K, s), unit)) * unit;
+    s = ceil_div(K, k_chunk);  // drop empty slices
+    if (s < 2) return none;
+    return FtTail{static_cast<int>(s), static_cast<int>(r), k_chunk};
 }
 // checksum vectors: one row per row group and per column group of the granularity
 static size_t ft_enc_bytes(const FtClass& fc, int granularity, int M, int N, int K) {
@@ -93,16 +94,20 @@ static size_t ft_enc_bytes(const FtClass& fc, int granularity, int M, int N, int
     const size_t b = static_cast<size_t>(ceil_div(M, fc.bm) * gm + ceil_div(N, fc.bn) * gn) * ft_enc_ld(K) * sizeof(float);
     return (b + 15) & ~static_cast<size_t>(15);
 }
-static size_t ft_tail_bytes(const FtClass& fc, const FtTail& t) {
+// the raw tile images of the K slices and their records (one per check tile of the workgroup tile)
+static size_t ft_tail_bytes(const FtClass& fc, int granularity, const FtTail& t) {
+    const int nct = granularity == HPCDNN_FT_GRAN_WAVE ? fc.wgm * fc.wgn : 1;
     return t.ways < 2 ? 0
-                      : static_cast<size_t>(t.tiles) * t.ways * (static_cast<size_t>(fc.bm) * fc.bn * sizeof(float) + sizeof(hpcdnn_ft_status));
+                      : static_cast<size_t>(t.tiles) * t.ways * (static_cast<size_t>(fc.bm) * fc.bn * sizeof(float) + nct * sizeof(hpcdnn_ft_status));
 }
 
 static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     const FtClass& fc = kFtClasses[tile_class];
-    const size_t tile_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_TILE, M, N, K) + ft_tail_bytes(fc, ft_tail_plan(fc, M, N, K));
-    const size_t wave_mode = fc.wave.plain ? ft_enc_bytes(fc, HPCDNN_FT_GRAN_WAVE, M, N, K) : 0;
+    // (a cadence kernel's slices are at most as many as these, and as long or longer: they fit as well)
+    const FtTail tail = ft_tail_plan(fc, M, N, K);
+    const size_t tile_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_TILE, M, N, K) + ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, tail);
+    const size_t wave_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_WAVE, M, N, K) + ft_tail_bytes(fc, HPCDNN_FT_GRAN_WAVE, tail);
     return tile_mode > wave_mode ? tile_mode : wave_mode;
 }
 
@@ -128,10 +133,8 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     if (opt.n_faults < 0 || opt.n_faults > HPCDNN_FT_MAX_FAULTS) return HPCDNN_ERR_INVALID_VALUE;
     const FtClass& fc = kFtClasses[opt.tile_class];
     const bool wave = opt.granularity == HPCDNN_FT_GRAN_WAVE;
-    if (wave && !fc.wave.plain) return HPCDNN_ERR_INVALID_VALUE;  // the 64-column classes check per workgroup tile only
     // an interval that covers all of K is a single verification after the loop
     const bool cadence = opt.check_interval > 0 && opt.check_interval < K;
-    if (cadence && (wave || !fc.pre_cad.plain)) return HPCDNN_ERR_INVALID_VALUE;
     if (M == 0 || N == 0) return HPCDNN_OK;
     if (wave && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
 
@@ -182,10 +185,9 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     if (ws && K > 0) {
         const size_t enc_bytes = ft_enc_bytes(fc, opt.granularity, M, N, K);
         if (ws_bytes < enc_bytes || (reinterpret_cast<uintptr_t>(ws) & 15u)) return HPCDNN_ERR_WORKSPACE;
-        // the K split of a partial last round is taken when the workspace has room for it (one checksum pair per
-        // workgroup tile and one verification only: a slice keeps one record)
-        FtTail tail = (wave || cadence) ? FtTail{1, 0} : ft_tail_plan(fc, M, N, K);
-        if (ws_bytes < enc_bytes + ft_tail_bytes(fc, tail)) tail = FtTail{1, 0};
+        // the K split of a partial last round is taken when the workspace has room for it
+        FtTail tail = ft_tail_plan(fc, M, N, K, cadence ? opt.check_interval : kGemmBK);
+        if (ws_bytes < enc_bytes + ft_tail_bytes(fc, opt.granularity, tail)) tail = FtTail{1, 0, 0};
         a.enc_ld = ft_enc_ld(K);
         const int row_groups = a.tiles_m * gm, col_groups = a.tiles_n * gn;
         float* enc_a = static_cast<float*>(ws);
@@ -195,24 +197,20 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
         const int b_blocks = static_cast<int>(ceil_div(N, 128));  // the pre-pass walks B in blocks of 128 columns
         // (ta: the same launch, with the blocks of the A half walking A^T)
-        const EncodeFn encode = ta ? ft_ta_encode(cm, cn) : wave ? fc.encode_wave : fc.encode;
+        const EncodeFn encode = ft_encode(opt.tile_class, ta, wave);
         if (!encode) return HPCDNN_ERR_INVALID_VALUE;
         hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(1024), 0, s, M, N, K,
                            A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;
-        const FtKernel ta_k = ta ? ft_ta_kernel(opt.tile_class, fc.bm, fc.bn, wave ? 1 : (cadence ? 2 : 0)) : FtKernel{nullptr, nullptr, 0, 0};
-        if (ta && !ta_k.plain) return HPCDNN_ERR_INVALID_VALUE;
-        const FtKernel& k = ta ? ta_k : wave ? fc.wave : (cadence ? fc.pre_cad : fc.pre);
+        const FtKernel k = ft_kernel(opt.tile_class, ta, wave ? (cadence ? kFtWaveCad : kFtWave) : (cadence ? kFtPreCad : kFtPre));
+        if (!k.plain) return HPCDNN_ERR_INVALID_VALUE;
         void (*fn)(const GemmArgs) = edge ? k.edge : k.plain;
         rc = enable_lds(fn, k.lds);
         if (rc != HPCDNN_OK) return rc;
         const int tiles = a.tiles_m * a.tiles_n;
         if (tail.ways >= 2) {
-            a.tail_k_chunk = static_cast<int>(ceil_div(ceil_div(K, tail.ways), kGemmBK)) * kGemmBK;
-            tail.ways = static_cast<int>(ceil_div(K, a.tail_k_chunk));  // drop empty slices
-        }
-        if (tail.ways >= 2) {
+            a.tail_k_chunk = tail.k_chunk;
             a.full_tiles = tiles - tail.tiles;
             a.tail_split = tail.ways;
             a.tail_partial = reinterpret_cast<float*>(static_cast<char*>(ws) + enc_bytes);
@@ -226,13 +224,12 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
                                                                          a.tail_split, a.tail_partial, C, ldc, alpha, beta);
         rc = launch_status();
         if (rc != HPCDNN_OK || !status) return rc;
-        ft_tail_status_kernel<><<<static_cast<int>(ceil_div(tail.tiles, 64)), 64, 0, s>>>(tail.tiles, a.tail_split, a.tiles_m, a.tiles_n,
-                                                                                        a.full_tiles, a.tail_status, status);
+        ft_tail_status_kernel<><<<static_cast<int>(ceil_div(tail.tiles * gm * gn, 64)), 64, 0, s>>>(
+            tail.tiles, a.tail_split, gm, gn, a.tiles_m, a.tiles_n, a.full_tiles, a.tail_status, status, a.status_rows, a.status_ld);
         return launch_status();
     }
-    const FtKernel ta_k = ta ? ft_ta_kernel(opt.tile_class, fc.bm, fc.bn, cadence ? 4 : 3) : FtKernel{nullptr, nullptr, 0, 0};
-    if (ta && !ta_k.plain) return HPCDNN_ERR_INVALID_VALUE;
-    const FtKernel& k = ta ? ta_k : cadence ? fc.fused_cad : fc.fused;
+    const FtKernel k = ft_kernel(opt.tile_class, ta, cadence ? kFtFusedCad : kFtFused);
+    if (!k.plain) return HPCDNN_ERR_INVALID_VALUE;
     void (*fn)(const GemmArgs) = edge ? k.edge : k.plain;
     rc = enable_lds(fn, k.lds);
     if (rc != HPCDNN_OK) return rc;
@@ -254,7 +251,6 @@ extern "C" int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn) {
 extern "C" int hpcdnn_ft_check_tile_info(int tile_class, int granularity, int* cm, int* cn) {
     if (tile_class < 0 || tile_class >= HPCDNN_FT_NUM_CLASSES) return HPCDNN_ERR_INVALID_VALUE;
     if (granularity != HPCDNN_FT_GRAN_TILE && granularity != HPCDNN_FT_GRAN_WAVE) return HPCDNN_ERR_INVALID_VALUE;
-    if (granularity == HPCDNN_FT_GRAN_WAVE && !kFtClasses[tile_class].wave.plain) return HPCDNN_ERR_INVALID_VALUE;
     int m = 0, n = 0;
     check_tile(kFtClasses[tile_class], granularity, &m, &n);
     if (cm) *cm = m;

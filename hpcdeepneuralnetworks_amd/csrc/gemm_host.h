@@ -61,14 +61,33 @@ struct FtKernel {
     int threads;
     size_t lds;
 };
-// The ABFT kernels of a tile class for a transposed left operand (ft_sgemm_ta.hip).  Checksum vectors from the
-// workspace: kind 0, one checksum pair per workgroup tile; 1, per wave tile; 2, per workgroup tile with a verification
-// every check_interval k.  Checksum vectors formed in the main loop: kind 3, per workgroup tile; 4, with the
-// verification cadence.  {nullptr, ...} where the class has no such kernel.
-FtKernel ft_ta_kernel(int tile_class, int bm, int bn, int kind);
-// Its pre-pass over both operands (row groups of `rows` rows, column groups of `cols` columns of the product), or nullptr
 typedef void (*EncodeFn)(int, int, int, const float*, int, const float*, int, float*, float*, int, int, int, int);
-EncodeFn ft_ta_encode(int rows, int cols);
+
+// ABFT tile classes: workgroup tile and the wave layout of the kernels that read their checksum vectors from the
+// workspace (the wave tile, (bm / wgm) x (bn / wgn), is the check tile of wave-tile granularity)
+struct FtGeom {
+    int bm, bn, wgm, wgn;
+};
+constexpr FtGeom kFtGeom[HPCDNN_FT_NUM_CLASSES] = {{256, 128, 2, 4}, {128, 128, 2, 2}, {64, 128, 2, 2}, {128, 64, 2, 2}, {64, 64, 2, 2}};
+
+// Kernel kinds of a class.  Fused: checksum vectors formed in the main loop (no workspace); pre: read from the
+// workspace the pre-pass filled; wave: pre, with one checksum pair per wave tile; cad: with a verification every
+// check_interval values of k.
+enum FtKind { kFtFused = 0, kFtFusedCad, kFtPre, kFtPreCad, kFtWave, kFtWaveCad, kFtKinds };
+
+// One getter pair per (class, operand layout): each lives in its own translation unit (ft_kernels.hip compiled with
+// -DHPCDNN_FT_CLASS / -DHPCDNN_FT_TA).  _ta1: the left operand is given transposed (K rows of M floats).
+#define HPCDNN_FT_DECLARE(c)                  \
+    FtKernel ft_kernel_c##c##_ta0(int kind);  \
+    FtKernel ft_kernel_c##c##_ta1(int kind);  \
+    EncodeFn ft_encode_c##c##_ta0(bool wave); \
+    EncodeFn ft_encode_c##c##_ta1(bool wave);
+HPCDNN_FT_DECLARE(0)
+HPCDNN_FT_DECLARE(1)
+HPCDNN_FT_DECLARE(2)
+HPCDNN_FT_DECLARE(3)
+HPCDNN_FT_DECLARE(4)
+#undef HPCDNN_FT_DECLARE
 
 // Kernels that use more than the default 64 KiB of LDS must opt in once per device.
 inline int enable_lds(void (*fn)(const GemmArgs), size_t bytes) {

@@ -66,7 +66,7 @@ struct GemmArgs {
     // ways along K (tail_k_chunk per slice) and write raw accumulators to tail_partial[tile - full_tiles][slice][BM*BN]
     int full_tiles, tail_split, tail_k_chunk;
     float* tail_partial;
-    hpcdnn_ft_status* tail_status;  // ABFT with a tail split: one record per slice, [tile - full_tiles][slice]
+    hpcdnn_ft_status* tail_status;  // ABFT with a tail split: [tile - full_tiles][slice][check tile of the workgroup tile]
     // ABFT
     float tau;      // absolute residual threshold; 0 = relative mode
     float tau_rel;  // relative mode: threshold of a line = tau_rel * sum |accumulators of the line| / sqrt(elements in it)
@@ -997,11 +997,14 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         // (run-time form of `t[2].x += error_inject`, ft_sgemm_huge.cuh:40,145).  A fault aimed at a row or column
         // of an edge tile that lies outside the matrix is ignored.  A kernel that verifies once injects every fault
         // before that verification.
-        // (a tile split along K verifies every slice on its own - the checksums are linear in K; the test faults go
-        // into its first slice)
+        // (a tile split along K verifies every slice on its own - the checksums are linear in K; a kernel that
+        // verifies once per slice takes the test faults into the tile's first slice, a cadence kernel, whose slices
+        // start on a multiple of the interval, into the slice and interval that verification number `check` of the
+        // whole K range falls into)
+        const int check_global = CADENCE ? k_first / p.check_interval + check : 0;
 #pragma unroll 1
         for (int f = 0; f < p.n_faults; ++f)
-            if (tile_linear == p.faults[f].tile && k_slice == 0 && (!CADENCE || p.faults[f].check == check) &&
+            if (tile_linear == p.faults[f].tile && (CADENCE ? p.faults[f].check == check_global : k_slice == 0) &&
                 m0 + p.faults[f].row < p.M && n0 + p.faults[f].col < p.N)
                 add_at(p.faults[f].row, p.faults[f].col, p.faults[f].delta);
 
@@ -1270,7 +1273,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 hpcdnn_ft_status st = rec;
                 if (st.flag == 2) { st.row = -1; st.col = -1; st.row_residual = 0.f; st.col_residual = 0.f; }
                 const int srow = tile_m * GM + gm, scol = tile_n * GN + gn;
-                if (tail_out) p.tail_status[tail_slot] = st;
+                if (tail_out) p.tail_status[tail_slot * NCT + ct] = st;
                 else if (srow < p.status_rows && scol < p.status_ld) p.status[srow * p.status_ld + scol] = st;
             }
         }
@@ -1476,16 +1479,19 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, 
     }
 }
 
-// ABFT with a tail split: the records of a tile's K slices become the tile's record.  Bad-line counts add up; a
-// slice that could not locate its fault makes the tile uncorrectable (2); otherwise the tile is corrected (1) if any
-// slice corrected an element, and reports the first such slice's location and residuals (more than one corrected
-// slice shows in the counts).
+// ABFT with a tail split: the records of a tile's K slices become the tile's records, one per check tile (gm x gn of
+// them per workgroup tile).  Bad-line counts add up; a slice that could not locate its fault makes the check tile
+// uncorrectable (2); otherwise it is corrected (1) if any slice corrected an element, and reports the first such
+// slice's location and residuals (more than one corrected slice shows in the counts).  Slices are K ranges in
+// ascending order, so with a verification cadence this is the order of the verifications.
 template <int kUnused = 0>
-__global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int splits, int tiles_m, int tiles_n,
+__global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int splits, int gm, int gn, int tiles_m, int tiles_n,
                                                             int full_tiles, const hpcdnn_ft_status* __restrict__ slices,
-                                                            hpcdnn_ft_status* __restrict__ status) {
-    const int t = blockIdx.x * 64 + threadIdx.x;
-    if (t >= tail_tiles) return;
+                                                            hpcdnn_ft_status* __restrict__ status, int status_rows, int status_ld) {
+    const int nct = gm * gn;
+    const int idx = blockIdx.x * 64 + threadIdx.x;
+    if (idx >= tail_tiles * nct) return;
+    const int t = idx / nct, ct = idx % nct;
     int tile_m, tile_n;
     tile_of_block(full_tiles + t, tiles_m, tiles_n, tile_m, tile_n);
     hpcdnn_ft_status out;
@@ -1493,7 +1499,7 @@ __global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int 
     out.row_residual = 0.f; out.col_residual = 0.f; out.max_clean_residual = 0.f;
     bool located = false;
     for (int z = 0; z < splits; ++z) {
-        const hpcdnn_ft_status s = slices[t * splits + z];
+        const hpcdnn_ft_status s = slices[(t * splits + z) * nct + ct];
         out.n_bad_rows += s.n_bad_rows;
         out.n_bad_cols += s.n_bad_cols;
         out.max_clean_residual = s.max_clean_residual > out.max_clean_residual ? s.max_clean_residual : out.max_clean_residual;
@@ -1505,7 +1511,8 @@ __global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int 
     }
     if (out.flag == 2) { out.row = -1; out.col = -1; out.row_residual = 0.f; out.col_residual = 0.f; }
     else if (located) out.flag = 1;
-    status[tile_m * tiles_n + tile_n] = out;
+    const int srow = tile_m * gm + ct / gn, scol = tile_n * gn + ct % gn;
+    if (srow < status_rows && scol < status_ld) status[srow * status_ld + scol] = out;
 }
 
 // ---- ABFT pre-encode: the checksum vectors of the operands, one per row group (RM rows) / column group (CN

@@ -221,7 +221,7 @@ int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
  * status record per workgroup tile of the class (what hpcdnn_ft_sgemm_ex does).
  * HPCDNN_FT_GRAN_WAVE: one per wave tile, the part of the workgroup tile one
  * 64-lane wave accumulates on the matrix cores (class 0: 128x32, class 1:
- * 64x64, class 2: 32x64; classes 3 and 4 have tile granularity only;
+ * 64x64, class 2: 32x64, class 3: 64x32, class 4: 32x32;
  * hpcdnn_ft_check_tile_info): every wave tile is
  * verified, located and corrected on its own, so one fault per wave tile is
  * correctable where tile granularity reports two faults in one 256x128 tile
@@ -241,7 +241,13 @@ int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
  * record of a check tile merges its verifications: bad-line counts add up,
  * flag 2 if any verification could not locate its fault, else 1 if any
  * corrected an element; row, col and the residuals are those of the first
- * correction.  Tile granularity, classes 0 and 1.
+ * correction.  Every class, either granularity, with or without workspace
+ * (the reference's kernels all carry the in-loop check,
+ * kernel/ft_sgemm/include/ft_sgemm_large.cuh:337, ft_sgemm_tall.cuh:18).
+ * Tiles of a partial last round that are split along K (see hpcdnn_ft_sgemm)
+ * are cut at multiples of check_interval, every slice verifying its own
+ * intervals, so the verifications of a tile are the same with and without
+ * the split.
  *
  * Check tiles are numbered row-major over the matrix,
  * t = (i / cm) * ceil(N / cn) + (j / cn); `status` holds

@@ -18,6 +18,14 @@ def _ws(blas, M, N, K):
     return torch.full((max(blas.ft_workspace_bytes(M, N, K) // 4, 4),), float("nan"), dtype=torch.float32, device="cuda")
 
 
+def _ws_checksums_only(blas, M, N, K, tile_class=0, granularity=0):
+    """A workspace with room for the checksum vectors and nothing else: the call cannot split tiles along K."""
+    bm, bn = blas.ft_tile(tile_class)
+    cm, cn = blas.ft_check_tile(tile_class, granularity)
+    words = (-(-M // bm) * (bm // cm) + -(-N // bn) * (bn // cn)) * ((-(-K // 16) + 2) * 16)
+    return torch.full(((words + 3) // 4 * 4,), float("nan"), dtype=torch.float32, device="cuda")
+
+
 def _problem(oracle_mod, M, N, K, seed, pad=(4, 4, 8)):
     a = oracle_mod.fill_uniform_matrix(M, K, seed, ld=K + pad[0])
     b = oracle_mod.fill_uniform_matrix(K, N, seed + 1, ld=N + pad[1])
@@ -40,13 +48,13 @@ def _assert_values(oracle_mod, M, N, K, a, b, c0, c, alpha, beta):
 
 
 def test_check_tile_table(blas):
-    assert [blas.ft_check_tile(c, blas.FT_GRAN_TILE) for c in range(3)] == [(256, 128), (128, 128), (64, 128)]
-    assert [blas.ft_check_tile(c, blas.FT_GRAN_WAVE) for c in range(3)] == [(128, 32), (64, 64), (32, 64)]
+    assert [blas.ft_check_tile(c, blas.FT_GRAN_TILE) for c in range(5)] == [(256, 128), (128, 128), (64, 128), (128, 64), (64, 64)]
+    assert [blas.ft_check_tile(c, blas.FT_GRAN_WAVE) for c in range(5)] == [(128, 32), (64, 64), (32, 64), (64, 32), (32, 32)]
     assert blas.ft_num_check_tiles(300, 300, 0, blas.FT_GRAN_WAVE) == 3 * 10
     assert blas.ft_num_check_tiles(300, 300, 0, blas.FT_GRAN_TILE) == blas.ft_num_tiles(300, 300) == 2 * 3
 
 
-@pytest.mark.parametrize("tile_class", [0, 1, 2])
+@pytest.mark.parametrize("tile_class", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("tau_kind", ["absolute", "scaled"])
 def test_wave_tiles_decisions_equal_the_model(blas, oracle_mod, tile_class, tau_kind):
     """One checksum pair, one verification and one record per wave tile; ragged in every dimension, so edge tiles have
@@ -151,7 +159,8 @@ def test_verification_cadence_corrects_one_fault_per_interval(blas, oracle_mod, 
             assert np.any(st1["flag"] == 2)
     # fault-free: the cadence changes nothing in C (same accumulation order as the plain kernel on this tile)
     da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
-    c_cad, _ = _device_run(blas, a, b, c0, M, N, K, 1.5, -1.0, tau, ws, check_interval=256)
+    # (with room in the workspace these six tiles would be split along K, which sums in another order)
+    c_cad, _ = _device_run(blas, a, b, c0, M, N, K, 1.5, -1.0, tau, ws if ws is None else _ws_checksums_only(blas, M, N, K), check_interval=256)
     plain = torch.from_numpy(c0).cuda()
     blas.sgemm(M, N, K, da, db, plain, 1.5, -1.0, tile=0, split_k=1)
     assert np.array_equal(c_cad[:, :N], plain.cpu().numpy()[:, :N])
@@ -172,6 +181,87 @@ def test_verification_cadence_on_the_128x128_class(blas, oracle_mod, mode):
             assert np.array_equal(st[f], st_model[f]), (faults, f, st[f], st_model[f])
         if not np.any(st["flag"] == 2):
             _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.5, -1.0)
+
+
+@pytest.mark.parametrize("tile_class", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("kind", ["tile-fused", "tile-workspace", "wave-workspace"])
+def test_every_class_granularity_and_cadence_equals_the_model(blas, oracle_mod, tile_class, kind):
+    """The whole option matrix: every tile class, both granularities, checksum vectors from the main loop or from the
+    workspace, with the verification every 256 k (the reference's scheme: every shape of its table has an ABFT kernel
+    with the in-loop check, kernel/ft_sgemm/sgemm.cu:186-192, ft_sgemm_large.cuh:337, ft_sgemm_tall.cuh:18) and, for
+    comparison, with one verification.  Ragged in every dimension; faults in check-tile units, in different intervals."""
+    gran = blas.FT_GRAN_WAVE if kind.startswith("wave") else blas.FT_GRAN_TILE
+    cm, cn = blas.ft_check_tile(tile_class, gran)
+    M, N, K = 333, 200, 900      # 4 verifications (k = 256, 512, 768, 900)
+    tau = blas.ft_default_tau(K)
+    a, b, c0 = _problem(oracle_mod, M, N, K, 1500 + tile_class)
+    # (no room for K slices: every element is summed by one workgroup, in the order the model below knows)
+    ws = _ws_checksums_only(blas, M, N, K, tile_class, gran) if kind.endswith("workspace") else None
+    ntm, ntn = -(-M // cm), -(-N // cn)
+    rng = np.random.default_rng(70 + tile_class)
+
+    def fault(tile, check):
+        tm, tn = min(cm, M - (tile // ntn) * cm), min(cn, N - (tile % ntn) * cn)
+        return (tile, int(rng.integers(tm)), int(rng.integers(tn)),
+                float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-1.0, 1.5))), check)
+
+    last = ntm * ntn - 1   # the corner check tile, clipped in both directions
+    cases = [[], [fault(0, 0)], [fault(last, 1), fault(last, 3)], [fault(1, 2), fault(ntn, 0), fault(ntn, 3)],
+             [fault(1, 2), fault(1, 2)]]                                     # same interval: uncorrectable
+    for faults in cases:
+        for interval in (256, 0):
+            c, st = _device_run(blas, a, b, c0, M, N, K, 1.5, -1.0, tau, ws, tile_class=tile_class, granularity=gran,
+                                check_interval=interval, faults=faults)
+            c_model = c0.copy()
+            st_model = oracle_mod.ft_sgemm_checked(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, cm, cn, tau, interval, faults)
+            assert len(st) == ntm * ntn
+            for f in DECISION_FIELDS:
+                assert np.array_equal(st[f], st_model[f]), (tile_class, kind, interval, faults, f, st[f], st_model[f])
+            if not np.any(st["flag"] == 2):
+                _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.5, -1.0)
+                # corrected or fault-free, C has the bits of the device's summation order
+                want = c0.copy()
+                oracle_mod.sgemm_device_order(M, N, K, a, K + 4, b, N + 4, want, N + 8, 1.5, -1.0)
+                assert np.array_equal(c[:, :N], want[:, :N]), (tile_class, kind, interval, faults)
+
+
+@pytest.mark.parametrize("tile_class,granularity", [(0, 0), (0, 1), (1, 1), (3, 0), (4, 1)])
+def test_partial_last_round_is_split_along_k_under_cadence_and_wave_granularity(blas, oracle_mod, tile_class, granularity):
+    """With room in the workspace the tiles of a partial last round of CUs are split along K; under a verification
+    cadence every slice is a whole number of intervals and verifies its own, with wave-tile granularity every slice
+    keeps one record per wave tile.  Decisions must equal the model's (which knows nothing of slices) and must not
+    depend on whether the split happened; C agrees to rounding (a split sums K in another order)."""
+    bm, bn = blas.ft_tile(tile_class)
+    cm, cn = blas.ft_check_tile(tile_class, granularity)
+    M, N, K = 2 * bm + bm // 2 + 3, 2 * bn + 5, 2048      # 3 x 3 workgroup tiles: fewer than half the CUs, all split
+    tau = blas.ft_default_tau(K)
+    a, b, c0 = _problem(oracle_mod, M, N, K, 1600 + tile_class)
+    need = blas.ft_workspace_bytes(M, N, K)
+    gm, gn = bm // cm, bn // cn
+    enc_only = 4 * (-(-M // bm) * gm + -(-N // bn) * gn) * ((-(-K // 16) + 2) * 16)
+    enc_only = (enc_only + 15) // 16 * 16
+    assert need > enc_only + 9 * 2 * bm * bn * 4
+    ntn = -(-N // cn)
+    corner = (-(-M // cm)) * ntn - 1
+    for interval, faults in [(0, [(corner, 1, 2, -0.75, 0)]),
+                             (128, [(corner, 1, 2, -0.75, 5), (corner, 2, 1, 3.0, 13), (ntn + 1, 17, 9, 12.5, 0)]),
+                             (512, [(0, 0, 0, 1.0, 3), (0, 5, 5, -1.0, 1)]),
+                             (128, [(1, 3, 3, 1.0, 9), (1, 4, 4, 1.0, 9)])]:      # same interval: uncorrectable
+        results = []
+        for nbytes in (need, enc_only):   # split, not split
+            ws = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+            results.append(_device_run(blas, a, b, c0, M, N, K, 1.5, -1.0, tau, ws, tile_class=tile_class,
+                                       granularity=granularity, check_interval=interval, faults=faults))
+        (c_split, st_split), (c_whole, st_whole) = results
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm_checked(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, cm, cn, tau, interval, faults)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st_split[f], st_model[f]), (interval, faults, f, st_split[f], st_model[f])
+            assert np.array_equal(st_whole[f], st_model[f]), (interval, faults, f, st_whole[f], st_model[f])
+        if not np.any(st_model["flag"] == 2):
+            _assert_values(oracle_mod, M, N, K, a, b, c0, c_split, 1.5, -1.0)
+            _assert_values(oracle_mod, M, N, K, a, b, c0, c_whole, 1.5, -1.0)
+            assert not np.array_equal(c_split[:, :N], c_whole[:, :N])   # the split did happen
 
 
 def test_cadence_with_data_scaled_threshold_and_interval_edge_cases(blas, oracle_mod):
@@ -196,8 +286,8 @@ def test_option_errors(blas):
     ws = torch.zeros(1 << 20, device="cuda")
     with pytest.raises(blas.HpcdnnError):   # wave-tile checksums come from the workspace
         blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, granularity=blas.FT_GRAN_WAVE)
-    with pytest.raises(blas.HpcdnnError):   # the cadence kernels exist for the 256 x 128 and 128 x 128 classes
-        blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, tile_class=2, check_interval=64, ws=ws)
+    with pytest.raises(blas.HpcdnnError):   # five classes
+        blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, tile_class=5, check_interval=64, ws=ws)
     with pytest.raises(blas.HpcdnnError):   # a multiple of the K step
         blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, check_interval=100, ws=ws)
     with pytest.raises(blas.HpcdnnError):   # wave tile 128 x 32: column 32 does not exist

@@ -38,17 +38,24 @@ def _ws(blas, M, N, K):
     return torch.full((max(nbytes // 4, 4),), float("nan"), dtype=torch.float32, device="cuda")   # poisoned
 
 
-def _run(blas, oracle_mod, M, N, K, alpha, beta, tau, faults=None, pad=(0, 0, 0), seed=600, mode="workspace", **opts):
+def _run(blas, oracle_mod, M, N, K, alpha, beta, tau, faults=None, pad=(0, 0, 0), seed=600, mode="workspace", values=True, **opts):
     abuf, bbuf, cbuf = _buffers(oracle_mod, M, N, K, pad, seed)
     da, db, dc = torch.from_numpy(abuf).cuda(), torch.from_numpy(bbuf).cuda(), torch.from_numpy(cbuf).cuda()
     tile_class, gran = opts.get("tile_class", 0), opts.get("granularity", 0)
     status = blas.ft_status_alloc(N, M, tile_class=tile_class, granularity=gran)
     ws = _ws(blas, M, N, K) if mode == "workspace" else None
+    if mode == "workspace" and opts.pop("no_split", False):
+        # room for the checksum vectors only: no tile can be split along K, every element is summed by one workgroup
+        bm, bn = blas.ft_tile(tile_class)
+        cm, cn = blas.ft_check_tile(tile_class, gran)
+        words = (-(-N // bm) * (bm // cm) + -(-M // bn) * (bn // cn)) * ((-(-K // 16) + 2) * 16)
+        ws = torch.full(((words + 3) // 4 * 4,), float("nan"), dtype=torch.float32, device="cuda")
+    opts.pop("no_split", None)
     blas.ft_sgemm_cm_nt(M, N, K, da, db, dc, alpha, beta, ws, tau=tau, status=status, faults=faults, **opts)
     c = dc.cpu().numpy()
     ref, den = oracle_mod.gemm_cm_nt_f64(M, N, K, abuf, abuf.shape[1], bbuf, bbuf.shape[1], cbuf, cbuf.shape[1], alpha, beta)
     err = oracle_mod.gemm_max_err(M, c, c.shape[1], ref, den)
-    assert err <= TOL, err
+    assert err <= TOL or not values, err   # (values=False: the caller leaves uncorrectable faults in C)
     assert np.all(np.isnan(c[:, M:]))
     return abuf, bbuf, cbuf, c, blas.ft_status_numpy(status), status
 
@@ -78,13 +85,10 @@ def test_against_the_row_major_call_on_a_transposed_copy(blas, oracle_mod, ft_mo
     for f in DECISION_FIELDS:
         assert np.array_equal(st[f], st2[f]), f
     assert np.allclose(st["row_residual"], st2["row_residual"], atol=2e-3) and np.allclose(st["col_residual"], st2["col_residual"], atol=2e-3)
-    if fault is None:
-        assert np.array_equal(c2[:, :M], c[:, :M])            # same summation order of every element
-    else:
+    # same summation order of every element, and a corrected element is computed again in that order
+    assert np.array_equal(c2[:, :M], c[:, :M])
+    if fault is not None:
         assert st["flag"][1] == 1 and (st["row"][1], st["col"][1]) == (5, 7)
-        differ = np.argwhere(c2[:, :M] != c[:, :M])           # only the corrected element may differ (by rounding of the residual)
-        assert all(tuple(d) == (5, 128 + 7) for d in differ)
-        assert abs(c2[5, 128 + 7] - c[5, 128 + 7]) < 1e-3
 
 
 def test_reference_known_answer_plus_one_at_0_1(blas, oracle_mod, ft_mode):
@@ -133,6 +137,42 @@ def test_other_classes_granularity_and_cadence(blas, oracle_mod):
     for mode in ("workspace", "fused"):
         *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 0.0, tau, faults=[(0, 3, 4, 2.0, 1)], check_interval=256, mode=mode)
         assert st["flag"][0] == 1 and (st["row"][0], st["col"][0]) == (3, 4)
+
+
+@pytest.mark.parametrize("tile_class", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("kind", ["tile-fused", "tile-workspace", "wave-workspace"])
+def test_every_class_granularity_and_cadence_equals_the_model(blas, oracle_mod, tile_class, kind):
+    """The option matrix on the column-major buffers: every class, both granularities, checksum vectors from the main
+    loop or the workspace, with the verification every 256 k and with a single one; decisions equal the CPU model of
+    the row-major problem C^T = (B^T)^T A^T, corrected values have the bits of the device's summation order."""
+    gran = blas.FT_GRAN_WAVE if kind.startswith("wave") else blas.FT_GRAN_TILE
+    cm, cn = blas.ft_check_tile(tile_class, gran)
+    M, N, K = 200, 333, 600      # C^T is 333 x 200; 3 verifications (k = 256, 512, 600)
+    tau = blas.ft_default_tau(K)
+    ntm, ntn = -(-N // cm), -(-M // cn)
+    last = ntm * ntn - 1
+    rng = np.random.default_rng(90 + tile_class)
+
+    def fault(tile, check):
+        tm, tn = min(cm, N - (tile // ntn) * cm), min(cn, M - (tile % ntn) * cn)
+        return (tile, int(rng.integers(tm)), int(rng.integers(tn)),
+                float(np.float32((1 if rng.integers(2) else -1) * 10.0 ** rng.uniform(-1.0, 1.5))), check)
+
+    for faults in ([], [fault(last, 0), fault(last, 2)], [fault(0, 1), fault(1, 1), fault(1, 2)], [fault(1, 1), fault(1, 1)]):
+        for interval in (256, 0):
+            abuf, bbuf, cbuf, c, st, _ = _run(blas, oracle_mod, M, N, K, 1.5, -1.0, tau, faults=faults, pad=(4, 4, 8), seed=1700 + tile_class,
+                                              mode="workspace" if kind.endswith("workspace") else "fused", tile_class=tile_class,
+                                              granularity=gran, check_interval=interval, no_split=True, values=False)
+            bt = np.ascontiguousarray(bbuf[:, :N].T)
+            c_model = cbuf.copy()
+            st_model = oracle_mod.ft_sgemm_checked(N, M, K, bt, K, abuf, abuf.shape[1], c_model, cbuf.shape[1], 1.5, -1.0,
+                                                   cm, cn, tau, interval, faults)
+            for f in DECISION_FIELDS:
+                assert np.array_equal(st[f], st_model[f]), (tile_class, kind, interval, faults, f, st[f], st_model[f])
+            if not np.any(st["flag"] == 2):
+                want = cbuf.copy()
+                oracle_mod.sgemm_device_order(N, M, K, bt, K, abuf, abuf.shape[1], want, cbuf.shape[1], 1.5, -1.0)
+                assert np.array_equal(c[:, :M], want[:, :M]), (tile_class, kind, interval, faults)
 
 
 def test_workspace_rules(blas, oracle_mod):
