@@ -65,7 +65,7 @@ static void check_tile(const FtClass& fc, int granularity, int* cm, int* cn) {
 
 // ABFT with a workspace splits the tiles of a partial last round of CUs along K, like plain SGEMM's tail split: every
 // slice is a workgroup that verifies (and corrects) its own partial product - the checksums are linear in K - and
-// writes it raw; tail_reduce_kernel adds the slices, ft_tail_status_kernel merges their records.  With fewer tiles
+// writes it raw; tail_reduce_kernel adds the slices and merges their records.  With fewer tiles
 // than half the CUs every tile is split.  A slice is a multiple of `unit` values of k long: the K step, or the
 // verification interval, so that every slice of a cadence kernel verifies whole intervals of the K range.  Returns
 // the number of ways (1: no split), the tiles it applies to and the slice length.
@@ -108,7 +108,14 @@ static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
     const FtTail tail = ft_tail_plan(fc, M, N, K);
     const size_t tile_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_TILE, M, N, K) + ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, tail);
     const size_t wave_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_WAVE, M, N, K) + ft_tail_bytes(fc, HPCDNN_FT_GRAN_WAVE, tail);
-    return tile_mode > wave_mode ? tile_mode : wave_mode;
+    size_t most = tile_mode > wave_mode ? tile_mode : wave_mode;
+    // a product one tile wide or high: every tile split up to eight ways by the kernels that need no pre-pass
+    const int64_t tiles = ceil_div(M, fc.bm) * ceil_div(N, fc.bn);
+    if (ceil_div(M, fc.bm) == 1 || ceil_div(N, fc.bn) == 1) {
+        const size_t all = ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, FtTail{8, static_cast<int>(tiles), 0});
+        if (all > most) most = all;
+    }
+    return most;
 }
 
 // K == 0 with wave-tile granularity: there is nothing to verify, every check tile gets a clean record
@@ -180,6 +187,48 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     }
     const bool edge = needs_edge(a, fc.bm, fc.bn, kGemmBK);
     dim3 grid(a.tiles_m * a.tiles_n, 1, 1);
+    // A product that is one tile wide (or one tile high) reads each row panel of A (column panel of B) in exactly one
+    // workgroup: a pre-pass would read that operand a second time for checksum vectors nobody shares, and on a tall
+    // product with few columns the operand is all the traffic there is.  Those products run the kernels that form the
+    // vectors in their main loop, and use the workspace only to split every tile along K until two workgroups per CU
+    // keep enough bytes on their way from memory.
+    const bool fused_split = ws && K > 0 && !wave && (a.tiles_n == 1 || a.tiles_m == 1) && a.tiles_m * a.tiles_n >= device_cus() / 8;
+    if (fused_split) {
+        if (reinterpret_cast<uintptr_t>(ws) & 15u) return HPCDNN_ERR_WORKSPACE;
+        const int unit = cadence ? opt.check_interval : kGemmBK;
+        const int tiles = a.tiles_m * a.tiles_n;
+        int64_t ways = ceil_div(2 * device_cus(), tiles);
+        const int64_t most = K / (16 * kGemmBK);
+        if (ways > most) ways = most;
+        if (ways > 8) ways = 8;
+        FtTail tail{1, 0, 0};
+        if (ways >= 2) {
+            const int k_chunk = static_cast<int>(ceil_div(ceil_div(K, ways), unit)) * unit;
+            ways = ceil_div(K, k_chunk);
+            if (ways >= 2) tail = FtTail{static_cast<int>(ways), tiles, k_chunk};
+        }
+        if (ws_bytes < ft_tail_bytes(fc, opt.granularity, tail)) tail = FtTail{1, 0, 0};
+        const FtKernel k = ft_kernel(opt.tile_class, ta, cadence ? kFtFusedCad : kFtFused);
+        if (!k.plain) return HPCDNN_ERR_INVALID_VALUE;
+        void (*fn)(const GemmArgs) = edge ? k.edge : k.plain;
+        rc = enable_lds(fn, k.lds);
+        if (rc != HPCDNN_OK) return rc;
+        if (tail.ways >= 2) {
+            a.tail_k_chunk = tail.k_chunk;
+            a.full_tiles = 0;
+            a.tail_split = tail.ways;
+            a.tail_partial = static_cast<float*>(ws);
+            a.tail_status = reinterpret_cast<hpcdnn_ft_status*>(a.tail_partial + static_cast<size_t>(tiles) * tail.ways * fc.bm * fc.bn);
+            grid = dim3(tiles * tail.ways, 1, 1);
+        }
+        hipLaunchKernelGGL(fn, grid, dim3(k.threads), k.lds, s, a);
+        rc = launch_status();
+        if (rc != HPCDNN_OK || a.tail_split < 2) return rc;
+        tail_reduce_kernel<><<<dim3(tiles, fc.bm / 32), 256, 0, s>>>(M, N, fc.bm, fc.bn, a.tiles_m, a.tiles_n, 0, a.tail_split,
+                                                                    a.tail_partial, C, ldc, alpha, beta, a.tail_status, status, 1, 1,
+                                                                    a.status_rows, a.status_ld);
+        return launch_status();
+    }
     // With a workspace the checksum vectors of A and B are formed once per row group / column group by a small
     // bandwidth-bound kernel and the main loop only reads them; without one every workgroup forms them itself.
     if (ws && K > 0) {
@@ -221,11 +270,8 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         rc = launch_status();
         if (rc != HPCDNN_OK || a.tail_split < 2) return rc;
         tail_reduce_kernel<><<<dim3(tail.tiles, fc.bm / 32), 256, 0, s>>>(M, N, fc.bm, fc.bn, a.tiles_m, a.tiles_n, a.full_tiles,
-                                                                         a.tail_split, a.tail_partial, C, ldc, alpha, beta);
-        rc = launch_status();
-        if (rc != HPCDNN_OK || !status) return rc;
-        ft_tail_status_kernel<><<<static_cast<int>(ceil_div(tail.tiles * gm * gn, 64)), 64, 0, s>>>(
-            tail.tiles, a.tail_split, gm, gn, a.tiles_m, a.tiles_n, a.full_tiles, a.tail_status, status, a.status_rows, a.status_ld);
+                                                                         a.tail_split, a.tail_partial, C, ldc, alpha, beta, a.tail_status,
+                                                                         status, gm, gn, a.status_rows, a.status_ld);
         return launch_status();
     }
     const FtKernel k = ft_kernel(opt.tile_class, ta, cadence ? kFtFusedCad : kFtFused);

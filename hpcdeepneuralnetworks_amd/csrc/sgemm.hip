@@ -380,7 +380,7 @@ static int run_sgemm(int M, int N, int K, const float* A, int lda, const float* 
     if (tail_tiles > 0) {
         tail_reduce_kernel<><<<dim3(tail_tiles, cfg.bm / 32), 256, 0, stream>>>(M, N, cfg.bm, cfg.bn, a.tiles_m, a.tiles_n,
                                                                              a.full_tiles, a.tail_split, a.tail_partial, C,
-                                                                             ldc, alpha, beta);
+                                                                             ldc, alpha, beta, nullptr, nullptr, 1, 1, 0, 0);
         return launch_status();
     }
     if (split == 1) return rc;

@@ -218,7 +218,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     int tile_id = blockIdx.x, k_slice = blockIdx.z, k_chunk = p.k_chunk;
     float* tail_out = nullptr;
     int tail_slot = 0;  // index of this slice among all tail slices
-    if (FT != 1 && p.tail_split > 1 && tile_id >= p.full_tiles) {
+    if (p.tail_split > 1 && tile_id >= p.full_tiles) {
         const int r = tile_id - p.full_tiles;
         tail_slot = r;
         tile_id = p.full_tiles + r / p.tail_split;
@@ -1302,7 +1302,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int row_base = m0 + wm * WM + lh * 4;  // + i*32 + 8*(v/4) + v%4
     const int col_base = n0 + wn * WN + lr;      // + j*32
 
-    if (FT != 1 && tail_out) {
+    if (tail_out) {
         // whole tile, no bounds: the reduction that reads these images skips rows and columns past the matrix
         float* out = tail_out + (wm * WM + lh * 4) * BN + wn * WN + lr;
 #pragma unroll
@@ -1443,10 +1443,19 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
 
 // Fixed-order second phase of the tail split: for the tiles after the first full_tiles, C = alpha * (slice 0 +
 // slice 1 + ...) + beta*C.  grid = (tail tiles, bm / 32): one block adds 32 rows of one tile, 4 columns per thread.
+//
+// ABFT (slices != nullptr): the first block of every tile also turns the records of the tile's K slices into the
+// tile's records, one per check tile (gm x gn of them per workgroup tile).  Bad-line counts add up; a slice that could
+// not locate its fault makes the check tile uncorrectable (2); otherwise it is corrected (1) if any slice corrected an
+// element, and reports the first such slice's location and residuals (more than one corrected slice shows in the
+// counts).  Slices are K ranges in ascending order, so with a verification cadence this is the order of the
+// verifications.
 template <int kUnused = 0>
 __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, int bn, int tiles_m, int tiles_n,
                                                           int full_tiles, int splits, const float* __restrict__ partial,
-                                                          float* __restrict__ C, int ldc, float alpha, float beta) {
+                                                          float* __restrict__ C, int ldc, float alpha, float beta,
+                                                          const hpcdnn_ft_status* __restrict__ slices, hpcdnn_ft_status* __restrict__ status,
+                                                          int gm, int gn, int status_rows, int status_ld) {
     int tile_m, tile_n;
     tile_of_block(full_tiles + blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
     const int m0 = tile_m * bm, n0 = tile_n * bn;
@@ -1477,42 +1486,28 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, 
                 dst[e] = (beta == 0.f) ? t : __builtin_fmaf(beta, dst[e], t);
             }
     }
-}
-
-// ABFT with a tail split: the records of a tile's K slices become the tile's records, one per check tile (gm x gn of
-// them per workgroup tile).  Bad-line counts add up; a slice that could not locate its fault makes the check tile
-// uncorrectable (2); otherwise it is corrected (1) if any slice corrected an element, and reports the first such
-// slice's location and residuals (more than one corrected slice shows in the counts).  Slices are K ranges in
-// ascending order, so with a verification cadence this is the order of the verifications.
-template <int kUnused = 0>
-__global__ __launch_bounds__(64) void ft_tail_status_kernel(int tail_tiles, int splits, int gm, int gn, int tiles_m, int tiles_n,
-                                                            int full_tiles, const hpcdnn_ft_status* __restrict__ slices,
-                                                            hpcdnn_ft_status* __restrict__ status, int status_rows, int status_ld) {
-    const int nct = gm * gn;
-    const int idx = blockIdx.x * 64 + threadIdx.x;
-    if (idx >= tail_tiles * nct) return;
-    const int t = idx / nct, ct = idx % nct;
-    int tile_m, tile_n;
-    tile_of_block(full_tiles + t, tiles_m, tiles_n, tile_m, tile_n);
-    hpcdnn_ft_status out;
-    out.flag = 0; out.row = -1; out.col = -1; out.n_bad_rows = 0; out.n_bad_cols = 0;
-    out.row_residual = 0.f; out.col_residual = 0.f; out.max_clean_residual = 0.f;
-    bool located = false;
-    for (int z = 0; z < splits; ++z) {
-        const hpcdnn_ft_status s = slices[(t * splits + z) * nct + ct];
-        out.n_bad_rows += s.n_bad_rows;
-        out.n_bad_cols += s.n_bad_cols;
-        out.max_clean_residual = s.max_clean_residual > out.max_clean_residual ? s.max_clean_residual : out.max_clean_residual;
-        if (s.flag == 2) out.flag = 2;
-        if (s.flag == 1 && !located) {
-            located = true;
-            out.row = s.row; out.col = s.col; out.row_residual = s.row_residual; out.col_residual = s.col_residual;
+    if (slices && status && blockIdx.y == 0 && static_cast<int>(threadIdx.x) < gm * gn) {
+        const int nct = gm * gn, ct = threadIdx.x, t = blockIdx.x;
+        hpcdnn_ft_status out;
+        out.flag = 0; out.row = -1; out.col = -1; out.n_bad_rows = 0; out.n_bad_cols = 0;
+        out.row_residual = 0.f; out.col_residual = 0.f; out.max_clean_residual = 0.f;
+        bool located = false;
+        for (int z = 0; z < splits; ++z) {
+            const hpcdnn_ft_status s = slices[(t * splits + z) * nct + ct];
+            out.n_bad_rows += s.n_bad_rows;
+            out.n_bad_cols += s.n_bad_cols;
+            out.max_clean_residual = s.max_clean_residual > out.max_clean_residual ? s.max_clean_residual : out.max_clean_residual;
+            if (s.flag == 2) out.flag = 2;
+            if (s.flag == 1 && !located) {
+                located = true;
+                out.row = s.row; out.col = s.col; out.row_residual = s.row_residual; out.col_residual = s.col_residual;
+            }
         }
+        if (out.flag == 2) { out.row = -1; out.col = -1; out.row_residual = 0.f; out.col_residual = 0.f; }
+        else if (located) out.flag = 1;
+        const int srow = tile_m * gm + ct / gn, scol = tile_n * gn + ct % gn;
+        if (srow < status_rows && scol < status_ld) status[srow * status_ld + scol] = out;
     }
-    if (out.flag == 2) { out.row = -1; out.col = -1; out.row_residual = 0.f; out.col_residual = 0.f; }
-    else if (located) out.flag = 1;
-    const int srow = tile_m * gm + ct / gn, scol = tile_n * gn + ct % gn;
-    if (srow < status_rows && scol < status_ld) status[srow * status_ld + scol] = out;
 }
 
 // ---- ABFT pre-encode: the checksum vectors of the operands, one per row group (RM rows) / column group (CN

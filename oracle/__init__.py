@@ -82,6 +82,10 @@ def _load():
     lib.oracle_gemm_max_err.argtypes = [C.c_int, fp, C.c_int, ip, C.c_int, dp, dp]
     lib.oracle_saxpy.restype = None
     lib.oracle_saxpy.argtypes = [C.c_int64, C.c_float, fp, fp]
+    lib.oracle_saxpy_omp.restype = None
+    lib.oracle_saxpy_omp.argtypes = [C.c_int64, C.c_float, fp, fp]
+    lib.oracle_sdot_f64_serial.restype = C.c_double
+    lib.oracle_sdot_f64_serial.argtypes = [C.c_int64, fp, fp]
     lib.oracle_sdot_f64.restype = C.c_double
     lib.oracle_sdot_f64.argtypes = [C.c_int64, fp, fp]
     lib.oracle_sdot_f32.restype = C.c_float
@@ -201,6 +205,17 @@ def saxpy(alpha: float, x: np.ndarray, y: np.ndarray) -> None:
     """In-place y = fmaf(alpha, x, y)."""
     assert x.size == y.size
     _load().oracle_saxpy(x.size, alpha, _f(x), _f(y))
+
+
+def saxpy_omp(alpha: float, x: np.ndarray, y: np.ndarray) -> None:
+    """In-place y = fmaf(alpha, x, y) on the OpenMP pool (same bits as ``saxpy``)."""
+    assert x.size == y.size
+    _load().oracle_saxpy_omp(x.size, alpha, _f(x), _f(y))
+
+
+def sdot_f64_serial(x: np.ndarray, y: np.ndarray) -> float:
+    """Double-accumulated dot product on one thread (``sdot_f64`` is the OpenMP form)."""
+    return float(_load().oracle_sdot_f64_serial(x.size, _f(x), _f(y)))
 
 
 def sdot_f64(x: np.ndarray, y: np.ndarray) -> float:

@@ -208,6 +208,21 @@ void oracle_saxpy(int64_t n, float alpha, const float* x, float* y) {
     for (int64_t i = 0; i < n; ++i) y[i] = fmaf(alpha, x[i], y[i]);
 }
 
+/* The same loop spread over the OpenMP pool (element-wise, so the bits do not depend on the thread count); the
+ * multi-threaded CPU baseline of the benchmark. */
+void oracle_saxpy_omp(int64_t n, float alpha, const float* x, float* y) {
+    #pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) y[i] = fmaf(alpha, x[i], y[i]);
+}
+
+/* Double-accumulated dot product on one thread, k ascending: the single-thread CPU baseline of the benchmark
+ * (oracle_sdot_f64 below is its OpenMP form, whose partial sums are added in thread order). */
+double oracle_sdot_f64_serial(int64_t n, const float* x, const float* y) {
+    double s = 0.0;
+    for (int64_t i = 0; i < n; ++i) s += (double)x[i] * (double)y[i];
+    return s;
+}
+
 /* Exact-as-possible dot product (double accumulate); the tolerance test for
  * kernel/sdot/sdot.cu:9-36 is relative to this. */
 double oracle_sdot_f64(int64_t n, const float* x, const float* y) {

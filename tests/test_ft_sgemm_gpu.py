@@ -451,6 +451,45 @@ def test_seeded_random_cases_equal_the_model(blas, oracle_mod):
                 assert np.array_equal(c[:, :N], want[:, :N]), what
 
 
+@pytest.mark.parametrize("M,N,K,tile_class", [(4200, 50, 600, 4), (8300, 64, 1030, 3), (40, 8200, 520, 2), (9000, 100, 512, 2)])
+def test_products_one_tile_wide_are_split_along_k_without_a_pre_pass(blas, oracle_mod, M, N, K, tile_class):
+    """A product one tile wide (or high) reads each operand panel in one workgroup only: with a workspace its tiles are
+    split along K by the kernels that form the checksum vectors in their main loop (no second pass over the operands).
+    Decisions equal the model's, values obey the criterion, and the result does not depend on run-to-run timing."""
+    bm, bn = blas.ft_tile(tile_class)
+    tau = blas.ft_default_tau(K)
+    a = oracle_mod.fill_uniform_matrix(M, K, 2200, ld=K + 4)
+    b = oracle_mod.fill_uniform_matrix(K, N, 2201, ld=N + 4)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, 2202, ld=N + 8)
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    ntm, ntn = -(-M // bm), -(-N // bn)
+    assert min(ntm, ntn) == 1
+    last = ntm * ntn - 1
+    tm, tn = M - (ntm - 1) * bm, N - (ntn - 1) * bn
+    for fault in [None, (last, tm - 1, tn - 1, -0.75), (ntm * ntn // 2, 17, 9, 12.5)]:
+        for t in (tau, 0.0):
+            results = []
+            for _ in range(2):
+                ws = torch.full((blas.ft_workspace_bytes(M, N, K) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+                dc = torch.from_numpy(c0).cuda()
+                status = blas.ft_status_alloc(M, N, tile_class=tile_class)
+                blas.ft_sgemm(M, N, K, da, db, dc, 1.5, -1.0, tau=t, fault=fault, status=status, ws=ws, tile_class=tile_class)
+                results.append((dc.cpu().numpy(), blas.ft_status_numpy(status)))
+            (c, st), (c2, st2) = results
+            assert np.array_equal(c[:, :N], c2[:, :N]) and np.array_equal(st, st2)
+            c_model = c0.copy()
+            st_model = oracle_mod.ft_sgemm(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, bm, bn, t, fault)
+            for f in DECISION_FIELDS:
+                assert np.array_equal(st[f], st_model[f]), (fault, t, f, st[f], st_model[f])
+            ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, K + 4, b, N + 4, c0, N + 8, 1.5, -1.0)
+            assert oracle_mod.gemm_max_err(N, c, c.shape[1], ref, den) <= TOL
+            assert np.all(np.isnan(c[:, N:]))
+            # the split did happen: C differs in the last bits from the unsplit call (no workspace)
+            dc = torch.from_numpy(c0).cuda()
+            blas.ft_sgemm(M, N, K, da, db, dc, 1.5, -1.0, tau=t, fault=fault, tile_class=tile_class)
+            assert not np.array_equal(dc.cpu().numpy()[:, :N], c[:, :N])
+
+
 def test_partial_last_round_is_split_along_k(blas, oracle_mod):
     """With room in the workspace the tiles of a partial last round of CUs are split along K; every slice verifies its
     own partial product, a second pass adds the slices and merges their records.  Decisions and C must not depend on

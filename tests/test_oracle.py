@@ -170,6 +170,22 @@ def test_saxpy_differs_from_unfused_where_it_must(oracle_mod):
     assert np.float32(np.float32(a * a) + np.float32(-1.0)) != y[0]
 
 
+def test_threaded_saxpy_and_serial_sdot_are_the_same_functions(oracle_mod):
+    """The two extra CPU baselines of the benchmark: SAXPY on the OpenMP pool has the bits of the one-thread loop, the
+    one-thread double-accumulated dot product agrees with numpy and with the OpenMP form to double rounding."""
+    n = (1 << 16) + 7
+    x, y = oracle_mod.fill_uniform(n, 5), oracle_mod.fill_uniform(n, 6)
+    y1, y2 = y.copy(), y.copy()
+    oracle_mod.saxpy(2.5, x, y1)
+    oracle_mod.saxpy_omp(2.5, x, y2)
+    assert np.array_equal(y1, y2) and not np.array_equal(y1, y)
+    want = float(np.dot(x.astype(np.float64), y.astype(np.float64)))
+    assert oracle_mod.sdot_f64_serial(x, y) == pytest.approx(want, rel=1e-13, abs=1e-12)
+    assert oracle_mod.sdot_f64(x, y) == pytest.approx(oracle_mod.sdot_f64_serial(x, y), rel=1e-13, abs=1e-12)
+    assert oracle_mod.sdot_f64_serial(np.array([3.0, 4.0], np.float32), np.array([5.0, -2.0], np.float32)) == 7.0
+    assert oracle_mod.sdot_f64_serial(x[:0], y[:0]) == 0.0
+
+
 def test_sdot_f64_and_f32(oracle_mod):
     rng = np.random.default_rng(3)
     n = 100003
