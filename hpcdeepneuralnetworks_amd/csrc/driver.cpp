@@ -170,7 +170,7 @@ int run_ft_sgemm(int start, int end, int gap, int first, int last) {
         if (f > ft_ws_bytes) ft_ws_bytes = f;
         if (o > off_ws_bytes) off_ws_bytes = o;
     }
-    for (int n = start; n <= end; n += gap) {  // the column-major ABFT series adds room for its transposed operand
+    for (int n = start; n <= end; n += gap) {  // the column-major ABFT series (its query is that of the transposed problem)
         const size_t f = hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM_CM_NT, n, n, K);
         if (f > ft_ws_bytes) ft_ws_bytes = f;
     }

@@ -414,7 +414,10 @@ extern "C" int hpcdnn_ft_sgemm_cm_nt(int M, int N, int K, const float* A, int ld
 // library runs on holds its own copy of the array at its own address, looked up once per device.
 static __device__ __align__(256) unsigned char scratch[HPCDNN_FT_STATIC_SCRATCH_BYTES];
 
-static int static_scratch_address(void** out) {
+// First call on a device: look the array's address up and let the two kernels the entry point launches (full-tile
+// and ragged-tile forms of the 256 x 128 class) use their LDS.  Neither belongs into a stream capture, so a first call
+// that finds its stream capturing is refused; any earlier eager call (M = 0 is enough) has done the set-up.
+static int static_scratch_address(void** out, hipStream_t stream) {
     constexpr int kMaxDevices = 64;
     static std::mutex mu;
     static void* address[kMaxDevices] = {};
@@ -424,10 +427,21 @@ static int static_scratch_address(void** out) {
     if (dev < 0 || dev >= kMaxDevices) return HPCDNN_ERR_INVALID_VALUE;
     std::lock_guard<std::mutex> lock(mu);
     if (!address[dev]) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &capturing);
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (capturing != hipStreamCaptureStatusNone) return HPCDNN_ERR_NOT_READY;
         void* p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // the address on the current device
         if (e != hipSuccess) return static_cast<int>(e);
         if (!p) return HPCDNN_ERR_WORKSPACE;
+        int rc = HPCDNN_OK;
+        for (int kind : {kFtPre, kFtFused}) {  // (kFtFused: products one tile wide or high)
+            const FtKernel k = ft_kernel(0, false, kind);
+            if (rc == HPCDNN_OK) rc = enable_lds(k.plain, k.lds);
+            if (rc == HPCDNN_OK) rc = enable_lds(k.edge, k.lds);
+        }
+        if (rc != HPCDNN_OK) return rc;
         address[dev] = p;
     }
     *out = address[dev];
@@ -439,14 +453,15 @@ extern "C" int hpcdnn_ft_sgemm_static(int M, int N, int K, const float* A, int l
                                       hpcdnn_ft_status* status, void* stream) {
     int rc = check_gemm_args(M, N, K, A, lda, B, ldb, C, ldc);
     if (rc != HPCDNN_OK) return rc;
+    void* ws = nullptr;
+    rc = static_scratch_address(&ws, static_cast<hipStream_t>(stream));
+    if (rc != HPCDNN_OK) return rc;
     if (M == 0 || N == 0) return HPCDNN_OK;
     // the checksum vectors of the 256 x 128 class must fit; beyond that the call is refused, never silently slower
     if (K > 0 && ft_enc_bytes(kFtClasses[0], HPCDNN_FT_GRAN_TILE, M, N, K) > HPCDNN_FT_STATIC_SCRATCH_BYTES) return HPCDNN_ERR_WORKSPACE;
-    void* ws = nullptr;
-    rc = static_scratch_address(&ws);
-    if (rc != HPCDNN_OK) return rc;
     // Nothing in the array has to start at zero: the pre-pass rewrites every word of the checksum vectors the GEMM
     // reads (their zero padding included), and the K slices and their records are written before they are read.
+    // (a product one tile wide or high runs the kernels that need no pre-pass; their K slices use the array alone)
     return hpcdnn_ft_sgemm_ex(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, tau, inject, status, ws,
                               HPCDNN_FT_STATIC_SCRATCH_BYTES, 0, stream);
 }

@@ -20,6 +20,7 @@ extern "C" const char* hpcdnn_error_string(int code) {
         case HPCDNN_OK: return "success";
         case HPCDNN_ERR_INVALID_VALUE: return "invalid argument";
         case HPCDNN_ERR_WORKSPACE: return "workspace missing or too small";
+        case HPCDNN_ERR_NOT_READY: return "one-time set-up needed: make one call outside stream capture first";
         default: return hipGetErrorString(static_cast<hipError_t>(code));
     }
 }

@@ -33,6 +33,7 @@ extern "C" {
 #define HPCDNN_OK 0
 #define HPCDNN_ERR_INVALID_VALUE 1      /* == hipErrorInvalidValue */
 #define HPCDNN_ERR_WORKSPACE 2          /* workspace missing or too small (== hipErrorOutOfMemory) */
+#define HPCDNN_ERR_NOT_READY 3          /* one-time set-up refused under stream capture (== hipErrorNotInitialized) */
 
 /* Output tile of the ABFT kernel: one checksum pair (256 row sums, 128 column
  * sums) and one status record per tile, tiles numbered row-major:
@@ -318,6 +319,11 @@ float hpcdnn_ft_default_tau(int K);
  * overlap in time on one device (different streams, different host threads)
  * race on it and must be serialised by the caller; the array needs no
  * initialisation and keeps nothing between calls.
+ * The first call on a device looks the array's address up and raises the LDS
+ * limit of its kernels, which does not belong into a stream capture: it
+ * returns HPCDNN_ERR_NOT_READY when its stream is capturing.  Make one eager
+ * call on the device beforehand (M = 0 is enough and launches nothing); every
+ * later call only enqueues kernels and can be captured.
  * No counterpart in the reference, whose driver allocates everything up front
  * (kernel/ft_sgemm/sgemm.cu:60-83). */
 #define HPCDNN_FT_STATIC_SCRATCH_BYTES (4u << 20)

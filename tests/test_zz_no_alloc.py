@@ -72,3 +72,84 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit(blas):
     L = _lib.lib()
     rc = L.hpcdnn_ft_sgemm_static(n, n, n, t.data_ptr(), n, t.data_ptr(), n, t.data_ptr(), n, 1.0, 0.0, 0.0, None, None, None)
     assert rc == 2 and b"workspace" in L.hpcdnn_error_string(rc)   # refused before anything is launched
+
+
+_CAPTURE_SCRIPT = r"""
+import sys
+import numpy as np
+import torch
+sys.path.insert(0, sys.argv[1])
+import oracle
+from hpcdeepneuralnetworks_amd import blas, _lib
+
+M, N, K = 300, 200, 420
+tau = blas.ft_default_tau(K)
+a = torch.from_numpy(oracle.fill_uniform_matrix(M, K, 1)).cuda()
+b = torch.from_numpy(oracle.fill_uniform_matrix(K, N, 2)).cuda()
+c0 = torch.from_numpy(oracle.fill_uniform_matrix(M, N, 3)).cuda()
+c = c0.clone()
+status = blas.ft_status_alloc(M, N)
+fault = (3, 40, 70, -0.75)
+side = torch.cuda.Stream()
+side.wait_stream(torch.cuda.current_stream())
+
+# 1. the very first call of the process under capture: refused with the set-up error, nothing enqueued
+graph = torch.cuda.CUDAGraph()
+refused = False
+with torch.cuda.stream(side):
+    with torch.cuda.graph(graph, stream=side):
+        try:
+            blas.ft_sgemm_static(M, N, K, a, b, c, 1.5, -1.0, tau=tau, fault=fault, status=status)
+        except blas.HpcdnnError as e:
+            refused = "set-up" in str(e)
+assert refused, "a first call under capture must be refused"
+torch.cuda.synchronize()
+
+# 2. the documented remedy: one eager call that launches nothing
+rc = _lib.lib().hpcdnn_ft_sgemm_static(0, 0, 0, None, 1, None, 1, None, 1, 1.0, 0.0, 0.0, None, None, None)
+assert rc == 0, rc
+
+# 3. now the call can be captured, without any eager call on these operands before
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.stream(side):
+    with torch.cuda.graph(graph, stream=side):
+        blas.ft_sgemm_static(M, N, K, a, b, c, 1.5, -1.0, tau=tau, fault=fault, status=status)
+torch.cuda.synchronize()
+
+def reference():
+    ws = torch.full((blas.FT_STATIC_SCRATCH_BYTES // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    c_ws, st_ws = c0.clone(), blas.ft_status_alloc(M, N)
+    blas.ft_sgemm(M, N, K, a, b, c_ws, 1.5, -1.0, tau=tau, fault=fault, status=st_ws, ws=ws)
+    torch.cuda.synchronize()
+    return c_ws, blas.ft_status_numpy(st_ws)
+
+for replay in range(3):
+    if replay:   # changed operands between the replays, and eager work on the device
+        a.mul_(-0.5)
+        b.add_(0.25)
+    c.copy_(c0)
+    status.zero_()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    c_ws, st_ws = reference()
+    assert torch.equal(c, c_ws), replay
+    st = blas.ft_status_numpy(status)
+    assert np.array_equal(st, st_ws), replay
+    assert st["flag"][3] == 1 and (st["row"][3], st["col"][3]) == (40, 70), replay
+print("CAPTURE-OK")
+"""
+
+
+def test_static_scratch_entry_point_under_stream_capture():
+    """The entry point is meant for code under HIP graph capture.  Its one-time set-up per device (address of the array,
+    LDS limit of its kernels) cannot be captured: a first call under capture is refused with HPCDNN_ERR_NOT_READY, and
+    after one eager call that launches nothing the call is captured and replayed - with changed operands between the
+    replays - bit for bit like the workspace entry point.  A process of its own, so that the call under capture really is
+    the first."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, "-c", _CAPTURE_SCRIPT, root], capture_output=True, text=True, timeout=280)
+    assert p.returncode == 0 and "CAPTURE-OK" in p.stdout, (p.stdout[-2000:], p.stderr[-4000:])
