@@ -360,8 +360,12 @@ def main() -> int:
                                                       granularity=blas.FT_GRAN_WAVE), st, wu)
         ms_cad = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ft_ws, check_interval=256), st, wu)
         ms_cad_fused = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, check_interval=256), st, wu)
+        # the reference's second scheme: two row sums of B (weights [1, 1, ...] and [1, 2, ...]), location from their ratio
+        ms_weighted = median_timed(lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=tau, status=status, ws=ft_ws,
+                                                         locator=blas.FT_LOCATE_WEIGHTED), st, wu)
         pct = lambda t: round((t - ms_plain) / ms_plain * 100.0, 2)
         extras["abft_granularity_4096"] = {
+            "weighted_locator_256x128_overhead_pct": pct(ms_weighted),
             "tile_256x128_overhead_pct": pct(ms_ft), "wave_tile_128x32_overhead_pct": pct(ms_wave),
             "wave_tile_64x64_of_128x128_class_overhead_pct": pct(ms_wave1),
             "tile_verify_every_256k_overhead_pct": pct(ms_cad), "tile_verify_every_256k_no_workspace_overhead_pct": pct(ms_cad_fused),
@@ -442,7 +446,10 @@ def main() -> int:
         tau_s = blas.ft_default_tau(kk)
         ms_cls = median_timed(lambda: blas.ft_sgemm(m, n_, kk, a, b, c, 1.0, 0.0, tau=tau_s, status=status_s, ws=ft_ws_s, tile_class=cls), st, wu)
         ms_c1 = median_timed(lambda: blas.ft_sgemm(m, n_, kk, a, b, c, 1.0, 0.0, tau=tau_s, status=status_1, ws=ft_ws_s, tile_class=1), st, wu)
+        ms_w = median_timed(lambda: blas.ft_sgemm(m, n_, kk, a, b, c, 1.0, 0.0, tau=tau_s, status=status_s, ws=ft_ws_s, tile_class=cls,
+                                                  locator=blas.FT_LOCATE_WEIGHTED), st, wu)
         extras["abft_16384x64x4096"] = {
+            "weighted_locator_overhead_pct_vs_sgemm": round((ms_w - ms_plain) / ms_plain * 100.0, 2),
             "picked_tile_class": cls, "picked_tile": list(blas.ft_tile(cls)),
             "sgemm_gflops": round(2.0 * m * n_ * kk / ms_plain / 1e6, 1),
             "ft_sgemm_gflops": round(2.0 * m * n_ * kk / ms_cls / 1e6, 1),

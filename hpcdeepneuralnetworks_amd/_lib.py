@@ -67,6 +67,8 @@ class Fault(C.Structure):
 
 
 FT_GRAN_TILE = 0
+FT_LOCATE_ROW_COL = 0
+FT_LOCATE_WEIGHTED = 1
 FT_GRAN_WAVE = 1
 FT_MAX_FAULTS = 4
 
@@ -77,7 +79,7 @@ class FaultAt(C.Structure):
 
 class FtOptions(C.Structure):
     _fields_ = [("tile_class", C.c_int32), ("granularity", C.c_int32), ("check_interval", C.c_int32),
-                ("n_faults", C.c_int32), ("faults", FaultAt * FT_MAX_FAULTS)]
+                ("n_faults", C.c_int32), ("faults", FaultAt * FT_MAX_FAULTS), ("locator", C.c_int32)]
 
 
 class HpcdnnError(RuntimeError):

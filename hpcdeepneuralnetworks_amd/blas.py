@@ -138,14 +138,16 @@ def sgemm_cm_nt(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: to
 
 def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
              tau: float = 0.0, fault=None, status: torch.Tensor | None = None, ws: torch.Tensor | None = None,
-             tile_class: int = 0, granularity: int = 0, check_interval: int = 0, faults=None) -> None:
+             tile_class: int = 0, granularity: int = 0, check_interval: int = 0, faults=None, locator: int = 0) -> None:
     """ABFT GEMM; ``fault`` = (tile, row, col, delta) or None; ``status`` = int32 tensor of 8*ft_num_check_tiles words;
     ``ws`` = optional scratch tensor of ``ft_workspace_bytes(M, N, K)`` bytes (checksum vectors are then formed
     by a pre-pass instead of inside the main loop); ``tile_class`` selects the ABFT tile (0 = 256x128, 1 = 128x128, 3 = 128x64, 4 = 64x64,
     2 = 64x128).  ``granularity`` FT_GRAN_TILE keeps one checksum pair, verification and status record per tile of the
     class, FT_GRAN_WAVE one per wave tile (``ft_check_tile``); ``check_interval`` > 0 also verifies every that many
     values of k inside the K loop, with re-synchronised references; ``faults`` = up to four
-    (tile, row, col, delta[, check]) in check-tile units, ``check`` = the verification each precedes.
+    (tile, row, col, delta[, check]) in check-tile units, ``check`` = the verification each precedes; ``locator``
+    FT_LOCATE_ROW_COL finds a fault where a faulty row meets a faulty column, FT_LOCATE_WEIGHTED from two row checksums
+    with weights [1, 1, ...] and [1, 2, ...] (the reference's "kernel 2", kernel/ft_sgemm/README.md:16-26; needs ``ws``).
 
     Counterpart of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)`` (kernel/ft_sgemm/sgemm.cu:159-165), of its
     warp- and thread-level variants and of its verification every 256 k (ft_sgemm_huge.cuh:143).
@@ -161,7 +163,7 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
             raise HpcdnnError(f"status must be a contiguous int32 GPU tensor with >= {need} elements")
         sp = status.data_ptr()
     wp, wb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
-    if granularity == 0 and check_interval == 0 and not faults:
+    if granularity == 0 and check_interval == 0 and not faults and locator == 0:
         f = None
         if fault is not None:
             f = C.byref(Fault(int(fault[0]), int(fault[1]), int(fault[2]), float(fault[3])))
@@ -173,6 +175,7 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
         raise HpcdnnError(f"at most {_lib.FT_MAX_FAULTS} faults per call")
     opt = _lib.FtOptions()
     opt.tile_class, opt.granularity, opt.check_interval, opt.n_faults = tile_class, granularity, check_interval, len(every)
+    opt.locator = locator
     for i, fl in enumerate(every):
         opt.faults[i] = _lib.FaultAt(int(fl[0]), int(fl[1]), int(fl[2]), float(fl[3]), int(fl[4]) if len(fl) > 4 else 0)
     check(L.hpcdnn_ft_sgemm_opt(M, N, K, pa, lda, pb, ldb, pc, ldc, alpha, beta, tau, C.byref(opt), sp, wp, wb, _stream()),
@@ -180,6 +183,7 @@ def ft_sgemm(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch
 
 
 FT_GRAN_TILE, FT_GRAN_WAVE = _lib.FT_GRAN_TILE, _lib.FT_GRAN_WAVE
+FT_LOCATE_ROW_COL, FT_LOCATE_WEIGHTED = _lib.FT_LOCATE_ROW_COL, _lib.FT_LOCATE_WEIGHTED
 FT_STATIC_SCRATCH_BYTES = 4 << 20
 
 
@@ -189,7 +193,7 @@ def ft_cm_nt_workspace_bytes(M: int, N: int, K: int) -> int:
 
 def ft_sgemm_cm_nt(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, alpha: float, beta: float,
                    ws: torch.Tensor | None, tau: float = 0.0, status: torch.Tensor | None = None, tile_class: int = 0,
-                   granularity: int = 0, check_interval: int = 0, faults=None) -> None:
+                   granularity: int = 0, check_interval: int = 0, faults=None, locator: int = 0) -> None:
     """ABFT GEMM on the column-major buffers of ``ft_sgemm_huge<<<...>>>(M, N, K, A, B, C, alpha, beta)``
     (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:21): ``C (M x N) = alpha*A (M x K) @ B (N x K).T + beta*C``.  The tensors hold
     the column-major matrices as their row-major transposes (``A`` K x M, ``B`` K x N, ``C`` N x M).  Tiles, status
@@ -210,6 +214,7 @@ def ft_sgemm_cm_nt(M: int, N: int, K: int, A: torch.Tensor, B: torch.Tensor, Cm:
         raise HpcdnnError(f"at most {_lib.FT_MAX_FAULTS} faults per call")
     opt = _lib.FtOptions()
     opt.tile_class, opt.granularity, opt.check_interval, opt.n_faults = tile_class, granularity, check_interval, len(every)
+    opt.locator = locator
     for i, fl in enumerate(every):
         opt.faults[i] = _lib.FaultAt(int(fl[0]), int(fl[1]), int(fl[2]), float(fl[3]), int(fl[4]) if len(fl) > 4 else 0)
     wp, wb = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)

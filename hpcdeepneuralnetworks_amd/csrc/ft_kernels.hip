@@ -37,6 +37,7 @@ FtKernel HPCDNN_FT_PASTE(ft_kernel_c, HPCDNN_FT_CLASS, _ta, HPCDNN_FT_TA)(int ki
         case kFtPreCad: return make_kernel<2, 0, true>();
         case kFtWave: return make_kernel<2, 1, false>();
         case kFtWaveCad: return make_kernel<2, 1, true>();
+        case kFtWeighted: return make_kernel<3, 0, false>();
         default: return FtKernel{nullptr, nullptr, 0, 0};
     }
 }

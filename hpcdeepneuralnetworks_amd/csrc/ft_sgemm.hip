@@ -88,10 +88,29 @@ static FtTail ft_tail_plan(const FtClass& fc, int M, int N, int K, int unit = kG
     if (s < 2) return none;
     return FtTail{static_cast<int>(s), static_cast<int>(r), k_chunk};
 }
+// A product one tile wide or high streams an operand that no other workgroup shares: all its tiles are split along K
+// until two workgroups per CU keep enough bytes on their way from memory (at most eight ways, at least 16 K steps per
+// slice, slices a multiple of `unit` long).
+static FtTail ft_split_all_plan(int tiles, int K, int unit) {
+    int64_t ways = ceil_div(2 * device_cus(), tiles);
+    const int64_t most = K / (16 * kGemmBK);
+    if (ways > most) ways = most;
+    if (ways > 8) ways = 8;
+    if (ways < 2) return FtTail{1, 0, 0};
+    const int k_chunk = static_cast<int>(ceil_div(ceil_div(K, ways), unit)) * unit;
+    ways = ceil_div(K, k_chunk);
+    if (ways < 2) return FtTail{1, 0, 0};
+    return FtTail{static_cast<int>(ways), tiles, k_chunk};
+}
 // checksum vectors: one row per row group and per column group of the granularity
 static size_t ft_enc_bytes(const FtClass& fc, int granularity, int M, int N, int K) {
     const int gm = granularity == HPCDNN_FT_GRAN_WAVE ? fc.wgm : 1, gn = granularity == HPCDNN_FT_GRAN_WAVE ? fc.wgn : 1;
     const size_t b = static_cast<size_t>(ceil_div(M, fc.bm) * gm + ceil_div(N, fc.bn) * gn) * ft_enc_ld(K) * sizeof(float);
+    return (b + 15) & ~static_cast<size_t>(15);
+}
+// the weighted locator's vectors: two rows (plain and weighted row sums of B) per tile column
+static size_t ft_weighted_enc_bytes(const FtClass& fc, int N, int K) {
+    const size_t b = static_cast<size_t>(2 * ceil_div(N, fc.bn)) * ft_enc_ld(K) * sizeof(float);
     return (b + 15) & ~static_cast<size_t>(15);
 }
 // the raw tile images of the K slices and their records (one per check tile of the workgroup tile)
@@ -109,10 +128,12 @@ static size_t ft_class_workspace_bytes(int tile_class, int M, int N, int K) {
     const size_t tile_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_TILE, M, N, K) + ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, tail);
     const size_t wave_mode = ft_enc_bytes(fc, HPCDNN_FT_GRAN_WAVE, M, N, K) + ft_tail_bytes(fc, HPCDNN_FT_GRAN_WAVE, tail);
     size_t most = tile_mode > wave_mode ? tile_mode : wave_mode;
+    const size_t weighted_mode = ft_weighted_enc_bytes(fc, N, K) + ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, tail);
+    if (weighted_mode > most) most = weighted_mode;
     // a product one tile wide or high: every tile split up to eight ways by the kernels that need no pre-pass
     const int64_t tiles = ceil_div(M, fc.bm) * ceil_div(N, fc.bn);
     if (ceil_div(M, fc.bm) == 1 || ceil_div(N, fc.bn) == 1) {
-        const size_t all = ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, FtTail{8, static_cast<int>(tiles), 0});
+        const size_t all = ft_weighted_enc_bytes(fc, N, K) + ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, FtTail{8, static_cast<int>(tiles), 0});
         if (all > most) most = all;
     }
     return most;
@@ -138,12 +159,15 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     if (opt.granularity != HPCDNN_FT_GRAN_TILE && opt.granularity != HPCDNN_FT_GRAN_WAVE) return HPCDNN_ERR_INVALID_VALUE;
     if (opt.check_interval < 0 || opt.check_interval % kGemmBK != 0) return HPCDNN_ERR_INVALID_VALUE;
     if (opt.n_faults < 0 || opt.n_faults > HPCDNN_FT_MAX_FAULTS) return HPCDNN_ERR_INVALID_VALUE;
+    if (opt.locator != HPCDNN_FT_LOCATE_ROW_COL && opt.locator != HPCDNN_FT_LOCATE_WEIGHTED) return HPCDNN_ERR_INVALID_VALUE;
     const FtClass& fc = kFtClasses[opt.tile_class];
     const bool wave = opt.granularity == HPCDNN_FT_GRAN_WAVE;
+    const bool weighted = opt.locator == HPCDNN_FT_LOCATE_WEIGHTED;
     // an interval that covers all of K is a single verification after the loop
     const bool cadence = opt.check_interval > 0 && opt.check_interval < K;
+    if (weighted && (wave || cadence)) return HPCDNN_ERR_INVALID_VALUE;  // one pair of checksums per workgroup tile, verified once
     if (M == 0 || N == 0) return HPCDNN_OK;
-    if (wave && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
+    if ((wave || weighted) && K > 0 && !ws) return HPCDNN_ERR_WORKSPACE;
 
     GemmArgs a = make_args(M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, fc.bm, fc.bn);
     // tau > 0: absolute; tau <= 0: scaled to the data, the threshold of a line of n elements being f * 4.3 FP32
@@ -192,21 +216,11 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     // product with few columns the operand is all the traffic there is.  Those products run the kernels that form the
     // vectors in their main loop, and use the workspace only to split every tile along K until two workgroups per CU
     // keep enough bytes on their way from memory.
-    const bool fused_split = ws && K > 0 && !wave && (a.tiles_n == 1 || a.tiles_m == 1) && a.tiles_m * a.tiles_n >= device_cus() / 8;
+    const bool fused_split = ws && K > 0 && !wave && !weighted && (a.tiles_n == 1 || a.tiles_m == 1) && a.tiles_m * a.tiles_n >= device_cus() / 8;
     if (fused_split) {
         if (reinterpret_cast<uintptr_t>(ws) & 15u) return HPCDNN_ERR_WORKSPACE;
-        const int unit = cadence ? opt.check_interval : kGemmBK;
         const int tiles = a.tiles_m * a.tiles_n;
-        int64_t ways = ceil_div(2 * device_cus(), tiles);
-        const int64_t most = K / (16 * kGemmBK);
-        if (ways > most) ways = most;
-        if (ways > 8) ways = 8;
-        FtTail tail{1, 0, 0};
-        if (ways >= 2) {
-            const int k_chunk = static_cast<int>(ceil_div(ceil_div(K, ways), unit)) * unit;
-            ways = ceil_div(K, k_chunk);
-            if (ways >= 2) tail = FtTail{static_cast<int>(ways), tiles, k_chunk};
-        }
+        FtTail tail = ft_split_all_plan(tiles, K, cadence ? opt.check_interval : kGemmBK);
         if (ws_bytes < ft_tail_bytes(fc, opt.granularity, tail)) tail = FtTail{1, 0, 0};
         const FtKernel k = ft_kernel(opt.tile_class, ta, cadence ? kFtFusedCad : kFtFused);
         if (!k.plain) return HPCDNN_ERR_INVALID_VALUE;
@@ -232,10 +246,13 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     // With a workspace the checksum vectors of A and B are formed once per row group / column group by a small
     // bandwidth-bound kernel and the main loop only reads them; without one every workgroup forms them itself.
     if (ws && K > 0) {
-        const size_t enc_bytes = ft_enc_bytes(fc, opt.granularity, M, N, K);
+        const size_t enc_bytes = weighted ? ft_weighted_enc_bytes(fc, N, K) : ft_enc_bytes(fc, opt.granularity, M, N, K);
         if (ws_bytes < enc_bytes || (reinterpret_cast<uintptr_t>(ws) & 15u)) return HPCDNN_ERR_WORKSPACE;
         // the K split of a partial last round is taken when the workspace has room for it
         FtTail tail = ft_tail_plan(fc, M, N, K, cadence ? opt.check_interval : kGemmBK);
+        // (the weighted locator on a product one tile wide or high: every tile split, as the kernels without a pre-pass do)
+        if (weighted && (a.tiles_n == 1 || a.tiles_m == 1) && a.tiles_m * a.tiles_n >= device_cus() / 8)
+            tail = ft_split_all_plan(a.tiles_m * a.tiles_n, K, kGemmBK);
         if (ws_bytes < enc_bytes + ft_tail_bytes(fc, opt.granularity, tail)) tail = FtTail{1, 0, 0};
         a.enc_ld = ft_enc_ld(K);
         const int row_groups = a.tiles_m * gm, col_groups = a.tiles_n * gn;
@@ -246,13 +263,26 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
         const int b_blocks = static_cast<int>(ceil_div(N, 128));  // the pre-pass walks B in blocks of 128 columns
         // (ta: the same launch, with the blocks of the A half walking A^T)
-        const EncodeFn encode = ft_encode(opt.tile_class, ta, wave);
-        if (!encode) return HPCDNN_ERR_INVALID_VALUE;
-        hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(1024), 0, s, M, N, K,
-                           A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
+        if (weighted) {
+            // the two row sums of B per tile column; nothing of A (enc_a carries the weighted vectors to the kernel)
+            a.enc_b = static_cast<float*>(ws);
+            a.enc_a = a.enc_b + static_cast<size_t>(col_groups) * a.enc_ld;
+            float* const wb = static_cast<float*>(ws);
+            if (fc.bn == 128)
+                abft_encode_weighted_kernel<128><<<dim3(k_blocks * b_blocks), dim3(1024), 0, s>>>(N, K, B, ldb, wb, wb + static_cast<size_t>(col_groups) * a.enc_ld,
+                                                                                             a.enc_ld, k_blocks, col_groups);
+            else
+                abft_encode_weighted_kernel<64><<<dim3(k_blocks * b_blocks), dim3(1024), 0, s>>>(N, K, B, ldb, wb, wb + static_cast<size_t>(col_groups) * a.enc_ld,
+                                                                                            a.enc_ld, k_blocks, col_groups);
+        } else {
+            const EncodeFn encode = ft_encode(opt.tile_class, ta, wave);
+            if (!encode) return HPCDNN_ERR_INVALID_VALUE;
+            hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(1024), 0, s, M, N, K,
+                               A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
+        }
         rc = launch_status();
         if (rc != HPCDNN_OK) return rc;
-        const FtKernel k = ft_kernel(opt.tile_class, ta, wave ? (cadence ? kFtWaveCad : kFtWave) : (cadence ? kFtPreCad : kFtPre));
+        const FtKernel k = ft_kernel(opt.tile_class, ta, weighted ? kFtWeighted : wave ? (cadence ? kFtWaveCad : kFtWave) : (cadence ? kFtPreCad : kFtPre));
         if (!k.plain) return HPCDNN_ERR_INVALID_VALUE;
         void (*fn)(const GemmArgs) = edge ? k.edge : k.plain;
         rc = enable_lds(fn, k.lds);

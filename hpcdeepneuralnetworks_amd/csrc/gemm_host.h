@@ -72,8 +72,8 @@ constexpr FtGeom kFtGeom[HPCDNN_FT_NUM_CLASSES] = {{256, 128, 2, 4}, {128, 128, 
 
 // Kernel kinds of a class.  Fused: checksum vectors formed in the main loop (no workspace); pre: read from the
 // workspace the pre-pass filled; wave: pre, with one checksum pair per wave tile; cad: with a verification every
-// check_interval values of k.
-enum FtKind { kFtFused = 0, kFtFusedCad, kFtPre, kFtPreCad, kFtWave, kFtWaveCad, kFtKinds };
+// check_interval values of k; weighted: the weighted-checksum locator (two row sums of B from the workspace).
+enum FtKind { kFtFused = 0, kFtFusedCad, kFtPre, kFtPreCad, kFtWave, kFtWaveCad, kFtWeighted, kFtKinds };
 
 // One getter pair per (class, operand layout): each lives in its own translation unit (ft_kernels.hip compiled with
 // -DHPCDNN_FT_CLASS / -DHPCDNN_FT_TA).  _ta1: the left operand is given transposed (K rows of M floats).

@@ -80,7 +80,8 @@ struct GemmArgs {
     int status_rows, status_ld;  // records are laid out as a status_rows x status_ld grid of check tiles
     hpcdnn_ft_status* status;
     const float* enc_a;  // FT == 2: [row groups][enc_ld] column sums of A over the rows of each check tile
-    const float* enc_b;  // FT == 2: [column groups][enc_ld] row sums of B over the columns of each check tile
+                         // FT == 3: [column groups][enc_ld] weighted row sums of B (weights 1, 2, ... over the tile's columns)
+    const float* enc_b;  // FT >= 2: [column groups][enc_ld] row sums of B over the columns of each check tile
     int enc_ld;          // row length: K rounded up to the K step, plus two K steps of zeros
 };
 
@@ -99,12 +100,17 @@ constexpr int b_stage_stride() {
 // LDS the ABFT verification needs (it reuses the staging buffers once the K loop has drained): FP64 partials of the
 // reference checksums, observed line sums and their absolute counterparts per wave row / wave column, one residual
 // per line, one record per check tile, per-wave sums of |acc| per check tile.  GM x GN check tiles per workgroup tile.
-template <int BM, int BN, int WGM, int WGN, int GM, int GN>
+// (the weighted locator keeps, in place of everything about columns, the weighted row sums: its reference partials
+// fit where the column partials would be, its observed sums get WGN x BM words of their own, its lines are 2 BM)
+template <int BM, int BN, int WGM, int WGN, int GM, int GN, bool WEIGHTED = false>
 constexpr size_t ft_verify_lds_bytes() {
     constexpr size_t threads = static_cast<size_t>(WGM) * WGN * 64;
-    constexpr size_t ccp = threads / (BN / 4), crp = kGemmBK / 4, lines = static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
+    constexpr size_t ccp = threads / (BN / 4), crp = kGemmBK / 4;
+    constexpr size_t lines = WEIGHTED ? 2 * static_cast<size_t>(BM) : static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
+    static_assert(!WEIGHTED || GM * ccp * BN >= crp * BM, "the weighted reference partials fit in the column partials' place");
     return sizeof(double) * (GM * ccp * BN + GN * crp * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + lines) +
-           32 * GM * GN + sizeof(float) * GM * GN * (threads / 64) + 2 * sizeof(float) * GM * GN;
+           32 * GM * GN + sizeof(float) * GM * GN * (threads / 64) + 2 * sizeof(float) * GM * GN +
+           (WEIGHTED ? sizeof(float) * WGN * BM : 0);
 }
 
 template <int BM, int BN, int FT = 0, int THREADS = 256, int WGM = 2, int WGN = 2, int GRAN = 0>
@@ -114,7 +120,7 @@ constexpr size_t gemm_lds_bytes() {
     // publish nothing (one word per thread plus the reach of the strided writes)
     constexpr size_t staging = sizeof(float) * 2 * (static_cast<size_t>(BM) * (kGemmBK + 4) + static_cast<size_t>(kGemmBK) * b_stage_stride<BN, FT>()) +
            (FT == 1 ? sizeof(float) * (2 * (kGemmBK * (THREADS / 64) + kGemmBK) + THREADS + 2 * kGemmBK * (THREADS / 64)) : 0);
-    constexpr size_t verify = FT ? ft_verify_lds_bytes<BM, BN, WGM, WGN, GRAN ? WGM : 1, GRAN ? WGN : 1>() : 0;
+    constexpr size_t verify = FT ? ft_verify_lds_bytes<BM, BN, WGM, WGN, GRAN ? WGM : 1, GRAN ? WGN : 1, FT == 3>() : 0;
     return staging > verify ? staging : verify;
 }
 
@@ -151,7 +157,11 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
 }
 
 // FT: 0 = plain SGEMM; 1 = ABFT, checksum vectors e^T A and B e formed inside the main loop; 2 = ABFT, checksum
-// vectors read from a workspace filled by abft_encode_kernel (fewer VALU instructions in the main loop).
+// vectors read from a workspace filled by abft_encode_kernel (fewer VALU instructions in the main loop); 3 = ABFT with
+// the weighted-checksum locator (the reference's "kernel 2", kernel/ft_sgemm/README.md:16-26: two row sums of B,
+// e1 = [1, 1, ...] and e2 = [1, 2, ...], and nothing from A): references A (B e1) and A (B e2) against the plain and
+// the weighted row sums of the accumulators; a faulty row is found by the first pair, the column inside it as the
+// ratio of the two residuals; both vectors of B come from the workspace (abft_encode_weighted_kernel).
 //
 // NSLOT: staging register sets.  K step t + 1 waits in one of them while steps up to t + NSLOT are on their way from
 // memory.  Two are enough while a K step takes longer than a trip to memory (big tiles) or the operands come from
@@ -178,6 +188,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     static_assert(NSLOT == 2 || (FT == 0 && NSLOT % 2 == 0), "the ABFT loop is written for two staging sets");
     static_assert(FT != 0 || (GRAN == 0 && !CADENCE), "granularity and cadence belong to the ABFT kernels");
     static_assert(GRAN == 0 || FT == 2, "wave-tile checksums come from the pre-encoded vectors");
+    static_assert(FT != 3 || (GRAN == 0 && !CADENCE), "the weighted locator checks a workgroup tile once, after the K loop");
+    constexpr bool kWeighted = FT == 3;
     constexpr int GM = GRAN ? WGM : 1, GN = GRAN ? WGN : 1;  // check tiles per workgroup tile
     constexpr int CM = BM / GM, CN = BN / GN;                // check tile
     static_assert(CM % 32 == 0 && CN % 32 == 0, "check tiles are made of 32x32 blocks");
@@ -302,9 +314,12 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // (with wave-tile checksums the tile's GM / GN rows of the vectors follow each other: one descriptor over all
     // of them, the row chosen by the scalar offset)
     const __amdgpu_buffer_rsrc_t enc_a_rsrc =
-        make_rsrc(FT == 2 ? p.enc_a + static_cast<int64_t>(tile_m) * GM * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * GM * 4);
+        make_rsrc(FT == 2   ? p.enc_a + static_cast<int64_t>(tile_m) * GM * p.enc_ld
+                  : FT == 3 ? p.enc_a + static_cast<int64_t>(tile_n) * p.enc_ld  // the weighted row sums of B
+                            : nullptr,
+                  static_cast<int64_t>(p.enc_ld) * GM * 4);
     const __amdgpu_buffer_rsrc_t enc_b_rsrc =
-        make_rsrc(FT == 2 ? p.enc_b + static_cast<int64_t>(tile_n) * GN * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * GN * 4);
+        make_rsrc(FT >= 2 ? p.enc_b + static_cast<int64_t>(tile_n) * GN * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * GN * 4);
     const int enc_row_bytes = p.enc_ld * 4;
     // a_c of the k rows of B this thread stages: k = tid / (BN / 4) (and k + 8 when it stages two), which the
     // pre-encode kernel stores side by side (order 0, 8, 1, 9, ... inside each K step)
@@ -313,6 +328,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     int enc_off = kbeg * 4;
     float g_ac[2][GM][B_SLOTS];
     v4f g_br[2][GN];
+    v4f g_bw[2];  // FT == 3: the weighted row sums of B for the four k values of A this thread stages
     auto gload1 = [&](auto slot, auto part, auto bulk) {  // bulk: this K step is not the slice's last (kLazyBounds)
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P == 0) k_slot[S] = k_loaded;
@@ -322,6 +338,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         } else {
             if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc(a_base, a_left), a_voff[P]);
             else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc(b_base, b_left), b_voff[P - A_SLOTS]);
+        }
+        if constexpr (FT == 3 && P == NGL - 1) {
+            g_br[S][0] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_b_rsrc, enc_b_voff, enc_off, 0));
+            g_bw[S] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_a_rsrc, enc_b_voff, enc_off, 0));
         }
         if constexpr (FT == 2 && P == NGL - 1) {
             static_assert(FT != 2 || B_SLOTS <= 2, "a thread stages one or two k rows of B");
@@ -413,7 +433,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             b_left = more ? b_left - b_step * 4 : 0;
         }
         k_loaded += more ? BK : 0;
-        if constexpr (FT == 2) enc_off += BK * 4;
+        if constexpr (FT >= 2) enc_off += BK * 4;
     };
     // The same in two parts, so that the short-step schedule can place them apart.  Its full tiles keep no bounds at
     // all: nothing they fetch lies outside the matrix, and past the end of the slice they fetch its last K step
@@ -555,6 +575,15 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         for (int sl = 0; sl < A_SLOTS; ++sl)
 #pragma unroll
             for (int e = 0; e < 4; ++e) cr_lo[gn][sl][e] = 0.f;
+    double crw_ref[A_SLOTS];  // FT == 3: the weighted row checksum references of this thread's rows
+    float crw_lo[A_SLOTS][4];
+#pragma unroll
+    for (int sl = 0; sl < A_SLOTS; ++sl) {
+        crw_ref[sl] = 0.0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) crw_lo[sl][e] = 0.f;
+    }
+    v4f e_bwv;
     float e_pa[4], e_sw[4];
     v4f e_t[kPartV4 * B_SLOTS], e_brv[GN];
     v4f e_a[TA ? A_SLOTS : 1];  // TA: this thread's rows of the staged K step (four k each), read back from LDS
@@ -663,12 +692,16 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         constexpr bool kFlush = decltype(flush)::value;
         const float* ap = s_apart + par * BK * kParts;
         const float* br = s_br + par * BK;
-        if constexpr (FT == 2 && E <= 1) {
+        if constexpr (FT >= 2 && E <= 1) {
             if constexpr (E == 0) {
+                if constexpr (FT == 2) {
 #pragma unroll
-                for (int gm = 0; gm < GM; ++gm)
+                    for (int gm = 0; gm < GM; ++gm)
 #pragma unroll
-                    for (int sl = 0; sl < B_SLOTS; ++sl) e_ac[gm][sl] = g_ac[S][gm][sl];
+                        for (int sl = 0; sl < B_SLOTS; ++sl) e_ac[gm][sl] = g_ac[S][gm][sl];
+                } else {
+                    e_bwv = g_bw[S];
+                }
 #pragma unroll
                 for (int gn = 0; gn < GN; ++gn) e_brv[gn] = g_br[S][gn];
                 // (the barrier before the second half has made stage `par`, which holds this K step, complete)
@@ -698,6 +731,20 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 e_ac[0][sl] = (u.x + u.y) + (u.z + u.w);
                 HPCDNN_PIN(e_ac[0][sl]);
             }
+        } else if constexpr (kWeighted && E < 2 + GM) {
+            // the weighted row checksums take the place of the column checksums
+#pragma unroll
+            for (int sl = 0; sl < A_SLOTS; ++sl) {
+                const v4f av = TA ? e_a[TA ? sl : 0] : ra[S][sl];
+                crw_lo[sl][0] = __builtin_fmaf(av.x, e_bwv.x, crw_lo[sl][0]);
+                crw_lo[sl][1] = __builtin_fmaf(av.y, e_bwv.y, crw_lo[sl][1]);
+                crw_lo[sl][2] = __builtin_fmaf(av.z, e_bwv.z, crw_lo[sl][2]);
+                crw_lo[sl][3] = __builtin_fmaf(av.w, e_bwv.w, crw_lo[sl][3]);
+            }
+#pragma unroll
+            for (int sl = 0; sl < A_SLOTS; ++sl)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) HPCDNN_PIN(crw_lo[sl][e]);
         } else if constexpr (E < 2 + GM) {
             // independent accumulators: a wave alone on its SIMD cannot hide the latency of dependent VALU
             // instructions behind other waves
@@ -733,8 +780,16 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             // every 16th K step (and after the last one): FP32 partials -> FP64 running sums.  FP64 VALU
             // instructions are twice as expensive as FP32 ones, so this is kept rare.
             if (flush_now) {
+                if constexpr (kWeighted) {
 #pragma unroll
-                for (int gm = 0; gm < GM; ++gm)
+                    for (int sl = 0; sl < A_SLOTS; ++sl) {
+                        crw_ref[sl] += static_cast<double>((crw_lo[sl][0] + crw_lo[sl][1]) + (crw_lo[sl][2] + crw_lo[sl][3]));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) crw_lo[sl][e] = 0.f;
+                    }
+                }
+#pragma unroll
+                for (int gm = 0; gm < (kWeighted ? 0 : GM); ++gm)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         float t = cc_lo[gm][0][e];
@@ -934,7 +989,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;   // partials per column / per row checksum
     constexpr int NCT = GM * GN;                          // check tiles per workgroup tile
     constexpr int kRowLines = GN * BM;                    // row lines (gn, m) come first, column lines (gm, n) after them
-    constexpr int kLines = kRowLines + GM * BN;
+    // (weighted locator: the BM row lines, then the BM weighted row lines; there are no column lines)
+    constexpr int kLines = kWeighted ? 2 * BM : kRowLines + GM * BN;
     constexpr int LPT = (kLines + kGemmThreads - 1) / kGemmThreads;  // lines per thread
     static_assert(NCT <= kGemmThreads, "one thread per check tile keeps its record");
     double line_off[LPT];          // CADENCE: what re-synchronisation has taken out of each of this thread's lines
@@ -956,7 +1012,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         int* const s_meta = reinterpret_cast<int*>(s_dr + kLines);      // [NCT][8] nbr, nbc, bad row, bad col, max clean (float bits)
         float* const s_tsum = reinterpret_cast<float*>(s_meta + 8 * NCT);  // [NCT][waves] partial sums of |acc| over a check tile
         float* const s_fix = s_tsum + NCT * (kGemmThreads / kWave);        // [NCT][2] recomputed element, and what it changed
-        static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads, WGM, WGN, GRAN>() >= ft_verify_lds_bytes<BM, BN, WGM, WGN, GM, GN>(),
+        float* const s_crwobs = s_fix + 2 * NCT;                           // weighted locator: [WGN][BM] observed weighted row sums
+        double* const s_crwref = s_ccref;                                  // weighted locator: [CRP][BM] weighted reference partials
+        static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads, WGM, WGN, GRAN>() >= ft_verify_lds_bytes<BM, BN, WGM, WGN, GM, GN, kWeighted>(),
                       "verification scratch fits in the kernel's LDS");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
 
@@ -1012,10 +1070,16 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 
         // reference checksums: every thread publishes its partial sums (columns nc..nc+3 over its k rows, its
         // rows over its k group); the residual step below adds the partials in a fixed order
+        if constexpr (kWeighted) {
 #pragma unroll
-        for (int gm = 0; gm < GM; ++gm)
+            for (int sl = 0; sl < A_SLOTS; ++sl)
+                s_crwref[e_class * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = crw_ref[sl];
+        } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) s_ccref[(gm * CCP + e_hw) * BN + (tid % B_V4_PER_ROW) * 4 + e] = cc_ref[gm][e];
+            for (int gm = 0; gm < GM; ++gm)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s_ccref[(gm * CCP + e_hw) * BN + (tid % B_V4_PER_ROW) * 4 + e] = cc_ref[gm][e];
+        }
 #pragma unroll
         for (int gn = 0; gn < GN; ++gn)
 #pragma unroll
@@ -1025,7 +1089,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         // sums of absolute values go with them: they scale the threshold to the data.
         const bool relative = p.tau <= 0.f;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+        for (int j = 0; j < (kWeighted ? 0 : TN); ++j) {
             float s = 0.f, sa = 0.f;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
@@ -1084,6 +1148,20 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 s_crobs[wn * BM + row] = rs[0];
                 s_crabs[wn * BM + row] = ra_[0];
             }
+            if constexpr (kWeighted) {
+                // the same rows with column n of the tile weighted by n + 1 (kernel/ft_sgemm/README.md:16-26, e2 = [1, 2, ...])
+                float rw[RG];
+#pragma unroll
+                for (int e2 = 0; e2 < RG; ++e2) {
+                    const int i = (g * RG + e2) / 16, v = (g * RG + e2) % 16;
+                    float s = acc[i][0][v] * static_cast<float>(wn * WN + lr + 1);
+#pragma unroll
+                    for (int j = 1; j < TN; ++j) s = __builtin_fmaf(acc[i][j][v], static_cast<float>(wn * WN + j * 32 + lr + 1), s);
+                    rw[e2] = s;
+                }
+                half32_transpose_sum<RG>(rw, lane);
+                if (RG == 32 || lr < RG) s_crwobs[wn * BM + row] = rw[0];
+            }
         }
         __syncthreads();
 
@@ -1116,16 +1194,22 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             if (line < kLines) {
                 const bool is_row = line < kRowLines;
                 // row line (gn, idx): row idx of the tile against wave column gn; column line (gm, idx) likewise
-                const int grp = is_row ? line / BM : (line - kRowLines) / BN;
-                const int idx = is_row ? line - grp * BM : (line - kRowLines) - grp * BN;
-                const int gm = is_row ? idx / CM : grp, gn = is_row ? grp : idx / CN;
+                const int grp = kWeighted ? 0 : is_row ? line / BM : (line - kRowLines) / BN;
+                const int idx = kWeighted ? (is_row ? line : line - BM) : is_row ? line - grp * BM : (line - kRowLines) - grp * BN;
+                const int gm = kWeighted ? 0 : is_row ? idx / CM : grp, gn = kWeighted ? 0 : is_row ? grp : idx / CN;
                 const int ct = gm * GN + gn;
                 int rows_in = p.M - (m0 + gm * CM), cols_in = p.N - (n0 + gn * CN);
                 rows_in = rows_in < CM ? rows_in : CM;
                 cols_in = cols_in < CN ? cols_in : CN;
                 double ref = 0.0, obs = 0.0;
                 float mag = 0.f;
-                if (is_row) {
+                if (kWeighted && !is_row) {
+                    // weighted row line idx: its residual locates the column, it is not tested against a threshold
+#pragma unroll
+                    for (int w = 0; w < CRP; ++w) ref += s_crwref[w * BM + idx];
+#pragma unroll
+                    for (int w = 0; w < WGN; ++w) obs += static_cast<double>(s_crwobs[w * BM + idx]);
+                } else if (is_row) {
 #pragma unroll
                     for (int w = 0; w < CRP; ++w) ref += s_crref[(grp * CRP + w) * BM + idx];
 #pragma unroll
@@ -1142,7 +1226,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 }
                 const double d = (CADENCE ? ref - line_off[it] : ref) - obs;
                 d_line[it] = d;
-                if (rows_in > 0 && cols_in > 0) {  // check tiles of an edge tile that lie outside the matrix have no lines
+                if (rows_in > 0 && cols_in > 0 && !(kWeighted && !is_row)) {  // check tiles of an edge tile that lie outside the matrix have no lines
                     double tau = static_cast<double>(p.tau);
                     if (relative) {
                         float total = 0.f;
@@ -1157,6 +1241,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     if (fabs(d) > tau) {
                         atomicAdd(&s_meta[8 * ct + (is_row ? 0 : 1)], 1);
                         atomicMax(&s_meta[8 * ct + (is_row ? 2 : 3)], idx);
+                        if constexpr (kWeighted) s_meta[8 * ct + 5] = __float_as_int(static_cast<float>(tau));  // (used when it is the only one)
                     } else {
                         clean = static_cast<float>(fabs(d));
                     }
@@ -1180,6 +1265,27 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         // the bits a fault-free run gives it.  The operand row and column are staged through the LDS the reference
         // partials no longer need, a chunk of kFixChunk values of k at a time, by all threads (the condition is
         // uniform over the workgroup); zeros pad the last K step.
+        // Weighted locator (kernel/ft_sgemm/README.md:16-26): one faulty row; with a fault delta in column n its two
+        // residuals are -delta and -(n + 1) delta, so their ratio names the column.  The element found that way is
+        // computed again like any located element; the location counts as confirmed when that changed the element by
+        // what the row's residual says (computing a healthy element again changes nothing, so a wrong guess does no
+        // harm: the tile is then reported as detected, not corrected).
+        float w_d1 = 0.f;
+        bool w_located = false;
+        if constexpr (kWeighted) {
+            w_located = s_meta[0] == 1;
+            if (w_located) {
+                const int bad_r = s_meta[2];
+                w_d1 = s_dr[bad_r];
+                int cols_in = p.N - n0;
+                cols_in = cols_in < BN ? cols_in : BN;
+                int col = static_cast<int>(__builtin_rintf(s_dr[BM + bad_r] / w_d1)) - 1;
+                col = col < 0 ? 0 : (col >= cols_in ? cols_in - 1 : col);
+                __syncthreads();  // everybody has read the line counts
+                if (tid == 0) { s_meta[1] = 1; s_meta[3] = col; }
+                __syncthreads();
+            }
+        }
         bool any_fixed = false;
 #pragma unroll 1
         for (int ct = 0; ct < NCT; ++ct) {
@@ -1233,6 +1339,13 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             }
         }
         if (CADENCE && any_fixed) __syncthreads();  // s_fix[2 ct + 1] = corrected - faulty value, for the resync below
+        if constexpr (kWeighted) {
+            if (w_located) {
+                __syncthreads();  // s_fix[1] = what computing the element again changed
+                const bool confirmed = __builtin_fabsf(s_fix[1] - w_d1) <= __int_as_float(s_meta[5]);
+                if (!confirmed && tid == 0) s_meta[1] = 0;  // (read again by this same thread below)
+            }
+        }
         if constexpr (CADENCE) {
             // re-synchronise (ft_sgemm_huge.cuh:268-271): every line starts the next interval with what is left of
             // its residual after the correction taken out of its reference
@@ -1267,7 +1380,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 rec.row = bad_r - gm * CM;
                 rec.col = bad_c - gn * CN;
                 rec.row_residual = s_dr[gn * BM + bad_r];
-                rec.col_residual = s_dr[kRowLines + gm * BN + bad_c];
+                rec.col_residual = kWeighted ? s_dr[BM + bad_r] : s_dr[kRowLines + gm * BN + bad_c];
             }
             if (last && p.status) {
                 hpcdnn_ft_status st = rec;
@@ -1632,6 +1745,73 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
             const int k = kb + half + kHalves * in_group;
             // (the last block of 128 columns may reach past the last column group)
             if (k < enc_ld && group < col_groups) enc_b[static_cast<int64_t>(group) * enc_ld + k] = out;
+        }
+    }
+}
+
+// ---- Pre-pass of the weighted-checksum locator: the two row sums of B per column group of CN columns,
+//   enc_b[g][k]  = sum over the group's columns n of B[k][n]             (B e1, e1 = [1, 1, ...])
+//   enc_bw[g][k] = sum over the group's columns n of (n' + 1) B[k][n]    (B e2, e2 = [1, 2, ...], n' counted inside the group)
+// (kernel/ft_sgemm/README.md:16-26); zero for K <= k < enc_ld.  Nothing of A is needed.  Layout of the work as in the
+// B half of abft_encode_kernel: 1024-thread blocks over 256 values of k and 128 columns, a half wave per k row.
+template <int CN>
+__global__ __launch_bounds__(1024) void abft_encode_weighted_kernel(int N, int K, const float* __restrict__ B, int ldb,
+                                                                    float* __restrict__ enc_b, float* __restrict__ enc_bw,
+                                                                    int enc_ld, int k_blocks, int col_groups) {
+    static_assert(CN == 128 || CN == 64, "column groups are 16 or 32 lanes of a half wave");
+    constexpr int kHalves = 32, kRowsPerHalf = 256 / kHalves;
+    constexpr int kGroupLanes = CN / 4, kGroupsPer128 = 128 / CN;
+    const int bid = blockIdx.x;
+    const int lr = threadIdx.x & 31, half = threadIdx.x >> 5;
+    const int tile_n = bid / k_blocks, n0 = tile_n * 128;
+    const int kb = (bid % k_blocks) * 256;
+    const int in_group = lr % kGroupLanes;
+    const float w0 = static_cast<float>(in_group * 4 + 1);  // weight of this lane's first column
+    float s[kRowsPerHalf], sw[kRowsPerHalf];
+    v4f v[kRowsPerHalf];
+#pragma unroll
+    for (int i = 0; i < kRowsPerHalf; ++i) {
+        const int k = kb + half + kHalves * i;
+        const int kc = k < K ? k : K - 1;
+        const float* base = B + static_cast<int64_t>(kc) * ldb + n0;
+        v[i] = buffer_load_v4f(make_rsrc(base, static_cast<int64_t>(N - n0) * 4), lr * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < kRowsPerHalf; ++i) {
+        const int k = kb + half + kHalves * i;
+        float t = (v[i].x + v[i].y) + (v[i].z + v[i].w);
+        float tw = __builtin_fmaf(v[i].x, w0, v[i].y * (w0 + 1.f)) + __builtin_fmaf(v[i].z, w0 + 2.f, v[i].w * (w0 + 3.f));
+        t = k < K ? t : 0.f;
+        tw = k < K ? tw : 0.f;
+        // sums over the lanes of the column group; every lane of the group gets them
+        t += dpp_mov<kDppXor1>(t);
+        tw += dpp_mov<kDppXor1>(tw);
+        t += dpp_mov<kDppXor2>(t);
+        tw += dpp_mov<kDppXor2>(tw);
+        t += dpp_mov<kDppHalfMirror>(t);
+        tw += dpp_mov<kDppHalfMirror>(tw);
+        t += dpp_mov<kDppMirror>(t);
+        tw += dpp_mov<kDppMirror>(tw);
+        if constexpr (kGroupLanes >= 32) {
+            t += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, t), 0x401F));
+            tw += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, tw), 0x401F));
+        }
+        s[i] = t;
+        sw[i] = tw;
+    }
+    // lane l of a group writes the group's sums of k row l of this half wave
+    const int group = tile_n * kGroupsPer128 + lr / kGroupLanes;
+    if (in_group < kRowsPerHalf) {
+        float out = s[0], outw = sw[0];
+#pragma unroll
+        for (int i = 1; i < kRowsPerHalf; ++i) {
+            out = (in_group == i) ? s[i] : out;
+            outw = (in_group == i) ? sw[i] : outw;
+        }
+        const int k = kb + half + kHalves * in_group;
+        if (k < enc_ld && group < col_groups) {
+            enc_b[static_cast<int64_t>(group) * enc_ld + k] = out;
+            enc_bw[static_cast<int64_t>(group) * enc_ld + k] = outw;
         }
     }
 }

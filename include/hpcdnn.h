@@ -250,6 +250,28 @@ int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
  * intervals, so the verifications of a tile are the same with and without
  * the split.
  *
+ * locator HPCDNN_FT_LOCATE_ROW_COL: a faulty row and a faulty column of a
+ * check tile meet in the faulty element (what everything above describes).
+ * HPCDNN_FT_LOCATE_WEIGHTED: the reference's second scheme ("kernel 2",
+ * kernel/ft_sgemm/README.md:16-26; its weighted locator is left in comments
+ * at kernel/ft_sgemm/include/ft_sgemm_huge.cuh:299-310): two row sums of B,
+ * with weights e1 = [1, 1, ...] and e2 = [1, 2, ...] over the tile's columns,
+ * and nothing from A.  The references A (B e1), A (B e2) are compared with the
+ * plain and the weighted row sums of the accumulators: a row whose plain
+ * residual d1 exceeds the threshold is faulty, and with one fault delta in
+ * column n of it the residuals are d1 = -delta, d2 = -(n + 1) delta, so the
+ * column is round(d2 / d1) - 1.  One faulty row: that element is computed
+ * again; if that changed it by d1 (to within the row's threshold) the fault is
+ * located and corrected (flag 1, n_bad_cols = 1), else - two faults in the
+ * row, or a fault too small against the rounding noise of the weighted sums,
+ * which is about 0.6 x the tile's width x that of the plain sums - the tile
+ * is reported as detected, not corrected (flag 2, n_bad_cols = 0; computing a
+ * healthy element again changes nothing, so a wrong guess does no harm).  More
+ * faulty rows: flag 2.  The record's col_residual is d2 of the located row.
+ * The pre-pass reads B only, which is what a tall product with few columns
+ * wants.  Needs the workspace; tile granularity, one verification (the other
+ * combinations return HPCDNN_ERR_INVALID_VALUE).
+ *
  * Check tiles are numbered row-major over the matrix,
  * t = (i / cm) * ceil(N / cn) + (j / cn); `status` holds
  * hpcdnn_ft_num_check_tiles() records, and the tile / row / col of a fault
@@ -258,6 +280,8 @@ int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
  * that verification.  Faults aimed outside the matrix are ignored. */
 #define HPCDNN_FT_GRAN_TILE 0
 #define HPCDNN_FT_GRAN_WAVE 1
+#define HPCDNN_FT_LOCATE_ROW_COL 0
+#define HPCDNN_FT_LOCATE_WEIGHTED 1
 #define HPCDNN_FT_MAX_FAULTS 4
 typedef struct hpcdnn_ft_fault_at {
     int32_t tile;
@@ -271,6 +295,7 @@ typedef struct hpcdnn_ft_options {
     int32_t check_interval;  /* 0, or a positive multiple of 16 */
     int32_t n_faults;        /* 0 .. HPCDNN_FT_MAX_FAULTS */
     hpcdnn_ft_fault_at faults[HPCDNN_FT_MAX_FAULTS];
+    int32_t locator;         /* HPCDNN_FT_LOCATE_* */
 } hpcdnn_ft_options;
 /* hpcdnn_ft_sgemm_ex with the options above (`opt` is a HOST pointer, NULL =
  * class 0, tile granularity, one verification, no faults). */

@@ -114,6 +114,9 @@ def _load():
     lib.oracle_ft_sgemm_checked.restype = None
     lib.oracle_ft_sgemm_checked.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
                                             C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.oracle_ft_sgemm_weighted.restype = None
+    lib.oracle_ft_sgemm_weighted.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, C.c_float,
+                                             C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p]
     lib.oracle_abft_relative_thresholds.restype = None
     lib.oracle_abft_relative_thresholds.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, C.c_float, dp, dp]
     lib.oracle_sgemv_f64.restype = None
@@ -309,6 +312,19 @@ def ft_sgemm_checked(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, tile_m, tile_
     _load().oracle_ft_sgemm_checked(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, tile_m, tile_n, tau,
                                     int(check_interval), len(faults), fa.ctypes.data_as(C.c_void_p),
                                     status.ctypes.data_as(C.c_void_p))
+    return status
+
+
+def ft_sgemm_weighted(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, tile_m, tile_n, tau, faults=()):
+    """In-place ABFT GEMM model with the weighted-checksum locator (two row sums of B, weights [1, 1, ...] and
+    [1, 2, ...] over each tile's columns); ``faults`` = iterable of (tile, i, j, delta).  Returns the per-tile status."""
+    ntiles = ((M + tile_m - 1) // tile_m) * ((N + tile_n - 1) // tile_n)
+    status = np.zeros(ntiles, dtype=FT_STATUS_DTYPE)
+    fa = np.zeros(max(len(faults), 1), dtype=FAULT_AT_DTYPE)
+    for i, f in enumerate(faults):
+        fa[i] = (int(f[0]), int(f[1]), int(f[2]), float(f[3]), 0)
+    _load().oracle_ft_sgemm_weighted(M, N, K, _f(a), lda, _f(b), ldb, _f(c), ldc, alpha, beta, tile_m, tile_n, tau,
+                                     len(faults), fa.ctypes.data_as(C.c_void_p), status.ctypes.data_as(C.c_void_p))
     return status
 
 

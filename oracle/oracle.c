@@ -33,6 +33,13 @@
  *     (AB)e = A(Be)) and to the one known-answer case the reference holds
  *     (+1.0 at tile-local (0,1), threshold 0.1 -> row 0, col 1, magnitude 1;
  *     kernel/ft_sgemm/include/ft_sgemm_huge.cuh:40,145,263,358).
+ *   oracle_ft_sgemm_weighted (the reference's second scheme, two row sums of
+ *     B with weights [1,1,...] and [1,2,...], README.md:16-26): pinned by
+ *     closed forms on exact-integer data (d1 = -delta, d2 = -(n+1) delta,
+ *     every column of a tile located; two faults in a row detected, not
+ *     corrected) and against an independent numpy composition; the reference
+ *     only ever ran this scheme offline through cuBLAS and printed nothing,
+ *     so it holds no expected values for it.
  *   oracle_recompute_element (the correction: the located accumulator formed
  *     again): pinned by K = 1 and exact-integer cases in which a corrected
  *     product must equal the fault-free one bit for bit.
@@ -497,6 +504,108 @@ typedef struct {
     float delta;
     int32_t check;
 } oracle_fault_at;
+
+/* The whole-matrix model of the reference's second scheme ("kernel 2", kernel/ft_sgemm/README.md:16-26: double row
+ * sums of B with e1 = [1, 1, ...] and e2 = [1, 2, ..., N]; its locator is left in comments at
+ * kernel/ft_sgemm/include/ft_sgemm_huge.cuh:299-310): per tile the references r1 = A (B e1), r2 = A (B e2) - weights
+ * counted over the tile's columns - are compared with the plain and the weighted row sums of the accumulators.  A row
+ * whose plain residual d1 exceeds its threshold is faulty; with one fault delta in column n its residuals are
+ * d1 = -delta, d2 = -(n + 1) delta, so the column is round(d2 / d1) - 1 (clamped into the tile).  One faulty row: that
+ * element is computed again (oracle_recompute_element); the location is confirmed when that changed the element by d1
+ * to within the row's threshold -> flag 1, n_bad_cols 1, row/col set, row_residual = d1, col_residual = d2.  Not
+ * confirmed (two faults in the row, or a fault lost in the rounding of the weighted sums) or more faulty rows ->
+ * flag 2, n_bad_cols 0.  Computing a healthy element again changes nothing, so a wrong column does no harm.
+ * tau as for oracle_ft_sgemm; every fault is added before the one verification. */
+void oracle_ft_sgemm_weighted(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                              int ldc, float alpha, float beta, int tile_m, int tile_n, float tau,
+                              int n_faults, const oracle_fault_at* faults, oracle_ft_status* status) {
+    int ntm = (M + tile_m - 1) / tile_m, ntn = (N + tile_n - 1) / tile_n;
+    #pragma omp parallel for schedule(dynamic, 1)
+    for (int t = 0; t < ntm * ntn; ++t) {
+        int bm = t / ntn, bn = t % ntn;
+        int m0 = bm * tile_m, n0 = bn * tile_n;
+        int tm = (M - m0 < tile_m) ? M - m0 : tile_m;
+        int tn = (N - n0 < tile_n) ? N - n0 : tile_n;
+        float* acc = (float*)calloc((size_t)tm * tn, sizeof(float));
+        double* buf = (double*)calloc((size_t)(3 * tm + tn) + 2 * (size_t)(K > 0 ? K : 1), sizeof(double));
+        double *d1 = buf, *d2 = buf + tm, *thr = buf + 2 * tm;      /* thr: tm row thresholds, then tn column ones (unused) */
+        double *b1 = buf + 3 * tm + tn, *b2 = b1 + (K > 0 ? K : 1);
+        for (int m = 0; m < tm; ++m)
+            for (int k = 0; k < K; ++k) {
+                float a = A[(size_t)(m0 + m) * lda + k];
+                const float* brow = B + (size_t)k * ldb + n0;
+                float* arow = acc + (size_t)m * tn;
+                for (int n = 0; n < tn; ++n) arow[n] = fmaf(a, brow[n], arow[n]);
+            }
+        for (int f = 0; f < n_faults; ++f)
+            if (faults[f].tile == t && faults[f].row < tm && faults[f].col < tn)
+                acc[(size_t)faults[f].row * tn + faults[f].col] += faults[f].delta;
+        for (int k = 0; k < K; ++k) {
+            double s1 = 0.0, s2 = 0.0;
+            for (int n = 0; n < tn; ++n) {
+                double v = (double)B[(size_t)k * ldb + n0 + n];
+                s1 += v;
+                s2 += (double)(n + 1) * v;
+            }
+            b1[k] = s1;
+            b2[k] = s2;
+        }
+        for (int m = 0; m < tm; ++m) {
+            double r1 = 0.0, r2 = 0.0, o1 = 0.0, o2 = 0.0;
+            for (int k = 0; k < K; ++k) {
+                double a = (double)A[(size_t)(m0 + m) * lda + k];
+                r1 += a * b1[k];
+                r2 += a * b2[k];
+            }
+            for (int n = 0; n < tn; ++n) {
+                double v = (double)acc[(size_t)m * tn + n];
+                o1 += v;
+                o2 += (double)(n + 1) * v;
+            }
+            d1[m] = r1 - o1;
+            d2[m] = r2 - o2;
+        }
+        if (tau <= 0.0f) oracle_abft_relative_thresholds(tm, tn, K, acc, tn, tau < 0.0f ? -tau : 1.0f, thr, thr + tm);
+        else for (int m = 0; m < tm; ++m) thr[m] = (double)tau;
+        oracle_ft_status st;
+        memset(&st, 0, sizeof st);
+        st.row = st.col = -1;
+        int nbr = 0, r = -1;
+        double clean = 0.0;
+        for (int m = 0; m < tm; ++m) {
+            if (fabs(d1[m]) > thr[m]) { ++nbr; r = m; }
+            else if (fabs(d1[m]) > clean) clean = fabs(d1[m]);
+        }
+        st.n_bad_rows = nbr;
+        st.max_clean_residual = (float)clean;
+        if (nbr == 1) {
+            float f1 = (float)d1[r], f2 = (float)d2[r];
+            int c = (int)rintf(f2 / f1) - 1;
+            c = c < 0 ? 0 : (c >= tn ? tn - 1 : c);
+            float* e = &acc[(size_t)r * tn + c];
+            float again = oracle_recompute_element(0, K, A + (size_t)(m0 + r) * lda, B + n0 + c, ldb);
+            float change = again - *e;
+            *e = again;
+            if (fabsf(change - f1) <= (float)thr[r]) {
+                st.flag = 1; st.n_bad_cols = 1; st.row = r; st.col = c;
+                st.row_residual = f1; st.col_residual = f2;
+            } else {
+                st.flag = 2;
+            }
+        } else if (nbr > 1) {
+            st.flag = 2;
+        }
+        status[t] = st;
+        for (int m = 0; m < tm; ++m)
+            for (int n = 0; n < tn; ++n) {
+                float* c = &C[(size_t)(m0 + m) * ldc + n0 + n];
+                float v = alpha * acc[(size_t)m * tn + n];
+                *c = (beta == 0.0f) ? v : fmaf(beta, *c, v);
+            }
+        free(acc);
+        free(buf);
+    }
+}
 
 /* The whole-matrix model with the reference's verification cadence: the accumulators of a tile are verified every
  * check_interval values of k inside the K loop (kernel/ft_sgemm/include/ft_sgemm_huge.cuh:143, `if (k % 256 == 0)`)

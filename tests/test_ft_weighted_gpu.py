@@ -1,0 +1,169 @@
+"""GPU parity of the weighted-checksum locator (the reference's second scheme, "kernel 2": two row sums of B with weights
+[1, 1, ...] and [1, 2, ...], kernel/ft_sgemm/README.md:16-26; locator left in comments at
+kernel/ft_sgemm/include/ft_sgemm_huge.cuh:299-310) against the CPU model ``oracle.ft_sgemm_weighted``.
+
+Decisions (flag, located row and column, bad-line counts) must equal the model's; values obey the 1e-5 componentwise
+criterion once the fault is corrected, and a corrected product has the bits of a fault-free one."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+DECISION_FIELDS = ("flag", "row", "col", "n_bad_rows", "n_bad_cols")
+
+
+def _ws(blas, M, N, K, split=True, tile_class=0):
+    if split:
+        nbytes = blas.ft_workspace_bytes(M, N, K)
+    else:   # the two vectors per tile column and nothing else: no tile can be split along K
+        bn = blas.ft_tile(tile_class)[1]
+        nbytes = 4 * 2 * -(-N // bn) * ((-(-K // 16) + 2) * 16)
+    return torch.full((max((nbytes + 15) // 16 * 4, 4),), float("nan"), dtype=torch.float32, device="cuda")
+
+
+def _run(blas, a, b, c0, M, N, K, alpha, beta, tau, ws, tile_class, faults):
+    da, db, dc = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), torch.from_numpy(c0).cuda()
+    status = blas.ft_status_alloc(M, N, tile_class=tile_class)
+    blas.ft_sgemm(M, N, K, da, db, dc, alpha, beta, tau=tau, status=status, ws=ws, tile_class=tile_class, faults=faults,
+                  locator=blas.FT_LOCATE_WEIGHTED)
+    return dc.cpu().numpy(), blas.ft_status_numpy(status)
+
+
+@pytest.mark.parametrize("tile_class", [0, 1, 2, 3, 4])
+def test_exact_integer_operands_every_class(blas, oracle_mod, tile_class):
+    """Small-integer operands: accumulators, checksums and weighted checksums are exact, so d1 = -delta and
+    d2 = -(n + 1) delta exactly and every column is located, in full and in clipped tiles."""
+    bm, bn = blas.ft_tile(tile_class)
+    M, N, K = 2 * bm + 37, 2 * bn + 21, 200
+    rng = np.random.default_rng(300 + tile_class)
+    a = rng.integers(-4, 5, (M, K + 3)).astype(np.float32)
+    b = rng.integers(-4, 5, (K, N + 5)).astype(np.float32)
+    c0 = np.zeros((M, N + 2), np.float32)
+    exact = (a[:, :K].astype(np.float64) @ b[:, :N].astype(np.float64)).astype(np.float32)
+    ws = _ws(blas, M, N, K, tile_class=tile_class)
+    ntn = -(-N // bn)
+    ntiles = -(-M // bm) * ntn
+    cases = [[]]
+    for tile in (0, ntn - 1, ntiles - 1, ntiles // 2):
+        rows, cols = min(bm, M - (tile // ntn) * bm), min(bn, N - (tile % ntn) * bn)
+        for n in (0, 1, cols // 2, cols - 1):
+            cases.append([(tile, int(rng.integers(rows)), n, float(rng.choice([-1, 1]) * rng.integers(3, 40)))])
+    cases.append([(0, 5, 2, 8.0), (0, 5, 6, 8.0)])       # two in one row: the ratio names a healthy column, not confirmed
+    cases.append([(1, 5, 2, 8.0), (1, 6, 2, -4.0)])      # two rows
+    cases.append([(0, 1, 1, 0.25)])                      # below the threshold
+    for faults in cases:
+        c, st = _run(blas, a, b, c0, M, N, K, 1.0, 0.0, 0.5, ws, tile_class, faults)
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm_weighted(M, N, K, a, K + 3, b, N + 5, c_model, N + 2, 1.0, 0.0, bm, bn, 0.5, faults)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (tile_class, faults, f, st[f], st_model[f])
+        assert np.array_equal(c[:, :N], c_model[:, :N]), (tile_class, faults)
+        if len(faults) == 1 and abs(faults[0][3]) > 0.5:
+            t, m, n, delta = faults[0]
+            assert st["flag"][t] == 1 and (st["row"][t], st["col"][t]) == (m, n)
+            assert (st["row_residual"][t], st["col_residual"][t]) == (-delta, -(n + 1) * delta)
+            assert np.array_equal(c[:, :N], exact)
+
+
+@pytest.mark.parametrize("tile_class", [0, 1, 3])
+@pytest.mark.parametrize("tau_kind", ["absolute", "default"])
+def test_uniform_operands_decisions_equal_the_model(blas, oracle_mod, tile_class, tau_kind):
+    """Uniform operands, ragged shape, padded leading dimensions, alpha and beta: faults large against the rounding
+    noise of the weighted sums are located and corrected (bits of the device's summation order), decisions equal the
+    model's; a small fault is detected."""
+    bm, bn = blas.ft_tile(tile_class)
+    M, N, K = 333, 200, 420
+    tau = blas.ft_default_tau(K) if tau_kind == "absolute" else 0.0
+    a = oracle_mod.fill_uniform_matrix(M, K, 1900, ld=K + 4)
+    b = oracle_mod.fill_uniform_matrix(K, N, 1901, ld=N + 4)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, 1902, ld=N + 8)
+    ws = _ws(blas, M, N, K, split=False, tile_class=tile_class)
+    ntn = -(-N // bn)
+    ntiles = -(-M // bm) * ntn
+    rng = np.random.default_rng(500 + tile_class)
+    want = c0.copy()
+    oracle_mod.sgemm_device_order(M, N, K, a, K + 4, b, N + 4, want, N + 8, 1.5, -1.0)
+    for trial in range(8):
+        faults = []
+        if trial:
+            tile = int(rng.integers(ntiles))
+            rows, cols = min(bm, M - (tile // ntn) * bm), min(bn, N - (tile % ntn) * bn)
+            faults = [(tile, int(rng.integers(rows)), int(rng.integers(cols)), float(np.float32(rng.choice([-1, 1]) * 10.0 ** rng.uniform(0.3, 2))))]
+        c, st = _run(blas, a, b, c0, M, N, K, 1.5, -1.0, tau, ws, tile_class, faults)
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm_weighted(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, bm, bn, tau, faults)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (tile_class, faults, f, st[f], st_model[f])
+        if faults:
+            t, m, n, delta = faults[0]
+            assert st["flag"][t] == 1 and (st["row"][t], st["col"][t]) == (m, n) and np.count_nonzero(st["flag"]) == 1
+            assert abs(st["row_residual"][t] + delta) < 2e-3 + 1e-6 * abs(delta)
+            assert abs(st["col_residual"][t] + (n + 1) * delta) < (2e-3 + 1e-6 * abs(delta)) * bn
+        else:
+            assert not st["flag"].any()
+        assert np.array_equal(c[:, :N], want[:, :N]), (tile_class, faults)     # fault-free or corrected: the same bits
+        assert np.all(np.isnan(c[:, N:]))
+    # a fault of five thresholds: detected in its row for certain; located or not depends on the rounding of the
+    # weighted sums, and computing the guessed element again does no harm either way
+    small = 5 * blas.ft_default_tau(K)
+    c, st = _run(blas, a, b, c0, M, N, K, 1.5, -1.0, blas.ft_default_tau(K), ws, tile_class, [(0, 7, 30, small)])
+    assert st["flag"][0] in (1, 2) and st["n_bad_rows"][0] == 1 and not st["flag"][1:].any()
+    differ = np.argwhere(c[:, :N] != want[:, :N])
+    assert (len(differ) == 0 and st["flag"][0] == 1) or (differ.tolist() == [[7, 30]] and st["flag"][0] == 2)
+
+
+def test_partial_last_round_split_along_k_and_column_major_operands(blas, oracle_mod):
+    M, N, K = 700, 300, 2048       # 3 x 3 tiles of 256 x 128: all split along K when the workspace has the room
+    tau = blas.ft_default_tau(K)
+    a = oracle_mod.fill_uniform_matrix(M, K, 2300)
+    b = oracle_mod.fill_uniform_matrix(K, N, 2301)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, 2302)
+    faults = [(8, 700 - 512 - 1, 300 - 256 - 1, -7.5)]
+    results = [_run(blas, a, b, c0, M, N, K, 1.0, 1.0, tau, _ws(blas, M, N, K, split=s), 0, faults) for s in (True, False)]
+    c_model = c0.copy()
+    st_model = oracle_mod.ft_sgemm_weighted(M, N, K, a, K, b, N, c_model, N, 1.0, 1.0, 256, 128, tau, faults)
+    for c, st in results:
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), f
+        ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, K, b, N, c0, N, 1.0, 1.0)
+        assert oracle_mod.gemm_max_err(N, c, N, ref, den) <= TOL
+    assert not np.array_equal(results[0][0], results[1][0])     # the split did happen
+    # the reference family's column-major buffers: the row-major problem C^T = (B^T)^T A^T, tiles and faults of that problem
+    Mc, Nc, Kc = 200, 333, 300
+    abuf = oracle_mod.fill_uniform_matrix(Kc, Mc, 2400)
+    bbuf = oracle_mod.fill_uniform_matrix(Kc, Nc, 2401)
+    cbuf = oracle_mod.fill_uniform_matrix(Nc, Mc, 2402)
+    status = blas.ft_status_alloc(Nc, Mc)
+    dc = torch.from_numpy(cbuf).cuda()
+    fault = (3, 60, 40, 9.0)
+    blas.ft_sgemm_cm_nt(Mc, Nc, Kc, torch.from_numpy(abuf).cuda(), torch.from_numpy(bbuf).cuda(), dc, 1.0, 0.0,
+                        _ws(blas, Nc, Mc, Kc), tau=blas.ft_default_tau(Kc), status=status, faults=[fault], locator=blas.FT_LOCATE_WEIGHTED)
+    st = blas.ft_status_numpy(status)
+    bt = np.ascontiguousarray(bbuf.T)
+    c_model = cbuf.copy()
+    st_model = oracle_mod.ft_sgemm_weighted(Nc, Mc, Kc, bt, Kc, abuf, Mc, c_model, Mc, 1.0, 0.0, 256, 128, blas.ft_default_tau(Kc), [fault])
+    for f in DECISION_FIELDS:
+        assert np.array_equal(st[f], st_model[f]), f
+    assert st["flag"][3] == 1 and (st["row"][3], st["col"][3]) == (60, 40)
+    ref, den = oracle_mod.gemm_cm_nt_f64(Mc, Nc, Kc, abuf, Mc, bbuf, Nc, cbuf, Mc, 1.0, 0.0)
+    assert oracle_mod.gemm_max_err(Mc, dc.cpu().numpy(), Mc, ref, den) <= TOL
+
+
+def test_option_errors(blas):
+    t = torch.zeros(256, 256, device="cuda")
+    ws = torch.zeros(1 << 20, device="cuda")
+    with pytest.raises(blas.HpcdnnError):   # the two vectors of B come from the workspace
+        blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, locator=blas.FT_LOCATE_WEIGHTED)
+    with pytest.raises(blas.HpcdnnError):   # one checksum pair per workgroup tile
+        blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, locator=blas.FT_LOCATE_WEIGHTED, granularity=blas.FT_GRAN_WAVE, ws=ws)
+    with pytest.raises(blas.HpcdnnError):   # verified once
+        blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, locator=blas.FT_LOCATE_WEIGHTED, check_interval=64, ws=ws)
+    with pytest.raises(blas.HpcdnnError):
+        blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, locator=2, ws=ws)
+    # K = 0 needs no workspace and flags nothing
+    c = torch.full((256, 256), 2.0, device="cuda")
+    status = blas.ft_status_alloc(256, 256)
+    blas.ft_sgemm(256, 256, 0, t[:, :0], t[:0, :], c, 1.0, 0.5, locator=blas.FT_LOCATE_WEIGHTED, status=status)
+    assert torch.equal(c, torch.full((256, 256), 1.0, device="cuda")) and not blas.ft_status_numpy(status)["flag"].any()

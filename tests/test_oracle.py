@@ -618,6 +618,86 @@ def test_checked_model_corrects_one_fault_per_verification(oracle_mod):
     assert np.array_equal(c, want.astype(np.float32))
 
 
+def test_weighted_locator_model_closed_forms(oracle_mod):
+    """The reference's second scheme (two row sums of B, weights [1, 1, ...] and [1, 2, ...]; README.md:16-26) on
+    small-integer operands, where accumulators and checksums are exact: a fault delta at (m, n) of a tile gives
+    d1 = -delta and d2 = -(n + 1) delta, every column of every tile is located (also in the clipped edge tiles), the
+    corrected product is the fault-free one, and the record carries the two residuals."""
+    M, N, K, tm, tn = 20, 27, 48, 8, 12     # 3 x 3 tiles, the last row of tiles 4 high, the last column 3 wide
+    a, b, exact = _exact_problem(M, N, K, 31)
+    ntn = -(-N // tn)
+    for tile in range(9):
+        rows, cols = min(tm, M - (tile // ntn) * tm), min(tn, N - (tile % ntn) * tn)
+        for n in range(cols):
+            m, delta = (3 * n + tile) % rows, float((-1) ** n * (5 + n))
+            c = np.zeros((M, N), np.float32)
+            st = oracle_mod.ft_sgemm_weighted(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, [(tile, m, n, delta)])
+            want = [0] * 9
+            want[tile] = 1
+            assert st["flag"].tolist() == want
+            assert (st["row"][tile], st["col"][tile], st["n_bad_rows"][tile], st["n_bad_cols"][tile]) == (m, n, 1, 1)
+            assert (st["row_residual"][tile], st["col_residual"][tile]) == (-delta, -(n + 1) * delta)
+            assert np.array_equal(c, exact.astype(np.float32))
+    # fault-free: nothing flagged, exact residuals
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_weighted(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, [])
+    assert not st["flag"].any() and st["max_clean_residual"].max() == 0.0 and np.array_equal(c, exact.astype(np.float32))
+    # below the threshold: not flagged, left in C
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_weighted(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, [(4, 1, 1, 0.25)])
+    assert not st["flag"].any() and st["max_clean_residual"][4] == 0.25 and c[9, 13] == exact[9, 13] + 0.25
+    # two equal faults in one row, columns 2 and 6: the ratio points at column 4, which is healthy - computing it again
+    # changes nothing, the location is not confirmed, the tile is reported detected and both faults stay
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_weighted(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, [(0, 5, 2, 8.0), (0, 5, 6, 8.0)])
+    assert st["flag"][0] == 2 and (st["n_bad_rows"][0], st["n_bad_cols"][0], st["row"][0], st["col"][0]) == (1, 0, -1, -1)
+    want = exact.copy()
+    want[5, 2] += 8.0
+    want[5, 6] += 8.0
+    assert np.array_equal(c, want.astype(np.float32))
+    # two faults in different rows: two bad rows, nothing located
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_weighted(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, 0.5, [(0, 5, 2, 8.0), (0, 6, 2, -4.0)])
+    assert st["flag"][0] == 2 and st["n_bad_rows"][0] == 2
+    # alpha / beta are applied after the correction
+    c0 = np.arange(M * N, dtype=np.float32).reshape(M, N)
+    c = c0.copy()
+    oracle_mod.ft_sgemm_weighted(M, N, K, a, K, b, N, c, N, 2.0, -1.0, tm, tn, 0.5, [(8, 3, 2, 64.0)])
+    assert np.array_equal(c, (2.0 * exact - c0).astype(np.float32))
+
+
+def test_weighted_locator_model_against_numpy_composition(oracle_mod):
+    """Uniform operands, padded leading dimensions: the residuals the record reports equal an independent numpy FP64
+    composition (references from A and the two row sums of B, observed sums from the FP32 accumulator model), the
+    data-scaled threshold is that of the row x column model's rows, and a fault is located where its size allows."""
+    M, N, K, tm, tn, lda, ldb = 24, 40, 96, 16, 32, 100, 43
+    a = oracle_mod.fill_uniform_matrix(M, K, 71, ld=lda)
+    b = oracle_mod.fill_uniform_matrix(K, N, 72, ld=ldb)
+    tile, m, n, delta = 1, 5, 6, 0.5        # tile 1: rows 0..15, columns 32..39 (8 wide)
+    for tau in (1e-4, 0.0, -1.0):
+        c = np.zeros((M, N), np.float32)
+        st = oracle_mod.ft_sgemm_weighted(M, N, K, a, lda, b, ldb, c, N, 1.0, 0.0, tm, tn, tau, [(tile, m, n, delta)])
+        assert st["flag"].tolist() == [0, 1, 0, 0] and (st["row"][1], st["col"][1]) == (m, n)
+        at, bt = a[:16, :K], b[:, 32:40]
+        acc = oracle_mod.tile_acc(at, lda, bt, ldb, 16, 8, K)
+        acc[m, n] += np.float32(delta)
+        w = np.arange(1, 9, dtype=np.float64)
+        r1 = at.astype(np.float64) @ bt.astype(np.float64).sum(axis=1)
+        r2 = at.astype(np.float64) @ (bt.astype(np.float64) @ w)
+        d1 = r1 - acc.astype(np.float64).sum(axis=1)
+        d2 = r2 - acc.astype(np.float64) @ w
+        assert st["row_residual"][1] == np.float32(d1[m]) and st["col_residual"][1] == np.float32(d2[m])
+        assert st["max_clean_residual"][1] == np.float32(np.abs(np.delete(d1, m)).max())
+        assert abs(d1[m] + delta) < 1e-5 and abs(d2[m] + (n + 1) * delta) < 1e-4
+        ref = a[:, :K].astype(np.float64) @ b[:, :N].astype(np.float64)
+        assert np.max(np.abs(c - ref)) < 5e-6     # corrected: the fault is gone
+    # a fault just above the threshold but far below the rounding noise of the weighted sums x the tile width is
+    # detected, whether or not the ratio happens to hit its column
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_weighted(M, N, K, a, lda, b, ldb, c, N, 1.0, 0.0, tm, tn, 2e-5, [(0, 3, 17, 4e-5)])
+    assert st["flag"][0] in (1, 2) and st["n_bad_rows"][0] == 1 and not st["flag"][1:].any()
+
+
 def test_checked_model_resynchronises_after_every_verification(oracle_mod):
     """Two faults of 0.75 tau in one row, in different intervals: each verification sees one of them and absorbs it,
     so nothing is ever flagged (and both stay in C); a single verification at the end sees 1.5 tau in that row and in
