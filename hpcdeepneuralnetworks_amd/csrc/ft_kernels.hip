@@ -17,11 +17,15 @@ constexpr FtGeom kGeom = kFtGeom[HPCDNN_FT_CLASS];
 constexpr bool kTa = HPCDNN_FT_TA != 0;
 
 // the kernels without a workspace run four waves (2 x 2), those with one the class's own wave layout (ft_sgemm.hip)
+// (two staging sets in every class: the ABFT loop with four of them, tried on the 64-column classes for the products that
+// stream an operand from memory, measured 10-20 % slower on every shape)
+constexpr int kSlots = 2;
+
 template <int FT, int GRAN, bool CAD>
 FtKernel make_kernel() {
     constexpr int WGM = FT == 1 ? 2 : kGeom.wgm, WGN = FT == 1 ? 2 : kGeom.wgn;
-    return FtKernel{sgemm_kernel<kGeom.bm, kGeom.bn, WGM, WGN, false, FT, 1, 2, GRAN, CAD, kTa>,
-                    sgemm_kernel<kGeom.bm, kGeom.bn, WGM, WGN, true, FT, 1, 2, GRAN, CAD, kTa>, WGM * WGN * kWave,
+    return FtKernel{sgemm_kernel<kGeom.bm, kGeom.bn, WGM, WGN, false, FT, 1, kSlots, GRAN, CAD, kTa>,
+                    sgemm_kernel<kGeom.bm, kGeom.bn, WGM, WGN, true, FT, 1, kSlots, GRAN, CAD, kTa>, WGM * WGN * kWave,
                     gemm_lds_bytes<kGeom.bm, kGeom.bn, FT, WGM * WGN * kWave, WGM, WGN, GRAN>()};
 }
 }  // namespace

@@ -185,7 +185,8 @@ template <int BM, int BN, int WGM, int WGN, bool EDGE, int FT, int MIN_BLOCKS, i
           bool TA = false>
 __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(const GemmArgs p) {
     constexpr int BK = kGemmBK;
-    static_assert(NSLOT == 2 || (FT == 0 && NSLOT % 2 == 0), "the ABFT loop is written for two staging sets");
+    static_assert(NSLOT >= 2 && NSLOT % 2 == 0, "an even number of staging sets: LDS stages alternate with the K steps");
+    static_assert(NSLOT == 2 || FT == 0, "the ABFT kernels are instantiated and tested with two staging sets");
     static_assert(FT != 0 || (GRAN == 0 && !CADENCE), "granularity and cadence belong to the ABFT kernels");
     static_assert(GRAN == 0 || FT == 2, "wave-tile checksums come from the pre-encoded vectors");
     static_assert(FT != 3 || (GRAN == 0 && !CADENCE), "the weighted locator checks a workgroup tile once, after the K loop");
@@ -304,9 +305,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 
     // One staging load (part P of the K step at a_base/b_base) into slot S.  Nothing here touches the loaded
     // value, so the load stays in flight until the slot is consumed a K step later.
-    int k_slot[NSLOT];  // absolute k of the K step held by each staging slot
-#pragma unroll
-    for (int i = 0; i < NSLOT; ++i) k_slot[i] = kbeg;
+    int k_mask = kbeg;  // ragged tiles: absolute k of the K step whose staged data goes to LDS next (the one the masks see)
     // FT == 2: the K step's slice of the pre-encoded checksum vectors travels with it (same run-ahead, same
     // slots).  The rows of enc_a / enc_b end with two K steps of zeros, so the fetches that run ahead past the
     // end need no bounds: one descriptor per row, a per-thread offset, and a scalar offset that moves on by one
@@ -326,12 +325,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int enc_a_voff = B_SLOTS == 2 ? (tid / B_V4_PER_ROW) * 8 : ((((tid / B_V4_PER_ROW) & 7) * 2 + (tid / B_V4_PER_ROW) / 8) * 4);
     const int enc_b_voff = (tid & 3) * 16;  // b_r of the four k values of A this thread stages
     int enc_off = kbeg * 4;
-    float g_ac[2][GM][B_SLOTS];
-    v4f g_br[2][GN];
-    v4f g_bw[2];  // FT == 3: the weighted row sums of B for the four k values of A this thread stages
-    auto gload1 = [&](auto slot, auto part, auto bulk) {  // bulk: this K step is not the slice's last (kLazyBounds)
+    float g_ac[NSLOT][GM][B_SLOTS];
+    v4f g_br[NSLOT][GN];
+    v4f g_bw[NSLOT];  // FT == 3: the weighted row sums of B for the four k values of A this thread stages
+    auto gload1 = [&](auto slot, auto part, auto bulk) __attribute__((always_inline)) {  // bulk: this K step is not the slice's last (kLazyBounds)
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
-        if constexpr (P == 0) k_slot[S] = k_loaded;
         if constexpr (kNoBounds || (kLazyBounds && decltype(bulk)::value)) {
             if constexpr (P < A_SLOTS) ra[S][P] = buffer_load_v4f(make_rsrc_unbounded(a_base), a_voff[P]);
             else rb[S][P - A_SLOTS] = buffer_load_v4f(make_rsrc_unbounded(b_base), b_voff[P - A_SLOTS]);
@@ -367,7 +365,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // descriptor).  Columns n >= N of B hold the next row or padding too, but they only ever reach accumulators of
     // columns n >= N, which are never stored: plain SGEMM leaves them alone, the ABFT kernels (whose row sums of B
     // run over the whole tile width) force them to 0 as well.
-    auto gmask1 = [&](auto slot, auto part) {
+    auto gmask1 = [&](auto slot, auto part) __attribute__((always_inline)) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P < A_SLOTS && TA) {
             // rows k >= K of A^T read as 0, and a K slice ends on a K step unless it ends with K; columns m >= M
@@ -382,7 +380,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 ra[S][P] = v;
             }
         } else if constexpr (P < A_SLOTS) {
-            const int left = kend - (k_slot[S] + a_kc[P]);
+            const int left = kend - (k_mask + a_kc[P]);
             v4f v = ra[S][P];
             v.x = left > 0 ? v.x : 0.f;
             v.y = left > 1 ? v.y : 0.f;
@@ -391,7 +389,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             ra[S][P] = v;
         } else if constexpr (FT != 0) {
             constexpr int Q = P - A_SLOTS;
-            const int nv = (k_slot[S] + b_row[Q] < kend) ? b_nvalid[Q] : 0;
+            const int nv = (k_mask + b_row[Q] < kend) ? b_nvalid[Q] : 0;
             v4f v = rb[S][Q];
             v.x = nv > 0 ? v.x : 0.f;
             v.y = nv > 1 ? v.y : 0.f;
@@ -403,18 +401,18 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // After the last part of a K step: move to the next one, unless that would leave the slice; then the
     // descriptors are emptied, so the fetches that run ahead past the end all return 0 (never multiplied, and
     // neutral for the checksums).
-    auto gload_advance_bulk = [&]() {  // kLazyBounds, a step that is not the slice's last: no end to look out for
+    auto gload_advance_bulk = [&]() __attribute__((always_inline)) {  // kLazyBounds, a step that is not the slice's last: no end to look out for
         if constexpr (TA) a_base += a_step;
         else a_base += BK;
         b_base += b_step;
         k_loaded += BK;
     };
     // kLazyBounds, at the end of the bulk steps: the byte counts from the current bases to the ends of A and B
-    auto bounds_from_position = [&]() {
+    auto bounds_from_position = [&]() __attribute__((always_inline)) {
         a_left = a_bytes_left(k_loaded);
         b_left = (static_cast<int64_t>(p.K - 1 - k_loaded) * p.ldb + (p.N - n0)) * 4;
     };
-    auto gload_advance = [&]() {
+    auto gload_advance = [&]() __attribute__((always_inline)) {
         const bool more = k_loaded + BK < kend;
         if constexpr (TA) {
             // the bases move on regardless (an emptied descriptor returns 0 wherever it starts): with both steps
@@ -438,15 +436,15 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // The same in two parts, so that the short-step schedule can place them apart.  Its full tiles keep no bounds at
     // all: nothing they fetch lies outside the matrix, and past the end of the slice they fetch its last K step
     // again instead of zeros.
-    auto gload_advance_a_bulk = [&]() {
+    auto gload_advance_a_bulk = [&]() __attribute__((always_inline)) {
         if constexpr (TA) a_base += a_step;
         else a_base += BK;
     };
-    auto gload_advance_b_bulk = [&]() {
+    auto gload_advance_b_bulk = [&]() __attribute__((always_inline)) {
         b_base += b_step;
         k_loaded += BK;
     };
-    auto gload_advance_a = [&]() {
+    auto gload_advance_a = [&]() __attribute__((always_inline)) {
         const bool more = k_loaded + BK < kend;
         if constexpr (TA) {
             a_base += more ? a_step : 0;
@@ -456,13 +454,13 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             if constexpr (!kNoBounds) a_left = more ? a_left - BK * 4 : 0;
         }
     };
-    auto gload_advance_b = [&]() {
+    auto gload_advance_b = [&]() __attribute__((always_inline)) {
         const bool more = k_loaded + BK < kend;
         b_base += more ? b_step : 0;
         if constexpr (!kNoBounds) b_left = more ? b_left - b_step * 4 : 0;
         k_loaded += more ? BK : 0;
     };
-    auto lstore1 = [&](auto slot, auto part, int stage) {
+    auto lstore1 = [&](auto slot, auto part, int stage) __attribute__((always_inline)) {
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (P < A_SLOTS && TA) {
             float* const dst = As + stage * A_STAGE + a_lds[P];
@@ -477,14 +475,13 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     };
 
     // CADENCE: point the staging state at the start of the next verification interval [kbeg, kend)
-    auto k_range_reset = [&]() {
+    auto k_range_reset = [&]() __attribute__((always_inline)) {
         a_base = a_origin(kbeg);
         b_base = p.B + static_cast<int64_t>(kbeg) * p.ldb + n0;
         a_left = a_bytes_left(kbeg);
         b_left = (static_cast<int64_t>(p.K - 1 - kbeg) * p.ldb + (p.N - n0)) * 4;
         k_loaded = kbeg;
-#pragma unroll
-        for (int i = 0; i < NSLOT; ++i) k_slot[i] = kbeg;
+        k_mask = kbeg;
         enc_off = kbeg * 4;
     };
 
@@ -502,7 +499,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     const int a_frag_off = (wm * WM + lr) * AS + lh * 4;
     const int b_frag_off = (lh * 4) * BS + wn * WN + lr;
 
-    auto fread1 = [&](auto buf, auto part, int stage, int g) {  // part < TM: A block `part`; else B block `part - TM`
+    auto fread1 = [&](auto buf, auto part, int stage, int g) __attribute__((always_inline)) {  // part < TM: A block `part`; else B block `part - TM`
         constexpr int Bf = decltype(buf)::value, P = decltype(part)::value;
         if constexpr (P < TM) {
             fa[Bf][P] = *reinterpret_cast<const v4f*>(As + stage * A_STAGE + a_frag_off + g * 8 + P * 32 * AS);
@@ -513,7 +510,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             for (int q = 0; q < 4; ++q) fb[Bf][j][q] = bs[q * BS];
         }
     };
-    auto mfma1 = [&](auto buf, auto idx) {
+    auto mfma1 = [&](auto buf, auto idx) __attribute__((always_inline)) {
         constexpr int Bf = decltype(buf)::value, I = decltype(idx)::value;
         constexpr int q = I / (TM * TN), i = (I / TN) % TM, j = I % TN;
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[Bf][i][q], fb[Bf][j][q], acc[i][j], 0, 0, 0);
@@ -597,7 +594,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int NCONS = FT ? 2 + GM + NCR + 1 : 0;
     constexpr int kDppRor4 = 0x124, kDppRor8 = 0x128;  // rotate right inside each row of 16 lanes
 
-    auto produce1 = [&](auto slot, auto piece, int par) {
+    auto produce1 = [&](auto slot, auto piece, int par) __attribute__((always_inline)) {
         constexpr int S = decltype(slot)::value, E = decltype(piece)::value;
         if constexpr (TA && E <= 3) {
             // column sums of A^T's staged K step: a lane holds four m of one k per slot, the four lanes of a quad
@@ -687,7 +684,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         }
     };
     bool flush_now = true;  // uniform; set by the main loop before each K step that may flush
-    auto consume1 = [&](auto slot, auto piece, int par, auto flush) {
+    auto consume1 = [&](auto slot, auto piece, int par, auto flush) __attribute__((always_inline)) {
         constexpr int S = decltype(slot)::value, E = decltype(piece)::value;
         constexpr bool kFlush = decltype(flush)::value;
         const float* ap = s_apart + par * BK * kParts;
@@ -823,7 +820,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     //                (+ consume the checksum partials of step kt+1)
     // Work past the end of the slice (kt+1, kt+2 >= nkt) moves duplicate data that is never multiplied, which
     // keeps the loop free of branches (and lets the loads stay two steps ahead).
-    auto step_in = [&](auto sl_next, auto sl_free, auto stage, auto flush, auto masked, auto bulk) {
+    auto step_in = [&](auto sl_next, auto sl_free, auto stage, auto flush, auto masked, auto bulk) __attribute__((always_inline)) {
         constexpr int st = decltype(stage)::value;
         constexpr bool kBulk = kLazyBounds && decltype(bulk)::value;
         constexpr int NMASK = (EDGE && decltype(masked)::value) ? (FT ? NGL : A_SLOTS) : 0;
@@ -870,6 +867,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             __builtin_amdgcn_sched_barrier(0);
         });
         __syncthreads();
+        if constexpr (EDGE) k_mask += BK;  // the next step's masks belong to the K step after this one's successor
         __builtin_amdgcn_sched_barrier(0);
         static_for<NMG>([&](auto m) {
             constexpr int Mi = decltype(m)::value;
@@ -898,14 +896,14 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     };
 
     // with two staging sets steps alternate between (next = slot 1, LDS stage 0) and (next = slot 0, LDS stage 1)
-    auto step = [&](auto sl_next, auto sl_free, auto flush, auto masked, auto bulk) {
+    auto step = [&](auto sl_next, auto sl_free, auto flush, auto masked, auto bulk) __attribute__((always_inline)) {
         step_in(sl_next, sl_free, std::integral_constant<int, (decltype(sl_next)::value == 1) ? 0 : 1>{}, flush, masked, bulk);
     };
     // step number kt with kt % NSLOT == phase: its successor waits in slot (phase + 1) % NSLOT, slot phase is free
-    auto step_at = [&](auto phase, auto masked, auto bulk) {
+    auto step_at = [&](auto phase, auto masked, auto bulk, auto flush) __attribute__((always_inline)) {
         constexpr int Ph = decltype(phase)::value;
         step_in(std::integral_constant<int, (Ph + 1) % NSLOT>{}, std::integral_constant<int, Ph % NSLOT>{},
-                std::integral_constant<int, Ph % 2>{}, std::false_type{}, masked, bulk);
+                std::integral_constant<int, Ph % 2>{}, flush, masked, bulk);
     };
 
     // One pass of the software pipeline over [kbeg, kend).
@@ -915,6 +913,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         static_for<NGL>([&](auto s) { gload1(S0{}, s, std::false_type{}); });
         gload_advance();
         if constexpr (EDGE) static_for<NGL>([&](auto s) { gmask1(S0{}, s); });
+        if constexpr (EDGE) k_mask += BK;
         static_for<NGL>([&](auto s) { lstore1(S0{}, s, 0); });
         static_for<NPROD>([&](auto e) { produce1(S0{}, e, 0); });
         static_for<NGL>([&](auto s) { gload1(S1{}, s, std::false_type{}); });
@@ -934,14 +933,24 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             if constexpr (kLazyBounds) {
                 // groups whose loads (NSLOT steps ahead) all stay before the slice's last K step
                 for (; lazy_ok && kt + 2 * NSLOT + 1 <= nkt; kt += NSLOT)
-                    static_for<NSLOT>([&](auto ph) { step_at(ph, std::false_type{}, std::true_type{}); });
+                    static_for<NSLOT>([&](auto ph) { step_at(ph, std::false_type{}, std::true_type{}, std::false_type{}); });
                 if (kt > 0) bounds_from_position();
             }
-            for (; kt + NSLOT <= bulk_end; kt += NSLOT)
-                static_for<NSLOT>([&](auto ph) { step_at(ph, std::false_type{}, std::false_type{}); });
+            // (ABFT: the checksums of a ragged problem want zeros in the columns n >= N of every step, so its groups
+            // run with the masks; the FP32 partial sums are flushed with the last step of every fourth group of four)
+            for (; kt + NSLOT <= bulk_end; kt += NSLOT) {
+                if constexpr (FT != 0) flush_now = (kt & 12) == 12;
+                static_for<NSLOT>([&](auto ph) {
+                    step_at(ph, std::integral_constant<bool, EDGE && FT != 0>{}, std::false_type{},
+                            std::integral_constant<bool, FT != 0 && decltype(ph)::value == NSLOT - 1>{});
+                });
+            }
             // what is left (fewer than a group, plus the two last steps of a ragged tile), one step at a time
+            flush_now = true;
             static_for<NSLOT + (EDGE ? 1 : -1)>([&](auto i) {
-                if (kt + decltype(i)::value < nkt) step_at(std::integral_constant<int, decltype(i)::value % NSLOT>{}, std::true_type{}, std::false_type{});
+                if (kt + decltype(i)::value < nkt)
+                    step_at(std::integral_constant<int, decltype(i)::value % NSLOT>{}, std::true_type{}, std::false_type{},
+                            std::integral_constant<bool, FT != 0>{});
             });
         } else {
             if constexpr (EDGE && FT == 0) {
