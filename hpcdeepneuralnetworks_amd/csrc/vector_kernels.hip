@@ -72,12 +72,14 @@ __global__ __launch_bounds__(kVecThreads) void saxpy_dword_kernel(int64_t n, flo
 // ------------------------------------------------------------------- SDOT --
 // Stands in for _sdot (grid-stride + shared-memory tree + float atomicAdd,
 // kernel/sdot/sdot.cu:9-36) and for the sdot + reduction multi-launch chain
-// (:38-67).  One launch, no float atomics: every block writes one partial,
-// takes a ticket, and the block that draws the last ticket adds the partials
-// in index order, so the result is reproducible bit for bit.
+// (:38-67).  One launch, no float atomics: every block publishes one partial,
+// and block 0 collects the partials and adds them in index order, so the result
+// is reproducible bit for bit.
 //
-// Workspace layout: [0] ticket (uint32, zero between calls), [64..] one double
-// per block.
+// Workspace layout: [0] epoch (uint32: the number of calls completed on this
+// workspace), [64..] two 64-bit words per block, each holding the epoch tag of
+// the call that wrote it in its upper half and one half of the block's double
+// partial in its lower half.
 constexpr int kSdotMaxBlocks = 4096;
 constexpr int kSdotVecBlocks = 256;  // one workgroup per CU of an MI355X: fewest tickets and partials, full bandwidth
 constexpr size_t kSdotPartialOffset = 64;
@@ -97,12 +99,17 @@ __device__ __forceinline__ double block_sum_to_thread0(double v, double* lds) {
     return s;
 }
 
+constexpr int kSdotSpinLimit = 1 << 20;  // polls before block 0 gives up on a block (about a second)
+
 template <int UNROLL, bool VEC>
 __global__ __launch_bounds__(kVecThreads) void sdot_kernel(int64_t n, const float* __restrict__ x,
                                                            const float* __restrict__ y, float* __restrict__ out,
-                                                           unsigned int* ticket, double* partials) {
+                                                           unsigned int* epoch, unsigned long long* slots) {
     __shared__ double lds[kVecThreads / kWave];
-    __shared__ bool is_last;
+    __shared__ unsigned int s_tag;
+    // this call's number: one more than the calls completed on this workspace (read now, needed after the sums)
+    unsigned int tag = 0;
+    if (threadIdx.x == 0) tag = __hip_atomic_load(epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
     float acc[UNROLL][4];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) acc[u][0] = acc[u][1] = acc[u][2] = acc[u][3] = 0.0f;
@@ -157,33 +164,44 @@ __global__ __launch_bounds__(kVecThreads) void sdot_kernel(int64_t n, const floa
     const double block_total = block_sum_to_thread0(v, lds);
 
     // Cross-block hand-off without cache-wide fences (a device-scope release/acquire fence writes back and
-    // invalidates the whole L2 of the XCD, which costs a streaming kernel a quarter of its bandwidth).  All
-    // traffic on the partials and the ticket is device-scope atomic read-modify-write.  Hardware assumption: a
-    // device-scope read-modify-write is performed at the point of coherence shared by the 8 XCDs, and its return
-    // value leaves that point only after the operation has been performed there.  The ticket's increment is made
-    // to depend on the value the exchange returned, so the ticket cannot issue before the exchange that
-    // published the partial has been performed; the last block reads the partials back with atomic adds of zero.
+    // invalidates the whole L2 of the XCD, which costs a streaming kernel a quarter of its bandwidth) and without a
+    // chain of dependent read-modify-writes (exchange, ticket, read-back: three trips to the point of coherence, which
+    // is most of a short call).  Every block stores its partial as two device-scope 64-bit words, each tagged with
+    // this call's number; block 0 polls the words of every block until both carry the tag - a word is written whole,
+    // so a matching tag means its payload is this call's - and adds the partials in index order.  No value of a
+    // partial is special: stale words are told apart by their tag, which differs from call to call.  Hardware
+    // assumption: device-scope (sc1) stores and loads of an aligned 64-bit word are single accesses at the point of
+    // coherence shared by the XCDs.  Every block but block 0 ends without waiting; block 0 waits for blocks that are
+    // running or will run once a CU is free, and gives up (NaN result) after a bounded number of polls.
     if (threadIdx.x == 0) {
-        const double old = __hip_atomic_exchange(&partials[blockIdx.x], block_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // zero for every bit pattern of `old`, through an instruction the compiler cannot see into: a data
-        // dependency without a special value
-        unsigned int dep = static_cast<unsigned int>(__builtin_bit_cast(unsigned long long, old));
-        asm volatile("v_and_b32 %0, 0, %0" : "+v"(dep));
-        const unsigned int one = 1u + dep;
-        const unsigned int t = __hip_atomic_fetch_add(ticket, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = (t == gridDim.x - 1);
+        const unsigned long long bits = __builtin_bit_cast(unsigned long long, block_total);
+        const unsigned long long tag_hi = static_cast<unsigned long long>(tag) << 32;
+        __hip_atomic_store(&slots[2 * blockIdx.x], tag_hi | (bits & 0xffffffffull), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&slots[2 * blockIdx.x + 1], tag_hi | (bits >> 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_tag = tag;
     }
+    if (blockIdx.x != 0) return;
     __syncthreads();
-    if (!is_last) return;
-
+    const unsigned int want = s_tag;
     double s = 0.0;
-    for (unsigned int b = threadIdx.x; b < gridDim.x; b += kVecThreads)
-        s += __hip_atomic_fetch_add(&partials[b], 0.0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();  // lds reuse
+    int missing = 0;
+    for (unsigned int b = threadIdx.x; b < gridDim.x; b += kVecThreads) {
+        unsigned long long lo = 0, hi = 0;
+        int spin = 0;
+        for (; spin < kSdotSpinLimit; ++spin) {
+            lo = __hip_atomic_load(&slots[2 * b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            hi = __hip_atomic_load(&slots[2 * b + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (static_cast<unsigned int>(lo >> 32) == want && static_cast<unsigned int>(hi >> 32) == want) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        missing += spin == kSdotSpinLimit;
+        s += __builtin_bit_cast(double, (hi << 32) | (lo & 0xffffffffull));
+    }
+    missing = __syncthreads_or(missing);  // (also the barrier before lds is reused)
     const double total = block_sum_to_thread0(s, lds);
     if (threadIdx.x == 0) {
-        *out = static_cast<float>(total);
-        __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next stream-ordered call
+        *out = missing ? __builtin_nanf("") : static_cast<float>(total);
+        __hip_atomic_store(epoch, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // the next stream-ordered call is number want + 1
     }
 }
 
@@ -260,8 +278,8 @@ extern "C" int hpcdnn_sdot(int64_t n, const float* x, const float* y, float* out
     if (!ws || ws_bytes < hpcdnn_workspace_bytes(HPCDNN_OP_SDOT, 0, 0, 0)) return HPCDNN_ERR_WORKSPACE;
     if (reinterpret_cast<uintptr_t>(ws) & 7u) return HPCDNN_ERR_INVALID_VALUE;  // the block partials are doubles
     hipStream_t s = static_cast<hipStream_t>(stream);
-    unsigned int* ticket = static_cast<unsigned int*>(ws);
-    double* partials = reinterpret_cast<double*>(static_cast<char*>(ws) + kSdotPartialOffset);
+    unsigned int* ticket = static_cast<unsigned int*>(ws);  // the epoch word
+    unsigned long long* partials = reinterpret_cast<unsigned long long*>(static_cast<char*>(ws) + kSdotPartialOffset);
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
     if (aligned) {
         // one slice of >= 4096 elements per workgroup, 256 workgroups at most: a function of n only, so the

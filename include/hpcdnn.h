@@ -419,14 +419,17 @@ int hpcdnn_saxpy(int64_t n, float alpha, const float* x, float* y, void* stream)
 /* *out = sum_i x[i]*y[i] (device scalar, overwritten; deterministic: the same
  * inputs give the same bits on every run).  `ws` must hold
  * hpcdnn_workspace_bytes(HPCDNN_OP_SDOT,...) bytes and have been passed through
- * hpcdnn_workspace_init once; calls sharing a workspace must be stream-ordered.
+ * hpcdnn_workspace_init once (it holds the number of calls completed, by
+ * which a call tells the partial sums of its own blocks from older ones);
+ * calls sharing a workspace must be stream-ordered, and nothing else may
+ * write to it.
  * Replaces _sdot <<<min(1024,ceil(n/tpb)),tpb>>>(N,x,y,out) with its
  * pre-zeroed atomicAdd target, and the sdot + reduction multi-launch chain
  * (kernel/sdot/sdot.cu:9-67, launches :156,:177-187). */
 int hpcdnn_sdot(int64_t n, const float* x, const float* y, float* out, void* ws, size_t ws_bytes, void* stream);
 
 /* Scratch size for an operation (SGEMM: split-K partials for the split
- * hpcdnn_sgemm would choose, 0 if none; SDOT: block partials + ticket; M,N,K
+ * hpcdnn_sgemm would choose, 0 if none; SDOT: the blocks' tagged partials + the call counter; M,N,K
  * ignored for SDOT). */
 size_t hpcdnn_workspace_bytes(int op, int M, int N, int K);
 /* Zero a freshly allocated workspace (fill kernel, safe to capture). */
