@@ -49,7 +49,7 @@ def main() -> int:
     ap.add_argument("--ft-launches", type=int, default=1000, help="launches of the ABFT fault campaign")
     ap.add_argument("--kernel", default="all", choices=["all", "sgemm", "sgemm_1024", "sgemm_lowk", "sgemm_cm_nt", "ft_sgemm_cm_nt", "ft_sgemm", "ft_sgemm_fused", "ft_sgemm_wave", "offline_ft", "saxpy", "sdot", "copy",
                              "sgemv_n", "sgemv_t", "sgemm_deepk", "sgemm_1000", "sgemm_512", "sgemm_skinny", "ft_sgemm_skinny", "ft_sgemm_cadence",
-                             "ft_sgemm_cadence_fused", "ft_sgemm_2048x1024", "saxpy_tail", "sdot_tail"],
+                             "ft_sgemm_cadence_fused", "ft_sgemm_2048x1024", "ft_sgemm_weighted", "saxpy_tail", "sdot_tail"],
                     help="run one kernel only for --steps launches (for profiling with rocprofv3) and print a short line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -128,6 +128,15 @@ def main() -> int:
             ft_ws = blas.workspace(blas.ft_workspace_bytes(mm, nn, kk))
             fn = lambda: blas.ft_sgemm(mm, nn, kk, a, b, c, 1.0, 0.0, tau=blas.ft_default_tau(kk), status=status, ws=ft_ws, tile_class=cls)
             work, unit = 2.0 * mm * nn * kk, "GFLOP/s"
+        elif args.kernel == "ft_sgemm_weighted":
+            # the reference's second scheme: two row sums of B, location from the ratio of the two residuals
+            m = 4096
+            a, b, c = operands(m, m, m, 20)
+            status = blas.ft_status_alloc(m, m)
+            ft_ws = blas.workspace(blas.ft_workspace_bytes(m, m, m))
+            fn = lambda: blas.ft_sgemm(m, m, m, a, b, c, 1.0, 0.0, tau=blas.ft_default_tau(m), status=status, ws=ft_ws,
+                                       locator=blas.FT_LOCATE_WEIGHTED)
+            work, unit = 2.0 * m ** 3, "GFLOP/s"
         elif args.kernel in ("ft_sgemm_cadence", "ft_sgemm_cadence_fused"):
             # the reference's scheme: a verification every 256 values of k (ft_sgemm_huge.cuh:143)
             m = 4096
