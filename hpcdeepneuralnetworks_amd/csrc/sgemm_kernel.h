@@ -156,6 +156,53 @@ __device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, 
     tn = in_group / gsz;
 }
 
+// One element of A * B computed again, for the ABFT correction: the sum over k in [k0, k1) of
+// a[k * a_stride] * b[k * b_stride] as one chain of fused multiply-adds in the order the matrix core adds them (per K
+// step of 16 and half step g, the pairs k = 8g + q, 8g + 4 + q for q = 0..3: a 32x32x2 FP32 MFMA is two chained FMAs,
+// lanes 0-31's k first; zeros pad the last K step), so the element gets exactly the bits a fault-free run gives it.
+// All `threads` threads of the workgroup call it together: they stage the operand row and column through LDS
+// (`stage`: 2 * chunk floats, chunk a multiple of 16), thread 0 walks them, and only thread 0's return value means
+// anything.  Kept out of line on purpose: inlined into the GEMM kernels, the address arithmetic of this (cold) code
+// changed the register assignment of their main loops, which cost the 256x128 kernel 1 % of a 4096^3 product.
+static __device__ __attribute__((noinline)) float recompute_element(const float* a, int64_t a_stride, const float* b, int64_t b_stride,
+                                                           int k0, int k1, float* stage, int chunk, int tid, int threads) {
+    float* const s_fa = stage;
+    float* const s_fb = stage + chunk;
+    float val = 0.f;
+#pragma unroll 1
+    for (int kc = k0; kc < k1; kc += chunk) {
+        const int len = (k1 - kc < chunk) ? k1 - kc : chunk;
+        const int padded = (len + kGemmBK - 1) / kGemmBK * kGemmBK;
+#pragma unroll 1
+        for (int i = tid; i < padded; i += threads) {
+            const int k = kc + i;
+            s_fa[i] = i < len ? a[static_cast<int64_t>(k) * a_stride] : 0.f;
+            s_fb[i] = i < len ? b[static_cast<int64_t>(k) * b_stride] : 0.f;
+        }
+        __syncthreads();
+        if (tid == 0) {
+#pragma unroll 1
+            for (int i = 0; i < padded; i += kGemmBK) {
+                float av[kGemmBK], bv[kGemmBK];
+#pragma unroll
+                for (int e = 0; e < kGemmBK; e += 4) {
+                    *reinterpret_cast<v4f*>(av + e) = *reinterpret_cast<const v4f*>(s_fa + i + e);
+                    *reinterpret_cast<v4f*>(bv + e) = *reinterpret_cast<const v4f*>(s_fb + i + e);
+                }
+#pragma unroll
+                for (int g = 0; g < 2; ++g)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        val = __builtin_fmaf(av[8 * g + q], bv[8 * g + q], val);
+                        val = __builtin_fmaf(av[8 * g + 4 + q], bv[8 * g + 4 + q], val);
+                    }
+            }
+        }
+        __syncthreads();
+    }
+    return val;
+}
+
 // FT: 0 = plain SGEMM; 1 = ABFT, checksum vectors e^T A and B e formed inside the main loop; 2 = ABFT, checksum
 // vectors read from a workspace filled by abft_encode_kernel (fewer VALU instructions in the main loop); 3 = ABFT with
 // the weighted-checksum locator (the reference's "kernel 2", kernel/ft_sgemm/README.md:16-26: two row sums of B,
@@ -1268,12 +1315,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         // locate: one faulty row x one faulty column of a check tile (ft_sgemm_huge.cuh:273-296).  Correct: the
         // reference subtracts round(|residual|) (:352-371), which only fits its +1.0 test fault, and the signed row
         // residual would leave the fault-free rounding noise of a whole row in one element; the located accumulator
-        // is computed again from A and B instead.  One lane walks the k range done so far with one fused multiply-add
-        // per k in the order the matrix core adds them (per K step and half step g, the pairs k = 8g + q, 8g + 4 + q
-        // for q = 0..3: a 32x32x2 FP32 MFMA is two chained FMAs, lanes 0-31's k first), so the element gets exactly
-        // the bits a fault-free run gives it.  The operand row and column are staged through the LDS the reference
-        // partials no longer need, a chunk of kFixChunk values of k at a time, by all threads (the condition is
-        // uniform over the workgroup); zeros pad the last K step.
+        // is computed again from A and B instead (recompute_element: one chain of fused multiply-adds over the k range
+        // done so far, in the matrix core's order, so the element gets exactly the bits a fault-free run gives it).  The
+        // operand row and column are staged through the LDS the reference partials no longer need, a chunk of kFixChunk
+        // values of k at a time, by all threads (the condition is uniform over the workgroup).
         // Weighted locator (kernel/ft_sgemm/README.md:16-26): one faulty row; with a fault delta in column n its two
         // residuals are -delta and -(n + 1) delta, so their ratio names the column.  The element found that way is
         // computed again like any located element; the location counts as confirmed when that changed the element by
@@ -1302,42 +1347,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 const int bad_r = s_meta[8 * ct + 2], bad_c = s_meta[8 * ct + 3];
                 if (m0 + bad_r >= p.M || n0 + bad_c >= p.N) continue;  // (lines outside the matrix are all zeros: not reached)
                 constexpr int kFixChunk = static_cast<int>(sizeof(double) * (GM * CCP * BN + GN * CRP * BM) / (2 * sizeof(float))) / BK * BK;
-                float* const s_fa = smem;
-                float* const s_fb = smem + kFixChunk;
                 const float* const a_src = TA ? p.A + (m0 + bad_r) : p.A + static_cast<int64_t>(m0 + bad_r) * p.lda;
                 const float* const b_src = p.B + (n0 + bad_c);
-                float fixed_val = 0.f;
-#pragma unroll 1
-                for (int kc = k_first; kc < kend; kc += kFixChunk) {
-                    const int len = (kend - kc < kFixChunk) ? kend - kc : kFixChunk;
-                    const int padded = (len + BK - 1) / BK * BK;
-#pragma unroll 1
-                    for (int i = tid; i < padded; i += kGemmThreads) {
-                        const int k = kc + i;
-                        s_fa[i] = i < len ? (TA ? a_src[static_cast<int64_t>(k) * p.lda] : a_src[k]) : 0.f;
-                        s_fb[i] = i < len ? b_src[static_cast<int64_t>(k) * p.ldb] : 0.f;
-                    }
-                    __syncthreads();
-                    if (tid == 0) {
-#pragma unroll 1
-                        for (int i = 0; i < padded; i += BK) {
-                            float av[BK], bv[BK];
-#pragma unroll
-                            for (int e = 0; e < BK; e += 4) {
-                                *reinterpret_cast<v4f*>(av + e) = *reinterpret_cast<const v4f*>(s_fa + i + e);
-                                *reinterpret_cast<v4f*>(bv + e) = *reinterpret_cast<const v4f*>(s_fb + i + e);
-                            }
-#pragma unroll
-                            for (int g = 0; g < 2; ++g)
-#pragma unroll
-                                for (int q = 0; q < 4; ++q) {
-                                    fixed_val = __builtin_fmaf(av[8 * g + q], bv[8 * g + q], fixed_val);
-                                    fixed_val = __builtin_fmaf(av[8 * g + 4 + q], bv[8 * g + 4 + q], fixed_val);
-                                }
-                        }
-                    }
-                    __syncthreads();
-                }
+                const float fixed_val = recompute_element(a_src, TA ? p.lda : 1, b_src, p.ldb, k_first, kend, smem, kFixChunk, tid, kGemmThreads);
                 // thread 0 hands the value to the accumulator's owner, who reports what the correction changed
                 // (the re-synchronisation takes exactly that out of the two lines' residuals)
                 if (tid == 0) s_fix[2 * ct] = fixed_val;
