@@ -166,13 +166,16 @@ static Plan choose_plan(int M, int N, int K, bool allow_split, size_t ws_bytes, 
         Plan plan;
         double cost;
     };
-    Candidate cand[kNumTiles * 8];
+    Candidate cand[kNumTiles * 10];
     int n_cand = 0;
     double best_cost = 1e300;
     for (int t = 0; t < kNumTiles; ++t) {
         const TileConfig& cfg = kTiles[t];
         if (cfg.eff <= 0.f || (same_bits_only && cfg.wave_split_k)) continue;
-        for (int split = 1; split <= 64; split *= 2) {
+        // (more than 64 slices only for the tiles of at most 64 x 64: they are for products too small to fill the CUs
+        // otherwise; measured on 96..256-square products with K up to 262144, the larger tiles lost with them)
+        const int max_split = cfg.bm * cfg.bn <= 64 * 64 ? 256 : 64;
+        for (int split = 1; split <= max_split; split *= 2) {
             if (split > 1) {
                 if (!allow_split) break;
                 if (ceil_div(K, split) < 8 * cfg.bk) break;

@@ -219,6 +219,27 @@ def test_split_k_forced_matches_and_is_deterministic(blas, oracle_mod):
     assert np.array_equal(outs[-1][:, :N], again[:, :N])
 
 
+@pytest.mark.parametrize("tile", [1, 4])
+def test_split_k_slices_are_the_products_of_their_k_ranges(blas, tile):
+    """Eight slices (a multiple of the XCD count: the launch hands whole K slices to each XCD): the result has the bits of
+    the eight products over the K ranges, each computed by an unsplit call, added in slice order."""
+    M, N, K, split = 200, 136, 2048, 8
+    g = torch.Generator(device="cpu").manual_seed(77 + tile)
+    a = (torch.rand(M, K, generator=g) * 2 - 1).cuda()
+    b = (torch.rand(K, N, generator=g) * 2 - 1).cuda()
+    ws = blas.workspace(M * N * split * 4)
+    c = torch.full((M, N), 3.0, device="cuda")
+    blas.sgemm(M, N, K, a, b, c, 1.0, 0.0, ws=ws, tile=tile, split_k=split)
+    kc = K // split
+    total = None
+    for i in range(split):
+        part = torch.empty(M, N, device="cuda")
+        blas.sgemm(M, N, kc, a[:, i * kc:(i + 1) * kc], b[i * kc:(i + 1) * kc, :], part, 1.0, 0.0, tile=tile, split_k=1)
+        total = part if total is None else total + part
+    torch.cuda.synchronize()
+    assert torch.equal(c, total)
+
+
 @pytest.mark.parametrize("M,N,K,split", [(200, 136, 4200, 13), (200, 136, 4200, 32), (77, 132, 9000, 64), (200, 138, 4200, 16)])
 def test_split_k_many_slices(blas, oracle_mod, M, N, K, split):
     """More than eight slices are added by the reduction whose lanes share the slices of a group of elements (N a
