@@ -1061,11 +1061,17 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int kRowLines = GN * BM;                    // row lines (gn, m) come first, column lines (gm, n) after them
     // (weighted locator: the BM row lines, then the BM weighted row lines; there are no column lines)
     constexpr int kLines = kWeighted ? 2 * BM : kRowLines + GM * BN;
-    constexpr int LPT = (kLines + kGemmThreads - 1) / kGemmThreads;  // lines per thread
+    // lines per thread in the pass over the column lines and in the pass over the row lines (with the weighted locator
+    // the second pass also takes the weighted row lines)
+    constexpr int kColPass = kWeighted ? 0 : GM * BN, kRowPass = kWeighted ? kLines : kRowLines;
+    constexpr int LPT_C = (kColPass + kGemmThreads - 1) / kGemmThreads > 0 ? (kColPass + kGemmThreads - 1) / kGemmThreads : 1;
+    constexpr int LPT_R = (kRowPass + kGemmThreads - 1) / kGemmThreads;
     static_assert(NCT <= kGemmThreads, "one thread per check tile keeps its record");
-    double line_off[LPT];          // CADENCE: what re-synchronisation has taken out of each of this thread's lines
+    double off_col[LPT_C], off_row[LPT_R];  // CADENCE: what re-synchronisation has taken out of each of this thread's lines
 #pragma unroll
-    for (int it = 0; it < LPT; ++it) line_off[it] = 0.0;
+    for (int it = 0; it < LPT_C; ++it) off_col[it] = 0.0;
+#pragma unroll
+    for (int it = 0; it < LPT_R; ++it) off_row[it] = 0.0;
     const int k_first = kbeg;      // first k of this workgroup's K range (kbeg moves on from interval to interval)
     hpcdnn_ft_status rec;          // thread ct < NCT: the record of check tile ct, merged over the verifications
     rec.flag = 0; rec.row = -1; rec.col = -1; rec.n_bad_rows = 0; rec.n_bad_cols = 0;
@@ -1138,194 +1144,250 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 
         if (tid < NCT) { s_meta[8 * tid] = 0; s_meta[8 * tid + 1] = 0; s_meta[8 * tid + 2] = -1; s_meta[8 * tid + 3] = -1; s_meta[8 * tid + 4] = 0; s_fix[2 * tid + 1] = 0.f; }
 
-        // reference checksums: every thread publishes its partial sums (columns nc..nc+3 over its k rows, its
-        // rows over its k group); the residual step below adds the partials in a fixed order
-        if constexpr (kWeighted) {
-#pragma unroll
-            for (int sl = 0; sl < A_SLOTS; ++sl)
-                s_crwref[e_class * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = crw_ref[sl];
-        } else {
+        // Two stages (the reference acts on a tile only when a column checksum AND a row checksum disagree,
+        // ft_sgemm_huge.cuh:263-296 `if (error > err_bound1 && error1 > err_bound1)`): the column checksums screen -
+        // observed column sums are in-lane additions, the cheap half of the work -, and the row checksums of the
+        // workgroup tile are formed and compared only when some column was flagged.  A check tile none of whose
+        // columns is flagged is clean; its rows are not looked at (nor counted, nor re-synchronised).  The weighted
+        // locator has no column lines: there the plain row checksums are the screen, evaluated every time.
+        // Reference checksums: every thread publishes its partial sums (columns nc..nc+3 over its k rows, its rows
+        // over its k group); the residual passes below add the partials in a fixed order.
+        auto publish_col_refs = [&]() {
 #pragma unroll
             for (int gm = 0; gm < GM; ++gm)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) s_ccref[(gm * CCP + e_hw) * BN + (tid % B_V4_PER_ROW) * 4 + e] = cc_ref[gm][e];
-        }
+        };
+        auto publish_row_refs = [&]() {
+            if constexpr (kWeighted) {
 #pragma unroll
-        for (int gn = 0; gn < GN; ++gn)
+                for (int sl = 0; sl < A_SLOTS; ++sl)
+                    s_crwref[e_class * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = crw_ref[sl];
+            }
 #pragma unroll
-            for (int sl = 0; sl < A_SLOTS; ++sl)
-                s_crref[(gn * CRP + e_class) * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = cr_ref[gn][sl];
+            for (int gn = 0; gn < GN; ++gn)
+#pragma unroll
+                for (int sl = 0; sl < A_SLOTS; ++sl)
+                    s_crref[(gn * CRP + e_class) * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = cr_ref[gn][sl];
+        };
         // observed column sums of the accumulators (ft_sgemm_huge.cuh:147-154): lane = column.  In relative mode the
         // sums of absolute values go with them: they scale the threshold to the data.
         const bool relative = p.tau <= 0.f;
+        auto observe_cols = [&]() {
 #pragma unroll
-        for (int j = 0; j < (kWeighted ? 0 : TN); ++j) {
-            float s = 0.f, sa = 0.f;
+            for (int j = 0; j < TN; ++j) {
+                float s = 0.f, sa = 0.f;
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                float si = 0.f;
+                for (int i = 0; i < TM; ++i) {
+                    float si = 0.f;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) si += acc[i][j][v];
-                s += si;
+                    for (int v = 0; v < 16; ++v) si += acc[i][j][v];
+                    s += si;
+                }
+                s += __shfl_xor(s, 32, kWave);
+                if (relative) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) sa += __builtin_fabsf(acc[i][j][v]);
+                    sa += __shfl_xor(sa, 32, kWave);
+                }
+                if (lh == 0) {
+                    s_ccobs[wm * BN + wn * WN + j * 32 + lr] = s;
+                    s_ccabs[wm * BN + wn * WN + j * 32 + lr] = sa;
+                }
             }
-            s += __shfl_xor(s, 32, kWave);
-            if (relative) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) sa += __builtin_fabsf(acc[i][j][v]);
-                sa += __shfl_xor(sa, 32, kWave);
-            }
-            if (lh == 0) {
-                s_ccobs[wm * BN + wn * WN + j * 32 + lr] = s;
-                s_ccabs[wm * BN + wn * WN + j * 32 + lr] = sa;
-            }
-        }
+        };
         // observed row sums (ft_sgemm_huge.cuh:156-171): register = row, summed over the 32 column lanes.  The
         // TM * 16 sums of a lane are reduced together, 32 (or 16) at a time: afterwards lane lr of each half holds
         // the sum of row number lr of the group, and every lane stores one
-        constexpr int RG = TM >= 2 ? 32 : 16;      // rows reduced together
-        constexpr int NRG = TM * 16 / RG;          // groups per wave tile
+        auto observe_rows = [&]() {
+            constexpr int RG = TM >= 2 ? 32 : 16;      // rows reduced together
+            constexpr int NRG = TM * 16 / RG;          // groups per wave tile
 #pragma unroll
-        for (int g = 0; g < NRG; ++g) {
-            float rs[RG], ra_[RG];
-#pragma unroll
-            for (int e = 0; e < RG; ++e) {
-                const int i = (g * RG + e) / 16, v = (g * RG + e) % 16;
-                float s = acc[i][0][v];
-#pragma unroll
-                for (int j = 1; j < TN; ++j) s += acc[i][j][v];
-                rs[e] = s;
-            }
-            half32_transpose_sum<RG>(rs, lane);
-            if (relative) {
+            for (int g = 0; g < NRG; ++g) {
+                float rs[RG], ra_[RG];
 #pragma unroll
                 for (int e = 0; e < RG; ++e) {
                     const int i = (g * RG + e) / 16, v = (g * RG + e) % 16;
-                    float sa = 0.f;
+                    float s = acc[i][0][v];
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) sa += __builtin_fabsf(acc[i][j][v]);
-                    ra_[e] = sa;
+                    for (int j = 1; j < TN; ++j) s += acc[i][j][v];
+                    rs[e] = s;
                 }
-                half32_transpose_sum<RG>(ra_, lane);
-            } else {
-                ra_[0] = 0.f;
-            }
-            // this lane's row: number e = lr % RG of the group -> block i, register v
-            const int e = g * RG + (lr & (RG - 1)), v = e & 15;
-            const int row = wm * WM + (e >> 4) * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (RG == 32 || lr < RG) {
-                s_crobs[wn * BM + row] = rs[0];
-                s_crabs[wn * BM + row] = ra_[0];
-            }
-            if constexpr (kWeighted) {
-                // the same rows with column n of the tile weighted by n + 1 (kernel/ft_sgemm/README.md:16-26, e2 = [1, 2, ...])
-                float rw[RG];
+                half32_transpose_sum<RG>(rs, lane);
+                if (relative) {
 #pragma unroll
-                for (int e2 = 0; e2 < RG; ++e2) {
-                    const int i = (g * RG + e2) / 16, v = (g * RG + e2) % 16;
-                    float s = acc[i][0][v] * static_cast<float>(wn * WN + lr + 1);
+                    for (int e = 0; e < RG; ++e) {
+                        const int i = (g * RG + e) / 16, v = (g * RG + e) % 16;
+                        float sa = 0.f;
 #pragma unroll
-                    for (int j = 1; j < TN; ++j) s = __builtin_fmaf(acc[i][j][v], static_cast<float>(wn * WN + j * 32 + lr + 1), s);
-                    rw[e2] = s;
+                        for (int j = 0; j < TN; ++j) sa += __builtin_fabsf(acc[i][j][v]);
+                        ra_[e] = sa;
+                    }
+                    half32_transpose_sum<RG>(ra_, lane);
+                } else {
+                    ra_[0] = 0.f;
                 }
-                half32_transpose_sum<RG>(rw, lane);
-                if (RG == 32 || lr < RG) s_crwobs[wn * BM + row] = rw[0];
+                // this lane's row: number e = lr % RG of the group -> block i, register v
+                const int e = g * RG + (lr & (RG - 1)), v = e & 15;
+                const int row = wm * WM + (e >> 4) * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+                if (RG == 32 || lr < RG) {
+                    s_crobs[wn * BM + row] = rs[0];
+                    s_crabs[wn * BM + row] = ra_[0];
+                }
+                if constexpr (kWeighted) {
+                    // the same rows with column n of the tile weighted by n + 1 (kernel/ft_sgemm/README.md:16-26, e2 = [1, 2, ...])
+                    float rw[RG];
+#pragma unroll
+                    for (int e2 = 0; e2 < RG; ++e2) {
+                        const int i = (g * RG + e2) / 16, v = (g * RG + e2) % 16;
+                        float s = acc[i][0][v] * static_cast<float>(wn * WN + lr + 1);
+#pragma unroll
+                        for (int j = 1; j < TN; ++j) s = __builtin_fmaf(acc[i][j][v], static_cast<float>(wn * WN + j * 32 + lr + 1), s);
+                        rw[e2] = s;
+                    }
+                    half32_transpose_sum<RG>(rw, lane);
+                    if (RG == 32 || lr < RG) s_crwobs[wn * BM + row] = rw[0];
+                }
             }
-        }
-        __syncthreads();
-
-        // residual = reference - observed per line; |d| > tau marks the line (ft_sgemm_huge.cuh:200-271).  Relative
-        // mode: tau of a line of n elements inside the matrix = tau_rel * sqrt(n) * max(mean |acc| of the line, mean
-        // |acc| of the check tile): the rounding noise of a sum of n accumulators grows like sqrt(n) times their
+        };
+        // Relative mode: tau of a line of n elements inside the matrix = tau_rel * sqrt(n) * max(mean |acc| of the line,
+        // mean |acc| of the check tile): the rounding noise of a sum of n accumulators grows like sqrt(n) times their
         // magnitude, and the tile mean stands in for a short or cancelling line whose own accumulators say little about
-        // the size of its terms.  The tile sum is formed in a fixed order (per wave, then wave by wave).
+        // the size of its terms.  The tile sum is formed in a fixed order (per wave, then wave by wave) from the sums
+        // of the screening lines: columns, or rows with the weighted locator.
         constexpr int WPGM = WGM / GM, WPGN = WGN / GN;  // wave rows / wave columns per check tile
-        if (relative) {
+        auto tile_abs_sums = [&]() {
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct) {
                 const int gm = ct / GN, gn = ct % GN;
                 float part = 0.f;
-                for (int r = tid; r < CM; r += kGemmThreads)
+                if constexpr (kWeighted) {
+                    for (int r = tid; r < CM; r += kGemmThreads)
 #pragma unroll
-                    for (int w = 0; w < WPGN; ++w) part += s_crabs[(gn * WPGN + w) * BM + gm * CM + r];
+                        for (int w = 0; w < WPGN; ++w) part += s_crabs[(gn * WPGN + w) * BM + gm * CM + r];
+                } else {
+                    for (int c = tid; c < CN; c += kGemmThreads)
+#pragma unroll
+                        for (int w = 0; w < WPGM; ++w) part += s_ccabs[(gm * WPGM + w) * BN + gn * CN + c];
+                }
                 part = wave_sum_lane63(part);
                 if (lane == kWave - 1) s_tsum[ct * (kGemmThreads / kWave) + wave] = part;
             }
-            __syncthreads();
-        }
-        double d_line[LPT];
+        };
+        // One pass over the lines [first, first + count): residual = reference - observed; |d| > tau marks the line
+        // (ft_sgemm_huge.cuh:200-271).  gated: a row line counts only if its check tile has a flagged column.
+        auto residual_pass = [&](auto first_c, auto count_c, auto gated_c, double* d_out, const double* off) {
+            constexpr int kFirst = decltype(first_c)::value, kCount = decltype(count_c)::value;
+            constexpr bool kGated = decltype(gated_c)::value;
+            constexpr int kPer = (kCount + kGemmThreads - 1) / kGemmThreads;
 #pragma unroll
-        for (int it = 0; it < LPT; ++it) {
-            const int line = tid + it * kGemmThreads;
-            d_line[it] = 0.0;
-            float clean = 0.f;
-            int line_ct = -1;  // check tile of this line, if it has one inside the matrix
-            if (line < kLines) {
-                const bool is_row = line < kRowLines;
-                // row line (gn, idx): row idx of the tile against wave column gn; column line (gm, idx) likewise
-                const int grp = kWeighted ? 0 : is_row ? line / BM : (line - kRowLines) / BN;
-                const int idx = kWeighted ? (is_row ? line : line - BM) : is_row ? line - grp * BM : (line - kRowLines) - grp * BN;
-                const int gm = kWeighted ? 0 : is_row ? idx / CM : grp, gn = kWeighted ? 0 : is_row ? grp : idx / CN;
-                const int ct = gm * GN + gn;
-                int rows_in = p.M - (m0 + gm * CM), cols_in = p.N - (n0 + gn * CN);
-                rows_in = rows_in < CM ? rows_in : CM;
-                cols_in = cols_in < CN ? cols_in : CN;
-                double ref = 0.0, obs = 0.0;
-                float mag = 0.f;
-                if (kWeighted && !is_row) {
-                    // weighted row line idx: its residual locates the column, it is not tested against a threshold
+            for (int it = 0; it < kPer; ++it) {
+                const int line = kFirst + tid + it * kGemmThreads;
+                d_out[it] = 0.0;
+                float clean = 0.f;
+                int line_ct = -1;  // check tile of this line, if it has one inside the matrix (and is looked at)
+                if (line < kFirst + kCount) {
+                    const bool is_row = line < kRowLines;
+                    // row line (gn, idx): row idx of the tile against wave column gn; column line (gm, idx) likewise
+                    const int grp = kWeighted ? 0 : is_row ? line / BM : (line - kRowLines) / BN;
+                    const int idx = kWeighted ? (is_row ? line : line - BM) : is_row ? line - grp * BM : (line - kRowLines) - grp * BN;
+                    const int gm = kWeighted ? 0 : is_row ? idx / CM : grp, gn = kWeighted ? 0 : is_row ? grp : idx / CN;
+                    const int ct = gm * GN + gn;
+                    int rows_in = p.M - (m0 + gm * CM), cols_in = p.N - (n0 + gn * CN);
+                    rows_in = rows_in < CM ? rows_in : CM;
+                    cols_in = cols_in < CN ? cols_in : CN;
+                    double ref = 0.0, obs = 0.0;
+                    float mag = 0.f;
+                    if (kWeighted && !is_row) {
+                        // weighted row line idx: its residual locates the column, it is not tested against a threshold
 #pragma unroll
-                    for (int w = 0; w < CRP; ++w) ref += s_crwref[w * BM + idx];
+                        for (int w = 0; w < CRP; ++w) ref += s_crwref[w * BM + idx];
 #pragma unroll
-                    for (int w = 0; w < WGN; ++w) obs += static_cast<double>(s_crwobs[w * BM + idx]);
-                } else if (is_row) {
+                        for (int w = 0; w < WGN; ++w) obs += static_cast<double>(s_crwobs[w * BM + idx]);
+                    } else if (is_row) {
 #pragma unroll
-                    for (int w = 0; w < CRP; ++w) ref += s_crref[(grp * CRP + w) * BM + idx];
+                        for (int w = 0; w < CRP; ++w) ref += s_crref[(grp * CRP + w) * BM + idx];
 #pragma unroll
-                    for (int w = 0; w < WPGN; ++w) obs += static_cast<double>(s_crobs[(grp * WPGN + w) * BM + idx]);
+                        for (int w = 0; w < WPGN; ++w) obs += static_cast<double>(s_crobs[(grp * WPGN + w) * BM + idx]);
 #pragma unroll
-                    for (int w = 0; w < WPGN; ++w) mag += s_crabs[(grp * WPGN + w) * BM + idx];
-                } else {
-#pragma unroll
-                    for (int w = 0; w < CCP; ++w) ref += s_ccref[(grp * CCP + w) * BN + idx];
-#pragma unroll
-                    for (int w = 0; w < WPGM; ++w) obs += static_cast<double>(s_ccobs[(grp * WPGM + w) * BN + idx]);
-#pragma unroll
-                    for (int w = 0; w < WPGM; ++w) mag += s_ccabs[(grp * WPGM + w) * BN + idx];
-                }
-                const double d = (CADENCE ? ref - line_off[it] : ref) - obs;
-                d_line[it] = d;
-                if (rows_in > 0 && cols_in > 0 && !(kWeighted && !is_row)) {  // check tiles of an edge tile that lie outside the matrix have no lines
-                    double tau = static_cast<double>(p.tau);
-                    if (relative) {
-                        float total = 0.f;
-#pragma unroll
-                        for (int w = 0; w < kGemmThreads / kWave; ++w) total += s_tsum[ct * (kGemmThreads / kWave) + w];
-                        const float mean = total / (static_cast<float>(rows_in) * static_cast<float>(cols_in));
-                        const float n_line = static_cast<float>(is_row ? cols_in : rows_in);
-                        const float own = mag * (p.tau_rel / __builtin_sqrtf(n_line));
-                        const float floor = p.tau_rel * __builtin_sqrtf(n_line) * mean;
-                        tau = static_cast<double>(own > floor ? own : floor);
-                    }
-                    if (fabs(d) > tau) {
-                        atomicAdd(&s_meta[8 * ct + (is_row ? 0 : 1)], 1);
-                        atomicMax(&s_meta[8 * ct + (is_row ? 2 : 3)], idx);
-                        if constexpr (kWeighted) s_meta[8 * ct + 5] = __float_as_int(static_cast<float>(tau));  // (used when it is the only one)
+                        for (int w = 0; w < WPGN; ++w) mag += s_crabs[(grp * WPGN + w) * BM + idx];
                     } else {
-                        clean = static_cast<float>(fabs(d));
+#pragma unroll
+                        for (int w = 0; w < CCP; ++w) ref += s_ccref[(grp * CCP + w) * BN + idx];
+#pragma unroll
+                        for (int w = 0; w < WPGM; ++w) obs += static_cast<double>(s_ccobs[(grp * WPGM + w) * BN + idx]);
+#pragma unroll
+                        for (int w = 0; w < WPGM; ++w) mag += s_ccabs[(grp * WPGM + w) * BN + idx];
                     }
-                    line_ct = ct;
+                    const double d = (CADENCE ? ref - off[it] : ref) - obs;
+                    d_out[it] = d;
+                    const bool looked_at = !kGated || s_meta[8 * ct + 1] > 0;
+                    if (rows_in > 0 && cols_in > 0 && looked_at && !(kWeighted && !is_row)) {  // check tiles of an edge tile that lie outside the matrix have no lines
+                        double tau = static_cast<double>(p.tau);
+                        if (relative) {
+                            float total = 0.f;
+#pragma unroll
+                            for (int w = 0; w < kGemmThreads / kWave; ++w) total += s_tsum[ct * (kGemmThreads / kWave) + w];
+                            const float mean = total / (static_cast<float>(rows_in) * static_cast<float>(cols_in));
+                            const float n_line = static_cast<float>(is_row ? cols_in : rows_in);
+                            const float own = mag * (p.tau_rel / __builtin_sqrtf(n_line));
+                            const float floor = p.tau_rel * __builtin_sqrtf(n_line) * mean;
+                            tau = static_cast<double>(own > floor ? own : floor);
+                        }
+                        if (fabs(d) > tau) {
+                            atomicAdd(&s_meta[8 * ct + (is_row ? 0 : 1)], 1);
+                            atomicMax(&s_meta[8 * ct + (is_row ? 2 : 3)], idx);
+                            if constexpr (kWeighted) s_meta[8 * ct + 5] = __float_as_int(static_cast<float>(tau));  // (used when it is the only one)
+                        } else {
+                            clean = static_cast<float>(fabs(d));
+                        }
+                        line_ct = ct;
+                    }
+                    s_dr[line] = static_cast<float>(d);
                 }
-                s_dr[line] = static_cast<float>(d);
+                // largest residual among the clean lines: the 32 lines of a half wave belong to one check tile (check
+                // tiles are multiples of 32 rows and columns), so one lane per half records their maximum
+                const float half_max = half32_allmax(clean);
+                if (lr == 0 && line_ct >= 0) atomicMax(&s_meta[8 * line_ct + 4], __float_as_int(half_max));
             }
-            // largest residual among the clean lines: the 32 lines of a half wave belong to one check tile (check
-            // tiles are multiples of 32 rows and columns), so one lane per half records their maximum
-            const float half_max = half32_allmax(clean);
-            if (lr == 0 && line_ct >= 0) atomicMax(&s_meta[8 * line_ct + 4], __float_as_int(half_max));
+        };
+        constexpr int kColLines = kColPass, kScreenedRowLines = kRowPass;
+        double d_col[LPT_C], d_row[LPT_R];  // this verification's residuals of this thread's lines
+        bool rows_done = kWeighted;
+        if constexpr (kWeighted) {
+            publish_row_refs();
+            observe_rows();
+            __syncthreads();
+            if (relative) {
+                tile_abs_sums();
+                __syncthreads();
+            }
+            residual_pass(std::integral_constant<int, 0>{}, std::integral_constant<int, kScreenedRowLines>{}, std::false_type{}, d_row, off_row);
+            __syncthreads();
+        } else {
+            publish_col_refs();
+            observe_cols();
+            __syncthreads();
+            if (relative) {
+                tile_abs_sums();
+                __syncthreads();
+            }
+            residual_pass(std::integral_constant<int, kRowLines>{}, std::integral_constant<int, kColLines>{}, std::false_type{}, d_col, off_col);
+            __syncthreads();
+            int flagged_cols = 0;
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) flagged_cols |= s_meta[8 * ct + 1];
+            rows_done = __builtin_amdgcn_readfirstlane(flagged_cols) > 0;  // the same in every thread of the workgroup
+            if (rows_done) {
+                publish_row_refs();
+                observe_rows();
+                __syncthreads();
+                residual_pass(std::integral_constant<int, 0>{}, std::integral_constant<int, kScreenedRowLines>{}, std::true_type{}, d_row, off_row);
+                __syncthreads();
+            }
         }
-        __syncthreads();
-
         // locate: one faulty row x one faulty column of a check tile (ft_sgemm_huge.cuh:273-296).  Correct: the
         // reference subtracts round(|residual|) (:352-371), which only fits its +1.0 test fault, and the signed row
         // residual would leave the fault-free rounding noise of a whole row in one element; the located accumulator
@@ -1382,21 +1444,33 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             }
         }
         if constexpr (CADENCE) {
-            // re-synchronise (ft_sgemm_huge.cuh:268-271): every line starts the next interval with what is left of
-            // its residual after the correction taken out of its reference
+            // re-synchronise (ft_sgemm_huge.cuh:268-271): every line that was looked at starts the next interval with
+            // what is left of its residual after the correction taken out of its reference
+            constexpr int kColPer = (kColLines + kGemmThreads - 1) / kGemmThreads, kRowPer = (kRowLines + kGemmThreads - 1) / kGemmThreads;
 #pragma unroll
-            for (int it = 0; it < LPT; ++it) {
-                const int line = tid + it * kGemmThreads;
-                if (line < kLines) {
-                    const bool is_row = line < kRowLines;
-                    const int grp = is_row ? line / BM : (line - kRowLines) / BN;
-                    const int idx = is_row ? line - grp * BM : (line - kRowLines) - grp * BN;
-                    const int gm = is_row ? idx / CM : grp, gn = is_row ? grp : idx / CN;
-                    const int ct = gm * GN + gn;
+            for (int it = 0; it < kColPer; ++it) {
+                const int cl = tid + it * kGemmThreads;
+                if (cl < kColLines) {
+                    const int gm = cl / BN, idx = cl - gm * BN;
+                    const int ct = gm * GN + idx / CN;
                     double fixed = 0.0;
-                    if (s_meta[8 * ct] == 1 && s_meta[8 * ct + 1] == 1 && idx == s_meta[8 * ct + (is_row ? 2 : 3)])
-                        fixed = static_cast<double>(s_fix[2 * ct + 1]);
-                    line_off[it] += d_line[it] - fixed;
+                    if (s_meta[8 * ct] == 1 && s_meta[8 * ct + 1] == 1 && idx == s_meta[8 * ct + 3]) fixed = static_cast<double>(s_fix[2 * ct + 1]);
+                    off_col[it] += d_col[it] - fixed;
+                }
+            }
+            if (rows_done) {
+#pragma unroll
+                for (int it = 0; it < kRowPer; ++it) {
+                    const int line = tid + it * kGemmThreads;
+                    if (line < kRowLines) {
+                        const int gn = line / BM, idx = line - gn * BM;
+                        const int ct = (idx / CM) * GN + gn;
+                        if (s_meta[8 * ct + 1] > 0) {
+                            double fixed = 0.0;
+                            if (s_meta[8 * ct] == 1 && s_meta[8 * ct + 1] == 1 && idx == s_meta[8 * ct + 2]) fixed = static_cast<double>(s_fix[2 * ct + 1]);
+                            off_row[it] += d_row[it] - fixed;
+                        }
+                    }
                 }
             }
         }

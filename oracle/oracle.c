@@ -330,19 +330,27 @@ void oracle_abft_residuals(int tm, int tn, int K, const float* A, int lda, const
  * magnitude, but adding it back would leave the row's fault-free rounding
  * noise in one element, so the models below compute the located accumulator
  * again (oracle_recompute_element) and use the residual as a report only.
+ * Like the reference, which acts on a tile only when a column checksum AND a
+ * row checksum disagree (`if (error > err_bound1 && error1 > err_bound1)`,
+ * ft_sgemm_huge.cuh:289), the column checksums screen: a tile none of whose
+ * columns exceeds its threshold is clean (flag 0, no bad lines), and its rows
+ * are not looked at - neither counted nor part of max_clean_residual.  With a
+ * flagged column the rows are thresholded too: one faulty row x one faulty
+ * column -> located (flag 1), anything else -> detected only (flag 2).
  * Returns the signed row residual of the located row (0 when nothing is located). */
 /* Per-line thresholds: tau_r[m] for row m, tau_c[n] for column n. */
 float oracle_abft_decide_lines(int tm, int tn, const double* dr, const double* dc, const double* tau_r,
                                const double* tau_c, oracle_ft_status* st) {
     int nbr = 0, nbc = 0, r = -1, c = -1;
     double clean = 0.0;
-    for (int m = 0; m < tm; ++m) {
-        if (fabs(dr[m]) > tau_r[m]) { ++nbr; r = m; }
-        else if (fabs(dr[m]) > clean) clean = fabs(dr[m]);
-    }
     for (int n = 0; n < tn; ++n) {
         if (fabs(dc[n]) > tau_c[n]) { ++nbc; c = n; }
         else if (fabs(dc[n]) > clean) clean = fabs(dc[n]);
+    }
+    /* the rows are looked at only when a column checksum disagrees (see the comment above) */
+    for (int m = 0; m < tm && nbc > 0; ++m) {
+        if (fabs(dr[m]) > tau_r[m]) { ++nbr; r = m; }
+        else if (fabs(dr[m]) > clean) clean = fabs(dr[m]);
     }
     st->n_bad_rows = nbr;
     st->n_bad_cols = nbc;
@@ -613,7 +621,8 @@ void oracle_ft_sgemm_weighted(int M, int N, int K, const float* A, int lda, cons
  * verification the references are re-synchronised with the accumulators (`C_c -= C_c_`, ft_sgemm_huge.cuh:263-271):
  * what is left of each line's residual after the correction is absorbed, so the next verification sees only what
  * happened since this one.  (The reference leaves a line that exceeded the threshold unsynchronised and has no
- * working locate/correct step; here every line is re-synchronised, a located element is corrected first, and a
+ * working locate/correct step; here every line that a verification looked at is re-synchronised - the columns always,
+ * the rows when a column was flagged, see oracle_abft_decide_lines -, a located element is corrected first, and a
  * verification that could not locate its fault marks the tile uncorrectable for good.)
  * check_interval <= 0: one verification after the K loop (then this is oracle_ft_sgemm with several faults).
  * The tile's record merges its verifications: bad-line counts add up, flag 2 if any verification was
@@ -680,8 +689,9 @@ void oracle_ft_sgemm_checked(int M, int N, int K, const float* A, int lda, const
                 changed = (double)again - (double)*e;
                 *e = again;
             }
-            /* re-synchronise every line with what it shows after the correction */
-            for (int m = 0; m < tm; ++m) off_r[m] += dr[m] - ((cur.flag == 1 && m == cur.row) ? changed : 0.0);
+            /* re-synchronise every line that was looked at (the columns; the rows when a column was flagged) with
+             * what it shows after the correction */
+            for (int m = 0; m < tm && cur.n_bad_cols > 0; ++m) off_r[m] += dr[m] - ((cur.flag == 1 && m == cur.row) ? changed : 0.0);
             for (int n = 0; n < tn; ++n) off_c[n] += dc[n] - ((cur.flag == 1 && n == cur.col) ? changed : 0.0);
             /* merge */
             rec.n_bad_rows += cur.n_bad_rows;

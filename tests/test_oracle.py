@@ -295,24 +295,33 @@ def test_abft_decide_cases(oracle_mod):
     z_r, z_c = np.zeros(tm), np.zeros(tn)
     st, fix = oracle_mod.abft_decide(z_r, z_c, 0.01)
     assert st["flag"] == 0 and fix == 0.0 and st["row"] == -1 and st["col"] == -1
-    # below threshold -> clean, recorded as the largest clean residual
-    r = z_r.copy(); r[2] = -0.009
-    st, fix = oracle_mod.abft_decide(r, z_c, 0.01)
+    # below threshold -> clean, recorded as the largest clean residual (of the columns: they are the screen)
+    c = z_c.copy(); c[2] = -0.009
+    st, fix = oracle_mod.abft_decide(z_r, c, 0.01)
     assert st["flag"] == 0 and st["max_clean_residual"] == pytest.approx(0.009)
     # exactly at the threshold is clean (strict >), as in the reference (fabsf(x) > err_bound)
-    r[2] = float(np.float32(0.01))
-    assert oracle_mod.abft_decide(r, z_c, np.float32(0.01))[0]["flag"] == 0
+    c[2] = float(np.float32(0.01))
+    assert oracle_mod.abft_decide(z_r, c, np.float32(0.01))[0]["flag"] == 0
     # single fault: correction is the signed row residual
     r = z_r.copy(); c = z_c.copy(); r[4] = -0.5; c[1] = -0.5001
     st, fix = oracle_mod.abft_decide(r, c, 0.01)
     assert (st["flag"], st["row"], st["col"]) == (1, 4, 1) and fix == pytest.approx(-0.5)
     assert st["row_residual"] == pytest.approx(-0.5) and st["col_residual"] == pytest.approx(-0.5001)
-    # row without column, or two rows: detected but not correctable
+    # the columns screen, as in the reference, which acts only when a column AND a row disagree
+    # (ft_sgemm_huge.cuh:289): a row without any column is not looked at - not flagged, not counted, and not part of
+    # the largest clean residual either
     st, fix = oracle_mod.abft_decide(r, z_c, 0.01)
-    assert st["flag"] == 2 and fix == 0.0 and (st["n_bad_rows"], st["n_bad_cols"]) == (1, 0)
+    assert st["flag"] == 0 and fix == 0.0 and (st["n_bad_rows"], st["n_bad_cols"]) == (0, 0) and st["max_clean_residual"] == 0.0
+    # column without row, two rows, or two columns: detected but not correctable
+    st, fix = oracle_mod.abft_decide(z_r, c, 0.01)
+    assert st["flag"] == 2 and fix == 0.0 and (st["n_bad_rows"], st["n_bad_cols"]) == (0, 1)
     r[0] = 0.3
     st, _ = oracle_mod.abft_decide(r, c, 0.01)
-    assert st["flag"] == 2 and st["n_bad_rows"] == 2
+    assert st["flag"] == 2 and (st["n_bad_rows"], st["n_bad_cols"]) == (2, 1)
+    c[3] = 0.3
+    r[0] = 0.0
+    st, _ = oracle_mod.abft_decide(r, c, 0.01)
+    assert st["flag"] == 2 and (st["n_bad_rows"], st["n_bad_cols"]) == (1, 2)
 
 
 def test_tile_acc_matches_numpy_on_a_padded_rectangular_tile(oracle_mod):
@@ -356,14 +365,22 @@ def test_decide_lines_uses_each_lines_own_threshold(oracle_mod):
     dr, dc = np.zeros(tm), np.zeros(tn)
     tau_r = np.array([1.0, 0.1, 1.0, 0.01, 1.0])
     tau_c = np.array([0.5, 0.05, 0.5, 0.5])
-    # 0.2 is above row 1's threshold but below its neighbours'; the same residual in row 2 is clean
-    dr[1] = -0.2
+    # 0.2 is above column 1's threshold but below its neighbours'; the same residual in column 2 is clean
+    dc[1] = -0.2
     st, fix = oracle_mod.abft_decide_lines(dr, dc, tau_r, tau_c)
-    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"]) == (2, 1, 0) and fix == 0.0
-    dr[:] = 0.0
-    dr[2] = -0.2
+    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"]) == (2, 0, 1) and fix == 0.0
+    dc[:] = 0.0
+    dc[2] = -0.2
     st, fix = oracle_mod.abft_decide_lines(dr, dc, tau_r, tau_c)
     assert st["flag"] == 0 and st["max_clean_residual"] == pytest.approx(0.2)
+    # with a flagged column the rows get their own thresholds: 0.2 flags row 1 (0.1) and is clean in row 2 (1.0)
+    dc[:] = [0.0, -0.2, 0.0, 0.0]
+    dr[:] = [0.0, 0.0, -0.2, 0.0, 0.0]
+    st, fix = oracle_mod.abft_decide_lines(dr, dc, tau_r, tau_c)
+    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"]) == (2, 0, 1) and st["max_clean_residual"] == pytest.approx(0.2)
+    dr[:] = [0.0, -0.2, 0.0, 0.0, 0.0]
+    st, fix = oracle_mod.abft_decide_lines(dr, dc, tau_r, tau_c)
+    assert (st["flag"], st["row"], st["col"]) == (1, 1, 1)
     # row 1 and column 1 flagged by their own thresholds, the equally large residuals of row 0 / column 0 are clean
     dr[:] = [0.2, -0.2, 0.0, 0.0, 0.0]
     dc[:] = [0.2, -0.21, 0.0, 0.0]
@@ -371,9 +388,9 @@ def test_decide_lines_uses_each_lines_own_threshold(oracle_mod):
     assert (st["flag"], st["row"], st["col"], st["n_bad_rows"], st["n_bad_cols"]) == (1, 1, 1, 1, 1)
     assert fix == pytest.approx(-0.2) and st["col_residual"] == pytest.approx(-0.21)
     assert st["max_clean_residual"] == pytest.approx(0.2)
-    # rows and columns are not mixed up: tau_c applied to rows would flag row 0 (0.2 > 0.05 is column 1's threshold)
-    st, _ = oracle_mod.abft_decide_lines(dr, dc, tau_r, np.array([0.5, 0.5, 0.5, 0.5]))
-    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"]) == (2, 1, 0)
+    # rows and columns are not mixed up: tau_c applied to rows would flag row 0 too (0.2 > 0.05 is column 1's threshold)
+    st, _ = oracle_mod.abft_decide_lines(dr, dc, tau_r, np.array([0.1, 0.05, 0.5, 0.5]))
+    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"]) == (2, 1, 2)
     # the uniform form is the special case
     st_u, fix_u = oracle_mod.abft_decide(dr, dc, 0.1)
     st_l, fix_l = oracle_mod.abft_decide_lines(dr, dc, np.full(tm, np.float32(0.1), np.float64), np.full(tn, np.float32(0.1), np.float64))
@@ -699,23 +716,27 @@ def test_weighted_locator_model_against_numpy_composition(oracle_mod):
 
 
 def test_checked_model_resynchronises_after_every_verification(oracle_mod):
-    """Two faults of 0.75 tau in one row, in different intervals: each verification sees one of them and absorbs it,
-    so nothing is ever flagged (and both stay in C); a single verification at the end sees 1.5 tau in that row and in
-    two columns.  The residual a verification reports is what happened since the one before."""
+    """Two faults of 0.75 tau in one column, in different intervals: each verification sees one of them and absorbs it,
+    so nothing is ever flagged (and both stay in C); a single verification at the end sees 1.5 tau in that column and
+    0.75 tau in two rows.  The residual a verification reports is what happened since the one before."""
     M, N, K, tm, tn = 8, 8, 64, 8, 8
     a, b, exact = _exact_problem(M, N, K, 22)
     tau = 1.0
-    faults = [(0, 2, 1, 0.75, 0), (0, 2, 6, 0.75, 1)]
+    faults = [(0, 1, 2, 0.75, 0), (0, 6, 2, 0.75, 1)]
     c = np.zeros((M, N), np.float32)
     st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, tau, 32, faults)
     assert st["flag"][0] == 0 and st["max_clean_residual"][0] == 0.75
     want = exact.copy()
-    want[2, 1] += 0.75
-    want[2, 6] += 0.75
+    want[1, 2] += 0.75
+    want[6, 2] += 0.75
     assert np.array_equal(c, want.astype(np.float32))
     c = np.zeros((M, N), np.float32)
     st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, tau, 0, faults)
-    assert (st["flag"][0], st["n_bad_rows"][0], st["n_bad_cols"][0]) == (2, 1, 0) and st["max_clean_residual"][0] == 0.75
+    assert (st["flag"][0], st["n_bad_rows"][0], st["n_bad_cols"][0]) == (2, 0, 1) and st["max_clean_residual"][0] == 0.75
+    # (the same two faults in one row would go unnoticed by a single verification: the columns, 0.75 tau each, screen)
+    c = np.zeros((M, N), np.float32)
+    st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, tau, 0, [(0, 2, 1, 0.75, 0), (0, 2, 6, 0.75, 1)])
+    assert (st["flag"][0], st["n_bad_rows"][0], st["n_bad_cols"][0]) == (0, 0, 0)
     # the interval boundaries are k = 32, 64: a fault before verification 1 is seen by verification 1, not 0
     c = np.zeros((M, N), np.float32)
     st = oracle_mod.ft_sgemm_checked(M, N, K, a, K, b, N, c, N, 1.0, 0.0, tm, tn, tau, 32, [(0, 4, 4, 8.0, 1)])
