@@ -68,15 +68,20 @@ typedef struct hpcdnn_fault {
     float delta;
 } hpcdnn_fault;
 
-/* Verification record of one output tile (32 bytes, device memory). */
+/* Verification record of one output tile (32 bytes, device memory).
+ * The column checksums screen: a tile none of whose columns exceeds its
+ * threshold is clean, and its row checksums are not looked at (the reference
+ * acts on a tile only when a column AND a row checksum disagree,
+ * kernel/ft_sgemm/include/ft_sgemm_huge.cuh:289).  With a flagged column the
+ * rows are thresholded too: one row x one column locates the element. */
 typedef struct hpcdnn_ft_status {
     int32_t flag;             /* 0 clean; 1 single fault located and corrected; 2 detected, not correctable */
     int32_t row, col;         /* tile-local location of the corrected element, -1 if none */
     int32_t n_bad_rows;       /* lines whose |reference - observed| checksum residual exceeded the threshold */
-    int32_t n_bad_cols;
-    float row_residual;       /* signed residual of the located row (the correction that was added), else 0 */
+    int32_t n_bad_cols;       /* (rows are counted only when a column was flagged) */
+    float row_residual;       /* signed residual of the located row (the size of the fault, negated), else 0 */
     float col_residual;       /* signed residual of the located column, else 0 */
-    float max_clean_residual; /* largest |residual| among the lines judged clean */
+    float max_clean_residual; /* largest |residual| among the lines looked at and judged clean */
 } hpcdnn_ft_status;
 
 const char* hpcdnn_version(void);
