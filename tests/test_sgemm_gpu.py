@@ -201,7 +201,8 @@ def test_largest_square_sizes(blas, oracle_mod, n, beta):
     _sampled_check(oracle_mod, blas, n, n, n, 1.0, beta, nrows=24)
 
 
-@pytest.mark.parametrize("M,N,K", [(8192, 8192, 256), (16384, 64, 4096), (128, 128, 65536)])
+@pytest.mark.parametrize("M,N,K", [(8192, 8192, 256), (16384, 64, 4096), (128, 128, 65536), (64, 64, 131072), (40, 52, 200000),
+                                   (192, 192, 65536)])
 def test_skinny_and_deep_shapes(blas, oracle_mod, M, N, K):
     ws = blas.workspace(max(blas.sgemm_workspace_bytes(M, N, K), 4))
     c1 = _sampled_check(oracle_mod, blas, M, N, K, 1.0, 0.0, nrows=16, ws=ws)
