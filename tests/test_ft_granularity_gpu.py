@@ -294,3 +294,40 @@ def test_option_errors(blas):
         blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, granularity=blas.FT_GRAN_WAVE, ws=ws, faults=[(0, 0, 32, 1.0)])
     with pytest.raises(blas.HpcdnnError):
         blas.ft_sgemm(256, 256, 256, t, t, t.clone(), 1.0, 0.0, granularity=2, ws=ws)
+
+
+@pytest.mark.parametrize("mode", ["workspace", "fused"])
+@pytest.mark.parametrize("tile_class", [0, 1, 3])
+def test_columns_screen_and_rows_locate(blas, oracle_mod, mode, tile_class):
+    """The column checksums screen (the reference acts only when a column and a row disagree,
+    ft_sgemm_huge.cuh:289): two faults of 0.75 tau in one ROW show in no column and leave the tile clean, with both
+    faults still in C; the same two faults in one COLUMN add up to 1.5 tau there, are detected and cannot be located
+    (no row passes its threshold); with a verification every 256 k each of them is seen alone and absorbed."""
+    bm, bn = blas.ft_tile(tile_class)
+    M, N, K = 2 * bm + 40, bn + 24, 768
+    a, b, c0 = _problem(oracle_mod, M, N, K, 640 + tile_class)
+    tau, d = 0.05, 0.0375
+    ws = _ws(blas, M, N, K) if mode == "workspace" else None
+    clean, _ = _device_run(blas, a, b, c0, M, N, K, 1.0, 0.0, tau, ws, tile_class=tile_class)
+    tile = 2  # second tile row, first tile column
+    cases = {
+        "one row": ([(tile, 9, 4, d, 0), (tile, 9, 61, d, 1)], 0, (0, 0, 0)),
+        "one column": ([(tile, 9, 4, d, 0), (tile, 33, 4, d, 1)], 0, (2, 0, 1)),
+        "one column, cadence": ([(tile, 9, 4, d, 0), (tile, 33, 4, d, 1)], 256, (0, 0, 0)),
+        "row and column": ([(tile, 9, 4, 4 * d, 0)], 0, (1, 1, 1)),
+    }
+    for name, (faults, interval, want) in cases.items():
+        c, st = _device_run(blas, a, b, c0, M, N, K, 1.0, 0.0, tau, ws, tile_class=tile_class, check_interval=interval, faults=faults)
+        c_model = c0.copy()
+        st_model = oracle_mod.ft_sgemm_checked(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.0, 0.0, bm, bn, tau, interval, faults)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (name, f, st[f], st_model[f])
+        assert (st["flag"][tile], st["n_bad_rows"][tile], st["n_bad_cols"][tile]) == want, name
+        assert np.count_nonzero(st["flag"]) == (1 if want[0] else 0), name
+        if want[0] == 1:
+            assert np.array_equal(c[:, :N], clean[:, :N]), name   # corrected: the bits of the fault-free product
+        else:
+            # not corrected: the faults are still in C, everything else has the fault-free bits
+            diff = np.argwhere(c[:, :N] != clean[:, :N])
+            rows0 = (tile // -(-N // bn)) * bm
+            assert sorted(map(tuple, diff)) == sorted((rows0 + r, col) for (_, r, col, _, _) in faults), name
