@@ -1353,7 +1353,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 if (lr == 0 && line_ct >= 0) atomicMax(&s_meta[8 * line_ct + 4], __float_as_int(half_max));
             }
         };
-        constexpr int kColLines = kColPass, kScreenedRowLines = kRowPass;
         double d_col[LPT_C], d_row[LPT_R];  // this verification's residuals of this thread's lines
         bool rows_done = kWeighted;
         if constexpr (kWeighted) {
@@ -1364,7 +1363,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 tile_abs_sums();
                 __syncthreads();
             }
-            residual_pass(std::integral_constant<int, 0>{}, std::integral_constant<int, kScreenedRowLines>{}, std::false_type{}, d_row, off_row);
+            residual_pass(std::integral_constant<int, 0>{}, std::integral_constant<int, kRowPass>{}, std::false_type{}, d_row, off_row);
             __syncthreads();
         } else {
             publish_col_refs();
@@ -1374,7 +1373,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 tile_abs_sums();
                 __syncthreads();
             }
-            residual_pass(std::integral_constant<int, kRowLines>{}, std::integral_constant<int, kColLines>{}, std::false_type{}, d_col, off_col);
+            residual_pass(std::integral_constant<int, kRowLines>{}, std::integral_constant<int, kColPass>{}, std::false_type{}, d_col, off_col);
             __syncthreads();
             int flagged_cols = 0;
 #pragma unroll
@@ -1384,7 +1383,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 publish_row_refs();
                 observe_rows();
                 __syncthreads();
-                residual_pass(std::integral_constant<int, 0>{}, std::integral_constant<int, kScreenedRowLines>{}, std::true_type{}, d_row, off_row);
+                residual_pass(std::integral_constant<int, 0>{}, std::integral_constant<int, kRowPass>{}, std::true_type{}, d_row, off_row);
                 __syncthreads();
             }
         }
@@ -1446,11 +1445,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         if constexpr (CADENCE) {
             // re-synchronise (ft_sgemm_huge.cuh:268-271): every line that was looked at starts the next interval with
             // what is left of its residual after the correction taken out of its reference
-            constexpr int kColPer = (kColLines + kGemmThreads - 1) / kGemmThreads, kRowPer = (kRowLines + kGemmThreads - 1) / kGemmThreads;
+            constexpr int kColPer = (kColPass + kGemmThreads - 1) / kGemmThreads, kRowPer = (kRowLines + kGemmThreads - 1) / kGemmThreads;
 #pragma unroll
             for (int it = 0; it < kColPer; ++it) {
                 const int cl = tid + it * kGemmThreads;
-                if (cl < kColLines) {
+                if (cl < kColPass) {
                     const int gm = cl / BN, idx = cl - gm * BN;
                     const int ct = gm * GN + idx / CN;
                     double fixed = 0.0;
