@@ -168,7 +168,11 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * sqrt(n) * m, m being the larger of the mean |accumulator| of the line and
  * of the whole tile and f = -tau, or 1 for `tau` == 0, the default (f = 1 is
  * calibrated to twice the largest fault-free residual of uniform operands and
- * follows the data when it is scaled or shifted); `inject` is a HOST
+ * follows the data when it is scaled or shifted; a check tile that is a single
+ * element - the corner of a product ragged in both dimensions - has nothing to
+ * take a scale from but that element, and rounding noise flags about 2 % of
+ * such tiles when the element is small against its terms: the recomputation
+ * then leaves its value unchanged); `inject` is a HOST
  * pointer to one fault or NULL; `status` is DEVICE memory for
  * hpcdnn_ft_num_tiles(M,N) records or NULL.
  * `ws`/`ws_bytes`: optional DEVICE scratch of
@@ -266,7 +270,7 @@ int hpcdnn_ft_tile_info(int tile_class, int* bm, int* bn);
  * residual d1 exceeds the threshold is faulty, and with one fault delta in
  * column n of it the residuals are d1 = -delta, d2 = -(n + 1) delta, so the
  * column is round(d2 / d1) - 1.  One faulty row: that element is computed
- * again; if that changed it by d1 (to within the row's threshold) the fault is
+ * again; if that changed it by d1 (to within the row's threshold + 2^-20 |d1|) the fault is
  * located and corrected (flag 1, n_bad_cols = 1), else - two faults in the
  * row, or a fault too small against the rounding noise of the weighted sums,
  * which is about 0.6 x the tile's width x that of the plain sums - the tile

@@ -520,7 +520,7 @@ typedef struct {
  * whose plain residual d1 exceeds its threshold is faulty; with one fault delta in column n its residuals are
  * d1 = -delta, d2 = -(n + 1) delta, so the column is round(d2 / d1) - 1 (clamped into the tile).  One faulty row: that
  * element is computed again (oracle_recompute_element); the location is confirmed when that changed the element by d1
- * to within the row's threshold -> flag 1, n_bad_cols 1, row/col set, row_residual = d1, col_residual = d2.  Not
+ * to within the row's threshold + 2^-20 |d1| -> flag 1, n_bad_cols 1, row/col set, row_residual = d1, col_residual = d2.  Not
  * confirmed (two faults in the row, or a fault lost in the rounding of the weighted sums) or more faulty rows ->
  * flag 2, n_bad_cols 0.  Computing a healthy element again changes nothing, so a wrong column does no harm.
  * tau as for oracle_ft_sgemm; every fault is added before the one verification. */
@@ -594,7 +594,9 @@ void oracle_ft_sgemm_weighted(int M, int N, int K, const float* A, int lda, cons
             float again = oracle_recompute_element(0, K, A + (size_t)(m0 + r) * lda, B + n0 + c, ldb);
             float change = again - *e;
             *e = again;
-            if (fabsf(change - f1) <= (float)thr[r]) {
+            /* (the row's threshold plus sixteen rounding units of the residual: the observed sums of a row that
+             * holds a fault of thousands of thresholds are themselves only good to a few units of its size) */
+            if (fabsf(change - f1) <= (float)thr[r] + 0x1p-20f * fabsf(f1)) {
                 st.flag = 1; st.n_bad_cols = 1; st.row = r; st.col = c;
                 st.row_residual = f1; st.col_residual = f2;
             } else {

@@ -167,3 +167,26 @@ def test_option_errors(blas):
     status = blas.ft_status_alloc(256, 256)
     blas.ft_sgemm(256, 256, 0, t[:, :0], t[:0, :], c, 1.0, 0.5, locator=blas.FT_LOCATE_WEIGHTED, status=status)
     assert torch.equal(c, torch.full((256, 256), 1.0, device="cuda")) and not blas.ft_status_numpy(status)["flag"].any()
+
+
+@pytest.mark.parametrize("M,N,K,tile_class,fault", [(512, 300, 7, 3, (17, 65, 7, 2540.80859375)), (31, 200, 33, 3, (2, 17, 50, -2940.299072265625)),
+                                                     (300, 64, 64, 4, (4, 0, 33, -712.3224487304688))])
+def test_fault_of_millions_of_thresholds_is_still_confirmed(blas, oracle_mod, M, N, K, tile_class, fault):
+    """A fault ten million times the threshold: the observed row sums that contain it are good to a few rounding units
+    of ITS size only, far more than the threshold, so the confirmation allows 2^-20 of the residual on top of the
+    threshold (found by a randomized sweep: device and model used to disagree on these)."""
+    a = oracle_mod.fill_uniform_matrix(M, K, 9001, ld=K)
+    b = oracle_mod.fill_uniform_matrix(K, N, 9002, ld=N)
+    c0 = np.zeros((M, N), np.float32)
+    tau = blas.ft_default_tau(K)
+    assert abs(fault[3]) > 1e6 * tau
+    bm, bn = blas.ft_tile(tile_class)
+    ws = _ws(blas, M, N, K, tile_class=tile_class)
+    clean, _ = _run(blas, a, b, c0, M, N, K, 1.0, 0.0, tau, ws, tile_class, None)
+    c, st = _run(blas, a, b, c0, M, N, K, 1.0, 0.0, tau, ws, tile_class, [fault])
+    c_model = c0.copy()
+    st_model = oracle_mod.ft_sgemm_weighted(M, N, K, a, K, b, N, c_model, N, 1.0, 0.0, bm, bn, tau, [fault])
+    for f in DECISION_FIELDS:
+        assert np.array_equal(st[f], st_model[f]), (f, st[f], st_model[f])
+    assert st["flag"][fault[0]] == 1 and (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3]
+    assert np.array_equal(c, clean)
