@@ -3,6 +3,9 @@
 
 namespace hpcdnn {
 
+// the pre-pass runs blocks over 64 values of k instead of 256 while the latter would be fewer than this (two per CU)
+constexpr int kEncodeFineBelow = 512;
+
 // row length of the pre-encoded checksum vectors: K rounded up to the K step, plus two K steps of zeros for the
 // fetches that run ahead of the main loop
 static int ft_enc_ld(int K) { return (static_cast<int>(ceil_div(K, kGemmBK)) + 2) * kGemmBK; }
@@ -41,18 +44,18 @@ static FtKernel ft_kernel(int tile_class, bool ta, int kind) {
         default: return FtKernel{nullptr, nullptr, 0, 0};
     }
 }
-static EncodeFn ft_encode(int tile_class, bool ta, bool wave) {
+static EncodeFn ft_encode(int tile_class, bool ta, bool wave, bool fine) {
     switch (tile_class * 2 + (ta ? 1 : 0)) {
-        case 0: return ft_encode_c0_ta0(wave);
-        case 1: return ft_encode_c0_ta1(wave);
-        case 2: return ft_encode_c1_ta0(wave);
-        case 3: return ft_encode_c1_ta1(wave);
-        case 4: return ft_encode_c2_ta0(wave);
-        case 5: return ft_encode_c2_ta1(wave);
-        case 6: return ft_encode_c3_ta0(wave);
-        case 7: return ft_encode_c3_ta1(wave);
-        case 8: return ft_encode_c4_ta0(wave);
-        case 9: return ft_encode_c4_ta1(wave);
+        case 0: return ft_encode_c0_ta0(wave, fine);
+        case 1: return ft_encode_c0_ta1(wave, fine);
+        case 2: return ft_encode_c1_ta0(wave, fine);
+        case 3: return ft_encode_c1_ta1(wave, fine);
+        case 4: return ft_encode_c2_ta0(wave, fine);
+        case 5: return ft_encode_c2_ta1(wave, fine);
+        case 6: return ft_encode_c3_ta0(wave, fine);
+        case 7: return ft_encode_c3_ta1(wave, fine);
+        case 8: return ft_encode_c4_ta0(wave, fine);
+        case 9: return ft_encode_c4_ta1(wave, fine);
         default: return nullptr;
     }
 }
@@ -260,7 +263,7 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         float* enc_b = enc_a + static_cast<size_t>(row_groups) * a.enc_ld;
         a.enc_a = enc_a;
         a.enc_b = enc_b;
-        const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
+        int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
         const int b_blocks = static_cast<int>(ceil_div(N, 128));  // the pre-pass walks B in blocks of 128 columns
         // (ta: the same launch, with the blocks of the A half walking A^T)
         if (weighted) {
@@ -275,9 +278,12 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
                 abft_encode_weighted_kernel<64><<<dim3(k_blocks * b_blocks), dim3(1024), 0, s>>>(N, K, B, ldb, wb, wb + static_cast<size_t>(col_groups) * a.enc_ld,
                                                                                             a.enc_ld, k_blocks, col_groups);
         } else {
-            const EncodeFn encode = ft_encode(opt.tile_class, ta, wave);
+            const bool fine = k_blocks * (row_groups + b_blocks) < kEncodeFineBelow;
+            const int kb = fine ? 64 : 256;
+            k_blocks = static_cast<int>(ceil_div(a.enc_ld, kb));
+            const EncodeFn encode = ft_encode(opt.tile_class, ta, wave, fine);
             if (!encode) return HPCDNN_ERR_INVALID_VALUE;
-            hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(1024), 0, s, M, N, K,
+            hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(kb * 4), 0, s, M, N, K,
                                A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
         }
         rc = launch_status();

@@ -1734,42 +1734,44 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, 
 }
 
 // ---- ABFT pre-encode: the checksum vectors of the operands, one per row group (RM rows) / column group (CN
-// columns), in one launch of 1024-thread blocks that each cover 256 values of k: the first k_blocks * row_groups
-// blocks encode A, the rest B (one block per 128 columns of B, i.e. 128 / CN column groups).  A group is a workgroup tile's
-// rows or columns, or a wave tile's with wave-tile checksums.
+// columns), in one launch of blocks of 4 KB threads that each cover KB values of k (256, or 64 for operands so small
+// that blocks of 256 would leave most CUs idle; the sums are the same, bit for bit): the first k_blocks * row_groups
+// blocks encode A, the rest B (one block per 128 columns of B, i.e. 128 / CN column groups).  A group is a workgroup
+// tile's rows or columns, or a wave tile's with wave-tile checksums.
 //
 // enc_a[g][k'] = sum over the rows m of row group g (m < M) of A[m][k]; zero for K <= k < enc_ld; k' is k with
-// the order inside each group of 16 changed to 0, 8, 1, 9, ...  Lane q of a wave owns 4 consecutive k, wave w (16
-// of them) owns RM / 16 of the group's rows; the 16 partials are added in wave order, so the result does not depend
-// on timing.
+// the order inside each group of 16 changed to 0, 8, 1, 9, ...  A thread owns 4 consecutive k and the RM / 16 rows of
+// one of 16 row slices (a wave per slice with KB = 256, a quarter wave with KB = 64); the 16 partials are added in
+// slice order, so the result does not depend on timing.
 //
 // enc_b[g][k] = sum over the columns n of column group g (n < N) of B[k][n]; zero for K <= k < enc_ld.  A half
-// wave reads 128 columns of one k row (32 lanes x 4 columns) and owns 8 of the block's 256 rows; CN / 4 neighbouring
+// wave reads 128 columns of one k row (32 lanes x 4 columns) and owns 8 of the block's KB rows; CN / 4 neighbouring
 // lanes share a column group.
 //
 // TA: A is given transposed (K rows of M floats, row length lda).  A row then holds a group's RM values side by side:
 // the 16 lanes of a DPP row read them 16 at a time (64 contiguous bytes; the four rows of a wave four different k) and
-// add their partial sums across the row; a block covers 256 values of k of one row group, 64 per pass.
-template <int RM, int CN, bool TA = false>
-__global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
-                                                           const float* __restrict__ B, int ldb,
-                                                           float* __restrict__ enc_a, float* __restrict__ enc_b,
-                                                           int enc_ld, int k_blocks, int row_groups, int col_groups) {
+// add their partial sums across the row; a block covers KB values of k of one row group, KB / 4 per pass.
+template <int RM, int CN, bool TA = false, int KB = 256>
+__global__ __launch_bounds__(KB * 4) void abft_encode_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
+                                                             const float* __restrict__ B, int ldb,
+                                                             float* __restrict__ enc_a, float* __restrict__ enc_b,
+                                                             int enc_ld, int k_blocks, int row_groups, int col_groups) {
     static_assert(CN == 128 || CN == 64 || CN == 32, "column groups are 8, 16 or 32 lanes of a half wave");
-    static_assert(RM % 16 == 0, "the rows of a group split evenly over 16 waves");
-    constexpr int kWaves = 16, kRows = RM / kWaves;
-    constexpr int kHalves = 2 * kWaves, kRowsPerHalf = 256 / kHalves;
+    static_assert(RM % 16 == 0, "the rows of a group split evenly over 16 slices");
+    static_assert(KB == 256 || KB == 64, "a row slice is a wave or a quarter of one");
+    constexpr int kSlices = 16, kRows = RM / kSlices, kSliceLanes = KB / 4;
+    constexpr int kHalves = KB / 8, kRowsPerHalf = KB / kHalves;
     constexpr int kGroupLanes = CN / 4, kGroupsPer128 = 128 / CN;
     static_assert(kRowsPerHalf <= kGroupLanes, "every k row of a half wave has a lane of each group to write it");
-    __shared__ v4f part[kWaves][kWave];
+    __shared__ v4f part[kSlices][kSliceLanes];
     const int a_blocks = k_blocks * row_groups;
     if (TA && static_cast<int>(blockIdx.x) < a_blocks) {
         static_assert(RM % 16 == 0, "a row group is read 16 values at a time");
-        const int l16 = threadIdx.x & 15, krow = threadIdx.x >> 4;  // 64 rows of k per pass
+        const int l16 = threadIdx.x & 15, krow = threadIdx.x >> 4;  // KB / 4 rows of k per pass
         const int group = blockIdx.x / k_blocks, m0 = group * RM;
 #pragma unroll
         for (int pass = 0; pass < 4; ++pass) {
-            const int k = (blockIdx.x % k_blocks) * 256 + pass * 64 + krow;
+            const int k = (blockIdx.x % k_blocks) * KB + pass * (KB / 4) + krow;
             float t = 0.f;
             if (k < K) {
                 const float* row = A + static_cast<int64_t>(k) * lda + m0;
@@ -1786,9 +1788,9 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
             }
         }
     } else if (static_cast<int>(blockIdx.x) < a_blocks) {
-        const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+        const int lane = threadIdx.x % kSliceLanes, slice = threadIdx.x / kSliceLanes;
         const int group = blockIdx.x / k_blocks, m0 = group * RM;
-        const int k = ((blockIdx.x % k_blocks) * kWave + lane) * 4;
+        const int k = ((blockIdx.x % k_blocks) * kSliceLanes + lane) * 4;
         const float* base = A + static_cast<int64_t>(m0) * lda;
         // a group past the last row (the lower wave tiles of an edge tile) reads nothing and is all zeros
         const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base, m0 < M ? (static_cast<int64_t>(M - 1 - m0) * lda + K) * 4 : 0);
@@ -1796,7 +1798,7 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
         if (k < K && m0 < M) {
             v4f v[kRows];
 #pragma unroll
-            for (int r = 0; r < kRows; ++r) v[r] = buffer_load_v4f(rsrc, ((wave * kRows + r) * lda + k) * 4);
+            for (int r = 0; r < kRows; ++r) v[r] = buffer_load_v4f(rsrc, ((slice * kRows + r) * lda + k) * 4);
 #pragma unroll
             for (int r = 0; r < kRows; ++r) s += v[r];
             // the group's tail beyond K holds the next row's first elements
@@ -1804,12 +1806,12 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
             s.z = (k + 2 < K) ? s.z : 0.f;
             s.w = (k + 3 < K) ? s.w : 0.f;
         }
-        part[wave][lane] = s;
+        part[slice][lane] = s;
         __syncthreads();
-        if (wave == 0 && k < enc_ld) {
+        if (slice == 0 && k < enc_ld) {
             v4f t = part[0][lane];
 #pragma unroll
-            for (int w = 1; w < kWaves; ++w) t += part[w][lane];
+            for (int w = 1; w < kSlices; ++w) t += part[w][lane];
             // within each K step of 16, k and k + 8 sit side by side: the GEMM thread that stages rows k and
             // k + 8 of the B tile fetches both with one 8-byte load
             float* dst = enc_a + static_cast<int64_t>(group) * enc_ld + (k & ~15);
@@ -1823,7 +1825,7 @@ __global__ __launch_bounds__(1024) void abft_encode_kernel(int M, int N, int K, 
         const int bid = blockIdx.x - a_blocks;
         const int lr = threadIdx.x & 31, half = threadIdx.x >> 5;
         const int tile_n = bid / k_blocks, n0 = tile_n * 128;
-        const int kb = (bid % k_blocks) * 256;
+        const int kb = (bid % k_blocks) * KB;
         float s[kRowsPerHalf];
         v4f v[kRowsPerHalf];
 #pragma unroll

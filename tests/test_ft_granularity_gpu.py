@@ -87,6 +87,29 @@ def test_wave_tiles_decisions_equal_the_model(blas, oracle_mod, tile_class, tau_
         _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 1.0)
 
 
+@pytest.mark.parametrize("tile_class,granularity", [(4, 1), (2, 0)])
+def test_long_k_takes_the_pre_pass_with_blocks_over_256_values_of_k(blas, oracle_mod, tile_class, granularity):
+    """The pre-pass covers 64 values of k per block on small operands and 256 once that gives 512 blocks or more; the
+    other tests here are all of the first kind.  34 row groups and 2 blocks of 128 columns, times 16 blocks of k."""
+    cm, cn = blas.ft_check_tile(tile_class, granularity)
+    M, N, K = 17 * (64 if granularity else 128) - 3, 250, 3900
+    bm, _ = blas.ft_tile(tile_class)
+    assert -(-(K + 32) // 256) * (-(-M // bm) * (bm // cm) + -(-N // 128)) >= 512
+    tau = blas.ft_default_tau(K)
+    ntn = -(-N // cn)
+    a, b, c0 = _problem(oracle_mod, M, N, K, 4100 + tile_class)
+    fault = (5 * ntn + 1, 7, 9, -2.5)
+    c, st = _device_run(blas, a, b, c0, M, N, K, 1.0, 1.0, tau, _ws(blas, M, N, K), tile_class=tile_class, granularity=granularity,
+                        fault=fault)
+    c_model = c0.copy()
+    st_model = oracle_mod.ft_sgemm(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.0, 1.0, cm, cn, tau, fault)
+    for f in DECISION_FIELDS:
+        assert np.array_equal(st[f], st_model[f]), (f, st[f], st_model[f])
+    assert np.count_nonzero(st["flag"]) == 1 and (st["row"][fault[0]], st["col"][fault[0]]) == fault[1:3]
+    assert st["max_clean_residual"].max() < 0.6 * tau
+    _assert_values(oracle_mod, M, N, K, a, b, c0, c, 1.0, 1.0)
+
+
 def test_two_faults_in_one_workgroup_tile_need_wave_granularity(blas, oracle_mod):
     """Two simultaneous faults in different wave tiles of one 256 x 128 tile: tile granularity sees two bad rows and two
     bad columns and reports the tile uncorrectable; wave-tile granularity corrects both."""

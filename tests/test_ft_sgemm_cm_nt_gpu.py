@@ -139,6 +139,17 @@ def test_other_classes_granularity_and_cadence(blas, oracle_mod):
         assert st["flag"][0] == 1 and (st["row"][0], st["col"][0]) == (3, 4)
 
 
+def test_long_k_takes_the_pre_pass_with_blocks_over_256_values_of_k(blas, oracle_mod):
+    """The pre-pass walks 64 values of k per block on small operands and 256 once that gives 512 blocks or more: here
+    34 row groups (wave tiles of the 64 x 64 class over the 1085 rows of C^T) and 2 blocks of 128 columns, 16 blocks of k."""
+    M, N, K = 250, 1085, 3900
+    tau = blas.ft_default_tau(K)
+    *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 1.0, tau, faults=[(41, 3, 4, 2.0)], pad=(4, 8, 4), tile_class=4,
+                     granularity=blas.FT_GRAN_WAVE)
+    assert np.count_nonzero(st["flag"]) == 1 and st["flag"][41] == 1 and (st["row"][41], st["col"][41]) == (3, 4)
+    assert st["max_clean_residual"].max() < 0.6 * tau
+
+
 @pytest.mark.parametrize("tile_class", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("kind", ["tile-fused", "tile-workspace", "wave-workspace"])
 def test_every_class_granularity_and_cadence_equals_the_model(blas, oracle_mod, tile_class, kind):
