@@ -48,6 +48,7 @@ EXPORTS = (
     "hpcdnn_ft_tile_info",
     "hpcdnn_ft_num_tiles_ex",
     "hpcdnn_ft_pick_class",
+    "hpcdnn_ft_pick_class_ws",
     "hpcdnn_ft_default_tau",
     "hpcdnn_sgemv",
     "hpcdnn_offline_ft_sgemm",
@@ -149,6 +150,8 @@ def lib():
     L.hpcdnn_ft_num_tiles_ex.argtypes = [i, i, i]
     L.hpcdnn_ft_pick_class.restype = i
     L.hpcdnn_ft_pick_class.argtypes = [i, i, i]
+    L.hpcdnn_ft_pick_class_ws.restype = i
+    L.hpcdnn_ft_pick_class_ws.argtypes = [i, i, i, C.c_size_t]
     L.hpcdnn_ft_num_tiles.restype = i
     L.hpcdnn_ft_num_tiles.argtypes = [i, i]
     L.hpcdnn_ft_default_tau.restype = f

@@ -305,8 +305,12 @@ def ft_tile(tile_class: int = 0):
     return bm.value, bn.value
 
 
-def ft_pick_class(M: int, N: int, K: int) -> int:
-    return int(_lib.lib().hpcdnn_ft_pick_class(M, N, K))
+def ft_pick_class(M: int, N: int, K: int, ws_bytes: int | None = None) -> int:
+    """The tile class with the shortest predicted run: for a call with the full workspace, or with one of ``ws_bytes``
+    (0: none)."""
+    if ws_bytes is None:
+        return int(_lib.lib().hpcdnn_ft_pick_class(M, N, K))
+    return int(_lib.lib().hpcdnn_ft_pick_class_ws(M, N, K, ws_bytes))
 
 
 def ft_default_tau(K: int) -> float:

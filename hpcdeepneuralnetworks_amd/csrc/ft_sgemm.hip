@@ -352,16 +352,20 @@ extern "C" int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N) {
 
 extern "C" int hpcdnn_ft_num_tiles(int M, int N) { return hpcdnn_ft_num_tiles_ex(0, M, N); }
 
-// The class with the shortest predicted run (workspace variant).  Matrix-core time: rounds of tiles over the CUs
-// times the tile's flops, a partial last round counting for what its K split leaves of it plus the second pass over
-// those tiles, with the measured efficiency of the smaller tiles relative to the 256-row one.  An operand that is
-// read once cannot arrive faster than the bytes in flight allow (two K steps of the tile's rows per resident
-// workgroup and trip to memory), which is what decides between the classes on tall products with few columns.
-extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
+// The class with the shortest predicted run of a call that passes a workspace of ws_bytes (0: none).  Matrix-core
+// time: rounds of tiles over the CUs times the tile's flops, a partial last round counting for what its K split leaves
+// of it plus the second pass over those tiles (when the workspace has room for the split), with the measured
+// efficiency of the smaller tiles relative to the 256-row one.  An operand that is read once cannot arrive faster
+// than the bytes in flight allow (two K steps of the tile's rows per resident workgroup and trip to memory), which is
+// what decides between the classes on tall products with few columns.
+extern "C" int hpcdnn_ft_pick_class_ws(int M, int N, int K, size_t ws_bytes) {
     // measured on squares 1024 ... 6144: the 128-row class keeps up with the 256-row one (two of its workgroups share a CU
     // and cover each other's verification), the 64-row class runs 4-5 % behind; the 64-column classes move twice the
     // operand bytes per flop and only pay where the 128-column ones would multiply empty columns
     static const double rel_eff[HPCDNN_FT_NUM_CLASSES] = {1.0, 1.0, 0.955, 0.92, 0.88};
+    // without the pre-pass every workgroup forms the checksum vectors of its own tile in the main loop: additions per
+    // product grow as 1 / BM + 1 / BN (measured at 4096 and 2048 cubed)
+    static const double rel_eff_fused[HPCDNN_FT_NUM_CLASSES] = {1.0, 0.985, 0.91, 0.90, 0.78};
     static const int resident_max[HPCDNN_FT_NUM_CLASSES] = {1, 2, 2, 2, 3};  // workgroups of the class a CU holds
     constexpr double kPeakFlopsPerCu = 157.3e12 / 256.0, kTrip = 0.73e-6;
     const int cus = device_cus();
@@ -370,14 +374,26 @@ extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
     for (int c = 0; c < HPCDNN_FT_NUM_CLASSES; ++c) {
         const FtClass& fc = kFtClasses[c];
         const int64_t tiles = hpcdnn_ft_num_tiles_ex(c, M, N);
-        const FtTail tail = ft_tail_plan(fc, M, N, K);
+        const int tiles_m = static_cast<int>(ceil_div(M, fc.bm)), tiles_n = static_cast<int>(ceil_div(N, fc.bn));
+        // as run_ft_sgemm decides: a product one tile wide or high splits every tile and forms the vectors in the loop
+        const bool one_wide = K > 0 && (tiles_m == 1 || tiles_n == 1) && tiles >= cus / 8;
+        const size_t enc_bytes = ft_enc_bytes(fc, HPCDNN_FT_GRAN_TILE, M, N, K);
+        const bool pre = !one_wide && K > 0 && ws_bytes >= enc_bytes;
+        FtTail tail{1, 0, 0};
+        if (one_wide) {
+            tail = ft_split_all_plan(static_cast<int>(tiles), K, kGemmBK);
+            if (ws_bytes < ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, tail)) tail = FtTail{1, 0, 0};
+        } else if (pre) {
+            tail = ft_tail_plan(fc, M, N, K);
+            if (ws_bytes < enc_bytes + ft_tail_bytes(fc, HPCDNN_FT_GRAN_TILE, tail)) tail = FtTail{1, 0, 0};
+        }
         double rounds = static_cast<double>(ceil_div(tiles > 0 ? tiles : 1, cus));
         int64_t groups = tiles;  // workgroups of the launch
         if (tail.ways >= 2) {
-            rounds = static_cast<double>(tiles / cus) + static_cast<double>(ceil_div(static_cast<int64_t>(tail.tiles) * tail.ways, cus)) / tail.ways + 0.06;
+            rounds = static_cast<double>((tiles - tail.tiles) / cus) + static_cast<double>(ceil_div(static_cast<int64_t>(tail.tiles) * tail.ways, cus)) / tail.ways + 0.06;
             groups = tiles - tail.tiles + static_cast<int64_t>(tail.tiles) * tail.ways;
         }
-        double cost = rounds * 2.0 * fc.bm * fc.bn * (K > 0 ? K : 1) / kPeakFlopsPerCu / rel_eff[c];
+        double cost = rounds * 2.0 * fc.bm * fc.bn * (K > 0 ? K : 1) / kPeakFlopsPerCu / (pre ? rel_eff[c] : rel_eff_fused[c]);
         const double busy = static_cast<double>(groups < cus ? groups : cus);
         double resident = static_cast<double>(ceil_div(groups > 0 ? groups : 1, cus));
         if (resident > resident_max[c]) resident = resident_max[c];
@@ -390,6 +406,9 @@ extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) {
     }
     return best;
 }
+
+// (a workspace of hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM, ...) or more)
+extern "C" int hpcdnn_ft_pick_class(int M, int N, int K) { return hpcdnn_ft_pick_class_ws(M, N, K, ~static_cast<size_t>(0)); }
 
 // Fault-free residuals are the FP32 rounding of the accumulators added over a tile line; for operands uniform in
 // [-1, 1] their maximum over a whole matrix grows linearly with K (measured 4.0e-7 ... 4.9e-7 per unit of K from

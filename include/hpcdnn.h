@@ -332,6 +332,13 @@ int hpcdnn_ft_check_tile_info(int tile_class, int granularity, int* cm, int* cn)
 int hpcdnn_ft_num_check_tiles(int tile_class, int granularity, int M, int N);
 int hpcdnn_ft_num_tiles_ex(int tile_class, int M, int N);
 int hpcdnn_ft_pick_class(int M, int N, int K);
+/* The same for a call that passes a workspace of `ws_bytes` (0: none, the
+ * checksum vectors are then formed in the main loop and no tile can be split
+ * along K, which favours other classes: at 3072^3 without a workspace the
+ * 64x128 class runs 10 % ahead of the 128x128 one that the workspace variant
+ * takes).  The status records are those of the class returned.  No counterpart
+ * in the reference, which picks its kernel by name. */
+int hpcdnn_ft_pick_class_ws(int M, int N, int K, size_t ws_bytes);
 /* An absolute threshold for operands uniform in [-1, 1], to be passed as
  * `tau`: 1.1e-6 * max(K, 64), twice the largest fault-free residual measured
  * for such operands (the rounding noise of the FP32 accumulators grows

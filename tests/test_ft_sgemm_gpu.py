@@ -240,6 +240,15 @@ def test_pick_class_and_bad_class(blas):
     assert blas.ft_pick_class(3072, 3072, 3072) in (0, 1)  # either class ends its partial round with a K split
     assert blas.ft_pick_class(3072, 3072, 128) in (2, 4)  # too short a K to split: small tiles fill the rounds best
     assert blas.ft_pick_class(16384, 64, 4096) == 3       # 64 columns: the 128-column classes would multiply empty ones
+    # without a workspace no round can end in a K split, and the vectors formed in the loop cost the small tiles more
+    assert blas.ft_pick_class(4096, 4096, 4096, ws_bytes=0) == 0
+    assert blas.ft_pick_class(3072, 3072, 3072, ws_bytes=0) == 2   # 4.5 rounds of 64x128 against 2.25 of 128x128
+    assert blas.ft_pick_class(2560, 2560, 2560, ws_bytes=0) == 0   # 200 tiles of 256x128: one round
+    assert blas.ft_pick_class(1536, 1536, 1536, ws_bytes=0) == 4
+    assert blas.ft_pick_class(2048, 2048, 1024, ws_bytes=0) == 1
+    assert blas.ft_pick_class(16384, 64, 4096, ws_bytes=0) == 4    # 256 tiles of 64x64, none split
+    for shape in [(4096, 4096, 4096), (3072, 3072, 3072), (16384, 64, 4096), (1000, 1000, 1000)]:
+        assert blas.ft_pick_class(*shape, ws_bytes=blas.ft_workspace_bytes(*shape)) == blas.ft_pick_class(*shape)
     t = torch.zeros(64, 64, device="cuda")
     with pytest.raises(blas.HpcdnnError):
         blas.ft_sgemm(64, 64, 64, t, t, t.clone(), 1.0, 0.0, tile_class=5)
