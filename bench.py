@@ -471,7 +471,7 @@ def main() -> int:
 
         # ---- ABFT overhead across the square sweep (workspace variant, the tile class the library suggests)
         sweep = {}
-        for m in (2048, 3072, 5120, 6144):
+        for m in (2048, 3001, 3072, 5120, 6000, 6144):  # (3001, 6000: ragged tiles on the last tile row and column)
             a, b, c = operands(m, m, m, 26)
             cls = blas.ft_pick_class(m, m, m)
             status_s = blas.ft_status_alloc(m, m, tile_class=cls)

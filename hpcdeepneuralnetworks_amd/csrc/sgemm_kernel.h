@@ -264,6 +264,12 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // stored), so those steps run with unbounded descriptors and plain pointer steps; the byte counts that the range
     // checks need are formed only for the steps at the end of the slice.
     constexpr bool kLazyBounds = EDGE && FT == 0;
+    // ABFT with checksum vectors from the workspace, ragged tiles: the staged columns n >= N of B (TA: m >= M of A^T)
+    // hold the next row or padding.  The vectors cover the matrix only, so that data reaches nothing but the
+    // accumulators and reference sums of lines outside the matrix, which the verification sets to zero first; the K
+    // steps then need no masks but the last two of a slice.  (The kernels that form the vectors in the loop sum the
+    // staged data itself and keep the masks.)
+    constexpr bool kLazyOutside = EDGE && FT >= 2;
 
     extern __shared__ __align__(16) float smem[];
     float* const As = smem;
@@ -1031,8 +1037,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             if constexpr (EDGE && FT != 0) {
                 // ABFT on a ragged problem: a tile that does not hang over the last column needs the masks only where
                 // plain SGEMM does, in the slice's last two K steps (its checksums want zeros in columns k >= kend of
-                // A and rows k >= kend of B; the columns n >= N that the other steps would have to clear do not exist)
-                if (n0 + BN <= p.N && (!TA || m0 + BM <= p.M)) {
+                // A and rows k >= kend of B; the columns n >= N that the other steps would have to clear do not exist).
+                // With pre-encoded vectors a tile that does hang over runs the same way: what its columns n >= N (TA:
+                // rows m >= M) pick up reaches only their own accumulators and reference sums, and the verification
+                // clears those before it looks at anything (kLazyOutside).
+                if (kLazyOutside || (n0 + BN <= p.N && (!TA || m0 + BM <= p.M))) {
                     for (; kt + 3 < nkt; kt += 2) {
                         step(S1{}, S0{}, std::false_type{}, std::false_type{}, std::false_type{});
                         flush_now = (kt & 14) == 14;
@@ -1135,6 +1144,39 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         // verifies once per slice takes the test faults into the tile's first slice, a cadence kernel, whose slices
         // start on a multiple of the interval, into the slice and interval that verification number `check` of the
         // whole K range falls into)
+        if constexpr (kLazyOutside) {
+            if (n0 + BN > p.N) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const bool inside = n0 + wn * WN + j * 32 + lr < p.N;
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[i][j][v] = inside ? acc[i][j][v] : 0.f;
+                }
+#pragma unroll
+                for (int gm = 0; gm < GM; ++gm)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) cc_ref[gm][e] = e < b_nvalid[0] ? cc_ref[gm][e] : 0.0;
+            }
+            if (TA && m0 + BM > p.M) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const bool inside = m0 + wm * WM + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3) < p.M;
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) acc[i][j][v] = inside ? acc[i][j][v] : 0.f;
+                    }
+#pragma unroll
+                for (int sl = 0; sl < A_SLOTS; ++sl) {
+                    const bool inside = m0 + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl < p.M;
+#pragma unroll
+                    for (int gn = 0; gn < GN; ++gn) cr_ref[gn][sl] = inside ? cr_ref[gn][sl] : 0.0;
+                    crw_ref[sl] = inside ? crw_ref[sl] : 0.0;
+                }
+            }
+        }
         const int check_global = CADENCE ? k_first / p.check_interval + check : 0;
 #pragma unroll 1
         for (int f = 0; f < p.n_faults; ++f)
