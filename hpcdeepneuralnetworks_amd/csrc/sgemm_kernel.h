@@ -1064,6 +1064,76 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     if constexpr (FT == 0) {
         run_k_range();
     } else {
+    // the tile's epilogue as a function: these kernels call it before or after their last verification (early_store)
+    auto store_c = [&]() __attribute__((always_inline)) {
+        const int row_base = m0 + wm * WM + lh * 4;  // + i*32 + 8*(v/4) + v%4
+        const int col_base = n0 + wn * WN + lr;      // + j*32
+        // C = alpha*acc + beta*C.  With beta != 0 the 16 old values of a 32x32 block are fetched together before the
+        // first store, so that their latencies overlap instead of queueing behind each other.
+        // Tiles of at most 128x128 store C with the streaming hint: many small workgroups finish close together, and
+        // keeping their output out of the L2 leaves it to the operand panels (1 to 2 % on 1024^3, 2048^3, 4096x4096x256;
+        // the 256x128 tiles measured 0.2 % slower with it and keep the plain store).
+        constexpr bool kStreamC = BM * BN <= 128 * 128;
+        const float alpha = p.alpha, beta = p.beta;
+        if constexpr (EDGE) {
+            // Ragged tiles: a buffer descriptor from the tile's corner to the last element of C inside the tile, so the
+            // hardware drops stores to rows >= M (and returns 0 for loads there); the row offset has to be part of the
+            // vector offset for that (a scalar offset is not range-checked).  Columns >= N would land in the next row:
+            // they are switched off once per block column.  A compare, a branch and a 64-bit multiply per store, which
+            // is what the pointer form compiles to, cost a 64x64 tile 3200 cycles here.
+            const int64_t c_bytes = (static_cast<int64_t>(p.M - 1 - m0) * p.ldc + (p.N - n0)) * 4;
+            const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.C + static_cast<int64_t>(m0) * p.ldc + n0, c_bytes);
+            const int ldc_bytes = p.ldc * 4;  // BM * ldc * 4 < 2^31 (host check)
+            const int lane_off = (wm * WM + lh * 4) * ldc_bytes + (wn * WN + lr) * 4;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if (col_base + j * 32 >= p.N) continue;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    float old[16];
+                    if (beta != 0.f) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            old[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                         c_rsrc, lane_off + j * 128 + (i * 32 + 8 * (v / 4) + (v % 4)) * ldc_bytes, 0, 0));
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const float t = alpha * acc[i][j][v];
+                        const float out = (beta == 0.f) ? t : __builtin_fmaf(beta, old[v], t);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), c_rsrc,
+                                                              lane_off + j * 128 + (i * 32 + 8 * (v / 4) + (v % 4)) * ldc_bytes, 0,
+                                                              kStreamC ? 2 : 0);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int col = col_base + j * 32;
+                float* cbase = p.C + static_cast<size_t>(row_base + i * 32) * p.ldc + col;
+                float old[16];
+                if (beta != 0.f) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int r = 8 * (v / 4) + (v % 4);
+                        old[v] = cbase[static_cast<size_t>(r) * p.ldc];
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = 8 * (v / 4) + (v % 4);
+                    const float t = alpha * acc[i][j][v];
+                    const float out = (beta == 0.f) ? t : __builtin_fmaf(beta, old[v], t);
+                    if constexpr (kStreamC) __builtin_nontemporal_store(out, &cbase[static_cast<size_t>(r) * p.ldc]);
+                    else cbase[static_cast<size_t>(r) * p.ldc] = out;
+                }
+            }
+        }
+    };
+
     // ---- ABFT verification: inject (testing aid), observe, compare, locate, correct, re-synchronise
     constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;   // partials per column / per row checksum
     constexpr int NCT = GM * GN;                          // check tiles per workgroup tile
@@ -1082,6 +1152,12 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
     for (int it = 0; it < LPT_R; ++it) off_row[it] = 0.0;
     const int k_first = kbeg;      // first k of this workgroup's K range (kbeg moves on from interval to interval)
+    // With beta == 0 the tile goes to C before its (last) verification instead of after it, so that the stores are on
+    // their way while the checksums are compared; a located element is then written a second time, by its owner, with
+    // the value computed again.  (With beta != 0 the old value of C that the corrected element needs is gone once the
+    // tile is stored: the order stays verify, then store.  The K slices of a split tile write raw accumulators.  The
+    // cadence kernels, whose verification sits in a loop, spill 100-200 registers with the stores inside it.)
+    const bool early_store = !CADENCE && p.beta == 0.f && tail_out == nullptr;
     hpcdnn_ft_status rec;          // thread ct < NCT: the record of check tile ct, merged over the verifications
     rec.flag = 0; rec.row = -1; rec.col = -1; rec.n_bad_rows = 0; rec.n_bad_cols = 0;
     rec.row_residual = 0.f; rec.col_residual = 0.f; rec.max_clean_residual = 0.f;
@@ -1136,6 +1212,15 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             return old;
         };
 
+        // the element again, into C (tile already stored): the owner waits until its stores of the tile are written
+        auto rewrite_c = [&](int r, int c, float val) {
+            const int rr = r % 32;
+            if (wm == r / WM && wn == c / WN && lr == c % 32 && lh == (rr / 4) % 2) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+                p.C[static_cast<int64_t>(m0 + r) * p.ldc + (n0 + c)] = p.alpha * val;
+            }
+        };
+
         // Soft-error injection: one accumulator per fault, after the K loop (or interval), before the checks
         // (run-time form of `t[2].x += error_inject`, ft_sgemm_huge.cuh:40,145).  A fault aimed at a row or column
         // of an edge tile that lies outside the matrix is ignored.  A kernel that verifies once injects every fault
@@ -1183,6 +1268,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             if (tile_linear == p.faults[f].tile && (CADENCE ? p.faults[f].check == check_global : k_slice == 0) &&
                 m0 + p.faults[f].row < p.M && n0 + p.faults[f].col < p.N)
                 add_at(p.faults[f].row, p.faults[f].col, p.faults[f].delta);
+        if (last && early_store) store_c();
 
         if (tid < NCT) { s_meta[8 * tid] = 0; s_meta[8 * tid + 1] = 0; s_meta[8 * tid + 2] = -1; s_meta[8 * tid + 3] = -1; s_meta[8 * tid + 4] = 0; s_fix[2 * tid + 1] = 0.f; }
 
@@ -1473,6 +1559,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 __syncthreads();
                 const float old_val = set_at(bad_r, bad_c, s_fix[2 * ct], &s_fix[2 * ct + 1]);
                 (void)old_val;
+                if (last && early_store) rewrite_c(bad_r, bad_c, s_fix[2 * ct]);
                 any_fixed = true;
             }
         }
@@ -1560,6 +1647,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     } else {
         run_k_range();
         verify(0, true);
+    }
+    if (early_store) return;
+    if (!tail_out) {
+        store_c();
+        return;
     }
     }  // FT != 0
 
