@@ -52,12 +52,9 @@ FtKernel HPCDNN_FT_PASTE(ft_kernel_c, HPCDNN_FT_CLASS, _ta, HPCDNN_FT_TA)(int ki
 }
 
 // the pre-pass over both operands for this class's check tiles at either granularity
-// (fine: blocks over 64 values of k instead of 256, for operands that would not fill the CUs otherwise)
-EncodeFn HPCDNN_FT_PASTE(ft_encode_c, HPCDNN_FT_CLASS, _ta, HPCDNN_FT_TA)(bool wave, bool fine) {
-    if (wave)
-        return fine ? abft_encode_kernel<kGeom.bm / kGeom.wgm, kGeom.bn / kGeom.wgn, kTa, 64>
-                    : abft_encode_kernel<kGeom.bm / kGeom.wgm, kGeom.bn / kGeom.wgn, kTa, 256>;
-    return fine ? abft_encode_kernel<kGeom.bm, kGeom.bn, kTa, 64> : abft_encode_kernel<kGeom.bm, kGeom.bn, kTa, 256>;
+EncodeFn HPCDNN_FT_PASTE(ft_encode_c, HPCDNN_FT_CLASS, _ta, HPCDNN_FT_TA)(bool wave) {
+    if (wave) return abft_encode_kernel<kGeom.bm / kGeom.wgm, kGeom.bn / kGeom.wgn, kTa>;
+    return abft_encode_kernel<kGeom.bm, kGeom.bn, kTa>;
 }
 
 }  // namespace hpcdnn

@@ -3,8 +3,6 @@
 
 namespace hpcdnn {
 
-// the pre-pass runs blocks over 64 values of k instead of 256 while the latter would be fewer than this (two per CU)
-constexpr int kEncodeFineBelow = 512;
 
 // row length of the pre-encoded checksum vectors: K rounded up to the K step, plus two K steps of zeros for the
 // fetches that run ahead of the main loop
@@ -44,18 +42,18 @@ static FtKernel ft_kernel(int tile_class, bool ta, int kind) {
         default: return FtKernel{nullptr, nullptr, 0, 0};
     }
 }
-static EncodeFn ft_encode(int tile_class, bool ta, bool wave, bool fine) {
+static EncodeFn ft_encode(int tile_class, bool ta, bool wave) {
     switch (tile_class * 2 + (ta ? 1 : 0)) {
-        case 0: return ft_encode_c0_ta0(wave, fine);
-        case 1: return ft_encode_c0_ta1(wave, fine);
-        case 2: return ft_encode_c1_ta0(wave, fine);
-        case 3: return ft_encode_c1_ta1(wave, fine);
-        case 4: return ft_encode_c2_ta0(wave, fine);
-        case 5: return ft_encode_c2_ta1(wave, fine);
-        case 6: return ft_encode_c3_ta0(wave, fine);
-        case 7: return ft_encode_c3_ta1(wave, fine);
-        case 8: return ft_encode_c4_ta0(wave, fine);
-        case 9: return ft_encode_c4_ta1(wave, fine);
+        case 0: return ft_encode_c0_ta0(wave);
+        case 1: return ft_encode_c0_ta1(wave);
+        case 2: return ft_encode_c1_ta0(wave);
+        case 3: return ft_encode_c1_ta1(wave);
+        case 4: return ft_encode_c2_ta0(wave);
+        case 5: return ft_encode_c2_ta1(wave);
+        case 6: return ft_encode_c3_ta0(wave);
+        case 7: return ft_encode_c3_ta1(wave);
+        case 8: return ft_encode_c4_ta0(wave);
+        case 9: return ft_encode_c4_ta1(wave);
         default: return nullptr;
     }
 }
@@ -278,12 +276,10 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
                 abft_encode_weighted_kernel<64><<<dim3(k_blocks * b_blocks), dim3(1024), 0, s>>>(N, K, B, ldb, wb, wb + static_cast<size_t>(col_groups) * a.enc_ld,
                                                                                             a.enc_ld, k_blocks, col_groups);
         } else {
-            const bool fine = k_blocks * (row_groups + b_blocks) < kEncodeFineBelow;
-            const int kb = fine ? 64 : 256;
-            k_blocks = static_cast<int>(ceil_div(a.enc_ld, kb));
-            const EncodeFn encode = ft_encode(opt.tile_class, ta, wave, fine);
+            k_blocks = static_cast<int>(ceil_div(a.enc_ld, kEncodeKB));
+            const EncodeFn encode = ft_encode(opt.tile_class, ta, wave);
             if (!encode) return HPCDNN_ERR_INVALID_VALUE;
-            hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(kb * 4), 0, s, M, N, K,
+            hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(kEncodeKB * 4), 0, s, M, N, K,
                                A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
         }
         rc = launch_status();

@@ -80,8 +80,8 @@ enum FtKind { kFtFused = 0, kFtFusedCad, kFtPre, kFtPreCad, kFtWave, kFtWaveCad,
 #define HPCDNN_FT_DECLARE(c)                  \
     FtKernel ft_kernel_c##c##_ta0(int kind);  \
     FtKernel ft_kernel_c##c##_ta1(int kind);  \
-    EncodeFn ft_encode_c##c##_ta0(bool wave, bool fine); \
-    EncodeFn ft_encode_c##c##_ta1(bool wave, bool fine);
+    EncodeFn ft_encode_c##c##_ta0(bool wave); \
+    EncodeFn ft_encode_c##c##_ta1(bool wave);
 HPCDNN_FT_DECLARE(0)
 HPCDNN_FT_DECLARE(1)
 HPCDNN_FT_DECLARE(2)

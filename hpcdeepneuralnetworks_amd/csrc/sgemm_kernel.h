@@ -1868,31 +1868,33 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(int M, int N, int bm, 
 }
 
 // ---- ABFT pre-encode: the checksum vectors of the operands, one per row group (RM rows) / column group (CN
-// columns), in one launch of blocks of 4 KB threads that each cover KB values of k (256, or 64 for operands so small
-// that blocks of 256 would leave most CUs idle; the sums are the same, bit for bit): the first k_blocks * row_groups
-// blocks encode A, the rest B (one block per 128 columns of B, i.e. 128 / CN column groups).  A group is a workgroup
-// tile's rows or columns, or a wave tile's with wave-tile checksums.
+// columns), in one launch of 256-thread blocks that each cover kEncodeKB = 64 values of k: the first
+// k_blocks * row_groups blocks encode A, the rest B (one block per 128 columns of B, i.e. 128 / CN column groups).  A
+// group is a workgroup tile's rows or columns, or a wave tile's with wave-tile checksums.  (Blocks of 1024 threads
+// over 256 values of k, the first layout, left a partial last round of blocks on the CUs: 22 against 19 us at 4096
+// cubed, and most CUs idle on small operands.)
 //
 // enc_a[g][k'] = sum over the rows m of row group g (m < M) of A[m][k]; zero for K <= k < enc_ld; k' is k with
 // the order inside each group of 16 changed to 0, 8, 1, 9, ...  A thread owns 4 consecutive k and the RM / 16 rows of
-// one of 16 row slices (a wave per slice with KB = 256, a quarter wave with KB = 64); the 16 partials are added in
-// slice order, so the result does not depend on timing.
+// one of 16 row slices (a quarter wave per slice); the 16 partials are added in slice order, so the result does not
+// depend on timing.
 //
 // enc_b[g][k] = sum over the columns n of column group g (n < N) of B[k][n]; zero for K <= k < enc_ld.  A half
-// wave reads 128 columns of one k row (32 lanes x 4 columns) and owns 8 of the block's KB rows; CN / 4 neighbouring
+// wave reads 128 columns of one k row (32 lanes x 4 columns) and owns 8 of the block's rows; CN / 4 neighbouring
 // lanes share a column group.
 //
 // TA: A is given transposed (K rows of M floats, row length lda).  A row then holds a group's RM values side by side:
 // the 16 lanes of a DPP row read them 16 at a time (64 contiguous bytes; the four rows of a wave four different k) and
-// add their partial sums across the row; a block covers KB values of k of one row group, KB / 4 per pass.
-template <int RM, int CN, bool TA = false, int KB = 256>
+// add their partial sums across the row; a block covers kEncodeKB values of k of one row group, a quarter per pass.
+constexpr int kEncodeKB = 64;
+template <int RM, int CN, bool TA = false, int KB = kEncodeKB>
 __global__ __launch_bounds__(KB * 4) void abft_encode_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
                                                              const float* __restrict__ B, int ldb,
                                                              float* __restrict__ enc_a, float* __restrict__ enc_b,
                                                              int enc_ld, int k_blocks, int row_groups, int col_groups) {
     static_assert(CN == 128 || CN == 64 || CN == 32, "column groups are 8, 16 or 32 lanes of a half wave");
     static_assert(RM % 16 == 0, "the rows of a group split evenly over 16 slices");
-    static_assert(KB == 256 || KB == 64, "a row slice is a wave or a quarter of one");
+    static_assert(KB == 64 || KB == 256, "a row slice is a quarter wave (or a whole one)");
     constexpr int kSlices = 16, kRows = RM / kSlices, kSliceLanes = KB / 4;
     constexpr int kHalves = KB / 8, kRowsPerHalf = KB / kHalves;
     constexpr int kGroupLanes = CN / 4, kGroupsPer128 = 128 / CN;

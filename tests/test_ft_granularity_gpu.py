@@ -88,13 +88,11 @@ def test_wave_tiles_decisions_equal_the_model(blas, oracle_mod, tile_class, tau_
 
 
 @pytest.mark.parametrize("tile_class,granularity", [(4, 1), (2, 0)])
-def test_long_k_takes_the_pre_pass_with_blocks_over_256_values_of_k(blas, oracle_mod, tile_class, granularity):
-    """The pre-pass covers 64 values of k per block on small operands and 256 once that gives 512 blocks or more; the
-    other tests here are all of the first kind.  34 row groups and 2 blocks of 128 columns, times 16 blocks of k."""
+def test_long_k_and_many_row_groups_in_the_pre_pass(blas, oracle_mod, tile_class, granularity):
+    """The pre-pass with 34 row groups, 2 blocks of 128 columns and 62 blocks of k: K is not a multiple of its 64 values
+    of k per block, nor of the K step."""
     cm, cn = blas.ft_check_tile(tile_class, granularity)
     M, N, K = 17 * (64 if granularity else 128) - 3, 250, 3900
-    bm, _ = blas.ft_tile(tile_class)
-    assert -(-(K + 32) // 256) * (-(-M // bm) * (bm // cm) + -(-N // 128)) >= 512
     tau = blas.ft_default_tau(K)
     ntn = -(-N // cn)
     a, b, c0 = _problem(oracle_mod, M, N, K, 4100 + tile_class)

@@ -139,9 +139,9 @@ def test_other_classes_granularity_and_cadence(blas, oracle_mod):
         assert st["flag"][0] == 1 and (st["row"][0], st["col"][0]) == (3, 4)
 
 
-def test_long_k_takes_the_pre_pass_with_blocks_over_256_values_of_k(blas, oracle_mod):
-    """The pre-pass walks 64 values of k per block on small operands and 256 once that gives 512 blocks or more: here
-    34 row groups (wave tiles of the 64 x 64 class over the 1085 rows of C^T) and 2 blocks of 128 columns, 16 blocks of k."""
+def test_long_k_and_many_row_groups_in_the_pre_pass(blas, oracle_mod):
+    """The pre-pass over the K-major operands with 34 row groups (wave tiles of the 64 x 64 class over the 1085 rows of
+    C^T), 2 blocks of 128 columns and 62 blocks of k."""
     M, N, K = 250, 1085, 3900
     tau = blas.ft_default_tau(K)
     *_, st, _ = _run(blas, oracle_mod, M, N, K, 1.0, 1.0, tau, faults=[(41, 3, 4, 2.0)], pad=(4, 8, 4), tile_class=4,
