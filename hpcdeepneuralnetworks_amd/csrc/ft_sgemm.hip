@@ -261,7 +261,7 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         float* enc_b = enc_a + static_cast<size_t>(row_groups) * a.enc_ld;
         a.enc_a = enc_a;
         a.enc_b = enc_b;
-        int k_blocks = static_cast<int>(ceil_div(a.enc_ld, 256));
+        const int k_blocks = static_cast<int>(ceil_div(a.enc_ld, kEncodeKB));
         const int b_blocks = static_cast<int>(ceil_div(N, 128));  // the pre-pass walks B in blocks of 128 columns
         // (ta: the same launch, with the blocks of the A half walking A^T)
         if (weighted) {
@@ -270,13 +270,12 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
             a.enc_a = a.enc_b + static_cast<size_t>(col_groups) * a.enc_ld;
             float* const wb = static_cast<float*>(ws);
             if (fc.bn == 128)
-                abft_encode_weighted_kernel<128><<<dim3(k_blocks * b_blocks), dim3(1024), 0, s>>>(N, K, B, ldb, wb, wb + static_cast<size_t>(col_groups) * a.enc_ld,
+                abft_encode_weighted_kernel<128><<<dim3(k_blocks * b_blocks), dim3(kEncodeKB * 4), 0, s>>>(N, K, B, ldb, wb, wb + static_cast<size_t>(col_groups) * a.enc_ld,
                                                                                              a.enc_ld, k_blocks, col_groups);
             else
-                abft_encode_weighted_kernel<64><<<dim3(k_blocks * b_blocks), dim3(1024), 0, s>>>(N, K, B, ldb, wb, wb + static_cast<size_t>(col_groups) * a.enc_ld,
+                abft_encode_weighted_kernel<64><<<dim3(k_blocks * b_blocks), dim3(kEncodeKB * 4), 0, s>>>(N, K, B, ldb, wb, wb + static_cast<size_t>(col_groups) * a.enc_ld,
                                                                                             a.enc_ld, k_blocks, col_groups);
         } else {
-            k_blocks = static_cast<int>(ceil_div(a.enc_ld, kEncodeKB));
             const EncodeFn encode = ft_encode(opt.tile_class, ta, wave);
             if (!encode) return HPCDNN_ERR_INVALID_VALUE;
             hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(kEncodeKB * 4), 0, s, M, N, K,

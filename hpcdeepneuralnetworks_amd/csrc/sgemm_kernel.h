@@ -2001,18 +2001,18 @@ __global__ __launch_bounds__(KB * 4) void abft_encode_kernel(int M, int N, int K
 //   enc_b[g][k]  = sum over the group's columns n of B[k][n]             (B e1, e1 = [1, 1, ...])
 //   enc_bw[g][k] = sum over the group's columns n of (n' + 1) B[k][n]    (B e2, e2 = [1, 2, ...], n' counted inside the group)
 // (kernel/ft_sgemm/README.md:16-26); zero for K <= k < enc_ld.  Nothing of A is needed.  Layout of the work as in the
-// B half of abft_encode_kernel: 1024-thread blocks over 256 values of k and 128 columns, a half wave per k row.
-template <int CN>
-__global__ __launch_bounds__(1024) void abft_encode_weighted_kernel(int N, int K, const float* __restrict__ B, int ldb,
+// B half of abft_encode_kernel: 256-thread blocks over kEncodeKB values of k and 128 columns, a half wave per k row.
+template <int CN, int KB = kEncodeKB>
+__global__ __launch_bounds__(KB * 4) void abft_encode_weighted_kernel(int N, int K, const float* __restrict__ B, int ldb,
                                                                     float* __restrict__ enc_b, float* __restrict__ enc_bw,
                                                                     int enc_ld, int k_blocks, int col_groups) {
     static_assert(CN == 128 || CN == 64, "column groups are 16 or 32 lanes of a half wave");
-    constexpr int kHalves = 32, kRowsPerHalf = 256 / kHalves;
+    constexpr int kHalves = KB / 8, kRowsPerHalf = KB / kHalves;
     constexpr int kGroupLanes = CN / 4, kGroupsPer128 = 128 / CN;
     const int bid = blockIdx.x;
     const int lr = threadIdx.x & 31, half = threadIdx.x >> 5;
     const int tile_n = bid / k_blocks, n0 = tile_n * 128;
-    const int kb = (bid % k_blocks) * 256;
+    const int kb = (bid % k_blocks) * KB;
     const int in_group = lr % kGroupLanes;
     const float w0 = static_cast<float>(in_group * 4 + 1);  // weight of this lane's first column
     float s[kRowsPerHalf], sw[kRowsPerHalf];
