@@ -100,17 +100,15 @@ constexpr int b_stage_stride() {
 // LDS the ABFT verification needs (it reuses the staging buffers once the K loop has drained): FP64 partials of the
 // reference checksums, observed line sums and their absolute counterparts per wave row / wave column, one residual
 // per line, one record per check tile, per-wave sums of |acc| per check tile.  GM x GN check tiles per workgroup tile.
-// (the weighted locator keeps, in place of everything about columns, the weighted row sums: its reference partials
-// fit where the column partials would be, its observed sums get WGN x BM words of their own, its lines are 2 BM)
+// (the weighted locator has no column lines; its residual array has BM more words, of which the flagged row's holds that
+// row's weighted residual)
 template <int BM, int BN, int WGM, int WGN, int GM, int GN, bool WEIGHTED = false>
 constexpr size_t ft_verify_lds_bytes() {
     constexpr size_t threads = static_cast<size_t>(WGM) * WGN * 64;
     constexpr size_t ccp = threads / (BN / 4), crp = kGemmBK / 4;
     constexpr size_t lines = WEIGHTED ? 2 * static_cast<size_t>(BM) : static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
-    static_assert(!WEIGHTED || GM * ccp * BN >= crp * BM, "the weighted reference partials fit in the column partials' place");
     return sizeof(double) * (GM * ccp * BN + GN * crp * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + lines) +
-           32 * GM * GN + sizeof(float) * GM * GN * (threads / 64) + 2 * sizeof(float) * GM * GN +
-           (WEIGHTED ? sizeof(float) * WGN * BM : 0);
+           32 * GM * GN + sizeof(float) * GM * GN * (threads / 64) + 2 * sizeof(float) * GM * GN;
 }
 
 template <int BM, int BN, int FT = 0, int THREADS = 256, int WGM = 2, int WGN = 2, int GRAN = 0>
@@ -208,7 +206,9 @@ static __device__ __attribute__((noinline)) float recompute_element(const float*
 // the weighted-checksum locator (the reference's "kernel 2", kernel/ft_sgemm/README.md:16-26: two row sums of B,
 // e1 = [1, 1, ...] and e2 = [1, 2, ...], and nothing from A): references A (B e1) and A (B e2) against the plain and
 // the weighted row sums of the accumulators; a faulty row is found by the first pair, the column inside it as the
-// ratio of the two residuals; both vectors of B come from the workspace (abft_encode_weighted_kernel).
+// ratio of the two residuals; both vectors of B come from the workspace (abft_encode_weighted_kernel).  The main loop
+// accumulates the first reference only: the second pair is needed for one row, and only once that row is flagged, so
+// it is formed then (the row of A times the weighted vector, the weighted sum of the row's accumulators).
 //
 // NSLOT: staging register sets.  K step t + 1 waits in one of them while steps up to t + NSLOT are on their way from
 // memory.  Two are enough while a K step takes longer than a trip to memory (big tiles) or the operands come from
@@ -380,10 +380,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // (with wave-tile checksums the tile's GM / GN rows of the vectors follow each other: one descriptor over all
     // of them, the row chosen by the scalar offset)
     const __amdgpu_buffer_rsrc_t enc_a_rsrc =
-        make_rsrc(FT == 2   ? p.enc_a + static_cast<int64_t>(tile_m) * GM * p.enc_ld
-                  : FT == 3 ? p.enc_a + static_cast<int64_t>(tile_n) * p.enc_ld  // the weighted row sums of B
-                            : nullptr,
-                  static_cast<int64_t>(p.enc_ld) * GM * 4);
+        make_rsrc(FT == 2 ? p.enc_a + static_cast<int64_t>(tile_m) * GM * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * GM * 4);
     const __amdgpu_buffer_rsrc_t enc_b_rsrc =
         make_rsrc(FT >= 2 ? p.enc_b + static_cast<int64_t>(tile_n) * GN * p.enc_ld : nullptr, static_cast<int64_t>(p.enc_ld) * GN * 4);
     const int enc_row_bytes = p.enc_ld * 4;
@@ -394,7 +391,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     int enc_off = kbeg * 4;
     float g_ac[NSLOT][GM][B_SLOTS];
     v4f g_br[NSLOT][GN];
-    v4f g_bw[NSLOT];  // FT == 3: the weighted row sums of B for the four k values of A this thread stages
     auto gload1 = [&](auto slot, auto part, auto bulk) __attribute__((always_inline)) {  // bulk: this K step is not the slice's last (kLazyBounds)
         constexpr int S = decltype(slot)::value, P = decltype(part)::value;
         if constexpr (kNoBounds || (kLazyBounds && decltype(bulk)::value)) {
@@ -406,7 +402,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         }
         if constexpr (FT == 3 && P == NGL - 1) {
             g_br[S][0] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_b_rsrc, enc_b_voff, enc_off, 0));
-            g_bw[S] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_a_rsrc, enc_b_voff, enc_off, 0));
         }
         if constexpr (FT == 2 && P == NGL - 1) {
             static_assert(FT != 2 || B_SLOTS <= 2, "a thread stages one or two k rows of B");
@@ -639,15 +634,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         for (int sl = 0; sl < A_SLOTS; ++sl)
 #pragma unroll
             for (int e = 0; e < 4; ++e) cr_lo[gn][sl][e] = 0.f;
-    double crw_ref[A_SLOTS];  // FT == 3: the weighted row checksum references of this thread's rows
-    float crw_lo[A_SLOTS][4];
-#pragma unroll
-    for (int sl = 0; sl < A_SLOTS; ++sl) {
-        crw_ref[sl] = 0.0;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) crw_lo[sl][e] = 0.f;
-    }
-    v4f e_bwv;
     float e_pa[4], e_sw[4];
     v4f e_t[kPartV4 * B_SLOTS], e_brv[GN];
     v4f e_a[TA ? A_SLOTS : 1];  // TA: this thread's rows of the staged K step (four k each), read back from LDS
@@ -763,8 +749,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     for (int gm = 0; gm < GM; ++gm)
 #pragma unroll
                         for (int sl = 0; sl < B_SLOTS; ++sl) e_ac[gm][sl] = g_ac[S][gm][sl];
-                } else {
-                    e_bwv = g_bw[S];
                 }
 #pragma unroll
                 for (int gn = 0; gn < GN; ++gn) e_brv[gn] = g_br[S][gn];
@@ -796,19 +780,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 HPCDNN_PIN(e_ac[0][sl]);
             }
         } else if constexpr (kWeighted && E < 2 + GM) {
-            // the weighted row checksums take the place of the column checksums
-#pragma unroll
-            for (int sl = 0; sl < A_SLOTS; ++sl) {
-                const v4f av = TA ? e_a[TA ? sl : 0] : ra[S][sl];
-                crw_lo[sl][0] = __builtin_fmaf(av.x, e_bwv.x, crw_lo[sl][0]);
-                crw_lo[sl][1] = __builtin_fmaf(av.y, e_bwv.y, crw_lo[sl][1]);
-                crw_lo[sl][2] = __builtin_fmaf(av.z, e_bwv.z, crw_lo[sl][2]);
-                crw_lo[sl][3] = __builtin_fmaf(av.w, e_bwv.w, crw_lo[sl][3]);
-            }
-#pragma unroll
-            for (int sl = 0; sl < A_SLOTS; ++sl)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) HPCDNN_PIN(crw_lo[sl][e]);
+            // (no column checksums, and the weighted row checksum of a row is formed only once the row is flagged)
         } else if constexpr (E < 2 + GM) {
             // independent accumulators: a wave alone on its SIMD cannot hide the latency of dependent VALU
             // instructions behind other waves
@@ -844,14 +816,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             // every 16th K step (and after the last one): FP32 partials -> FP64 running sums.  FP64 VALU
             // instructions are twice as expensive as FP32 ones, so this is kept rare.
             if (flush_now) {
-                if constexpr (kWeighted) {
-#pragma unroll
-                    for (int sl = 0; sl < A_SLOTS; ++sl) {
-                        crw_ref[sl] += static_cast<double>((crw_lo[sl][0] + crw_lo[sl][1]) + (crw_lo[sl][2] + crw_lo[sl][3]));
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) crw_lo[sl][e] = 0.f;
-                    }
-                }
 #pragma unroll
                 for (int gm = 0; gm < (kWeighted ? 0 : GM); ++gm)
 #pragma unroll
@@ -1138,11 +1102,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;   // partials per column / per row checksum
     constexpr int NCT = GM * GN;                          // check tiles per workgroup tile
     constexpr int kRowLines = GN * BM;                    // row lines (gn, m) come first, column lines (gm, n) after them
-    // (weighted locator: the BM row lines, then the BM weighted row lines; there are no column lines)
+    // (weighted locator: the BM row lines, then BM words for the weighted residual of a flagged row; no column lines)
     constexpr int kLines = kWeighted ? 2 * BM : kRowLines + GM * BN;
-    // lines per thread in the pass over the column lines and in the pass over the row lines (with the weighted locator
-    // the second pass also takes the weighted row lines)
-    constexpr int kColPass = kWeighted ? 0 : GM * BN, kRowPass = kWeighted ? kLines : kRowLines;
+    // lines per thread in the pass over the column lines and in the pass over the row lines
+    constexpr int kColPass = kWeighted ? 0 : GM * BN, kRowPass = kRowLines;
     constexpr int LPT_C = (kColPass + kGemmThreads - 1) / kGemmThreads > 0 ? (kColPass + kGemmThreads - 1) / kGemmThreads : 1;
     constexpr int LPT_R = (kRowPass + kGemmThreads - 1) / kGemmThreads;
     static_assert(NCT <= kGemmThreads, "one thread per check tile keeps its record");
@@ -1173,8 +1136,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         int* const s_meta = reinterpret_cast<int*>(s_dr + kLines);      // [NCT][8] nbr, nbc, bad row, bad col, max clean (float bits)
         float* const s_tsum = reinterpret_cast<float*>(s_meta + 8 * NCT);  // [NCT][waves] partial sums of |acc| over a check tile
         float* const s_fix = s_tsum + NCT * (kGemmThreads / kWave);        // [NCT][2] recomputed element, and what it changed
-        float* const s_crwobs = s_fix + 2 * NCT;                           // weighted locator: [WGN][BM] observed weighted row sums
-        double* const s_crwref = s_ccref;                                  // weighted locator: [CRP][BM] weighted reference partials
         static_assert(gemm_lds_bytes<BM, BN, FT, kGemmThreads, WGM, WGN, GRAN>() >= ft_verify_lds_bytes<BM, BN, WGM, WGN, GM, GN, kWeighted>(),
                       "verification scratch fits in the kernel's LDS");
         const int tile_linear = tile_m * p.tiles_n + tile_n;
@@ -1258,7 +1219,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     const bool inside = m0 + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl < p.M;
 #pragma unroll
                     for (int gn = 0; gn < GN; ++gn) cr_ref[gn][sl] = inside ? cr_ref[gn][sl] : 0.0;
-                    crw_ref[sl] = inside ? crw_ref[sl] : 0.0;
                 }
             }
         }
@@ -1287,11 +1247,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 for (int e = 0; e < 4; ++e) s_ccref[(gm * CCP + e_hw) * BN + (tid % B_V4_PER_ROW) * 4 + e] = cc_ref[gm][e];
         };
         auto publish_row_refs = [&]() {
-            if constexpr (kWeighted) {
-#pragma unroll
-                for (int sl = 0; sl < A_SLOTS; ++sl)
-                    s_crwref[e_class * BM + (tid >> 2) + (kGemmThreads / A_V4_PER_ROW) * sl] = crw_ref[sl];
-            }
 #pragma unroll
             for (int gn = 0; gn < GN; ++gn)
 #pragma unroll
@@ -1364,20 +1319,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     s_crobs[wn * BM + row] = rs[0];
                     s_crabs[wn * BM + row] = ra_[0];
                 }
-                if constexpr (kWeighted) {
-                    // the same rows with column n of the tile weighted by n + 1 (kernel/ft_sgemm/README.md:16-26, e2 = [1, 2, ...])
-                    float rw[RG];
-#pragma unroll
-                    for (int e2 = 0; e2 < RG; ++e2) {
-                        const int i = (g * RG + e2) / 16, v = (g * RG + e2) % 16;
-                        float s = acc[i][0][v] * static_cast<float>(wn * WN + lr + 1);
-#pragma unroll
-                        for (int j = 1; j < TN; ++j) s = __builtin_fmaf(acc[i][j][v], static_cast<float>(wn * WN + j * 32 + lr + 1), s);
-                        rw[e2] = s;
-                    }
-                    half32_transpose_sum<RG>(rw, lane);
-                    if (RG == 32 || lr < RG) s_crwobs[wn * BM + row] = rw[0];
-                }
             }
         };
         // Relative mode: tau of a line of n elements inside the matrix = tau_rel * sqrt(n) * max(mean |acc| of the line,
@@ -1428,13 +1369,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     cols_in = cols_in < CN ? cols_in : CN;
                     double ref = 0.0, obs = 0.0;
                     float mag = 0.f;
-                    if (kWeighted && !is_row) {
-                        // weighted row line idx: its residual locates the column, it is not tested against a threshold
-#pragma unroll
-                        for (int w = 0; w < CRP; ++w) ref += s_crwref[w * BM + idx];
-#pragma unroll
-                        for (int w = 0; w < WGN; ++w) obs += static_cast<double>(s_crwobs[w * BM + idx]);
-                    } else if (is_row) {
+                    if (is_row) {
 #pragma unroll
                         for (int w = 0; w < CRP; ++w) ref += s_crref[(grp * CRP + w) * BM + idx];
 #pragma unroll
@@ -1452,7 +1387,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     const double d = (CADENCE ? ref - off[it] : ref) - obs;
                     d_out[it] = d;
                     const bool looked_at = !kGated || s_meta[8 * ct + 1] > 0;
-                    if (rows_in > 0 && cols_in > 0 && looked_at && !(kWeighted && !is_row)) {  // check tiles of an edge tile that lie outside the matrix have no lines
+                    if (rows_in > 0 && cols_in > 0 && looked_at) {  // check tiles of an edge tile that lie outside the matrix have no lines
                         double tau = static_cast<double>(p.tau);
                         if (relative) {
                             float total = 0.f;
@@ -1534,6 +1469,42 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             if (w_located) {
                 const int bad_r = s_meta[2];
                 w_d1 = s_dr[bad_r];
+                // The weighted residual of that one row, formed now: the weighted sum of its accumulators (column n of
+                // the tile weighted by n + 1) against the product of its row of A with the weighted row sums of B from
+                // the workspace.  Every thread takes a share of the k range and of the accumulators, thread 0 adds the
+                // shares in thread order.
+                __syncthreads();  // the reference partials at the start of the LDS are no longer read
+                double* const s_share = reinterpret_cast<double*>(smem);
+                static_assert(sizeof(double) * (GM * CCP * BN + GN * CRP * BM) >= sizeof(double) * kGemmThreads, "one share per thread fits");
+                float obs_share = 0.f;
+                {
+                    const int rr = bad_r % 32;
+                    const int fi = (bad_r % WM) / 32, fv = 4 * (rr / 8) + rr % 4;
+                    if (wm == bad_r / WM && lh == (rr / 4) % 2) {
+#pragma unroll
+                        for (int i = 0; i < TM; ++i)
+#pragma unroll
+                            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                                for (int v = 0; v < 16; ++v)
+                                    if (i == fi && v == fv)
+                                        obs_share = __builtin_fmaf(acc[i][j][v], static_cast<float>(wn * WN + j * 32 + lr + 1), obs_share);
+                    }
+                }
+                const float* const a_row = TA ? p.A + (m0 + bad_r) : p.A + static_cast<int64_t>(m0 + bad_r) * p.lda;
+                const int64_t a_stride = TA ? p.lda : 1;
+                const float* const bw = p.enc_a + static_cast<int64_t>(tile_n) * p.enc_ld;
+                double ref_share = 0.0;
+                for (int k = k_first + tid; k < kend; k += kGemmThreads)
+                    ref_share += static_cast<double>(a_row[k * a_stride]) * static_cast<double>(bw[k]);
+                s_share[tid] = ref_share - static_cast<double>(obs_share);
+                __syncthreads();
+                if (tid == 0) {
+                    double d2 = 0.0;
+                    for (int t = 0; t < kGemmThreads; ++t) d2 += s_share[t];
+                    s_dr[BM + bad_r] = static_cast<float>(d2);
+                }
+                __syncthreads();
                 int cols_in = p.N - n0;
                 cols_in = cols_in < BN ? cols_in : BN;
                 int col = static_cast<int>(__builtin_rintf(s_dr[BM + bad_r] / w_d1)) - 1;
