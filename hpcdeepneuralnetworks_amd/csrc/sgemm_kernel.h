@@ -270,6 +270,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // steps then need no masks but the last two of a slice.  (The kernels that form the vectors in the loop sum the
     // staged data itself and keep the masks.)
     constexpr bool kLazyOutside = EDGE && FT >= 2;
+    // ABFT with both checksum vectors from the workspace: the column checksums screen every verification, the row
+    // checksums are looked at only when a column is flagged - so the main loop carries the column references alone, and
+    // the row references of the tile (its rows of A times the row sums of B in the workspace) are formed when they are
+    // needed, by the whole workgroup, in the verification (lazy_row_refs).
+    constexpr bool kLazyRows = FT == 2;
 
     extern __shared__ __align__(16) float smem[];
     float* const As = smem;
@@ -417,9 +422,6 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                     g_ac[S][gm][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(enc_a_rsrc, enc_a_voff, soff, 0));
                 }
             }
-#pragma unroll
-            for (int gn = 0; gn < GN; ++gn)
-                g_br[S][gn] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(enc_b_rsrc, enc_b_voff, enc_off + gn * enc_row_bytes, 0));
         }
     };
     // Ragged tiles only, applied when the slot is consumed: columns k >= kend of A hold padding, the next K
@@ -750,12 +752,14 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
                         for (int sl = 0; sl < B_SLOTS; ++sl) e_ac[gm][sl] = g_ac[S][gm][sl];
                 }
+                if constexpr (!kLazyRows) {
 #pragma unroll
-                for (int gn = 0; gn < GN; ++gn) e_brv[gn] = g_br[S][gn];
-                // (the barrier before the second half has made stage `par`, which holds this K step, complete)
-                if constexpr (TA) {
+                    for (int gn = 0; gn < GN; ++gn) e_brv[gn] = g_br[S][gn];
+                    // (the barrier before the second half has made stage `par`, which holds this K step, complete)
+                    if constexpr (TA) {
 #pragma unroll
-                    for (int sl = 0; sl < A_SLOTS; ++sl) e_a[sl] = *reinterpret_cast<const v4f*>(As + par * A_STAGE + a_lds_rows[sl]);
+                        for (int sl = 0; sl < A_SLOTS; ++sl) e_a[sl] = *reinterpret_cast<const v4f*>(As + par * A_STAGE + a_lds_rows[sl]);
+                    }
                 }
             }
         } else if constexpr (E == 0) {
@@ -796,6 +800,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             for (int sl = 0; sl < B_SLOTS; ++sl)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) HPCDNN_PIN(cc_lo[gm][sl][e]);
+        } else if constexpr (kLazyRows && E < 2 + GM + NCR) {
+            // (the row references are formed in the verification, when a column is flagged)
         } else if constexpr (E < 2 + GM + NCR) {
             constexpr int piece = E - 2 - GM;
             constexpr int gn = GRAN ? piece : 0;
@@ -828,7 +834,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                         for (int sl = 0; sl < B_SLOTS; ++sl) cc_lo[gm][sl][e] = 0.f;
                     }
 #pragma unroll
-                for (int gn = 0; gn < GN; ++gn)
+                for (int gn = 0; gn < (kLazyRows ? 0 : GN); ++gn)
 #pragma unroll
                     for (int sl = 0; sl < A_SLOTS; ++sl) {
                         cr_ref[gn][sl] += static_cast<double>((cr_lo[gn][sl][0] + cr_lo[gn][sl][1]) + (cr_lo[gn][sl][2] + cr_lo[gn][sl][3]));
@@ -1247,6 +1253,69 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 for (int e = 0; e < 4; ++e) s_ccref[(gm * CCP + e_hw) * BN + (tid % B_V4_PER_ROW) * 4 + e] = cc_ref[gm][e];
         };
         auto publish_row_refs = [&]() {
+            if constexpr (kLazyRows) {
+                // Row references formed now: ref[gn][m] = sum over the k range done so far of A[m][k] * b_r[gn][k], b_r
+                // from the workspace, FP64.  Only run when a column is flagged, so its cost (a pass over the tile's rows
+                // of A by one workgroup) is that of a detection, not of a product.
+                constexpr int kWaves = kGemmThreads / kWave;
+                for (int i = tid; i < GN * CRP * BM; i += kGemmThreads) s_crref[i] = 0.0;
+                __syncthreads();
+                if constexpr (!TA) {
+                    // a wave per row, its lanes 4 values of k each: 1 KiB of the row per pass; the lanes' sums are added
+                    // by a butterfly, the same tree every time
+#pragma unroll 1
+                    for (int r = wave; r < BM; r += kWaves) {
+                        if (m0 + r >= p.M) break;
+                        const float* const a_row = p.A + static_cast<int64_t>(m0 + r) * p.lda;
+                        double sum[GN];
+#pragma unroll
+                        for (int gn = 0; gn < GN; ++gn) sum[gn] = 0.0;
+#pragma unroll 1
+                        for (int k = k_first + lane * 4; k < kend; k += kWave * 4) {
+                            float av[4];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) av[e] = (k + e < kend) ? a_row[k + e] : 0.f;
+#pragma unroll
+                            for (int gn = 0; gn < GN; ++gn) {
+                                const v4f b = *reinterpret_cast<const v4f*>(p.enc_b + (static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k);
+                                sum[gn] += static_cast<double>(av[0]) * static_cast<double>(b.x) + static_cast<double>(av[1]) * static_cast<double>(b.y) +
+                                           static_cast<double>(av[2]) * static_cast<double>(b.z) + static_cast<double>(av[3]) * static_cast<double>(b.w);
+                            }
+                        }
+#pragma unroll
+                        for (int gn = 0; gn < GN; ++gn) {
+                            double t = sum[gn];
+#pragma unroll
+                            for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, kWave);
+                            if (lane == 0) s_crref[(gn * CRP) * BM + r] = t;
+                        }
+                    }
+                } else {
+                    // A^T: a lane per row (64 neighbouring rows per wave, contiguous in memory for each k), the waves
+                    // that share a group of 64 rows take a part of the k range each: one partial per part
+                    constexpr int kGroups = BM / kWave, kKParts = kWaves / kGroups;
+                    static_assert(kWaves % kGroups == 0 && kKParts >= 1 && kKParts <= CRP, "the k parts of a row fit the partial slots");
+                    const int r = (wave % kGroups) * kWave + lane, part = wave / kGroups;
+                    const int per = ((kend - k_first + kKParts - 1) / kKParts + 3) & ~3;
+                    const int ka = k_first + part * per, kb = ka + per < kend ? ka + per : kend;
+                    if (m0 + r < p.M) {
+                        double sum[GN];
+#pragma unroll
+                        for (int gn = 0; gn < GN; ++gn) sum[gn] = 0.0;
+                        const float* a_col = p.A + static_cast<int64_t>(ka) * p.lda + (m0 + r);
+#pragma unroll 1
+                        for (int k = ka; k < kb; ++k, a_col += p.lda) {
+                            const double a = static_cast<double>(*a_col);
+#pragma unroll
+                            for (int gn = 0; gn < GN; ++gn)
+                                sum[gn] += a * static_cast<double>(p.enc_b[(static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k]);
+                        }
+#pragma unroll
+                        for (int gn = 0; gn < GN; ++gn) s_crref[(gn * CRP + part) * BM + r] = sum[gn];
+                    }
+                }
+                return;
+            }
 #pragma unroll
             for (int gn = 0; gn < GN; ++gn)
 #pragma unroll
