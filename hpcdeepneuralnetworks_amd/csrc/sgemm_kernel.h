@@ -267,14 +267,16 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // ABFT with checksum vectors from the workspace, ragged tiles: the staged columns n >= N of B (TA: m >= M of A^T)
     // hold the next row or padding.  The vectors cover the matrix only, so that data reaches nothing but the
     // accumulators and reference sums of lines outside the matrix, which the verification sets to zero first; the K
-    // steps then need no masks but the last two of a slice.  (The kernels that form the vectors in the loop sum the
-    // staged data itself and keep the masks.)
-    constexpr bool kLazyOutside = EDGE && FT >= 2;
-    // ABFT with both checksum vectors from the workspace: the column checksums screen every verification, the row
-    // checksums are looked at only when a column is flagged - so the main loop carries the column references alone, and
-    // the row references of the tile (its rows of A times the row sums of B in the workspace) are formed when they are
-    // needed, by the whole workgroup, in the verification (lazy_row_refs).
-    constexpr bool kLazyRows = FT == 2;
+    // steps then need no masks but the last two of a slice.  The kernels without a workspace sum the staged rows of A
+    // themselves - nothing of B, see kLazyRows -, so they run the same way unless A is given transposed (its staged
+    // columns m >= M would enter the column sums).
+    constexpr bool kLazyOutside = EDGE && (FT >= 2 || !TA);
+    // Row x column locator: the column checksums screen every verification, the row checksums are looked at only when
+    // a column is flagged - so the main loop carries the column references alone (a_c from the workspace or summed
+    // from the staged rows of A), and the row references of the tile (its rows of A times the row sums of B, from the
+    // workspace or summed from B then) are formed when they are needed, by the whole workgroup, in the verification.
+    // The weighted locator, whose screen is the plain row checksum, carries that one.
+    constexpr bool kLazyRows = FT == 1 || FT == 2;
 
     extern __shared__ __align__(16) float smem[];
     float* const As = smem;
@@ -696,6 +698,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         } else if constexpr (E == 3) {
             e_pa[0] += e_sw[0];
             e_sw[0] = lane_xor<16>(e_pa[0]);
+        } else if constexpr (kLazyRows && E >= 4 && E <= 7) {
+            // (the row sums of B are formed in the verification, when a column is flagged)
         } else if constexpr (E == 4) {
             // row sums of B: in-thread over the 4 columns, first butterfly step for each staged k row ...
             e_pb0 = (rb[S][0].x + rb[S][0].y) + (rb[S][0].z + rb[S][0].w);
@@ -726,8 +730,10 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 e_pa[0] += e_sw[0];
                 e_sw[0] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(x32_addr, __builtin_bit_cast(int, e_pa[0])));
             }
-            if constexpr (B_V4_PER_ROW == 32) e_pk += e_swb;
-            HPCDNN_PIN(e_pk);
+            if constexpr (!kLazyRows) {
+                if constexpr (B_V4_PER_ROW == 32) e_pk += e_swb;
+                HPCDNN_PIN(e_pk);
+            }
         } else if constexpr (E == 9) {
             if constexpr (!TA) e_pa[0] += e_sw[0];  // sum over the whole wave
             HPCDNN_PIN(e_pa[0]);
@@ -735,7 +741,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
             // lanes 0..15 of each wave publish the 16 column sums, the first lane (or two) of each k row of B its row sum;
             // the other lanes write to their dump word, which keeps the loop free of branches
             *(pub_a + par * (BK * kParts)) = e_pa[0];
-            *(pub_b + par * BK) = e_pk;
+            if constexpr (!kLazyRows) *(pub_b + par * BK) = e_pk;
         }
     };
     bool flush_now = true;  // uniform; set by the main loop before each K step that may flush
@@ -769,10 +775,12 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
                 for (int v = 0; v < kPartV4; ++v) e_t[kPartV4 * sl + v] = *reinterpret_cast<const v4f*>(row + 4 * v);
             }
-            e_brv[0] = *reinterpret_cast<const v4f*>(br + 4 * e_class);
-            if constexpr (TA) {
+            if constexpr (!kLazyRows) {
+                e_brv[0] = *reinterpret_cast<const v4f*>(br + 4 * e_class);
+                if constexpr (TA) {
 #pragma unroll
-                for (int sl = 0; sl < A_SLOTS; ++sl) e_a[sl] = *reinterpret_cast<const v4f*>(As + par * A_STAGE + a_lds_rows[sl]);
+                    for (int sl = 0; sl < A_SLOTS; ++sl) e_a[sl] = *reinterpret_cast<const v4f*>(As + par * A_STAGE + a_lds_rows[sl]);
+                }
             }
         } else if constexpr (E == 1) {
 #pragma unroll
@@ -1254,65 +1262,105 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         };
         auto publish_row_refs = [&]() {
             if constexpr (kLazyRows) {
-                // Row references formed now: ref[gn][m] = sum over the k range done so far of A[m][k] * b_r[gn][k], b_r
-                // from the workspace, FP64.  Only run when a column is flagged, so its cost (a pass over the tile's rows
-                // of A by one workgroup) is that of a detection, not of a product.
+                // Row references formed now: ref[gn][m] = sum over the k range done so far of A[m][k] * b_r[gn][k], FP64,
+                // b_r from the workspace or (FT == 1) summed here from B, 1024 values of k at a time, into the LDS the
+                // column partials no longer need.  Only run when a column is flagged, so its cost (a pass over the tile's
+                // rows of A, and of B without a workspace, by one workgroup) is that of a detection, not of a product.
                 constexpr int kWaves = kGemmThreads / kWave;
+                constexpr int kChunk = 1024;
+                static_assert(sizeof(double) * GM * CCP * BN >= sizeof(float) * kChunk, "a chunk of row sums fits in the column partials' place");
+                float* const s_b = reinterpret_cast<float*>(s_ccref);
                 for (int i = tid; i < GN * CRP * BM; i += kGemmThreads) s_crref[i] = 0.0;
                 __syncthreads();
-                if constexpr (!TA) {
-                    // a wave per row, its lanes 4 values of k each: 1 KiB of the row per pass; the lanes' sums are added
-                    // by a butterfly, the same tree every time
 #pragma unroll 1
-                    for (int r = wave; r < BM; r += kWaves) {
-                        if (m0 + r >= p.M) break;
-                        const float* const a_row = p.A + static_cast<int64_t>(m0 + r) * p.lda;
-                        double sum[GN];
-#pragma unroll
-                        for (int gn = 0; gn < GN; ++gn) sum[gn] = 0.0;
+                for (int kc = k_first, ke = k_first; kc < kend; kc = ke) {
+                    ke = (FT == 1 && kend - kc > kChunk) ? kc + kChunk : kend;  // (with a workspace: one pass)
+                    if constexpr (FT == 1) {
+                        // b_r[k] over the tile's columns inside the matrix: a half wave per k row, eight rows in flight
+                        constexpr int kHalfs = kGemmThreads / 32;
+                        const int hw = tid >> 5, l32 = tid & 31;
+                        int cols_in = p.N - n0;
+                        cols_in = cols_in < BN ? cols_in : BN;
+                        const int ke_pad = kc + ((ke - kc + 3) & ~3);  // the sums are read four at a time
 #pragma unroll 1
-                        for (int k = k_first + lane * 4; k < kend; k += kWave * 4) {
-                            float av[4];
+                        for (int kb = kc + hw * 8; kb < ke_pad; kb += kHalfs * 8) {
+                            float t[8];
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) av[e] = (k + e < kend) ? a_row[k + e] : 0.f;
+                            for (int i = 0; i < 8; ++i) {
+                                const int k = kb + i;
+                                const float* const brow = p.B + static_cast<int64_t>(k < ke ? k : kc) * p.ldb + n0 + l32 * 4;
+                                float x[4];
 #pragma unroll
-                            for (int gn = 0; gn < GN; ++gn) {
-                                const v4f b = *reinterpret_cast<const v4f*>(p.enc_b + (static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k);
-                                sum[gn] += static_cast<double>(av[0]) * static_cast<double>(b.x) + static_cast<double>(av[1]) * static_cast<double>(b.y) +
-                                           static_cast<double>(av[2]) * static_cast<double>(b.z) + static_cast<double>(av[3]) * static_cast<double>(b.w);
+                                for (int e = 0; e < 4; ++e) x[e] = (k < ke && l32 * 4 + e < cols_in) ? brow[e] : 0.f;
+                                t[i] = (x[0] + x[1]) + (x[2] + x[3]);
+                            }
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) {
+#pragma unroll
+                                for (int off = 16; off > 0; off >>= 1) t[i] += __shfl_xor(t[i], off, kWave);
+                                if (l32 == 0 && kb + i < ke_pad) s_b[kb + i - kc] = t[i];
                             }
                         }
-#pragma unroll
-                        for (int gn = 0; gn < GN; ++gn) {
-                            double t = sum[gn];
-#pragma unroll
-                            for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, kWave);
-                            if (lane == 0) s_crref[(gn * CRP) * BM + r] = t;
-                        }
+                        __syncthreads();
                     }
-                } else {
-                    // A^T: a lane per row (64 neighbouring rows per wave, contiguous in memory for each k), the waves
-                    // that share a group of 64 rows take a part of the k range each: one partial per part
-                    constexpr int kGroups = BM / kWave, kKParts = kWaves / kGroups;
-                    static_assert(kWaves % kGroups == 0 && kKParts >= 1 && kKParts <= CRP, "the k parts of a row fit the partial slots");
-                    const int r = (wave % kGroups) * kWave + lane, part = wave / kGroups;
-                    const int per = ((kend - k_first + kKParts - 1) / kKParts + 3) & ~3;
-                    const int ka = k_first + part * per, kb = ka + per < kend ? ka + per : kend;
-                    if (m0 + r < p.M) {
-                        double sum[GN];
-#pragma unroll
-                        for (int gn = 0; gn < GN; ++gn) sum[gn] = 0.0;
-                        const float* a_col = p.A + static_cast<int64_t>(ka) * p.lda + (m0 + r);
+                    if constexpr (!TA) {
+                        // a wave per row, its lanes 4 values of k each: 1 KiB of the row per pass; the lanes' sums are
+                        // added by a butterfly, the same tree every time
 #pragma unroll 1
-                        for (int k = ka; k < kb; ++k, a_col += p.lda) {
-                            const double a = static_cast<double>(*a_col);
+                        for (int r = wave; r < BM; r += kWaves) {
+                            if (m0 + r >= p.M) break;
+                            const float* const a_row = p.A + static_cast<int64_t>(m0 + r) * p.lda;
+                            double sum[GN];
 #pragma unroll
-                            for (int gn = 0; gn < GN; ++gn)
-                                sum[gn] += a * static_cast<double>(p.enc_b[(static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k]);
+                            for (int gn = 0; gn < GN; ++gn) sum[gn] = 0.0;
+#pragma unroll 1
+                            for (int k = kc + lane * 4; k < ke; k += kWave * 4) {
+                                float av[4];
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) av[e] = (k + e < ke) ? a_row[k + e] : 0.f;
+#pragma unroll
+                                for (int gn = 0; gn < GN; ++gn) {
+                                    const v4f b = FT == 1 ? *reinterpret_cast<const v4f*>(s_b + (k - kc))
+                                                          : *reinterpret_cast<const v4f*>(p.enc_b + (static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k);
+                                    sum[gn] += static_cast<double>(av[0]) * static_cast<double>(b.x) + static_cast<double>(av[1]) * static_cast<double>(b.y) +
+                                               static_cast<double>(av[2]) * static_cast<double>(b.z) + static_cast<double>(av[3]) * static_cast<double>(b.w);
+                                }
+                            }
+#pragma unroll
+                            for (int gn = 0; gn < GN; ++gn) {
+                                double t = sum[gn];
+#pragma unroll
+                                for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, kWave);
+                                if (lane == 0) s_crref[(gn * CRP) * BM + r] += t;
+                            }
                         }
+                    } else {
+                        // A^T: a lane per row (64 neighbouring rows per wave, contiguous in memory for each k), the waves
+                        // that share a group of 64 rows take a part of the k range each: one partial per part
+                        constexpr int kGroups = BM / kWave, kKParts = kWaves / kGroups;
+                        static_assert(kWaves % kGroups == 0 && kKParts >= 1 && kKParts <= CRP, "the k parts of a row fit the partial slots");
+                        const int r = (wave % kGroups) * kWave + lane, part = wave / kGroups;
+                        const int per = (ke - kc + kKParts - 1) / kKParts;
+                        const int ka = kc + part * per, kb = ka + per < ke ? ka + per : ke;
+                        if (m0 + r < p.M) {
+                            double sum[GN];
 #pragma unroll
-                        for (int gn = 0; gn < GN; ++gn) s_crref[(gn * CRP + part) * BM + r] = sum[gn];
+                            for (int gn = 0; gn < GN; ++gn) sum[gn] = 0.0;
+                            const float* a_col = p.A + static_cast<int64_t>(ka) * p.lda + (m0 + r);
+#pragma unroll 1
+                            for (int k = ka; k < kb; ++k, a_col += p.lda) {
+                                const double a = static_cast<double>(*a_col);
+#pragma unroll
+                                for (int gn = 0; gn < GN; ++gn) {
+                                    const float b = FT == 1 ? s_b[k - kc] : p.enc_b[(static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k];
+                                    sum[gn] += a * static_cast<double>(b);
+                                }
+                            }
+#pragma unroll
+                            for (int gn = 0; gn < GN; ++gn) s_crref[(gn * CRP + part) * BM + r] += sum[gn];
+                        }
                     }
+                    if constexpr (FT == 1) __syncthreads();  // the next chunk's sums go where these were
                 }
                 return;
             }
