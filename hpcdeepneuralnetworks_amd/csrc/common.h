@@ -159,6 +159,16 @@ __device__ __forceinline__ v4f buffer_load_v4f(__amdgpu_buffer_rsrc_t rsrc, int 
     return __builtin_bit_cast(v4f, v);
 }
 
+// Four consecutive floats from an address that is only 4-byte aligned and differs from lane to lane (a buffer
+// descriptor wants a wave-uniform base: with a per-lane one the compiler loops over the lanes).
+__device__ __forceinline__ v4f load_v4f_words(const float* p) {
+    struct __attribute__((aligned(4))) words {
+        float x, y, z, w;
+    };
+    const words t = *reinterpret_cast<const words*>(p);
+    return v4f{t.x, t.y, t.z, t.w};
+}
+
 // The same with the non-temporal hint, for data that is read once (aux bit 1 of the raw buffer instructions).
 __device__ __forceinline__ v4f buffer_load_v4f_nt(__amdgpu_buffer_rsrc_t rsrc, int byte_offset) {
     typedef unsigned v4u __attribute__((ext_vector_type(4)));

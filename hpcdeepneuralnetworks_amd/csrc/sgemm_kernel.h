@@ -1289,9 +1289,15 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                             for (int i = 0; i < 8; ++i) {
                                 const int k = kb + i;
                                 const float* const brow = p.B + static_cast<int64_t>(k < ke ? k : kc) * p.ldb + n0 + l32 * 4;
-                                float x[4];
+                                // (a lane whose four columns all lie inside loads them at once; the one lane of a row
+                                // that straddles the last column loads word by word; both predicated, nothing waits)
+                                const bool whole = k < ke && l32 * 4 + 3 < cols_in;
+                                v4f b4 = {0.f, 0.f, 0.f, 0.f};
+                                if (whole) b4 = load_v4f_words(brow);
+                                float x[4] = {b4.x, b4.y, b4.z, b4.w};
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) x[e] = (k < ke && l32 * 4 + e < cols_in) ? brow[e] : 0.f;
+                                for (int e = 0; e < 4; ++e)
+                                    if (!whole && k < ke && l32 * 4 + e < cols_in) x[e] = brow[e];
                                 t[i] = (x[0] + x[1]) + (x[2] + x[3]);
                             }
 #pragma unroll
@@ -1304,35 +1310,54 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                         __syncthreads();
                     }
                     if constexpr (!TA) {
-                        // a wave per row, its lanes 4 values of k each: 1 KiB of the row per pass; the lanes' sums are
-                        // added by a butterfly, the same tree every time
+                        // a wave per two rows, its lanes 4 values of k of each per pass (1 KiB of a row, one 16-byte load per
+                        // lane: four word loads move the same bytes in four times the instructions, and the vector memory
+                        // pipe of the one CU at work here is what limits this pass); the lanes' sums are added by a
+                        // butterfly, the same tree every time
 #pragma unroll 1
-                        for (int r = wave; r < BM; r += kWaves) {
-                            if (m0 + r >= p.M) break;
-                            const float* const a_row = p.A + static_cast<int64_t>(m0 + r) * p.lda;
-                            double sum[GN];
+                        for (int r0 = 2 * wave; r0 < BM; r0 += 2 * kWaves) {
+                            if (m0 + r0 >= p.M) break;
+                            const float* const a_row0 = p.A + static_cast<int64_t>(m0 + r0) * p.lda;
+                            const bool two = m0 + r0 + 1 < p.M;  // (else the second row reads the first again and is not kept)
+                            const float* const a_row1 = two ? a_row0 + p.lda : a_row0;
+                            double sum[2][GN];
 #pragma unroll
-                            for (int gn = 0; gn < GN; ++gn) sum[gn] = 0.0;
+                            for (int gn = 0; gn < GN; ++gn) sum[0][gn] = sum[1][gn] = 0.0;
 #pragma unroll 1
                             for (int k = kc + lane * 4; k < ke; k += kWave * 4) {
-                                float av[4];
+                                float av[2][4];
+                                if (k + 3 < ke) {
+                                    const v4f a0 = load_v4f_words(a_row0 + k);
+                                    const v4f a1 = load_v4f_words(a_row1 + k);
+                                    av[0][0] = a0.x; av[0][1] = a0.y; av[0][2] = a0.z; av[0][3] = a0.w;
+                                    av[1][0] = a1.x; av[1][1] = a1.y; av[1][2] = a1.z; av[1][3] = a1.w;
+                                } else {
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) av[e] = (k + e < ke) ? a_row[k + e] : 0.f;
+                                    for (int e = 0; e < 4; ++e) {
+                                        av[0][e] = (k + e < ke) ? a_row0[k + e] : 0.f;
+                                        av[1][e] = (k + e < ke) ? a_row1[k + e] : 0.f;
+                                    }
+                                }
 #pragma unroll
                                 for (int gn = 0; gn < GN; ++gn) {
                                     const v4f b = FT == 1 ? *reinterpret_cast<const v4f*>(s_b + (k - kc))
                                                           : *reinterpret_cast<const v4f*>(p.enc_b + (static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k);
-                                    sum[gn] += static_cast<double>(av[0]) * static_cast<double>(b.x) + static_cast<double>(av[1]) * static_cast<double>(b.y) +
-                                               static_cast<double>(av[2]) * static_cast<double>(b.z) + static_cast<double>(av[3]) * static_cast<double>(b.w);
+                                    const double bx = static_cast<double>(b.x), by = static_cast<double>(b.y), bz = static_cast<double>(b.z), bw = static_cast<double>(b.w);
+#pragma unroll
+                                    for (int j = 0; j < 2; ++j)
+                                        sum[j][gn] += static_cast<double>(av[j][0]) * bx + static_cast<double>(av[j][1]) * by +
+                                                      static_cast<double>(av[j][2]) * bz + static_cast<double>(av[j][3]) * bw;
                                 }
                             }
 #pragma unroll
-                            for (int gn = 0; gn < GN; ++gn) {
-                                double t = sum[gn];
+                            for (int j = 0; j < 2; ++j)
 #pragma unroll
-                                for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, kWave);
-                                if (lane == 0) s_crref[(gn * CRP) * BM + r] += t;
-                            }
+                                for (int gn = 0; gn < GN; ++gn) {
+                                    double t = sum[j][gn];
+#pragma unroll
+                                    for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, kWave);
+                                    if (lane == 0 && (j == 0 || two)) s_crref[(gn * CRP) * BM + r0 + j] += t;
+                                }
                         }
                     } else {
                         // A^T: a lane per row (64 neighbouring rows per wave, contiguous in memory for each k), the waves
@@ -1347,13 +1372,20 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
 #pragma unroll
                             for (int gn = 0; gn < GN; ++gn) sum[gn] = 0.0;
                             const float* a_col = p.A + static_cast<int64_t>(ka) * p.lda + (m0 + r);
+                            // (eight k rows' loads go out together)
 #pragma unroll 1
-                            for (int k = ka; k < kb; ++k, a_col += p.lda) {
-                                const double a = static_cast<double>(*a_col);
+                            for (int k0 = ka; k0 < kb; k0 += 8, a_col += 8 * static_cast<int64_t>(p.lda)) {
+                                float av[8];
 #pragma unroll
-                                for (int gn = 0; gn < GN; ++gn) {
-                                    const float b = FT == 1 ? s_b[k - kc] : p.enc_b[(static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k];
-                                    sum[gn] += a * static_cast<double>(b);
+                                for (int u = 0; u < 8; ++u) av[u] = k0 + u < kb ? a_col[u * static_cast<int64_t>(p.lda)] : 0.f;
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) {
+                                    const int k = k0 + u < kb ? k0 + u : kb - 1;  // (past the part: a zero times a value that exists)
+#pragma unroll
+                                    for (int gn = 0; gn < GN; ++gn) {
+                                        const float b = FT == 1 ? s_b[k - kc] : p.enc_b[(static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k];
+                                        sum[gn] += static_cast<double>(av[u]) * static_cast<double>(b);
+                                    }
                                 }
                             }
 #pragma unroll
