@@ -163,7 +163,8 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     if (opt.locator != HPCDNN_FT_LOCATE_ROW_COL && opt.locator != HPCDNN_FT_LOCATE_WEIGHTED) return HPCDNN_ERR_INVALID_VALUE;
     const FtClass& fc = kFtClasses[opt.tile_class];
     const bool wave = opt.granularity == HPCDNN_FT_GRAN_WAVE;
-    const bool weighted = opt.locator == HPCDNN_FT_LOCATE_WEIGHTED;
+    const bool user_weighted = opt.locator == HPCDNN_FT_LOCATE_WEIGHTED;
+    bool weighted = user_weighted;
     // an interval that covers all of K is a single verification after the loop
     const bool cadence = opt.check_interval > 0 && opt.check_interval < K;
     if (weighted && (wave || cadence)) return HPCDNN_ERR_INVALID_VALUE;  // one pair of checksums per workgroup tile, verified once
@@ -217,7 +218,17 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
     // product with few columns the operand is all the traffic there is.  Those products run the kernels that form the
     // vectors in their main loop, and use the workspace only to split every tile along K until two workgroups per CU
     // keep enough bytes on their way from memory.
-    const bool fused_split = ws && K > 0 && !wave && !weighted && (a.tiles_n == 1 || a.tiles_m == 1) && a.tiles_m * a.tiles_n >= device_cus() / 8;
+    const bool one_wide = K > 0 && (a.tiles_n == 1 || a.tiles_m == 1) && a.tiles_m * a.tiles_n >= device_cus() / 8;
+    // One tile wide, one verification per tile, row x column locator: the kernels of the weighted locator (row sums of B
+    // from a pre-pass over B, which is small here; the plain row checksum as the screen) with the column references
+    // formed when a row is flagged (locate_rc) - nothing of A is summed in the loop at all.
+    const bool row_screen = ws && one_wide && a.tiles_n == 1 && !wave && !cadence && !user_weighted &&
+                            ws_bytes >= ft_weighted_enc_bytes(fc, N, K) && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
+    if (row_screen) {
+        weighted = true;
+        a.locate_rc = 1;
+    }
+    const bool fused_split = ws && one_wide && !wave && !weighted;
     if (fused_split) {
         if (reinterpret_cast<uintptr_t>(ws) & 15u) return HPCDNN_ERR_WORKSPACE;
         const int tiles = a.tiles_m * a.tiles_n;

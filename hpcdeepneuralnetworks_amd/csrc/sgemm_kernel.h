@@ -77,6 +77,7 @@ struct GemmArgs {
         int check;
     } faults[kMaxFaults];
     int check_interval;          // CADENCE kernels: values of k between two verifications, a multiple of the K step
+    int locate_rc;               // FT == 3 kernels: 0 = the column from the weighted checksum; 1 = row x column, the rows as the screen
     int status_rows, status_ld;  // records are laid out as a status_rows x status_ld grid of check tiles
     hpcdnn_ft_status* status;
     const float* enc_a;  // FT == 2: [row groups][enc_ld] column sums of A over the rows of each check tile
@@ -100,13 +101,13 @@ constexpr int b_stage_stride() {
 // LDS the ABFT verification needs (it reuses the staging buffers once the K loop has drained): FP64 partials of the
 // reference checksums, observed line sums and their absolute counterparts per wave row / wave column, one residual
 // per line, one record per check tile, per-wave sums of |acc| per check tile.  GM x GN check tiles per workgroup tile.
-// (the weighted locator has no column lines; its residual array has BM more words, of which the flagged row's holds that
-// row's weighted residual)
+// (the kernels whose screen is the row checksum - the weighted locator, and row x column on products one tile wide -
+// keep, behind the BM row residuals, either the weighted residual of the flagged row or the BN column residuals)
 template <int BM, int BN, int WGM, int WGN, int GM, int GN, bool WEIGHTED = false>
 constexpr size_t ft_verify_lds_bytes() {
     constexpr size_t threads = static_cast<size_t>(WGM) * WGN * 64;
     constexpr size_t ccp = threads / (BN / 4), crp = kGemmBK / 4;
-    constexpr size_t lines = WEIGHTED ? 2 * static_cast<size_t>(BM) : static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
+    constexpr size_t lines = WEIGHTED ? static_cast<size_t>(BM) + (BM > BN ? BM : BN) : static_cast<size_t>(GN) * BM + static_cast<size_t>(GM) * BN;
     return sizeof(double) * (GM * ccp * BN + GN * crp * BM) + sizeof(float) * (2 * (WGM * BN + WGN * BM) + lines) +
            32 * GM * GN + sizeof(float) * GM * GN * (threads / 64) + 2 * sizeof(float) * GM * GN;
 }
@@ -1116,8 +1117,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     constexpr int CCP = kHalfWaves, CRP = A_V4_PER_ROW;   // partials per column / per row checksum
     constexpr int NCT = GM * GN;                          // check tiles per workgroup tile
     constexpr int kRowLines = GN * BM;                    // row lines (gn, m) come first, column lines (gm, n) after them
-    // (weighted locator: the BM row lines, then BM words for the weighted residual of a flagged row; no column lines)
-    constexpr int kLines = kWeighted ? 2 * BM : kRowLines + GM * BN;
+    // (row-screen kernels: the BM row lines, then the weighted residual of a flagged row or the BN column lines)
+    constexpr int kLines = kWeighted ? BM + (BM > BN ? BM : BN) : kRowLines + GM * BN;
     // lines per thread in the pass over the column lines and in the pass over the row lines
     constexpr int kColPass = kWeighted ? 0 : GM * BN, kRowPass = kRowLines;
     constexpr int LPT_C = (kColPass + kGemmThreads - 1) / kGemmThreads > 0 ? (kColPass + kGemmThreads - 1) / kGemmThreads : 1;
@@ -1614,7 +1615,98 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         float w_d1 = 0.f;
         bool w_located = false;
         if constexpr (kWeighted) {
-            w_located = s_meta[0] == 1;
+            if (p.locate_rc && s_meta[0] > 0) {
+                // Row x column with the rows as the screen (products one tile wide, whose operand A is read once and
+                // has no checksum vector): a row is flagged, so the column references are formed now, cc[n] = sum over
+                // the k range of a_c[k] * B[k][n] with a_c[k] the column sums of the tile's rows of A, a chunk of k at
+                // a time through the LDS the row partials have left; then the columns are observed and thresholded
+                // like the rows were.
+                constexpr int kWavesV = kGemmThreads / kWave;
+                constexpr int kChunkA = 8 * BM > 1024 ? 1024 : 8 * BM;  // floats in the place of GN * CRP * BM doubles
+                static_assert(sizeof(double) * GN * CRP * BM >= sizeof(float) * kChunkA, "a chunk of column sums of A fits in the row partials' place");
+                constexpr int kColGroups = BN / kWave, kKPartsV = kWavesV / kColGroups;
+                static_assert(BN % kWave == 0 && kWavesV % kColGroups == 0 && kKPartsV >= 1 && kKPartsV <= CCP, "the k parts of a column fit the partial slots");
+                float* const s_a = reinterpret_cast<float*>(s_crref);
+                int rows_in = p.M - m0, cols_in = p.N - n0;
+                rows_in = rows_in < BM ? rows_in : BM;
+                cols_in = cols_in < BN ? cols_in : BN;
+                __syncthreads();  // the row partials are no longer read
+                for (int i = tid; i < GM * CCP * BN; i += kGemmThreads) s_ccref[i] = 0.0;
+#pragma unroll 1
+                for (int kc = k_first, ke = k_first; kc < kend; kc = ke) {
+                    ke = kend - kc > kChunkA ? kc + kChunkA : kend;
+                    if constexpr (!TA) {
+                        // a thread per four values of k, four rows' loads in flight
+#pragma unroll 1
+                        for (int q = tid; q * 4 < ke - kc; q += kGemmThreads) {
+                            const int k = kc + q * 4;
+                            float t[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+                            for (int m = 0; m < rows_in; m += 4) {
+                                float v[4][4];
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    const float* const src = p.A + static_cast<int64_t>(m0 + (m + j < rows_in ? m + j : m)) * p.lda + k;
+                                    if (k + 3 < ke) {
+                                        const v4f a4 = load_v4f_words(src);
+                                        v[j][0] = a4.x; v[j][1] = a4.y; v[j][2] = a4.z; v[j][3] = a4.w;
+                                    } else {
+#pragma unroll
+                                        for (int e = 0; e < 4; ++e) v[j][e] = k + e < ke ? src[e] : 0.f;
+                                    }
+                                }
+#pragma unroll
+                                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) t[e] += m + j < rows_in ? v[j][e] : 0.f;
+                            }
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) s_a[q * 4 + e] = t[e];
+                        }
+                    } else {
+                        // A^T: row k holds the tile's rows side by side; a half wave per k
+                        const int hw = tid >> 5, l32 = tid & 31;
+#pragma unroll 1
+                        for (int k = kc + hw; k < ke; k += kGemmThreads / 32) {
+                            const float* const src = p.A + static_cast<int64_t>(k) * p.lda + m0;
+                            float t = 0.f;
+                            for (int m = l32; m < rows_in; m += 32) t += src[m];
+#pragma unroll
+                            for (int off = 16; off > 0; off >>= 1) t += __shfl_xor(t, off, kWave);
+                            if (l32 == 0) s_a[k - kc] = t;
+                        }
+                    }
+                    __syncthreads();
+                    {
+                        // a lane per column, the waves that share 64 columns a part of the chunk each
+                        const int n = (wave % kColGroups) * kWave + lane, part = wave / kColGroups;
+                        const int per = (ke - kc + kKPartsV - 1) / kKPartsV;
+                        const int ka = kc + part * per, kb = ka + per < ke ? ka + per : ke;
+                        if (n < cols_in) {
+                            double sum = 0.0;
+                            const float* bp = p.B + static_cast<int64_t>(ka) * p.ldb + n0 + n;
+#pragma unroll 1
+                            for (int k0 = ka; k0 < kb; k0 += 8, bp += 8 * static_cast<int64_t>(p.ldb)) {
+                                float bv[8];
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) bv[u] = k0 + u < kb ? bp[u * static_cast<int64_t>(p.ldb)] : 0.f;
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) {
+                                    const int k = k0 + u < kb ? k0 + u : kb - 1;
+                                    sum += static_cast<double>(bv[u]) * static_cast<double>(s_a[k - kc]);
+                                }
+                            }
+                            s_ccref[part * BN + n] += sum;
+                        }
+                    }
+                    __syncthreads();
+                }
+                observe_cols();
+                __syncthreads();
+                residual_pass(std::integral_constant<int, kRowLines>{}, std::integral_constant<int, BN>{}, std::false_type{}, d_col, off_col);
+                __syncthreads();
+            }
+            w_located = !p.locate_rc && s_meta[0] == 1;
             if (w_located) {
                 const int bad_r = s_meta[2];
                 w_d1 = s_dr[bad_r];
@@ -1739,7 +1831,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 rec.row = bad_r - gm * CM;
                 rec.col = bad_c - gn * CN;
                 rec.row_residual = s_dr[gn * BM + bad_r];
-                rec.col_residual = kWeighted ? s_dr[BM + bad_r] : s_dr[kRowLines + gm * BN + bad_c];
+                rec.col_residual = kWeighted ? s_dr[BM + (p.locate_rc ? bad_c : bad_r)] : s_dr[kRowLines + gm * BN + bad_c];
             }
             if (last && p.status) {
                 hpcdnn_ft_status st = rec;

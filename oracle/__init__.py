@@ -105,6 +105,8 @@ def _load():
     lib.oracle_abft_residuals.argtypes = [C.c_int, C.c_int, C.c_int, fp, C.c_int, fp, C.c_int, fp, C.c_int, dp, dp]
     lib.oracle_abft_decide.restype = C.c_float
     lib.oracle_abft_decide.argtypes = [C.c_int, C.c_int, dp, dp, C.c_float, C.POINTER(FtStatus)]
+    lib.oracle_abft_set_rows_screen.restype = None
+    lib.oracle_abft_set_rows_screen.argtypes = [C.c_int]
     lib.oracle_abft_decide_lines.restype = C.c_float
     lib.oracle_abft_decide_lines.argtypes = [C.c_int, C.c_int, dp, dp, dp, dp, C.POINTER(FtStatus)]
     lib.oracle_ft_sgemm.restype = None
@@ -286,6 +288,19 @@ def abft_decide_lines(dr: np.ndarray, dc: np.ndarray, tau_r: np.ndarray, tau_c: 
     assert len(tau_r) == len(dr) and len(tau_c) == len(dc)
     fix = _load().oracle_abft_decide_lines(len(dr), len(dc), _d(dr), _d(dc), _d(tau_r), _d(tau_c), C.byref(st))
     return {k: getattr(st, k) for k, _ in FtStatus._fields_}, float(fix)
+
+
+class rows_screen:
+    """Context manager: inside it the ABFT decision model takes the rows as the screen (columns looked at only when a
+    row is flagged), the library's rule for row x column location on products one tile wide with a workspace."""
+
+    def __enter__(self):
+        _load().oracle_abft_set_rows_screen(1)
+        return self
+
+    def __exit__(self, *exc):
+        _load().oracle_abft_set_rows_screen(0)
+        return False
 
 
 def ft_sgemm(M, N, K, a, lda, b, ldb, c, ldc, alpha, beta, tile_m, tile_n, tau, fault=None):

@@ -338,19 +338,37 @@ void oracle_abft_residuals(int tm, int tn, int K, const float* A, int lda, const
  * flagged column the rows are thresholded too: one faulty row x one faulty
  * column -> located (flag 1), anything else -> detected only (flag 2).
  * Returns the signed row residual of the located row (0 when nothing is located). */
+/* Which side screens.  0 (default): the columns, as described above.  1: the rows - the library's choice for
+ * products one tile wide with a workspace, whose operand A is streamed once and gets no checksum vector: there the
+ * row checksums (from the small B) are compared every time and the columns only when a row disagrees.  The rule is
+ * the same with the two sides exchanged. */
+static int g_rows_screen = 0;
+void oracle_abft_set_rows_screen(int on) { g_rows_screen = on != 0; }
+
 /* Per-line thresholds: tau_r[m] for row m, tau_c[n] for column n. */
 float oracle_abft_decide_lines(int tm, int tn, const double* dr, const double* dc, const double* tau_r,
                                const double* tau_c, oracle_ft_status* st) {
     int nbr = 0, nbc = 0, r = -1, c = -1;
     double clean = 0.0;
-    for (int n = 0; n < tn; ++n) {
-        if (fabs(dc[n]) > tau_c[n]) { ++nbc; c = n; }
-        else if (fabs(dc[n]) > clean) clean = fabs(dc[n]);
-    }
-    /* the rows are looked at only when a column checksum disagrees (see the comment above) */
-    for (int m = 0; m < tm && nbc > 0; ++m) {
-        if (fabs(dr[m]) > tau_r[m]) { ++nbr; r = m; }
-        else if (fabs(dr[m]) > clean) clean = fabs(dr[m]);
+    if (g_rows_screen) {
+        for (int m = 0; m < tm; ++m) {
+            if (fabs(dr[m]) > tau_r[m]) { ++nbr; r = m; }
+            else if (fabs(dr[m]) > clean) clean = fabs(dr[m]);
+        }
+        for (int n = 0; n < tn && nbr > 0; ++n) {
+            if (fabs(dc[n]) > tau_c[n]) { ++nbc; c = n; }
+            else if (fabs(dc[n]) > clean) clean = fabs(dc[n]);
+        }
+    } else {
+        for (int n = 0; n < tn; ++n) {
+            if (fabs(dc[n]) > tau_c[n]) { ++nbc; c = n; }
+            else if (fabs(dc[n]) > clean) clean = fabs(dc[n]);
+        }
+        /* the rows are looked at only when a column checksum disagrees (see the comment above) */
+        for (int m = 0; m < tm && nbc > 0; ++m) {
+            if (fabs(dr[m]) > tau_r[m]) { ++nbr; r = m; }
+            else if (fabs(dr[m]) > clean) clean = fabs(dr[m]);
+        }
     }
     st->n_bad_rows = nbr;
     st->n_bad_cols = nbc;

@@ -487,7 +487,11 @@ def test_products_one_tile_wide_are_split_along_k_without_a_pre_pass(blas, oracl
             (c, st), (c2, st2) = results
             assert np.array_equal(c[:, :N], c2[:, :N]) and np.array_equal(st, st2)
             c_model = c0.copy()
-            st_model = oracle_mod.ft_sgemm(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, bm, bn, t, fault)
+            if ntn == 1:   # one tile wide: the rows are the screen (B is small, A is never summed)
+                with oracle_mod.rows_screen():
+                    st_model = oracle_mod.ft_sgemm(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, bm, bn, t, fault)
+            else:
+                st_model = oracle_mod.ft_sgemm(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.5, -1.0, bm, bn, t, fault)
             for f in DECISION_FIELDS:
                 assert np.array_equal(st[f], st_model[f]), (fault, t, f, st[f], st_model[f])
             ref, den = oracle_mod.gemm_f64_rows(M, N, K, a, K + 4, b, N + 4, c0, N + 8, 1.5, -1.0)
@@ -497,6 +501,51 @@ def test_products_one_tile_wide_are_split_along_k_without_a_pre_pass(blas, oracl
             dc = torch.from_numpy(c0).cuda()
             blas.ft_sgemm(M, N, K, da, db, dc, 1.5, -1.0, tau=t, fault=fault, tile_class=tile_class)
             assert not np.array_equal(dc.cpu().numpy()[:, :N], c[:, :N])
+
+
+def test_one_tile_wide_takes_the_rows_as_the_screen(blas, oracle_mod):
+    """Row x column location on a product one tile wide with a workspace: the row checksums (from the small B) are the
+    screen and the column references are formed only when a row is flagged.  Two faults that cancel in their row are
+    not seen (with the columns as the screen they would be two flagged columns: detected, not correctable); two faults
+    in one column show as two rows and one column; a single fault is located and corrected to the bits of the clean
+    product."""
+    M, N, K, tile_class = 8300, 60, 530, 3
+    bm, bn = blas.ft_tile(tile_class)
+    tau = blas.ft_default_tau(K)
+    a = oracle_mod.fill_uniform_matrix(M, K, 2300, ld=K + 4)
+    b = oracle_mod.fill_uniform_matrix(K, N, 2301, ld=N + 4)
+    c0 = oracle_mod.fill_uniform_matrix(M, N, 2302, ld=N + 8)
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    ws = torch.full((blas.ft_workspace_bytes(M, N, K) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+
+    def run(faults):
+        dc = torch.from_numpy(c0).cuda()
+        status = blas.ft_status_alloc(M, N, tile_class=tile_class)
+        blas.ft_sgemm(M, N, K, da, db, dc, 1.0, 0.0, tau=tau, faults=faults, status=status, ws=ws, tile_class=tile_class)
+        return dc.cpu().numpy(), blas.ft_status_numpy(status)
+
+    clean, st = run(None)
+    assert not st["flag"].any() and not st["n_bad_rows"].any() and not st["n_bad_cols"].any()
+    cases = {"cancel in a row": [(5, 7, 3, 2.0), (5, 7, 40, -2.0)], "one column": [(9, 7, 3, 2.0), (9, 90, 3, 1.0)],
+             "single": [(64, 100, 59, -0.5)], "last tile": [(-(-M // bm) - 1, M - (-(-M // bm) - 1) * bm - 1, N - 1, 3.0)]}
+    for name, faults in cases.items():
+        c, st = run(faults)
+        c_model = c0.copy()
+        with oracle_mod.rows_screen():
+            st_model = oracle_mod.ft_sgemm_checked(M, N, K, a, K + 4, b, N + 4, c_model, N + 8, 1.0, 0.0, bm, bn, tau, 0, faults)
+        for f in DECISION_FIELDS:
+            assert np.array_equal(st[f], st_model[f]), (name, f, st[f], st_model[f])
+        t = faults[0][0]
+        if name == "cancel in a row":
+            assert st["flag"][t] == 0 and st["n_bad_cols"][t] == 0
+            assert not np.array_equal(c[:, :N], clean[:, :N])      # both faults are still in C
+        elif name == "one column":
+            assert st["flag"][t] == 2 and (st["n_bad_rows"][t], st["n_bad_cols"][t]) == (2, 1)
+        else:
+            assert st["flag"][t] == 1 and (st["row"][t], st["col"][t]) == faults[0][1:3]
+            assert abs(st["col_residual"][t] + faults[0][3]) < 2e-3 and abs(st["row_residual"][t] + faults[0][3]) < 2e-3
+            assert np.array_equal(c[:, :N], clean[:, :N]), name
+        assert np.count_nonzero(st["flag"]) == (0 if name == "cancel in a row" else 1)
 
 
 def test_partial_last_round_is_split_along_k(blas, oracle_mod):
