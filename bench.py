@@ -464,8 +464,9 @@ def main() -> int:
             "ft_sgemm_gflops": round(2.0 * m * n_ * kk / ms_cls / 1e6, 1),
             "overhead_pct_vs_sgemm": round((ms_cls - ms_plain) / ms_plain * 100.0, 2),
             "class1_128x128_ft_sgemm_gflops": round(2.0 * m * n_ * kk / ms_c1 / 1e6, 1),
-            "note": "one tile wide: every workgroup forms its checksum vectors in its main loop (no second pass over A) and "
-                    "the tiles are split along K, two workgroups per CU",
+            "note": "one tile wide: the row checksums (a pre-pass over B only) are the screen, the column references are "
+                    "formed when a row is flagged, nothing of A is summed in the loop; the tiles are split along K, two "
+                    "workgroups per CU",
         }
         del a, b, c
 

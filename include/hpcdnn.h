@@ -73,12 +73,19 @@ typedef struct hpcdnn_fault {
  * threshold is clean, and its row checksums are not looked at (the reference
  * acts on a tile only when a column AND a row checksum disagree,
  * kernel/ft_sgemm/include/ft_sgemm_huge.cuh:289).  With a flagged column the
- * rows are thresholded too: one row x one column locates the element. */
+ * rows are thresholded too: one row x one column locates the element.
+ * The other way round on a product one tile wide (N <= the tile's columns,
+ * 32 tiles or more) that is given a workspace and verified once per tile:
+ * its B is small and its A is read exactly once, so the row checksums, which
+ * need sums over B only, screen, and the columns are looked at (and counted)
+ * only when a row is flagged.  Either way the side that is not the screen
+ * costs nothing until it is needed: its references are formed in the
+ * verification, from A and B. */
 typedef struct hpcdnn_ft_status {
     int32_t flag;             /* 0 clean; 1 single fault located and corrected; 2 detected, not correctable */
     int32_t row, col;         /* tile-local location of the corrected element, -1 if none */
     int32_t n_bad_rows;       /* lines whose |reference - observed| checksum residual exceeded the threshold */
-    int32_t n_bad_cols;       /* (rows are counted only when a column was flagged) */
+    int32_t n_bad_cols;       /* (the side that is not the screen is counted only when the screen flagged a line) */
     float row_residual;       /* signed residual of the located row (the size of the fault, negated), else 0 */
     float col_residual;       /* signed residual of the located column, else 0 */
     float max_clean_residual; /* largest |residual| among the lines looked at and judged clean */
