@@ -381,9 +381,12 @@ extern "C" int hpcdnn_ft_pick_class_ws(int M, int N, int K, size_t ws_bytes) {
         const FtClass& fc = kFtClasses[c];
         const int64_t tiles = hpcdnn_ft_num_tiles_ex(c, M, N);
         const int tiles_m = static_cast<int>(ceil_div(M, fc.bm)), tiles_n = static_cast<int>(ceil_div(N, fc.bn));
-        // as run_ft_sgemm decides: a product one tile wide or high splits every tile and forms the vectors in the loop
+        // as run_ft_sgemm decides: a product one tile wide or high splits every tile; one tile wide with a workspace it
+        // takes the rows as the screen (a pre-pass over B only, nothing of A summed in the loop), else it forms the
+        // vectors in the loop
         const bool one_wide = K > 0 && (tiles_m == 1 || tiles_n == 1) && tiles >= cus / 8;
         const size_t enc_bytes = ft_enc_bytes(fc, HPCDNN_FT_GRAN_TILE, M, N, K);
+        const bool rows_screen = one_wide && tiles_n == 1 && ws_bytes >= ft_weighted_enc_bytes(fc, N, K);
         const bool pre = !one_wide && K > 0 && ws_bytes >= enc_bytes;
         FtTail tail{1, 0, 0};
         if (one_wide) {
@@ -399,7 +402,11 @@ extern "C" int hpcdnn_ft_pick_class_ws(int M, int N, int K, size_t ws_bytes) {
             rounds = static_cast<double>((tiles - tail.tiles) / cus) + static_cast<double>(ceil_div(static_cast<int64_t>(tail.tiles) * tail.ways, cus)) / tail.ways + 0.06;
             groups = tiles - tail.tiles + static_cast<int64_t>(tail.tiles) * tail.ways;
         }
-        double cost = rounds * 2.0 * fc.bm * fc.bn * (K > 0 ? K : 1) / kPeakFlopsPerCu / (pre ? rel_eff[c] : rel_eff_fused[c]);
+        double cost = rounds * 2.0 * fc.bm * fc.bn * (K > 0 ? K : 1) / kPeakFlopsPerCu / (pre || rows_screen ? rel_eff[c] : rel_eff_fused[c]);
+        // the pre-pass reads the operands it sums once more (about 5.5 TB/s), which counts on a product with few columns
+        constexpr double kPrePassBytesPerSecond = 5.5e12;
+        if (pre) cost += 4.0 * (static_cast<double>(M) * K + static_cast<double>(K) * N) / kPrePassBytesPerSecond;
+        if (rows_screen) cost += 4.0 * static_cast<double>(K) * N / kPrePassBytesPerSecond;
         const double busy = static_cast<double>(groups < cus ? groups : cus);
         double resident = static_cast<double>(ceil_div(groups > 0 ? groups : 1, cus));
         if (resident > resident_max[c]) resident = resident_max[c];
@@ -408,7 +415,9 @@ extern "C" int hpcdnn_ft_pick_class_ws(int M, int N, int K, size_t ws_bytes) {
         const double stream_b = static_cast<double>(N) * K * kTrip / (in_flight * fc.bn);
         const double stream = stream_a > stream_b ? stream_a : stream_b;
         if (stream > cost) cost = stream;
-        if (cost < best_cost) { best_cost = cost; best = c; }
+        // (a smaller tile has to promise 2 % to be taken: below that the model cannot tell them apart, and fewer, larger
+        // check tiles mean fewer records)
+        if (cost < best_cost * 0.98) { best_cost = cost; best = c; }
     }
     return best;
 }
