@@ -55,6 +55,9 @@
  *     compositions of the pieces above and to closed forms (faults in
  *     different intervals are each located; a corrected fault leaves no trace
  *     in the later intervals).
+ *   oracle_abft_set_rows_screen (the decision rule with the sides
+ *     exchanged, for products one tile wide): pinned by that symmetry on
+ *     random residual patterns and by the patterns that tell the screens apart.
  *   oracle_abft_relative_thresholds (data-scaled thresholds, an addition
  *     with no reference counterpart): pinned to closed forms (constant and
  *     single-entry tiles) and to its scaling laws.  Bit-level

@@ -397,6 +397,36 @@ def test_decide_lines_uses_each_lines_own_threshold(oracle_mod):
     assert st_u == st_l and fix_u == fix_l
 
 
+def test_rows_as_the_screen_is_the_same_rule_with_the_sides_exchanged(oracle_mod):
+    """The rule for products one tile wide: rows first, columns only when a row is flagged.  Pinned by symmetry (the
+    decision on (dr, dc) with the rows as the screen is the decision on (dc, dr) with the columns as the screen, rows
+    and columns renamed) and by the patterns that tell the two screens apart."""
+    rng = np.random.default_rng(7)
+    for _ in range(200):
+        tm, tn = int(rng.integers(1, 7)), int(rng.integers(1, 7))
+        dr = np.where(rng.random(tm) < 0.25, rng.normal(size=tm), 0.0)
+        dc = np.where(rng.random(tn) < 0.25, rng.normal(size=tn), 0.0)
+        tau_r, tau_c = rng.uniform(0.05, 0.5, tm), rng.uniform(0.05, 0.5, tn)
+        with oracle_mod.rows_screen():
+            st, fix = oracle_mod.abft_decide_lines(dr, dc, tau_r, tau_c)
+        sw, _ = oracle_mod.abft_decide_lines(dc, dr, tau_c, tau_r)     # columns as the screen, sides exchanged
+        assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"], st["row"], st["col"]) == \
+               (sw["flag"], sw["n_bad_cols"], sw["n_bad_rows"], sw["col"], sw["row"])
+        assert st["max_clean_residual"] == sw["max_clean_residual"]
+        assert st["row_residual"] == sw["col_residual"] and st["col_residual"] == sw["row_residual"]
+        assert fix == st["row_residual"]
+    # a residual pattern in the columns only: unseen with the rows as the screen, "detected" with the columns
+    dr, dc, t = np.zeros(4), np.array([0.0, 1.0, -1.0]), np.full(4, 0.1)
+    with oracle_mod.rows_screen():
+        st, _ = oracle_mod.abft_decide_lines(dr, dc, t, t[:3])
+    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"], st["max_clean_residual"]) == (0, 0, 0, 0.0)
+    st, _ = oracle_mod.abft_decide_lines(dr, dc, t, t[:3])
+    assert (st["flag"], st["n_bad_rows"], st["n_bad_cols"]) == (2, 0, 2)
+    # and the selector does not outlive the block
+    st, _ = oracle_mod.abft_decide_lines(np.array([1.0, 0.0, 0.0, 0.0]), np.zeros(3), t, t[:3])
+    assert st["flag"] == 0
+
+
 def _numpy_relative_decision(acc, cr_ref, cc_ref, K):
     """The data-scaled decision of one tile composed in numpy: thresholds rel * sqrt(n) * max(line mean |acc|, tile
     mean |acc|) with rel = 2.56e-7 * sqrt(max(K, 64)), residual = reference - line sum, strict comparison."""
