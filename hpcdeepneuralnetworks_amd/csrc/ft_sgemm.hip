@@ -289,7 +289,9 @@ static int run_ft_sgemm(int M, int N, int K, const float* A, int lda, const floa
         } else {
             const EncodeFn encode = ft_encode(opt.tile_class, ta, wave);
             if (!encode) return HPCDNN_ERR_INVALID_VALUE;
-            hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + b_blocks)), dim3(kEncodeKB * 4), 0, s, M, N, K,
+            // (one checksum pair per workgroup tile: the kernels need the column sums of A only - the row sums of B are
+            // formed in a verification that has flagged a column - so the blocks of the B half are not launched)
+            hipLaunchKernelGGL(encode, dim3(k_blocks * (row_groups + (wave ? b_blocks : 0))), dim3(kEncodeKB * 4), 0, s, M, N, K,
                                A, lda, B, ldb, enc_a, enc_b, a.enc_ld, k_blocks, row_groups, col_groups);
         }
         rc = launch_status();
@@ -405,7 +407,7 @@ extern "C" int hpcdnn_ft_pick_class_ws(int M, int N, int K, size_t ws_bytes) {
         double cost = rounds * 2.0 * fc.bm * fc.bn * (K > 0 ? K : 1) / kPeakFlopsPerCu / (pre || rows_screen ? rel_eff[c] : rel_eff_fused[c]);
         // the pre-pass reads the operands it sums once more (about 5.5 TB/s), which counts on a product with few columns
         constexpr double kPrePassBytesPerSecond = 5.5e12;
-        if (pre) cost += 4.0 * (static_cast<double>(M) * K + static_cast<double>(K) * N) / kPrePassBytesPerSecond;
+        if (pre) cost += 4.0 * static_cast<double>(M) * K / kPrePassBytesPerSecond;  // (the workgroup-tile pre-pass reads A only)
         if (rows_screen) cost += 4.0 * static_cast<double>(K) * N / kPrePassBytesPerSecond;
         const double busy = static_cast<double>(groups < cus ? groups : cus);
         double resident = static_cast<double>(ceil_div(groups > 0 ? groups : 1, cus));

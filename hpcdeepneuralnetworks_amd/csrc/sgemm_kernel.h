@@ -278,6 +278,9 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
     // workspace or summed from B then) are formed when they are needed, by the whole workgroup, in the verification.
     // The weighted locator, whose screen is the plain row checksum, carries that one.
     constexpr bool kLazyRows = FT == 1 || FT == 2;
+    // ... and the row sums of B they need are formed then as well, unless there is one per wave column (wave-tile
+    // checksums: those come from the workspace): the pre-pass of the workgroup-tile kernels reads A only.
+    constexpr bool kRowSumsAtDetection = FT == 1 || (FT == 2 && GRAN == 0);
 
     extern __shared__ __align__(16) float smem[];
     float* const As = smem;
@@ -1264,10 +1267,11 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
         auto publish_row_refs = [&]() {
             if constexpr (kLazyRows) {
                 // Row references formed now: ref[gn][m] = sum over the k range done so far of A[m][k] * b_r[gn][k], FP64,
-                // b_r from the workspace or (FT == 1) summed here from B, 1024 values of k at a time, into the LDS the
+                // b_r summed here from B, 1024 values of k at a time (with wave-tile checksums: read from the workspace), into the LDS the
                 // column partials no longer need.  Only run when a column is flagged, so its cost (a pass over the tile's
                 // rows of A, and of B without a workspace, by one workgroup) is that of a detection, not of a product.
                 constexpr int kWaves = kGemmThreads / kWave;
+                constexpr bool kFromB = kRowSumsAtDetection;
                 constexpr int kChunk = 1024;
                 static_assert(sizeof(double) * GM * CCP * BN >= sizeof(float) * kChunk, "a chunk of row sums fits in the column partials' place");
                 float* const s_b = reinterpret_cast<float*>(s_ccref);
@@ -1275,8 +1279,8 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                 __syncthreads();
 #pragma unroll 1
                 for (int kc = k_first, ke = k_first; kc < kend; kc = ke) {
-                    ke = (FT == 1 && kend - kc > kChunk) ? kc + kChunk : kend;  // (with a workspace: one pass)
-                    if constexpr (FT == 1) {
+                    ke = (kFromB && kend - kc > kChunk) ? kc + kChunk : kend;  // (b_r from the workspace: one pass)
+                    if constexpr (kFromB) {
                         // b_r[k] over the tile's columns inside the matrix: a half wave per k row, eight rows in flight
                         constexpr int kHalfs = kGemmThreads / 32;
                         const int hw = tid >> 5, l32 = tid & 31;
@@ -1341,7 +1345,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                                 }
 #pragma unroll
                                 for (int gn = 0; gn < GN; ++gn) {
-                                    const v4f b = FT == 1 ? *reinterpret_cast<const v4f*>(s_b + (k - kc))
+                                    const v4f b = kFromB ? *reinterpret_cast<const v4f*>(s_b + (k - kc))
                                                           : *reinterpret_cast<const v4f*>(p.enc_b + (static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k);
                                     const double bx = static_cast<double>(b.x), by = static_cast<double>(b.y), bz = static_cast<double>(b.z), bw = static_cast<double>(b.w);
 #pragma unroll
@@ -1384,7 +1388,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                                     const int k = k0 + u < kb ? k0 + u : kb - 1;  // (past the part: a zero times a value that exists)
 #pragma unroll
                                     for (int gn = 0; gn < GN; ++gn) {
-                                        const float b = FT == 1 ? s_b[k - kc] : p.enc_b[(static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k];
+                                        const float b = kFromB ? s_b[k - kc] : p.enc_b[(static_cast<int64_t>(tile_n) * GN + gn) * p.enc_ld + k];
                                         sum[gn] += static_cast<double>(av[u]) * static_cast<double>(b);
                                     }
                                 }
@@ -1393,7 +1397,7 @@ __global__ __launch_bounds__(WGM * WGN * kWave, MIN_BLOCKS) void sgemm_kernel(co
                             for (int gn = 0; gn < GN; ++gn) s_crref[(gn * CRP + part) * BM + r] += sum[gn];
                         }
                     }
-                    if constexpr (FT == 1) __syncthreads();  // the next chunk's sums go where these were
+                    if constexpr (kFromB) __syncthreads();  // the next chunk's sums go where these were
                 }
                 return;
             }
