@@ -184,10 +184,13 @@ int hpcdnn_sgemm_row_split(int M, int N, int K, size_t ws_bytes, int* rows_first
  * hpcdnn_ft_num_tiles(M,N) records or NULL.
  * `ws`/`ws_bytes`: optional DEVICE scratch of
  * hpcdnn_workspace_bytes(HPCDNN_OP_FT_SGEMM,M,N,K) bytes, 16-byte aligned, no
- * initialisation needed.  With it the checksum vectors of A and B are formed
- * once per tile row / tile column by a small kernel ahead of the GEMM
- * (faster); with ws == NULL each workgroup forms them in its main loop, as the
- * reference does.  Detection, location and correction are the same in both.
+ * initialisation needed.  With it the checksum vector of A that the main loop
+ * needs (its column sums per tile row) is formed once by a small kernel ahead
+ * of the GEMM (faster); with ws == NULL each workgroup forms it in its main
+ * loop, as the reference does.  What only a tile with a flagged line needs -
+ * the row sums of B and the row references - is formed in that tile's
+ * verification, from A and B, either way.  Detection, location and correction
+ * are the same in both.
  * The size the query returns also has room for the K slices of a partial last
  * round of tiles: those tiles are then split along K, every slice verifying
  * and correcting its own partial product (the checksums are linear in K), and
